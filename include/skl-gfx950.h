@@ -1,0 +1,199 @@
+/*
+ * skl-gfx950.h - kernel entry points of the MI355X (gfx950) implementation of
+ * SKL's gemm / pack / cvt families.
+ *
+ * Every function keeps the parameter list of the SKL routine it stands in for
+ * (cited as `path:line` below the reference checkout) and only changes the
+ * ISA suffix of the name to `gfx950`: dimensions and strides are `size_t` in
+ * ELEMENTS, alpha and beta have C's element type, all functions return void,
+ * buffers are owned by the caller, C is always read (`C = alpha*A*B + beta*C`,
+ * and `C = beta*C` when k == 0), elements outside the addressed set are never
+ * written. Pointers may be all device-accessible (asynchronous launch on the
+ * current stream) or all ordinary host memory (staged, synchronous); see
+ * skl-hip.h. Errors are reported through skl_hip_last_error().
+ *
+ * 16-bit floating types are passed as 16-bit patterns; where the compiler
+ * knows `__bf16` / `_Float16` the typedefs below are those types, so the
+ * reference's callers compile unchanged.
+ */
+#ifndef SKL_GFX950_H
+#define SKL_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "skl-hip.h"
+
+#if defined(__clang__) || (defined(__GNUC__) && __GNUC__ >= 13)
+typedef __bf16 skl_bf16_t;
+typedef _Float16 skl_f16_t;
+#else
+typedef uint16_t skl_bf16_t;
+typedef uint16_t skl_f16_t;
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ======================================================================== */
+/* GEMM - full-stride forms (the reference's defining routines)              */
+/* ======================================================================== */
+
+/* ref/gemm/gemm_i8rc_i8rc_i32rc.h:45 (skl_gemm_i8rc_i8rc_i32rc_ref) */
+void skl_gemm_i8rc_i8rc_i32rc_gfx950(size_t m, size_t n, size_t k, int32_t alpha, const int8_t *a,
+                                     size_t rsa, size_t csa, const int8_t *b, size_t rsb, size_t csb,
+                                     int32_t beta, int32_t *c, size_t rsc, size_t csc);
+/* ref/gemm/gemm_bf16rc_bf16rc_f32rc.h:44 */
+void skl_gemm_bf16rc_bf16rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const skl_bf16_t *a,
+                                         size_t rsa, size_t csa, const skl_bf16_t *b, size_t rsb,
+                                         size_t csb, float beta, float *c, size_t rsc, size_t csc);
+/* ref/gemm/gemm_f16rc_f16rc_f32rc.h:44 */
+void skl_gemm_f16rc_f16rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const skl_f16_t *a,
+                                       size_t rsa, size_t csa, const skl_f16_t *b, size_t rsb, size_t csb,
+                                       float beta, float *c, size_t rsc, size_t csc);
+/* ref/gemm/gemm_f8e4m3rc_f8e4m3rc_f32rc.h:48 */
+void skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
+                                             size_t rsa, size_t csa, const uint8_t *b, size_t rsb,
+                                             size_t csb, float beta, float *c, size_t rsc, size_t csc);
+/* ref/gemm/gemm_f8e5m2rc_f8e5m2rc_f32rc.h:48 */
+void skl_gemm_f8e5m2rc_f8e5m2rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
+                                             size_t rsa, size_t csa, const uint8_t *b, size_t rsb,
+                                             size_t csb, float beta, float *c, size_t rsc, size_t csc);
+/* Mixed formats: A is E4M3, B is E5M2. The reference has no such routine; the
+ * argument list is that of ref/gemm/gemm_f8e4m3rc_f8e4m3rc_f32rc.h:48 and the
+ * result is that of decoding both operands (ref/cvt/cvt_ofp8.c:18-95) and
+ * calling ref/gemm/gemm_f32rc_f32rc_f32rc.h:44. */
+void skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
+                                             size_t rsa, size_t csa, const uint8_t *b, size_t rsb,
+                                             size_t csb, float beta, float *c, size_t rsc, size_t csc);
+
+/* Blocked ("rcprc") forms: element (I,i ; P,p) of A is at
+ * a[I*rsa1 + P*csa1 + i*rsa0 + p*csa0], likewise B (rows k) and C. */
+#define SKL_GFX950_DECLARE_RCPRC(NAME, TA, TC)                                                       \
+  void NAME(size_t m0, size_t n0, size_t k0, size_t m1, size_t n1, size_t k1, TC alpha, const TA *a, \
+            size_t rsa0, size_t csa0, size_t rsa1, size_t csa1, const TA *b, size_t rsb0,            \
+            size_t csb0, size_t rsb1, size_t csb1, TC beta, TC *c, size_t rsc0, size_t csc0,         \
+            size_t rsc1, size_t csc1)
+/* ref/gemm/gemm_i8rcprc_i8rcprc_i32rcprc.h:50 */
+SKL_GFX950_DECLARE_RCPRC(skl_gemm_i8rcprc_i8rcprc_i32rcprc_gfx950, int8_t, int32_t);
+/* ref/gemm/gemm_bf16rcprc_bf16rcprc_f32rcprc.h:49 */
+SKL_GFX950_DECLARE_RCPRC(skl_gemm_bf16rcprc_bf16rcprc_f32rcprc_gfx950, skl_bf16_t, float);
+/* ref/gemm/gemm_f16rcprc_f16rcprc_f32rcprc.h:49 */
+SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f32rcprc_gfx950, skl_f16_t, float);
+/* ref/gemm/gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc.h:53 */
+SKL_GFX950_DECLARE_RCPRC(skl_gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950, uint8_t, float);
+/* ref/gemm/gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc.h:53 */
+SKL_GFX950_DECLARE_RCPRC(skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, float);
+
+/* ======================================================================== */
+/* GEMM - the optimized entry points of skl.h                                */
+/* ======================================================================== */
+
+/* Row-major A, B, C. M == 1 is served by the streaming (GEMV) kernels.
+ * src/gemm/gemm_i8_i8_i32_zve32x.h:50, src/gemm/gemm_i8_i8_i32_zve32x_x390.h:50 */
+void skl_gemm_i8_i8_i32_gfx950(size_t m, size_t n, size_t k, int32_t alpha, const int8_t *a, size_t rsa,
+                               const int8_t *b, size_t rsb, int32_t beta, int32_t *c, size_t rsc);
+/* src/gemm/gemm_bf16_bf16_f32_zvfbfwma.h:49, src/gemm/gemm_bf16_bf16_f32_zvfbfwma_x390.h:49 */
+void skl_gemm_bf16_bf16_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const skl_bf16_t *a,
+                                   size_t rsa, const skl_bf16_t *b, size_t rsb, float beta, float *c,
+                                   size_t rsc);
+/* src/gemm/gemm_f16_f16_f32_zvfh.h:49, src/gemm/gemm_f16_f16_f32_zvfh_x390.h:49 */
+void skl_gemm_f16_f16_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const skl_f16_t *a, size_t rsa,
+                                 const skl_f16_t *b, size_t rsb, float beta, float *c, size_t rsc);
+
+/* Column-major A (= A^T stored row-major with row stride csa), row-major B, C.
+ * src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:57 */
+void skl_gemm_i8c_i8_i32_gfx950(size_t m, size_t n, size_t k, int32_t alpha, const int8_t *a, size_t csa,
+                                const int8_t *b, size_t rsb, int32_t beta, int32_t *c, size_t rsc);
+/* src/gemm/gemm_bf16c_bf16_f32_xsfmm32a16f.h:56 */
+void skl_gemm_bf16c_bf16_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const skl_bf16_t *a,
+                                    size_t csa, const skl_bf16_t *b, size_t rsb, float beta, float *c,
+                                    size_t rsc);
+/* src/gemm/gemm_f16c_f16_f32_xsfmm32a16f.h:56 */
+void skl_gemm_f16c_f16_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const skl_f16_t *a, size_t csa,
+                                  const skl_f16_t *b, size_t rsb, float beta, float *c, size_t rsc);
+/* src/gemm/gemm_f8e4m3c_f8e4m3_f32_xsfmm32a8f.h:57 */
+void skl_gemm_f8e4m3c_f8e4m3_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
+                                        size_t csa, const uint8_t *b, size_t rsb, float beta, float *c,
+                                        size_t rsc);
+/* src/gemm/gemm_f8e5m2c_f8e5m2_f32_xsfmm32a8f.h:57 */
+void skl_gemm_f8e5m2c_f8e5m2_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
+                                        size_t csa, const uint8_t *b, size_t rsb, float beta, float *c,
+                                        size_t rsc);
+
+/* Panel-packed operands, TE = skl_hip_te() = 64: A in TE x 1 column panels
+ * (m0 = TE, k0 = 1, rsa0 = 1), B in 1 x TE row panels (n0 = TE, csb0 = 1), C in
+ * TE x TE blocks with free strides. m1 / n1 count blocks.
+ * src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:97 */
+#define SKL_GFX950_DECLARE_PANEL(NAME, TA, TC)                                                        \
+  void NAME(size_t m1, size_t n1, size_t k, TC alpha, const TA *a, size_t rsa1, size_t csa1,          \
+            const TA *b, size_t rsb1, size_t csb1, TC beta, TC *c, size_t rsc0, size_t csc0,          \
+            size_t rsc1, size_t csc1)
+SKL_GFX950_DECLARE_PANEL(skl_gemm_i8rcptex1c_i8rcp1xte_i32rcptexterc_gfx950, int8_t, int32_t);
+/* src/gemm/gemm_bf16c_bf16_f32_xsfmm32a16f.h:97 */
+SKL_GFX950_DECLARE_PANEL(skl_gemm_bf16rcptex1c_bf16rcp1xte_f32rcptexterc_gfx950, skl_bf16_t, float);
+/* src/gemm/gemm_f16c_f16_f32_xsfmm32a16f.h:97 */
+SKL_GFX950_DECLARE_PANEL(skl_gemm_f16rcptex1c_f16rcp1xte_f32rcptexterc_gfx950, skl_f16_t, float);
+/* src/gemm/gemm_f8e4m3c_f8e4m3_f32_xsfmm32a8f.h:98 */
+SKL_GFX950_DECLARE_PANEL(skl_gemm_f8e4m3rcptex1c_f8e4m3rcp1xte_f32rcptexterc_gfx950, uint8_t, float);
+/* src/gemm/gemm_f8e5m2c_f8e5m2_f32_xsfmm32a8f.h:98 */
+SKL_GFX950_DECLARE_PANEL(skl_gemm_f8e5m2rcptex1c_f8e5m2rcp1xte_f32rcptexterc_gfx950, uint8_t, float);
+
+/* K-packed int8 ("dot4") layout: A in 1 x 4 K-blocks (A(i, 4P+p) at i*rsa1 +
+ * P*csa1 + p), B in 4 x 1 K-blocks (B(4P+p, j) at P*rsb1 + 4*j + p), C row-major.
+ * src/gemm/gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.h:70 */
+void skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(size_t m, size_t n, size_t k1, int32_t alpha, const int8_t *a,
+                                          size_t rsa1, size_t csa1, const int8_t *b, size_t rsb1,
+                                          int32_t beta, int32_t *c, size_t rsc);
+
+/* ======================================================================== */
+/* pack / unpack / transpose                                                 */
+/* ======================================================================== */
+
+#define SKL_GFX950_DECLARE_PACK(W, T)                                                                  \
+  /* ref/pack/pack_e8rc_e8rcprc.h:44 (+ e16, e32); src/pack/pack_e8_zve32x.h:49 */                     \
+  void skl_pack_e##W##rc_e##W##rcprc_gfx950(size_t m, size_t n, const T *src, size_t rs, size_t cs,    \
+                                            size_t m0, size_t n0, T *dst, size_t rs0, size_t cs0,      \
+                                            size_t rs1, size_t cs1, T pad);                            \
+  /* ref/pack/unpack_e8rcprc_e8rc.h:48; src/pack/pack_e8_zve32x.h:88. The reference ships the */      \
+  /* 8-bit width only; the wider ones apply the same rule to wider elements. */                       \
+  void skl_unpack_e##W##rcprc_e##W##rc_gfx950(size_t m0, size_t n0, const T *src, size_t rs0,          \
+                                              size_t cs0, size_t rs1, size_t cs1, size_t m, size_t n,  \
+                                              T *dst, size_t rs, size_t cs);                           \
+  /* ref/pack/transpose_e8.h:33 (+ e16, e32); src/pack/pack_e8_zve32x.h:112, */                        \
+  /* src/pack/pack_e8_xsfmmbase.h:38 */                                                                \
+  void skl_transpose_e##W##_gfx950(size_t m, size_t n, const T *a, size_t rsa, T *at, size_t rsat);    \
+  /* TE x 1 column panels of a row-major matrix: src/pack/pack_e16_xsfmmbase.h:49, */                  \
+  /* src/pack/pack_e32_xsfmmbase.h:49 (the reference has no 8-bit one). */                             \
+  void skl_pack_e##W##_e##W##rcptex1c_gfx950(size_t m, size_t n, const T *src, size_t rs, T *dst,      \
+                                             size_t rs1, size_t cs1, T pad);
+SKL_GFX950_DECLARE_PACK(8, uint8_t)
+SKL_GFX950_DECLARE_PACK(16, uint16_t)
+SKL_GFX950_DECLARE_PACK(32, uint32_t)
+
+/* ======================================================================== */
+/* OFP8 / OFP4 conversions: (dst, src, scale, n)                             */
+/* ======================================================================== */
+
+/* src/cvt/cvt_f32_f8_zvfofp8min.h:61,78,94,111; ref/cvt/cvt_ofp8.h:59-95 */
+void skl_cvt_f32_f8e4m3_gfx950(uint8_t *dst, const float *src, float scale, size_t n);
+void skl_cvt_sat_f32_f8e4m3_gfx950(uint8_t *dst, const float *src, float scale, size_t n);
+void skl_cvt_f32_f8e5m2_gfx950(uint8_t *dst, const float *src, float scale, size_t n);
+void skl_cvt_sat_f32_f8e5m2_gfx950(uint8_t *dst, const float *src, float scale, size_t n);
+/* src/cvt/cvt_bf16_f8_zvfofp8min_zvfbfmin.h:67,84,102,119; ref/cvt/cvt_ofp8.h:106-141 */
+void skl_cvt_bf16_f8e4m3_gfx950(uint8_t *dst, const skl_bf16_t *src, float scale, size_t n);
+void skl_cvt_sat_bf16_f8e4m3_gfx950(uint8_t *dst, const skl_bf16_t *src, float scale, size_t n);
+void skl_cvt_bf16_f8e5m2_gfx950(uint8_t *dst, const skl_bf16_t *src, float scale, size_t n);
+void skl_cvt_sat_bf16_f8e5m2_gfx950(uint8_t *dst, const skl_bf16_t *src, float scale, size_t n);
+/* src/cvt/cvt_f8_bf16_zvfofp8min.h:39,52; ref/cvt/cvt_ofp8.h:150,158 */
+void skl_cvt_f8e4m3_bf16_gfx950(skl_bf16_t *dst, const uint8_t *src, size_t n);
+void skl_cvt_f8e5m2_bf16_gfx950(skl_bf16_t *dst, const uint8_t *src, size_t n);
+/* src/cvt/cvt_f4_f8_zvfofp4min.h:54; ref/cvt/cvt_ofp4.h:30. Two E2M1 values per
+ * source byte, low nibble first. */
+void skl_cvt_f4e2m1_f8e4m3_gfx950(uint8_t *dst, const uint8_t *src, size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SKL_GFX950_H */

@@ -1,0 +1,92 @@
+/*
+ * skl-hip.h - runtime shim of the gfx950 SKL library.
+ *
+ * The SKL kernel entry points (skl-gfx950.h) keep the reference's `void`
+ * signatures and caller-owned buffers. Everything a C caller needs around
+ * them on a GPU - device selection, device buffers, the stream kernels are
+ * launched on, synchronisation and an error channel - is in this header.
+ * All functions have C linkage and take only plain pointers and integers.
+ *
+ * The reference has no counterpart for this header: SKL has no runtime
+ * (README.md:9-10 of the reference) because it runs on the calling hart.
+ *
+ * Pointer convention of every kernel entry point:
+ *   - all pointers are device-accessible (device, managed or pinned-host
+ *     allocations): the kernel is enqueued on the current stream and the call
+ *     returns without waiting;
+ *   - all pointers are ordinary host memory: operands are staged through
+ *     temporary device buffers and the call returns after the result has been
+ *     copied back (a literal drop-in for a CPU caller);
+ *   - a mix of both: nothing is done and SKL_HIP_ERR_MIXED_POINTERS is recorded.
+ */
+#ifndef SKL_HIP_H
+#define SKL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Error codes recorded by the library (HIP's own codes are passed through as
+ * positive numbers; the library's own are negative). */
+#define SKL_HIP_OK 0
+#define SKL_HIP_ERR_MIXED_POINTERS (-1)
+#define SKL_HIP_ERR_BAD_ARGUMENT (-2)
+#define SKL_HIP_ERR_NO_DEVICE (-3)
+#define SKL_HIP_ERR_WORKSPACE (-4)
+
+/* Pointer-classification modes for skl_hip_set_pointer_mode(). */
+#define SKL_HIP_POINTERS_AUTO 0   /* ask the HIP runtime about every pointer (default) */
+#define SKL_HIP_POINTERS_DEVICE 1 /* caller promises device-accessible pointers: no queries */
+
+/* Selects `device` for the calling thread and creates the library's
+ * per-device state (workspace for split reductions). Returns 0 or an error. */
+int skl_hip_init(int device);
+/* Releases every per-device workspace. Outstanding work is waited for. */
+void skl_hip_shutdown(void);
+
+void *skl_hip_malloc(size_t bytes);
+void skl_hip_free(void *ptr);
+int skl_hip_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int skl_hip_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int skl_hip_memcpy_d2d(void *dst, const void *src, size_t bytes);
+int skl_hip_memset(void *dst, int byte, size_t bytes);
+
+/* The stream (a hipStream_t passed as void*) kernels of the calling thread are
+ * enqueued on; NULL selects the default stream. */
+void skl_hip_set_stream(void *stream);
+void *skl_hip_get_stream(void);
+/* Waits for the current stream. */
+int skl_hip_synchronize(void);
+
+void skl_hip_set_pointer_mode(int mode);
+int skl_hip_get_pointer_mode(void);
+/* 1 if `ptr` is device-accessible, 0 if it is ordinary host memory. */
+int skl_hip_pointer_is_device(const void *ptr);
+
+/* Thread-local, sticky until read: the only error channel of the `void`
+ * kernel entry points. Reading clears it. */
+int skl_hip_last_error(void);
+const char *skl_hip_last_error_string(void);
+
+/* Edge of the square tile the packed ("ptex1c / p1xte / ptexte") layouts are
+ * counted in. The reference reads it from the matrix engine at run time and
+ * its tests assume 64; here it is the constant 64 for every element width. */
+size_t skl_hip_te(void);
+
+/* Timing helpers on the current stream (hipEvent_t as void*). */
+void *skl_hip_event_create(void);
+void skl_hip_event_destroy(void *event);
+int skl_hip_event_record(void *event);
+/* Waits for `stop`, returns milliseconds between the two events (negative on error). */
+float skl_hip_event_elapsed_ms(void *start, void *stop);
+
+/* Name and compute-unit count of the current device (for reports). */
+int skl_hip_device_info(char *name, size_t name_len, int *compute_units, int *clock_mhz);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SKL_HIP_H */

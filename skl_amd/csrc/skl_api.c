@@ -1,0 +1,434 @@
+/*
+ * skl_api.c - the C host layer of the gfx950 SKL library: the public entry
+ * points of include/skl-gfx950.h. Like the reference's public functions
+ * (src/gemm/README.md:84,113-131 - dispatchers over private kernels), each one
+ * only normalises its arguments into a descriptor, stages host buffers when
+ * the caller passed ordinary host memory, and picks the kernel family:
+ *
+ *   M == 1                          -> HBM-streaming GEMV kernels
+ *   16-byte aligned canonical form  -> matrix-core (MFMA) kernels
+ *   anything else                   -> any-stride kernel
+ *
+ * No HIP header is included here; the GPU is reached only through the C-ABI of
+ * skl_launch.h and skl-hip.h.
+ */
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+#include "../../include/skl-gfx950.h"
+#include "skl_launch.h"
+
+#define SKL_TE 64u
+
+/* ------------------------------------------------------------------------ */
+/* helpers                                                                   */
+/* ------------------------------------------------------------------------ */
+
+static size_t elem_size(int dt) { return (dt == SKL_DT_BF16 || dt == SKL_DT_F16) ? 2u : 1u; }
+
+/* Number of elements between the first and one past the last addressed element
+ * of a 4-level strided array; 0 if any extent is 0. */
+static size_t span4(size_t d0, size_t s0, size_t d1, size_t s1, size_t d2, size_t s2, size_t d3,
+                    size_t s3) {
+  if (d0 == 0 || d1 == 0 || d2 == 0 || d3 == 0) return 0;
+  return (d0 - 1) * s0 + (d1 - 1) * s1 + (d2 - 1) * s2 + (d3 - 1) * s3 + 1;
+}
+
+/* Classifies up to three pointers (NULL entries are skipped).
+ * Returns 1 all device, 0 all host, -1 mixed (error recorded). */
+static int classify(const void *p0, const void *p1, const void *p2, const char *who) {
+  const void *p[3];
+  int n = 0, dev = 0;
+  if (p0) p[n++] = p0;
+  if (p1) p[n++] = p1;
+  if (p2) p[n++] = p2;
+  if (skl_hip_get_pointer_mode() == SKL_HIP_POINTERS_DEVICE) return 1;
+  for (int i = 0; i < n; ++i) dev += skl_hip_pointer_is_device(p[i]) ? 1 : 0;
+  if (dev == n) return 1;
+  if (dev == 0) return 0;
+  skl_hip_record_error(SKL_HIP_ERR_MIXED_POINTERS, who);
+  return -1;
+}
+
+/* Device copy of a host span (NULL on failure or empty span). */
+static void *stage_in(const void *host, size_t bytes) {
+  void *d;
+  if (bytes == 0) return NULL;
+  d = skl_hip_malloc(bytes);
+  if (d && skl_hip_memcpy_h2d(d, host, bytes) != 0) {
+    skl_hip_free(d);
+    d = NULL;
+  }
+  return d;
+}
+
+/* ------------------------------------------------------------------------ */
+/* GEMM                                                                      */
+/* ------------------------------------------------------------------------ */
+
+/* Blocked-by-64 view of one blocked dimension (block size b0, count b1, inner
+ * stride s0, block stride s1): index x = X*b0 + x0 lives at X*s1 + x0*s0. */
+static int block64(size_t b0, size_t b1, size_t s0, size_t s1, size_t *o0, size_t *o1) {
+  if (b0 == SKL_TE) {
+    *o0 = s0;
+    *o1 = s1;
+  } else if (b0 == 1) {
+    *o0 = s1;
+    *o1 = SKL_TE * s1;
+  } else if (b1 == 1 || s1 == b0 * s0) {
+    *o0 = s0;
+    *o1 = SKL_TE * s0;
+  } else {
+    return 0;
+  }
+  return 1;
+}
+
+/* Flat view of the K dimension (block size k0, count k1). */
+static int flat_k(size_t k0, size_t k1, size_t s0, size_t s1, size_t *sk) {
+  if (k0 == 1)
+    *sk = s1;
+  else if (k1 == 1 || s1 == k0 * s0)
+    *sk = s0;
+  else
+    return 0;
+  return 1;
+}
+
+static int canonicalize(const skl_gemm_desc *d, skl_gemm_canon *g) {
+  g->ta = d->ta;
+  g->tb = d->tb;
+  g->m = d->m0 * d->m1;
+  g->n = d->n0 * d->n1;
+  g->k = d->k0 * d->k1;
+  g->a = d->a;
+  g->b = d->b;
+  g->c = d->c;
+  g->alpha = d->alpha;
+  g->beta = d->beta;
+  if (!flat_k(d->k0, d->k1, d->csa0, d->csa1, &g->a_sk)) return 0;
+  if (!flat_k(d->k0, d->k1, d->rsb0, d->rsb1, &g->b_sk)) return 0;
+  if (!block64(d->m0, d->m1, d->rsa0, d->rsa1, &g->a_s0, &g->a_s1)) return 0;
+  if (!block64(d->n0, d->n1, d->csb0, d->csb1, &g->b_s0, &g->b_s1)) return 0;
+  if (!block64(d->m0, d->m1, d->rsc0, d->rsc1, &g->rsc0, &g->rsc1)) return 0;
+  if (!block64(d->n0, d->n1, d->csc0, d->csc1, &g->csc0, &g->csc1)) return 0;
+  return 1;
+}
+
+/* The K4-interleaved int8 layout of the dot4 entry point, M == 1 only. */
+static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g) {
+  if (d->ta != SKL_DT_I8 || d->m0 * d->m1 != 1 || d->k0 != 4 || d->n0 != 1) return 0;
+  if (d->rsb0 != 1 || d->csb1 != 4 || d->csa0 != 1) return 0;
+  if (!(d->k1 == 1 || d->csa1 == 4)) return 0;
+  memset(g, 0, sizeof *g);
+  g->ta = g->tb = SKL_DT_I8;
+  g->m = 1;
+  g->n = d->n1;
+  g->k = 4 * d->k1;
+  g->a = d->a;
+  g->a_sk = 1;
+  g->b = d->b;
+  g->b_sk = d->rsb1; /* stride between groups of four k */
+  g->c = d->c;
+  g->csc0 = d->csc1;
+  g->csc1 = SKL_TE * d->csc1;
+  g->alpha = d->alpha;
+  g->beta = d->beta;
+  return 1;
+}
+
+static void gemm_on_device(const skl_gemm_desc *d) {
+  skl_gemm_canon g;
+  if (d->k0 * d->k1 != 0) {
+    if (canonicalize_k4(d, &g) && skl_hip_gemv_supported(&g, 1)) {
+      skl_hip_launch_gemv(&g, 1);
+      return;
+    }
+    if (canonicalize(d, &g)) {
+      if (g.m == 1 && skl_hip_gemv_supported(&g, 0)) {
+        skl_hip_launch_gemv(&g, 0);
+        return;
+      }
+      if (skl_hip_gemm_mfma_supported(&g)) {
+        skl_hip_launch_gemm_mfma(&g);
+        return;
+      }
+    }
+  }
+  skl_hip_launch_gemm_generic(d);
+}
+
+static void gemm_run(const skl_gemm_desc *d, const char *who) {
+  const size_t M = d->m0 * d->m1, N = d->n0 * d->n1, K = d->k0 * d->k1;
+  int where;
+  if (M == 0 || N == 0) return; /* nothing is addressed */
+  where = classify(K ? d->a : NULL, K ? d->b : NULL, d->c, who);
+  if (where < 0) return;
+  if (where == 1) {
+    gemm_on_device(d);
+    return;
+  }
+  {
+    /* Ordinary host memory: stage the addressed spans. C's whole span travels
+     * both ways, so elements in its stride gaps come back unchanged. */
+    const size_t esa = elem_size(d->ta), esb = elem_size(d->tb);
+    const size_t na = K ? span4(d->m1, d->rsa1, d->k1, d->csa1, d->m0, d->rsa0, d->k0, d->csa0) : 0;
+    const size_t nb = K ? span4(d->k1, d->rsb1, d->n1, d->csb1, d->k0, d->rsb0, d->n0, d->csb0) : 0;
+    const size_t nc = span4(d->m1, d->rsc1, d->n1, d->csc1, d->m0, d->rsc0, d->n0, d->csc0);
+    skl_gemm_desc dd = *d;
+    void *da = stage_in(d->a, na * esa), *db = stage_in(d->b, nb * esb), *dc = stage_in(d->c, nc * 4);
+    if ((na && !da) || (nb && !db) || !dc) {
+      skl_hip_free(da);
+      skl_hip_free(db);
+      skl_hip_free(dc);
+      return;
+    }
+    dd.a = da;
+    dd.b = db;
+    dd.c = dc;
+    gemm_on_device(&dd);
+    skl_hip_memcpy_d2h(d->c, dc, nc * 4);
+    skl_hip_free(da);
+    skl_hip_free(db);
+    skl_hip_free(dc);
+  }
+}
+
+#define SCALAR_i32(x) .i = (x)
+#define SCALAR_f32(x) .f = (x)
+
+/* strided (rc) form: one element per block */
+#define DEFINE_GEMM_RC(NAME, TA_T, TC_T, DTA, DTB, SC)                                             \
+  void NAME(size_t m, size_t n, size_t k, TC_T alpha, const TA_T *a, size_t rsa, size_t csa,       \
+            const TA_T *b, size_t rsb, size_t csb, TC_T beta, TC_T *c, size_t rsc, size_t csc) {   \
+    skl_gemm_desc d = {DTA, DTB, 1,   1,   1,   m,    n,    k,   a,    0, 0, rsa, csa,             \
+                       b,   0,   0,   rsb, csb, c,    0,    0,   rsc,  csc, {SC(alpha)}, {SC(beta)}}; \
+    gemm_run(&d, #NAME);                                                                           \
+  }
+
+DEFINE_GEMM_RC(skl_gemm_i8rc_i8rc_i32rc_gfx950, int8_t, int32_t, SKL_DT_I8, SKL_DT_I8, SCALAR_i32)
+DEFINE_GEMM_RC(skl_gemm_bf16rc_bf16rc_f32rc_gfx950, skl_bf16_t, float, SKL_DT_BF16, SKL_DT_BF16, SCALAR_f32)
+DEFINE_GEMM_RC(skl_gemm_f16rc_f16rc_f32rc_gfx950, skl_f16_t, float, SKL_DT_F16, SKL_DT_F16, SCALAR_f32)
+DEFINE_GEMM_RC(skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950, uint8_t, float, SKL_DT_F8E4M3, SKL_DT_F8E4M3, SCALAR_f32)
+DEFINE_GEMM_RC(skl_gemm_f8e5m2rc_f8e5m2rc_f32rc_gfx950, uint8_t, float, SKL_DT_F8E5M2, SKL_DT_F8E5M2, SCALAR_f32)
+DEFINE_GEMM_RC(skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950, uint8_t, float, SKL_DT_F8E4M3, SKL_DT_F8E5M2, SCALAR_f32)
+
+/* blocked (rcprc) form */
+#define DEFINE_GEMM_RCPRC(NAME, TA_T, TC_T, DT, SC)                                                \
+  void NAME(size_t m0, size_t n0, size_t k0, size_t m1, size_t n1, size_t k1, TC_T alpha,          \
+            const TA_T *a, size_t rsa0, size_t csa0, size_t rsa1, size_t csa1, const TA_T *b,      \
+            size_t rsb0, size_t csb0, size_t rsb1, size_t csb1, TC_T beta, TC_T *c, size_t rsc0,   \
+            size_t csc0, size_t rsc1, size_t csc1) {                                               \
+    skl_gemm_desc d = {DT,   DT,   m0,   n0,   k0,   m1,   n1,   k1,   a,    rsa0, csa0, rsa1, csa1, \
+                       b,    rsb0, csb0, rsb1, csb1, c,    rsc0, csc0, rsc1, csc1, {SC(alpha)},    \
+                       {SC(beta)}};                                                                \
+    gemm_run(&d, #NAME);                                                                           \
+  }
+
+DEFINE_GEMM_RCPRC(skl_gemm_i8rcprc_i8rcprc_i32rcprc_gfx950, int8_t, int32_t, SKL_DT_I8, SCALAR_i32)
+DEFINE_GEMM_RCPRC(skl_gemm_bf16rcprc_bf16rcprc_f32rcprc_gfx950, skl_bf16_t, float, SKL_DT_BF16, SCALAR_f32)
+DEFINE_GEMM_RCPRC(skl_gemm_f16rcprc_f16rcprc_f32rcprc_gfx950, skl_f16_t, float, SKL_DT_F16, SCALAR_f32)
+DEFINE_GEMM_RCPRC(skl_gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950, uint8_t, float, SKL_DT_F8E4M3, SCALAR_f32)
+DEFINE_GEMM_RCPRC(skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, float, SKL_DT_F8E5M2, SCALAR_f32)
+
+/* row-major A, B, C: the rc form with csa = csb = csc = 1
+ * (src/gemm/gemm_i8_i8_i32_zve32x.h:38-48) */
+#define DEFINE_GEMM_ROWMAJOR(NAME, RC, TA_T, TC_T)                                                 \
+  void NAME(size_t m, size_t n, size_t k, TC_T alpha, const TA_T *a, size_t rsa, const TA_T *b,    \
+            size_t rsb, TC_T beta, TC_T *c, size_t rsc) {                                          \
+    RC(m, n, k, alpha, a, rsa, 1, b, rsb, 1, beta, c, rsc, 1);                                     \
+  }
+DEFINE_GEMM_ROWMAJOR(skl_gemm_i8_i8_i32_gfx950, skl_gemm_i8rc_i8rc_i32rc_gfx950, int8_t, int32_t)
+DEFINE_GEMM_ROWMAJOR(skl_gemm_bf16_bf16_f32_gfx950, skl_gemm_bf16rc_bf16rc_f32rc_gfx950, skl_bf16_t, float)
+DEFINE_GEMM_ROWMAJOR(skl_gemm_f16_f16_f32_gfx950, skl_gemm_f16rc_f16rc_f32rc_gfx950, skl_f16_t, float)
+
+/* column-major A: the rc form with rsa = 1
+ * (src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:38-48) */
+#define DEFINE_GEMM_COLMAJOR_A(NAME, RC, TA_T, TC_T)                                               \
+  void NAME(size_t m, size_t n, size_t k, TC_T alpha, const TA_T *a, size_t csa, const TA_T *b,    \
+            size_t rsb, TC_T beta, TC_T *c, size_t rsc) {                                          \
+    RC(m, n, k, alpha, a, 1, csa, b, rsb, 1, beta, c, rsc, 1);                                     \
+  }
+DEFINE_GEMM_COLMAJOR_A(skl_gemm_i8c_i8_i32_gfx950, skl_gemm_i8rc_i8rc_i32rc_gfx950, int8_t, int32_t)
+DEFINE_GEMM_COLMAJOR_A(skl_gemm_bf16c_bf16_f32_gfx950, skl_gemm_bf16rc_bf16rc_f32rc_gfx950, skl_bf16_t, float)
+DEFINE_GEMM_COLMAJOR_A(skl_gemm_f16c_f16_f32_gfx950, skl_gemm_f16rc_f16rc_f32rc_gfx950, skl_f16_t, float)
+DEFINE_GEMM_COLMAJOR_A(skl_gemm_f8e4m3c_f8e4m3_f32_gfx950, skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950, uint8_t, float)
+DEFINE_GEMM_COLMAJOR_A(skl_gemm_f8e5m2c_f8e5m2_f32_gfx950, skl_gemm_f8e5m2rc_f8e5m2rc_f32rc_gfx950, uint8_t, float)
+
+/* panel-packed: the rcprc form with (m0, n0, k0) = (TE, TE, 1), rsa0 = 1, csb0 = 1
+ * (src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:85-95) */
+#define DEFINE_GEMM_PANEL(NAME, RCPRC, TA_T, TC_T)                                                 \
+  void NAME(size_t m1, size_t n1, size_t k, TC_T alpha, const TA_T *a, size_t rsa1, size_t csa1,   \
+            const TA_T *b, size_t rsb1, size_t csb1, TC_T beta, TC_T *c, size_t rsc0, size_t csc0, \
+            size_t rsc1, size_t csc1) {                                                            \
+    RCPRC(SKL_TE, SKL_TE, 1, m1, n1, k, alpha, a, 1, 0, rsa1, csa1, b, 0, 1, rsb1, csb1, beta, c,  \
+          rsc0, csc0, rsc1, csc1);                                                                 \
+  }
+DEFINE_GEMM_PANEL(skl_gemm_i8rcptex1c_i8rcp1xte_i32rcptexterc_gfx950, skl_gemm_i8rcprc_i8rcprc_i32rcprc_gfx950, int8_t, int32_t)
+DEFINE_GEMM_PANEL(skl_gemm_bf16rcptex1c_bf16rcp1xte_f32rcptexterc_gfx950, skl_gemm_bf16rcprc_bf16rcprc_f32rcprc_gfx950, skl_bf16_t, float)
+DEFINE_GEMM_PANEL(skl_gemm_f16rcptex1c_f16rcp1xte_f32rcptexterc_gfx950, skl_gemm_f16rcprc_f16rcprc_f32rcprc_gfx950, skl_f16_t, float)
+DEFINE_GEMM_PANEL(skl_gemm_f8e4m3rcptex1c_f8e4m3rcp1xte_f32rcptexterc_gfx950, skl_gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950, uint8_t, float)
+DEFINE_GEMM_PANEL(skl_gemm_f8e5m2rcptex1c_f8e5m2rcp1xte_f32rcptexterc_gfx950, skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, float)
+
+/* K-packed int8: the rcprc form with (m0, n0, k0) = (1, 1, 4)
+ * (src/gemm/gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.h:43-53) */
+void skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(size_t m, size_t n, size_t k1, int32_t alpha, const int8_t *a,
+                                          size_t rsa1, size_t csa1, const int8_t *b, size_t rsb1,
+                                          int32_t beta, int32_t *c, size_t rsc) {
+  skl_gemm_i8rcprc_i8rcprc_i32rcprc_gfx950(1, 1, 4, m, n, k1, alpha, a, 0, 1, rsa1, csa1, b, 1, 0, rsb1, 4,
+                                           beta, c, 0, 0, rsc, 1);
+}
+
+/* ------------------------------------------------------------------------ */
+/* pack / unpack / transpose                                                 */
+/* ------------------------------------------------------------------------ */
+
+static void pack_run(int esize, size_t m, size_t n, const void *src, size_t rs, size_t cs, size_t m0,
+                     size_t n0, void *dst, size_t rs0, size_t cs0, size_t rs1, size_t cs1, uint32_t pad,
+                     const char *who) {
+  int where;
+  if (m == 0 || n == 0 || m0 == 0 || n0 == 0) return;
+  where = classify(src, dst, NULL, who);
+  if (where < 0) return;
+  if (where == 1) {
+    skl_hip_launch_pack(esize, m, n, src, rs, cs, m0, n0, dst, rs0, cs0, rs1, cs1, pad);
+    return;
+  }
+  {
+    const size_t m1 = (m + m0 - 1) / m0, n1 = (n + n0 - 1) / n0;
+    const size_t ns = span4(m, rs, n, cs, 1, 0, 1, 0);
+    const size_t nd = span4(m1, rs1, n1, cs1, m0, rs0, n0, cs0);
+    void *ds = stage_in(src, ns * esize), *dd = stage_in(dst, nd * esize);
+    if (ds && dd) {
+      skl_hip_launch_pack(esize, m, n, ds, rs, cs, m0, n0, dd, rs0, cs0, rs1, cs1, pad);
+      skl_hip_memcpy_d2h(dst, dd, nd * esize);
+    }
+    skl_hip_free(ds);
+    skl_hip_free(dd);
+  }
+}
+
+static void unpack_run(int esize, size_t m0, size_t n0, const void *src, size_t rs0, size_t cs0,
+                       size_t rs1, size_t cs1, size_t m, size_t n, void *dst, size_t rs, size_t cs,
+                       const char *who) {
+  int where;
+  if (m == 0 || n == 0 || m0 == 0 || n0 == 0) return;
+  where = classify(src, dst, NULL, who);
+  if (where < 0) return;
+  if (where == 1) {
+    skl_hip_launch_unpack(esize, m0, n0, src, rs0, cs0, rs1, cs1, m, n, dst, rs, cs);
+    return;
+  }
+  {
+    /* Only the in-range part of the blocks is read: the last block row/column
+     * may be shorter than m0 / n0 in the caller's buffer. The address is a row
+     * term plus a column term; the farthest element maximises each. */
+    const size_t m1 = (m + m0 - 1) / m0, n1 = (n + n0 - 1) / n0;
+    const size_t lm = m - (m1 - 1) * m0, ln = n - (n1 - 1) * n0; /* extent of the last block */
+    size_t max_r = (m1 - 1) * rs1 + (lm - 1) * rs0, max_c = (n1 - 1) * cs1 + (ln - 1) * cs0;
+    size_t ns;
+    const size_t nd = span4(m, rs, n, cs, 1, 0, 1, 0);
+    void *ds, *dd;
+    if (m1 > 1 && (m1 - 2) * rs1 + (m0 - 1) * rs0 > max_r) max_r = (m1 - 2) * rs1 + (m0 - 1) * rs0;
+    if (n1 > 1 && (n1 - 2) * cs1 + (n0 - 1) * cs0 > max_c) max_c = (n1 - 2) * cs1 + (n0 - 1) * cs0;
+    ns = max_r + max_c + 1;
+    ds = stage_in(src, ns * esize);
+    dd = stage_in(dst, nd * esize);
+    if (ds && dd) {
+      skl_hip_launch_unpack(esize, m0, n0, ds, rs0, cs0, rs1, cs1, m, n, dd, rs, cs);
+      skl_hip_memcpy_d2h(dst, dd, nd * esize);
+    }
+    skl_hip_free(ds);
+    skl_hip_free(dd);
+  }
+}
+
+#define DEFINE_PACK_FAMILY(W, T, ES)                                                                 \
+  void skl_pack_e##W##rc_e##W##rcprc_gfx950(size_t m, size_t n, const T *src, size_t rs, size_t cs, \
+                                            size_t m0, size_t n0, T *dst, size_t rs0, size_t cs0,   \
+                                            size_t rs1, size_t cs1, T pad) {                        \
+    pack_run(ES, m, n, src, rs, cs, m0, n0, dst, rs0, cs0, rs1, cs1, (uint32_t)pad, __func__);      \
+  }                                                                                                  \
+  void skl_unpack_e##W##rcprc_e##W##rc_gfx950(size_t m0, size_t n0, const T *src, size_t rs0,       \
+                                              size_t cs0, size_t rs1, size_t cs1, size_t m,         \
+                                              size_t n, T *dst, size_t rs, size_t cs) {             \
+    unpack_run(ES, m0, n0, src, rs0, cs0, rs1, cs1, m, n, dst, rs, cs, __func__);                   \
+  }                                                                                                  \
+  /* One m x n block written with strides (1, rsat): src/transpose/README.md:3-9 */                 \
+  void skl_transpose_e##W##_gfx950(size_t m, size_t n, const T *a, size_t rsa, T *at, size_t rsat) { \
+    pack_run(ES, m, n, a, rsa, 1, m, n, at, 1, rsat, 0, 0, 0, __func__);                            \
+  }                                                                                                  \
+  /* src/pack/pack_e16_xsfmmbase.h:34-43 */                                                          \
+  void skl_pack_e##W##_e##W##rcptex1c_gfx950(size_t m, size_t n, const T *src, size_t rs, T *dst,   \
+                                             size_t rs1, size_t cs1, T pad) {                       \
+    pack_run(ES, m, n, src, rs, 1, SKL_TE, 1, dst, 1, 0, rs1, cs1, (uint32_t)pad, __func__);        \
+  }
+DEFINE_PACK_FAMILY(8, uint8_t, 1)
+DEFINE_PACK_FAMILY(16, uint16_t, 2)
+DEFINE_PACK_FAMILY(32, uint32_t, 4)
+
+/* ------------------------------------------------------------------------ */
+/* cvt                                                                       */
+/* ------------------------------------------------------------------------ */
+
+/* kind: 0 f32->f8, 1 bf16->f8, 2 f8->bf16, 3 f4->f8e4m3 */
+static void cvt_run(int kind, int fmt, int sat, void *dst, const void *src, float scale, size_t n,
+                    const char *who) {
+  static const size_t src_num[4] = {4, 2, 1, 1}, dst_size[4] = {1, 1, 2, 1};
+  int where;
+  void *ds = NULL, *dd = NULL;
+  void *d = dst;
+  const void *s = src;
+  size_t src_bytes, dst_bytes;
+  if (n == 0) return;
+  where = classify(src, dst, NULL, who);
+  if (where < 0) return;
+  src_bytes = kind == 3 ? (n + 1) / 2 : n * src_num[kind];
+  dst_bytes = n * dst_size[kind];
+  if (where == 0) {
+    ds = stage_in(src, src_bytes);
+    dd = skl_hip_malloc(dst_bytes);
+    if (!ds || !dd) {
+      skl_hip_free(ds);
+      skl_hip_free(dd);
+      return;
+    }
+    d = dd;
+    s = ds;
+  }
+  switch (kind) {
+    case 0: skl_hip_launch_cvt_f32_f8(fmt, sat, (uint8_t *)d, (const float *)s, scale, n); break;
+    case 1: skl_hip_launch_cvt_bf16_f8(fmt, sat, (uint8_t *)d, (const uint16_t *)s, scale, n); break;
+    case 2: skl_hip_launch_cvt_f8_bf16(fmt, (uint16_t *)d, (const uint8_t *)s, n); break;
+    default: skl_hip_launch_cvt_f4_f8e4m3((uint8_t *)d, (const uint8_t *)s, n); break;
+  }
+  if (where == 0) {
+    skl_hip_memcpy_d2h(dst, dd, dst_bytes);
+    skl_hip_free(ds);
+    skl_hip_free(dd);
+  }
+}
+
+#define DEFINE_CVT_TO_F8(NAME, SRC_T, KIND, FMT, SAT)                               \
+  void NAME(uint8_t *dst, const SRC_T *src, float scale, size_t n) {                \
+    cvt_run(KIND, FMT, SAT, dst, src, scale, n, #NAME);                             \
+  }
+DEFINE_CVT_TO_F8(skl_cvt_f32_f8e4m3_gfx950, float, 0, SKL_DT_F8E4M3, 0)
+DEFINE_CVT_TO_F8(skl_cvt_sat_f32_f8e4m3_gfx950, float, 0, SKL_DT_F8E4M3, 1)
+DEFINE_CVT_TO_F8(skl_cvt_f32_f8e5m2_gfx950, float, 0, SKL_DT_F8E5M2, 0)
+DEFINE_CVT_TO_F8(skl_cvt_sat_f32_f8e5m2_gfx950, float, 0, SKL_DT_F8E5M2, 1)
+DEFINE_CVT_TO_F8(skl_cvt_bf16_f8e4m3_gfx950, skl_bf16_t, 1, SKL_DT_F8E4M3, 0)
+DEFINE_CVT_TO_F8(skl_cvt_sat_bf16_f8e4m3_gfx950, skl_bf16_t, 1, SKL_DT_F8E4M3, 1)
+DEFINE_CVT_TO_F8(skl_cvt_bf16_f8e5m2_gfx950, skl_bf16_t, 1, SKL_DT_F8E5M2, 0)
+DEFINE_CVT_TO_F8(skl_cvt_sat_bf16_f8e5m2_gfx950, skl_bf16_t, 1, SKL_DT_F8E5M2, 1)
+
+void skl_cvt_f8e4m3_bf16_gfx950(skl_bf16_t *dst, const uint8_t *src, size_t n) {
+  cvt_run(2, SKL_DT_F8E4M3, 0, dst, src, 1.0f, n, __func__);
+}
+void skl_cvt_f8e5m2_bf16_gfx950(skl_bf16_t *dst, const uint8_t *src, size_t n) {
+  cvt_run(2, SKL_DT_F8E5M2, 0, dst, src, 1.0f, n, __func__);
+}
+void skl_cvt_f4e2m1_f8e4m3_gfx950(uint8_t *dst, const uint8_t *src, size_t n) {
+  cvt_run(3, SKL_DT_F8E4M3, 0, dst, src, 1.0f, n, __func__);
+}

@@ -1,0 +1,72 @@
+// skl_fp8.hpp - OFP8 (E4M3 / E5M2) encode and decode on fp32 bit patterns,
+// shared by the conversion kernels and the scalar-path GEMM.
+//
+// Encode follows ref/cvt/cvt_ofp8.c:97-172 (round to nearest even, gradual
+// underflow, NaN -> 0x7F, overflow -> the format's overflow byte); decode
+// follows ref/cvt/cvt_ofp8.c:18-95 (NaN codes give the sign-less quiet NaN).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace skl_fp8 {
+
+struct E4M3 {
+  static constexpr int kMant = 3, kBias = 7, kEmin = -6;
+  static constexpr unsigned kMax = 0x7E;
+  __device__ static unsigned overflow(unsigned sign, bool sat) { return sat ? (sign | 0x7Eu) : 0x7Fu; }
+};
+struct E5M2 {
+  static constexpr int kMant = 2, kBias = 15, kEmin = -14;
+  static constexpr unsigned kMax = 0x7B;
+  __device__ static unsigned overflow(unsigned sign, bool sat) { return sign | (sat ? 0x7Bu : 0x7Cu); }
+};
+
+// fp32 bit pattern -> OFP8 byte, round to nearest even.
+template <class F>
+__device__ __forceinline__ unsigned encode_ofp8(unsigned bits, bool sat) {
+  const unsigned sign = (bits >> 24) & 0x80u;
+  const unsigned mag32 = bits & 0x7FFFFFFFu;
+  if (mag32 > 0x7F800000u) return 0x7Fu;                  // NaN
+  if (mag32 == 0x7F800000u) return F::overflow(sign, sat);  // +-inf
+  int e = (int)(mag32 >> 23) - 127;
+  unsigned sig = (mag32 & 0x7FFFFFu) | 0x800000u;
+  if ((mag32 >> 23) == 0) {  // fp32 subnormal: no hidden bit
+    e = -126;
+    sig = mag32;
+  }
+  const int te = e > F::kEmin ? e : F::kEmin;  // exponent of the target's quantum
+  int shift = (te - F::kMant) - (e - 23);      // low bits of sig that are dropped (> 0)
+  if (shift > 31) shift = 31;                  // sig < 2^24: everything rounds to 0
+  unsigned q = sig >> shift;
+  const unsigned rem = sig & ((1u << shift) - 1u);
+  const unsigned half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (q & 1u))) ++q;
+  // Adding q (which carries the hidden bit for normals) to the exponent field
+  // lets a mantissa carry bump the exponent and a subnormal round up to the
+  // smallest normal.
+  const unsigned mag = (e < F::kEmin) ? q : ((unsigned)(te + F::kBias - 1) << F::kMant) + q;
+  if (mag > F::kMax) return F::overflow(sign, sat);
+  return sign | mag;
+}
+
+// OFP8 byte -> fp32 bit pattern. NaN codes give the sign-less quiet NaN.
+template <class F>
+__device__ __forceinline__ unsigned decode_ofp8_bits(unsigned code) {
+  const unsigned sign = (code & 0x80u) << 24;
+  const unsigned e = (code & 0x7Fu) >> F::kMant;
+  const unsigned m = code & ((1u << F::kMant) - 1u);
+  constexpr unsigned emax = (1u << (7 - F::kMant)) - 1u;
+  if (F::kMant == 3) {
+    if ((code & 0x7Fu) == 0x7Fu) return 0x7FC00000u;
+  } else if (e == emax) {
+    return m ? 0x7FC00000u : (sign | 0x7F800000u);
+  }
+  if (e == 0) {
+    // m * 2^(emin - mant): exact in fp32
+    float v = (float)m * __uint_as_float((unsigned)(127 + F::kEmin - F::kMant) << 23);
+    return sign | __float_as_uint(v);
+  }
+  return sign | ((e + 127u - (unsigned)F::kBias) << 23) | (m << (23 - F::kMant));
+}
+
+}  // namespace skl_fp8

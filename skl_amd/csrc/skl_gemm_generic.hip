@@ -1,0 +1,122 @@
+// skl_gemm_generic.hip - the any-stride GEMM of the library: serves every call
+// the matrix-core and streaming kernels decline (odd strides, misaligned bases,
+// blocked layouts with k0 > 1, tiny shapes).
+//
+// It evaluates exactly the loop nest of the reference's blocked routine
+// (ref/gemm/gemm_i8rcprc_i8rcprc_i32rcprc.c:10-37 and its typed twins): one
+// thread per element of C, accumulator of C's type starting at zero, k1 outer
+// and k0 inner, products of the widened operands, then C = beta*C + alpha*acc
+// with C always read. Because every bf16/f16/fp8 product is exact in fp32 the
+// fused multiply-add used for the accumulation rounds exactly like the
+// reference's separate multiply and add, and the epilogue is kept as two
+// roundings, so for finite data the fp results are bit-identical to the
+// reference's, not merely within tolerance.
+#include <hip/hip_runtime.h>
+
+#include "skl_device.hpp"
+#include "skl_fp8.hpp"
+
+namespace {
+
+template <int DT>
+struct Elem;
+template <>
+struct Elem<SKL_DT_I8> {
+  using type = int8_t;
+  using acc = int32_t;
+  __device__ static acc widen(type v) { return (acc)v; }
+};
+template <>
+struct Elem<SKL_DT_BF16> {
+  using type = uint16_t;
+  using acc = float;
+  __device__ static acc widen(type v) { return __uint_as_float((unsigned)v << 16); }
+};
+template <>
+struct Elem<SKL_DT_F16> {
+  using type = _Float16;
+  using acc = float;
+  __device__ static acc widen(type v) { return (float)v; }
+};
+template <>
+struct Elem<SKL_DT_F8E4M3> {
+  using type = uint8_t;
+  using acc = float;
+  __device__ static acc widen(type v) { return __uint_as_float(skl_fp8::decode_ofp8_bits<skl_fp8::E4M3>(v)); }
+};
+template <>
+struct Elem<SKL_DT_F8E5M2> {
+  using type = uint8_t;
+  using acc = float;
+  __device__ static acc widen(type v) { return __uint_as_float(skl_fp8::decode_ofp8_bits<skl_fp8::E5M2>(v)); }
+};
+
+__device__ __forceinline__ int32_t axpby(int32_t alpha, int32_t acc, int32_t beta, int32_t c) {
+  return (int32_t)((uint32_t)beta * (uint32_t)c + (uint32_t)alpha * (uint32_t)acc);  // wraps like -fwrapv
+}
+__device__ __forceinline__ float axpby(float alpha, float acc, float beta, float c) {
+  return __fadd_rn(__fmul_rn(beta, c), __fmul_rn(alpha, acc));
+}
+
+template <int TA, int TB>
+__global__ void __launch_bounds__(256) gemm_generic_kernel(skl_gemm_desc d, unsigned tiles_n) {
+  using EA = Elem<TA>;
+  using EB = Elem<TB>;
+  using Acc = typename EA::acc;
+  const size_t M = d.m1 * d.m0, N = d.n1 * d.n0;
+  const size_t tile_i = blockIdx.x / tiles_n, tile_j = blockIdx.x % tiles_n;
+  const size_t i = tile_i * 16 + threadIdx.x / 16, j = tile_j * 16 + threadIdx.x % 16;
+  if (i >= M || j >= N) return;
+  const size_t I = i / d.m0, i0 = i % d.m0, J = j / d.n0, j0 = j % d.n0;
+  const typename EA::type *a = (const typename EA::type *)d.a + I * d.rsa1 + i0 * d.rsa0;
+  const typename EB::type *b = (const typename EB::type *)d.b + J * d.csb1 + j0 * d.csb0;
+  Acc acc = 0;
+  for (size_t P = 0; P < d.k1; ++P) {
+    const typename EA::type *ap = a + P * d.csa1;
+    const typename EB::type *bp = b + P * d.rsb1;
+    for (size_t p = 0; p < d.k0; ++p) {
+      const Acc av = EA::widen(ap[p * d.csa0]);
+      const Acc bv = EB::widen(bp[p * d.rsb0]);
+      if constexpr (TA == SKL_DT_I8)
+        acc = (Acc)((uint32_t)acc + (uint32_t)av * (uint32_t)bv);
+      else
+        acc = __fmaf_rn(av, bv, acc);
+    }
+  }
+  Acc *c = (Acc *)d.c + I * d.rsc1 + J * d.csc1 + i0 * d.rsc0 + j0 * d.csc0;
+  if constexpr (TA == SKL_DT_I8)
+    *c = axpby(d.alpha.i, acc, d.beta.i, *c);
+  else
+    *c = axpby(d.alpha.f, acc, d.beta.f, *c);
+}
+
+template <int TA, int TB>
+int launch(const skl_gemm_desc &d) {
+  const size_t M = d.m1 * d.m0, N = d.n1 * d.n0;
+  const size_t tm = (M + 15) / 16, tn = (N + 15) / 16;
+  if (tm * tn > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemm: too many tiles for one launch");
+    return -2;
+  }
+  gemm_generic_kernel<TA, TB><<<(unsigned)(tm * tn), 256, 0, skl_current_stream()>>>(d, (unsigned)tn);
+  return skl_check_launch("gemm_generic");
+}
+
+}  // namespace
+
+extern "C" int skl_hip_launch_gemm_generic(const skl_gemm_desc *d) {
+  if (d->m0 * d->m1 == 0 || d->n0 * d->n1 == 0) return 0;
+  const int key = d->ta * 8 + d->tb;
+  switch (key) {
+    case SKL_DT_I8 * 8 + SKL_DT_I8: return launch<SKL_DT_I8, SKL_DT_I8>(*d);
+    case SKL_DT_BF16 * 8 + SKL_DT_BF16: return launch<SKL_DT_BF16, SKL_DT_BF16>(*d);
+    case SKL_DT_F16 * 8 + SKL_DT_F16: return launch<SKL_DT_F16, SKL_DT_F16>(*d);
+    case SKL_DT_F8E4M3 * 8 + SKL_DT_F8E4M3: return launch<SKL_DT_F8E4M3, SKL_DT_F8E4M3>(*d);
+    case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E5M2: return launch<SKL_DT_F8E5M2, SKL_DT_F8E5M2>(*d);
+    case SKL_DT_F8E4M3 * 8 + SKL_DT_F8E5M2: return launch<SKL_DT_F8E4M3, SKL_DT_F8E5M2>(*d);
+    case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E4M3: return launch<SKL_DT_F8E5M2, SKL_DT_F8E4M3>(*d);
+    default:
+      skl_hip_record_error(-2, "gemm: operand type pair");
+      return -2;
+  }
+}

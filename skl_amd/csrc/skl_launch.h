@@ -1,0 +1,100 @@
+/*
+ * skl_launch.h - internal C-ABI between the C host layer (skl_api.c) and the
+ * HIP translation units. The host layer validates arguments, stages host
+ * buffers and decides which kernel family serves a call; the functions below
+ * compute grids and enqueue kernels on the calling thread's current stream.
+ * Every pointer handed to these functions is device-accessible.
+ *
+ * All launchers return 0 or an error code that has also been recorded for
+ * skl_hip_last_error().
+ */
+#ifndef SKL_LAUNCH_H
+#define SKL_LAUNCH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element kinds of GEMM operands. */
+enum {
+  SKL_DT_I8 = 0,
+  SKL_DT_BF16 = 1,
+  SKL_DT_F16 = 2,
+  SKL_DT_F8E4M3 = 3,
+  SKL_DT_F8E5M2 = 4
+};
+
+typedef union {
+  int32_t i;
+  float f;
+} skl_scalar;
+
+/* The fully general blocked GEMM of the reference (the `rcprc` form): element
+ * (I,i ; P,p) of A is at a + I*rsa1 + P*csa1 + i*rsa0 + p*csa0, and likewise
+ * for B (rows = k, columns = n) and C. Strides are in elements. */
+typedef struct {
+  int ta, tb; /* element kind of A and B; C is int32 for SKL_DT_I8, else f32 */
+  size_t m0, n0, k0, m1, n1, k1;
+  const void *a;
+  size_t rsa0, csa0, rsa1, csa1;
+  const void *b;
+  size_t rsb0, csb0, rsb1, csb1;
+  void *c;
+  size_t rsc0, csc0, rsc1, csc1;
+  skl_scalar alpha, beta;
+} skl_gemm_desc;
+
+/* Canonical form served by the matrix-core kernels: flat in K, blocked by 64
+ * in M and N. A(i,p) = a[(i/64)*a_s1 + (i%64)*a_s0 + p*a_sk] with exactly one of
+ * a_s0 / a_sk equal to 1; B(p,j) = b[(j/64)*b_s1 + (j%64)*b_s0 + p*b_sk]
+ * likewise; C(i,j) = c[(i/64)*rsc1 + (i%64)*rsc0 + (j/64)*csc1 + (j%64)*csc0]. */
+typedef struct {
+  int ta, tb;
+  size_t m, n, k;
+  const void *a;
+  size_t a_s1, a_s0, a_sk;
+  const void *b;
+  size_t b_s1, b_s0, b_sk;
+  void *c;
+  size_t rsc0, csc0, rsc1, csc1;
+  skl_scalar alpha, beta;
+} skl_gemm_canon;
+
+int skl_hip_launch_gemm_generic(const skl_gemm_desc *d);
+/* Returns 1 if the canonical problem meets the matrix-core kernels' alignment
+ * rules (16-byte aligned bases and strides along the non-unit dimensions). */
+int skl_hip_gemm_mfma_supported(const skl_gemm_canon *g);
+int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g);
+
+/* M == 1 streaming kernels: y[j*csc] = beta*y + alpha * sum_p x[p*x_sk] * B(p,j).
+ * `layout`: 0 = B row-major (b_s0 == 1 within 64-blocks), 1 = K4-interleaved
+ * int8 (`p4x1c`: B(p,j) at (p/4)*b_sk + j*4 + p%4). */
+int skl_hip_gemv_supported(const skl_gemm_canon *g, int layout);
+int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout);
+
+/* pack / unpack over elements of `esize` bytes (1, 2 or 4). */
+int skl_hip_launch_pack(int esize, size_t m, size_t n, const void *src, size_t rs, size_t cs,
+                        size_t m0, size_t n0, void *dst, size_t rs0, size_t cs0, size_t rs1,
+                        size_t cs1, uint32_t pad);
+int skl_hip_launch_unpack(int esize, size_t m0, size_t n0, const void *src, size_t rs0,
+                          size_t cs0, size_t rs1, size_t cs1, size_t m, size_t n, void *dst,
+                          size_t rs, size_t cs);
+
+/* OFP8 / OFP4 conversions. `fmt`: SKL_DT_F8E4M3 or SKL_DT_F8E5M2. */
+int skl_hip_launch_cvt_f32_f8(int fmt, int saturate, uint8_t *dst, const float *src, float scale,
+                              size_t n);
+int skl_hip_launch_cvt_bf16_f8(int fmt, int saturate, uint8_t *dst, const uint16_t *src,
+                               float scale, size_t n);
+int skl_hip_launch_cvt_f8_bf16(int fmt, uint16_t *dst, const uint8_t *src, size_t n);
+int skl_hip_launch_cvt_f4_f8e4m3(uint8_t *dst, const uint8_t *src, size_t n);
+
+/* Error recording shared by both layers. */
+void skl_hip_record_error(int code, const char *what);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SKL_LAUNCH_H */

@@ -1,0 +1,216 @@
+// skl_runtime.hip - the runtime shim declared in include/skl-hip.h: device
+// selection, buffers, the per-thread stream, pointer classification and the
+// thread-local error channel of the `void` kernel entry points.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+#include "../../include/skl-hip.h"
+#include "skl_device.hpp"
+
+namespace {
+
+constexpr int kMaxDevices = 16;
+
+struct DeviceState {
+  void *workspace = nullptr;
+  size_t workspace_bytes = 0;
+};
+
+std::mutex g_mutex;
+DeviceState g_devices[kMaxDevices];
+
+thread_local hipStream_t t_stream = nullptr;
+thread_local int t_pointer_mode = SKL_HIP_POINTERS_AUTO;
+thread_local int t_error = SKL_HIP_OK;
+thread_local char t_error_text[256] = "no error";
+
+}  // namespace
+
+extern "C" void skl_hip_record_error(int code, const char *what) {
+  if (code == SKL_HIP_OK || t_error != SKL_HIP_OK) return;  // keep the first error until it is read
+  t_error = code;
+  const char *detail = "";
+  if (code > 0) detail = hipGetErrorString((hipError_t)code);
+  else if (code == SKL_HIP_ERR_MIXED_POINTERS) detail = "host and device pointers mixed in one call";
+  else if (code == SKL_HIP_ERR_BAD_ARGUMENT) detail = "bad argument";
+  else if (code == SKL_HIP_ERR_NO_DEVICE) detail = "no usable GPU";
+  else if (code == SKL_HIP_ERR_WORKSPACE) detail = "workspace allocation failed";
+  snprintf(t_error_text, sizeof t_error_text, "%s: %s", what ? what : "skl", detail);
+}
+
+int skl_check_hip(hipError_t e, const char *what) {
+  if (e == hipSuccess) return SKL_HIP_OK;
+  skl_hip_record_error((int)e, what);
+  return (int)e;
+}
+
+hipStream_t skl_current_stream() { return t_stream; }
+
+void *skl_workspace(size_t bytes) {
+  int dev = 0;
+  if (skl_check_hip(hipGetDevice(&dev), "hipGetDevice") != 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  DeviceState &st = g_devices[dev];
+  if (st.workspace_bytes >= bytes) return st.workspace;
+  if (st.workspace) {
+    // Earlier launches may still read the old block.
+    if (skl_check_hip(hipDeviceSynchronize(), "workspace grow: synchronize") != 0) return nullptr;
+    (void)hipFree(st.workspace);
+    st.workspace = nullptr;
+    st.workspace_bytes = 0;
+  }
+  size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes;
+  void *p = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess) {
+    (void)hipGetLastError();
+    skl_hip_record_error(SKL_HIP_ERR_WORKSPACE, "skl_workspace");
+    return nullptr;
+  }
+  st.workspace = p;
+  st.workspace_bytes = want;
+  return p;
+}
+
+extern "C" {
+
+int skl_hip_init(int device) {
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+    (void)hipGetLastError();
+    skl_hip_record_error(SKL_HIP_ERR_NO_DEVICE, "skl_hip_init");
+    return SKL_HIP_ERR_NO_DEVICE;
+  }
+  if (device < 0 || device >= count || device >= kMaxDevices) {
+    skl_hip_record_error(SKL_HIP_ERR_BAD_ARGUMENT, "skl_hip_init: device index");
+    return SKL_HIP_ERR_BAD_ARGUMENT;
+  }
+  int rc = skl_check_hip(hipSetDevice(device), "hipSetDevice");
+  if (rc != 0) return rc;
+  return skl_workspace(1) ? SKL_HIP_OK : SKL_HIP_ERR_WORKSPACE;
+}
+
+void skl_hip_shutdown(void) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  int prev = 0;
+  if (hipGetDevice(&prev) != hipSuccess) {
+    (void)hipGetLastError();
+    return;
+  }
+  for (int d = 0; d < kMaxDevices; ++d) {
+    if (!g_devices[d].workspace) continue;
+    if (hipSetDevice(d) == hipSuccess) {
+      (void)hipDeviceSynchronize();
+      (void)hipFree(g_devices[d].workspace);
+    }
+    g_devices[d] = DeviceState{};
+  }
+  (void)hipSetDevice(prev);
+}
+
+void *skl_hip_malloc(size_t bytes) {
+  void *p = nullptr;
+  if (bytes == 0) bytes = 1;
+  if (skl_check_hip(hipMalloc(&p, bytes), "skl_hip_malloc") != 0) return nullptr;
+  return p;
+}
+
+void skl_hip_free(void *ptr) {
+  if (ptr) (void)skl_check_hip(hipFree(ptr), "skl_hip_free");
+}
+
+// Copies are ordered with the current stream and complete before returning, so
+// a caller can touch the host buffer immediately.
+static int copy_sync(void *dst, const void *src, size_t bytes, hipMemcpyKind kind, const char *what) {
+  if (bytes == 0) return SKL_HIP_OK;
+  int rc = skl_check_hip(hipMemcpyAsync(dst, src, bytes, kind, t_stream), what);
+  if (rc != 0) return rc;
+  return skl_check_hip(hipStreamSynchronize(t_stream), what);
+}
+
+int skl_hip_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+  return copy_sync(dst, src, bytes, hipMemcpyHostToDevice, "skl_hip_memcpy_h2d");
+}
+int skl_hip_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+  return copy_sync(dst, src, bytes, hipMemcpyDeviceToHost, "skl_hip_memcpy_d2h");
+}
+int skl_hip_memcpy_d2d(void *dst, const void *src, size_t bytes) {
+  if (bytes == 0) return SKL_HIP_OK;
+  return skl_check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, t_stream),
+                       "skl_hip_memcpy_d2d");
+}
+int skl_hip_memset(void *dst, int byte, size_t bytes) {
+  if (bytes == 0) return SKL_HIP_OK;
+  return skl_check_hip(hipMemsetAsync(dst, byte, bytes, t_stream), "skl_hip_memset");
+}
+
+void skl_hip_set_stream(void *stream) { t_stream = (hipStream_t)stream; }
+void *skl_hip_get_stream(void) { return (void *)t_stream; }
+int skl_hip_synchronize(void) { return skl_check_hip(hipStreamSynchronize(t_stream), "skl_hip_synchronize"); }
+
+void skl_hip_set_pointer_mode(int mode) {
+  t_pointer_mode = (mode == SKL_HIP_POINTERS_DEVICE) ? SKL_HIP_POINTERS_DEVICE : SKL_HIP_POINTERS_AUTO;
+}
+int skl_hip_get_pointer_mode(void) { return t_pointer_mode; }
+
+int skl_hip_pointer_is_device(const void *ptr) {
+  if (t_pointer_mode == SKL_HIP_POINTERS_DEVICE) return 1;
+  if (!ptr) return 0;
+  hipPointerAttribute_t attr;
+  memset(&attr, 0, sizeof attr);
+  hipError_t e = hipPointerGetAttributes(&attr, ptr);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();  // ordinary host memory is reported as an error: not ours to keep
+    return 0;
+  }
+  return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged ||
+         attr.type == hipMemoryTypeHost;
+}
+
+int skl_hip_last_error(void) {
+  int e = t_error;
+  t_error = SKL_HIP_OK;
+  return e;
+}
+
+const char *skl_hip_last_error_string(void) { return t_error_text; }
+
+size_t skl_hip_te(void) { return 64; }
+
+void *skl_hip_event_create(void) {
+  hipEvent_t ev = nullptr;
+  if (skl_check_hip(hipEventCreate(&ev), "hipEventCreate") != 0) return nullptr;
+  return (void *)ev;
+}
+void skl_hip_event_destroy(void *event) {
+  if (event) (void)skl_check_hip(hipEventDestroy((hipEvent_t)event), "hipEventDestroy");
+}
+int skl_hip_event_record(void *event) {
+  return skl_check_hip(hipEventRecord((hipEvent_t)event, t_stream), "hipEventRecord");
+}
+float skl_hip_event_elapsed_ms(void *start, void *stop) {
+  if (skl_check_hip(hipEventSynchronize((hipEvent_t)stop), "hipEventSynchronize") != 0) return -1.0f;
+  float ms = -1.0f;
+  if (skl_check_hip(hipEventElapsedTime(&ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime") != 0)
+    return -1.0f;
+  return ms;
+}
+
+int skl_hip_device_info(char *name, size_t name_len, int *compute_units, int *clock_mhz) {
+  int dev = 0;
+  int rc = skl_check_hip(hipGetDevice(&dev), "hipGetDevice");
+  if (rc != 0) return rc;
+  hipDeviceProp_t prop;
+  rc = skl_check_hip(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties");
+  if (rc != 0) return rc;
+  if (name && name_len) {
+    snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+  }
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  if (clock_mhz) *clock_mhz = prop.clockRate / 1000;
+  return SKL_HIP_OK;
+}
+
+}  // extern "C"

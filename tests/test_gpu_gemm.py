@@ -1,0 +1,137 @@
+"""GPU parity of the GEMM entry points with the CPU checker.
+
+Every row of the reference's gemm suites (tests/golden/ref_tables.json) is run
+through the entry point the reference's suite calls, with inputs drawn as the
+reference's harnesses draw them (int8 in [-128,127]; bf16/f16 in [-1,1]; fp8
+bytes 8..126 / 4..123). Integer results must equal the checker bit for bit over
+the whole C buffer (stride gaps included: the clobber check); floating-point
+results must satisfy the reference's elementwise bound
+2*((1+2^-24)^(K+2)-1)*(|alpha||A||B| + |beta||C|) and a relative Frobenius
+error <= 1e-3 against the fp64 result."""
+import numpy as np
+import pytest
+
+import skl_amd
+import support
+from gpu_support import MODES, run_gemm
+from support import colmajor_a_case, rowmajor_case, run_oracle_gemm
+from test_oracle_gemm import FP_SUITES, dot4_cases, panel_cases, rvv_cases, xsfmm_c_cases
+
+pytestmark = pytest.mark.gpu
+
+
+def check(gpu, kind, case, seed, mode):
+    a, b, c = case.make_inputs(seed)
+    got = run_gemm(gpu, kind, case, a, b, c, mode)
+    if case.is_int:
+        want = run_oracle_gemm(case, a, b, c)
+        assert np.array_equal(got, want), (kind, vars(case))
+    else:
+        support.assert_fp_gemm_close(case, a, b, c, got)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_int8_rowmajor_table(gpu, mode):
+    for path in ("test/gemm/rvv/skl_gemm_i8_i8_i32_zve32x.c", "test/gemm/rvv/skl_gemm_i8_i8_i32_zve32x_x390.c"):
+        for i, case in enumerate(rvv_cases(path, "i8")):
+            check(gpu, "rowmajor", case, 1000 + i, mode)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_int8_colmajor_a_table(gpu, mode):
+    for i, case in enumerate(xsfmm_c_cases("test/gemm/xsfmm/skl_gemm_i8c_i8_i32_xsfmm32a8i.c", "i8", max_k=8192)):
+        check(gpu, "colmajor_a", case, 2000 + i, mode)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_int8_panel_table(gpu, mode):
+    path = "test/gemm/xsfmm/skl_gemm_i8rcptex1c_i8rcp1xte_i32rcptexterc_xsfmm32a8i.c"
+    stride = 1 if mode == "device" else 5
+    for i, case in enumerate(panel_cases(path, "i8", stride=stride, max_k=8192)):
+        check(gpu, "panel", case, 3000 + i, mode)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_int8_dot4_table(gpu, mode):
+    for i, case in enumerate(dot4_cases()):
+        check(gpu, "dot4", case, 4000 + i, mode)
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("ta", list(FP_SUITES))
+def test_fp_tables(gpu, ta, mode):
+    rvv, xc, xp = FP_SUITES[ta]
+    seed = 5000
+    if rvv:
+        for path in (rvv, rvv.replace("_x390", "")):
+            for case in rvv_cases(path, ta):
+                seed += 1
+                check(gpu, "rowmajor", case, seed, mode)
+    for case in xsfmm_c_cases(xc, ta, max_k=8192):
+        seed += 1
+        check(gpu, "colmajor_a", case, seed, mode)
+    stride = 1 if mode == "device" else 7
+    for case in panel_cases(xp, ta, stride=stride, max_k=8192):
+        seed += 1
+        check(gpu, "panel", case, seed, mode)
+
+
+@pytest.mark.parametrize("kind", ("rc", "rcprc"))
+def test_general_strides(gpu, kind):
+    """Column-major B and C, gapped strides, blocked layouts with k0 > 1: the
+    layouts only the full-stride forms can express."""
+    rng = np.random.default_rng(77)
+    for ta in ("i8", "bf16", "f16", "f8e4m3", "f8e5m2"):
+        m, n, k = 37, 29, 53
+        if kind == "rc":
+            case = support.GemmCase(ta, None, 2, 3, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0,
+                                    rsa1=k + 3, csa1=1, rsb0=0, csb0=0, rsb1=1, csb1=k + 5, rsc0=0, csc0=0,
+                                    rsc1=2, csc1=2 * m + 1)
+        else:
+            case = support.GemmCase(ta, None, 2, 3, m0=3, n0=4, k0=5, m1=5, n1=3, k1=4, rsa0=5, csa0=1,
+                                    rsa1=100, csa1=15, rsb0=4, csb0=1, rsb1=20, csb1=90, rsc0=1, csc0=3,
+                                    rsc1=12, csc1=64)
+        check(gpu, kind, case, int(rng.integers(1 << 30)), "device")
+        check(gpu, kind, case, int(rng.integers(1 << 30)), "host")
+
+
+def test_mixed_e4m3_e5m2(gpu):
+    for (m, n, k) in ((13, 21, 37), (128, 192, 256)):
+        case = rowmajor_case("f8e4m3", m, n, k, 1.0, 0.0, tb="f8e5m2")
+        check(gpu, "rc", case, 6000 + m, "device")
+        case = colmajor_a_case("f8e4m3", m, n, k, 1.5, 0.5, tb="f8e5m2")
+        check(gpu, "rc", case, 6100 + m, "host")
+
+
+def test_config1_int8_512_cubed_bit_exact(gpu):
+    """BASELINE config 1: 512^3, row-major, C = 0, alpha = 1, beta = 0."""
+    case = rowmajor_case("i8", 512, 512, 512, 1, 0)
+    a, b, c = case.make_inputs(0x5EED0010)
+    c[:] = 0
+    for mode in MODES:
+        got = run_gemm(gpu, "rowmajor", case, a, b, c, mode)
+        assert np.array_equal(got, run_oracle_gemm(case, a, b, c))
+
+
+def test_k_zero_scales_c_without_reading_operands(gpu):
+    """k == 0: C = beta * C and A, B are never dereferenced
+    (test/gemm/rvv/skl_gemm_i8_i8_i32_zve32x_x390.c:59,68-69)."""
+    c = np.arange(33 * 33, dtype=np.int32)
+    out = c.copy()
+    gpu.skl_gemm_i8_i8_i32_gfx950(33, 33, 0, 1, None, 0, None, 33, 3, out, 33)
+    skl_amd.check_error()
+    assert np.array_equal(out, 3 * c)
+    cf = np.linspace(-1, 1, 16 * 16).astype(np.float32)
+    outf = cf.copy()
+    gpu.skl_gemm_bf16_bf16_f32_gfx950(16, 16, 0, 1.0, None, 0, None, 16, 0.5, outf, 16)
+    skl_amd.check_error()
+    assert np.array_equal(outf, np.float32(0.5) * cf)
+
+
+def test_zero_m_or_n_touches_nothing(gpu):
+    c = np.full(64, 7, np.int32)
+    a = np.ones(64, np.int8)
+    gpu.skl_gemm_i8_i8_i32_gfx950(0, 8, 8, 1, a, 8, a, 8, 0, c, 8)
+    gpu.skl_gemm_i8_i8_i32_gfx950(8, 0, 8, 1, a, 8, a, 8, 0, c, 8)
+    skl_amd.check_error()
+    assert np.all(c == 7)

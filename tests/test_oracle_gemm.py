@@ -1,0 +1,203 @@
+"""Pins the CPU checker's GEMMs: integer results against numpy's exact integer
+matmul, blocked == strided, the K-packed form, exactly-summable fp inputs that
+fix the result under any summation order, the fp64 bound, and bit-equality
+with the reference's own library on the reference's test tables.
+"""
+import numpy as np
+import pytest
+
+import support
+from support import (GemmCase, colmajor_a_case, dot4_case, oracle, panel_case, ref, rowmajor_case,
+                     run_oracle_gemm)
+
+
+def ref_gemm(case, a, b, c):
+    out = c.copy()
+    getattr(ref(), case.stem() + "_ref")(*case.rcprc_args(a, b, out))
+    return out
+
+
+def int_expect(case, a, b, c):
+    A, B, C, oc = case.dense(a, b, c)
+    acc = (A.astype(np.int64) @ B.astype(np.int64))
+    val = (case.beta * C.astype(np.int64) + case.alpha * acc)
+    out = c.copy()
+    if oc.size:
+        out[oc.ravel()] = (val & 0xFFFFFFFF).astype(np.uint32).view(np.int32).ravel()
+    return out
+
+
+def rvv_cases(path, ta):
+    out = []
+    for r in support.table_rows(path, ("TEST", "BENCH")):
+        out.append(rowmajor_case(ta, r["m1"], r["n1"], r["k1"], r.get("alpha", 0), r.get("beta", 0),
+                                 r.get("rsa1"), r.get("rsb1"), r.get("rsc1")))
+    return out
+
+
+def xsfmm_c_cases(path, ta, max_k=64):
+    out = []
+    for r in support.table_rows(path, ("TEST", "BENCH")):
+        k = min(r["k1"], max_k) if r["kind"] == "BENCH" else r["k1"]
+        out.append(colmajor_a_case(ta, r["m1"], r["n1"], k, r.get("alpha", 0), r.get("beta", 0),
+                                   r.get("csa1"), r.get("rsb1"), r.get("rsc1")))
+    return out
+
+
+def panel_cases(path, ta, stride=1, max_k=64):
+    rows = support.table_rows(path, ("TEST", "BENCH"))
+    out = []
+    for r in rows[::stride]:
+        k = min(r["k1"], max_k) if r["kind"] == "BENCH" else r["k1"]
+        out.append(panel_case(ta, r["m1"], r["n1"], k, r.get("alpha", 0), r.get("beta", 0),
+                              r.get("csa1", 0), r.get("rsa1", 0), r.get("rsb1", 0), r.get("csb1", 0),
+                              r.get("rsc0", 0), r.get("csc0", 0), r.get("rsc1", 0), r.get("csc1", 0)))
+    return out
+
+
+def dot4_cases():
+    out = []
+    for r in support.table_rows("test/gemm/xsfvqdotq/skl_gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.c", ("TEST", "BENCH")):
+        out.append(dot4_case(r["m1"], r["n1"], r["k1"], r.get("alpha", 0), r.get("beta", 0), r.get("rsa1", 0),
+                             r.get("csa1", 0), r.get("rsb1", 0), r.get("rsc1", 0)))
+    return out
+
+
+INT_CASES = (rvv_cases("test/gemm/rvv/skl_gemm_i8_i8_i32_zve32x_x390.c", "i8") +
+             xsfmm_c_cases("test/gemm/xsfmm/skl_gemm_i8c_i8_i32_xsfmm32a8i.c", "i8") +
+             panel_cases("test/gemm/xsfmm/skl_gemm_i8rcptex1c_i8rcp1xte_i32rcptexterc_xsfmm32a8i.c", "i8", stride=9) +
+             dot4_cases())
+
+
+def test_int8_against_exact_integer_matmul():
+    for idx, case in enumerate(INT_CASES):
+        a, b, c = case.make_inputs(100 + idx)
+        got = run_oracle_gemm(case, a, b, c)
+        assert np.array_equal(got, int_expect(case, a, b, c)), vars(case)
+        if ref() is not None:
+            assert np.array_equal(got, ref_gemm(case, a, b, c)), vars(case)
+
+
+def test_int8_config1_shape():
+    # BASELINE config 1: 512^3 row-major, alpha = 1, beta = 0, C = 0
+    case = rowmajor_case("i8", 512, 512, 512, 1, 0)
+    a, b, c = case.make_inputs(0x5EED0000)
+    c[:] = 0
+    got = run_oracle_gemm(case, a, b, c)
+    want = (a.reshape(512, 512).astype(np.int32) @ b.reshape(512, 512).astype(np.int32))
+    assert np.array_equal(got.reshape(512, 512), want)
+
+
+def test_int32_wraparound_in_epilogue():
+    case = rowmajor_case("i8", 3, 5, 8, alpha=0x7FFFFFF, beta=-0x12345678)
+    a, b, c = case.make_inputs(9)
+    c[:] = np.random.default_rng(2).integers(-2 ** 31, 2 ** 31, size=c.size)
+    assert np.array_equal(run_oracle_gemm(case, a, b, c), int_expect(case, a, b, c))
+
+
+def test_blocked_equals_strided():
+    # packed API with 1x1x1 blocks is the strided API (src/gemm/packed-gemm.md:77)
+    rng = np.random.default_rng(4)
+    m, n, k = 9, 11, 13
+    for ta in ("i8", "bf16", "f16", "f8e4m3", "f8e5m2"):
+        case = GemmCase(ta, None, 2, 3, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=k + 2, csa1=1,
+                        rsb0=0, csb0=0, rsb1=1, csb1=k + 1, rsc0=0, csc0=0, rsc1=2, csc1=2 * m + 3)
+        a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+        blocked = run_oracle_gemm(case, a, b, c)
+        strided = c.copy()
+        rc_name = case.stem().replace("rcprc", "rc") + "_oracle"
+        getattr(oracle(), rc_name)(m, n, k, case.alpha, a, case.rsa1, case.csa1, b, case.rsb1, case.csb1,
+                                   case.beta, strided, case.rsc1, case.csc1)
+        assert np.array_equal(blocked.view(np.uint32), strided.view(np.uint32)), ta
+
+
+FP_SUITES = {
+    "bf16": ("test/gemm/rvv/skl_gemm_bf16_bf16_f32_zvfbfwma_x390.c", "test/gemm/xsfmm/skl_gemm_bf16c_bf16_f32_xsfmm32a16f.c",
+             "test/gemm/xsfmm/skl_gemm_bf16rcptex1c_bf16rcp1xte_f32rcptexterc_xsfmm32a16f.c"),
+    "f16": ("test/gemm/rvv/skl_gemm_f16_f16_f32_zvfh_x390.c", "test/gemm/xsfmm/skl_gemm_f16c_f16_f32_xsfmm32a16f.c",
+            "test/gemm/xsfmm/skl_gemm_f16rcptex1c_f16rcp1xte_f32rcptexterc_xsfmm32a16f.c"),
+    "f8e4m3": (None, "test/gemm/xsfmm/skl_gemm_f8e4m3c_f8e4m3_f32_xsfmm32a8f.c",
+               "test/gemm/xsfmm/skl_gemm_f8e4m3rcptex1c_f8e4m3rcp1xte_f32rcptexterc_xsfmm32a8f.c"),
+    "f8e5m2": (None, "test/gemm/xsfmm/skl_gemm_f8e5m2c_f8e5m2_f32_xsfmm32a8f.c",
+               "test/gemm/xsfmm/skl_gemm_f8e5m2rcptex1c_f8e5m2rcp1xte_f32rcptexterc_xsfmm32a8f.c"),
+}
+
+
+def fp_cases(ta, panel_stride=17):
+    rvv, xc, xp = FP_SUITES[ta]
+    cases = []
+    if rvv:
+        cases += rvv_cases(rvv, ta)
+    cases += xsfmm_c_cases(xc, ta)
+    cases += panel_cases(xp, ta, stride=panel_stride)
+    return cases
+
+
+@pytest.mark.parametrize("ta", list(FP_SUITES))
+def test_fp_within_reference_bound_and_equal_to_reference(ta):
+    for idx, case in enumerate(fp_cases(ta)):
+        a, b, c = case.make_inputs(500 + idx)
+        got = run_oracle_gemm(case, a, b, c)
+        support.assert_fp_gemm_close(case, a, b, c, got)
+        if ref() is not None:
+            want = ref_gemm(case, a, b, c)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), vars(case)
+
+
+@pytest.mark.parametrize("ta", list(FP_SUITES))
+def test_fp_exactly_summable_inputs(ta):
+    """Small integers / powers of two: every partial sum is exact in fp32, so the
+    result is fixed by the mathematics whatever the summation order."""
+    rng = np.random.default_rng(21)
+    m, n, k = 17, 19, 40
+    vals = np.array([-2.0, -1.0, -0.5, 0.0, 0.5, 1.0, 2.0, 4.0])
+    A = rng.choice(vals, size=(m, k))
+    B = rng.choice(vals, size=(k, n))
+    C = rng.integers(-8, 9, size=(m, n)).astype(np.float64)
+
+    def enc(x):
+        x32 = x.astype(np.float32)
+        if ta == "bf16":
+            return support.f32_to_bf16_bits(x32)
+        if ta == "f16":
+            return x32.astype(np.float16).view(np.uint16)
+        out = np.zeros(x32.size, np.uint8)
+        getattr(oracle(), f"skl_cvt_f32_{ta}_oracle")(out, x32.ravel(), 1.0, x32.size)
+        return out.reshape(x.shape)
+
+    case = rowmajor_case(ta, m, n, k, alpha=2.0, beta=-3.0)
+    a, b, c = enc(A).ravel(), enc(B).ravel(), C.astype(np.float32).ravel()
+    got = run_oracle_gemm(case, a, b, c).reshape(m, n)
+    assert np.array_equal(got, (2.0 * (A @ B) - 3.0 * C).astype(np.float32))
+
+
+def test_mixed_fp8_equals_decode_then_f32_gemm():
+    m, n, k = 13, 21, 37
+    rng = np.random.default_rng(8)
+    a = rng.integers(8, 127, size=m * k, dtype=np.uint8)
+    b = rng.integers(4, 124, size=k * n, dtype=np.uint8)
+    c0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    got = c0.copy()
+    oracle().skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_oracle(m, n, k, 1.5, a, k, 1, b, n, 1, 0.5, got, n, 1)
+    af = support.decode_table("f8e4m3")[a].astype(np.float32)
+    bf = support.decode_table("f8e5m2")[b].astype(np.float32)
+    want = c0.copy()
+    oracle().skl_gemm_f32rc_f32rc_f32rc_oracle(m, n, k, 1.5, af, k, 1, bf, n, 1, 0.5, want, n, 1)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    if ref() is not None:
+        want2 = c0.copy()
+        ref().skl_gemm_f32rc_f32rc_f32rc_ref(m, n, k, 1.5, af, k, 1, bf, n, 1, 0.5, want2, n, 1)
+        assert np.array_equal(got.view(np.uint32), want2.view(np.uint32))
+
+
+def test_f64_helper_matches_numpy_and_reference():
+    m, n, k = 7, 9, 33
+    rng = np.random.default_rng(12)
+    A, B, C = rng.normal(size=(m, k)), rng.normal(size=(k, n)), rng.normal(size=(m, n))
+    got = C.copy().ravel()
+    oracle().skl_gemm_f64rc_f64rc_f64rc_oracle(m, n, k, 1.25, A.ravel(), k, 1, B.ravel(), n, 1, -0.5, got, n, 1)
+    assert np.allclose(got.reshape(m, n), 1.25 * A @ B - 0.5 * C, rtol=1e-13, atol=1e-13)
+    if ref() is not None:
+        want = C.copy().ravel()
+        ref().skl_gemm_f64rc_f64rc_f64rc_ref(m, n, k, 1.25, A.ravel(), k, 1, B.ravel(), n, 1, -0.5, want, n, 1)
+        assert np.array_equal(got, want)
