@@ -1,0 +1,320 @@
+#!/usr/bin/env python3
+"""Benchmark of the GEMM / GEMV / pack / cvt hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
+
+Prints ONE JSON line. The headline (`value`) is the int8 GEMV decode shape
+(1x4096 times 4096x11008, BASELINE config 2) in GB/s of algorithmic bytes with
+all operands resident in HBM; a "step" is one GEMV call on the next of several
+weight matrices (their total size exceeds the 256 MiB last-level cache, so the
+stream comes from HBM). `extra` carries the dense workloads (TOPS / TFLOP/s and
+fraction of the MFMA roofline) and the pack / cvt streams, each timed the same
+way. `cpu_baseline` is the reference's scalar routine (or, where that library
+was not built, the CPU checker) timed on this host for the same shape.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import skl_amd  # noqa: E402
+from skl_amd import DeviceBuffer  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TOPS = {"i8": 5000.0, "f8": 5000.0, "bf16": 2500.0, "f16": 2500.0}
+METRIC = "GEMM TOPS (int8/fp8/bf16) + GEMV HBM GB/s on 1 MI355X, % of roofline"
+
+
+class Timer:
+    """Times `steps` calls of fn(i) after `warmup` untimed ones: wall clock around a
+    synchronised region, and HIP events on the library's stream inside it."""
+
+    def __init__(self, lib):
+        self.lib = lib
+        self.e0, self.e1 = lib.skl_hip_event_create(), lib.skl_hip_event_create()
+
+    def run(self, fn, steps, warmup):
+        lib = self.lib
+        for i in range(warmup):
+            fn(i)
+        lib.skl_hip_synchronize()
+        t0 = time.perf_counter()
+        lib.skl_hip_event_record(self.e0)
+        for i in range(steps):
+            fn(warmup + i)
+        lib.skl_hip_event_record(self.e1)
+        ev_ms = lib.skl_hip_event_elapsed_ms(self.e0, self.e1)
+        lib.skl_hip_synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        skl_amd.check_error()
+        return wall_ms / steps, ev_ms / steps
+
+
+def rand_i8(rng, n):
+    return rng.integers(-128, 128, size=n, dtype=np.int8)
+
+
+def bf16_bits(x):
+    u = x.astype(np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+# ----------------------------------------------------------------------------
+# workloads: each returns (callable(i), per-step algorithmic bytes, per-step ops, bound, dtype key)
+# ----------------------------------------------------------------------------
+
+def wl_gemv(lib, rng):
+    k, n, nbuf = 4096, 11008, 8
+    w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(rand_i8(rng, k))
+    y = DeviceBuffer(4 * n)
+
+    def step(i):
+        lib.skl_gemm_i8_i8_i32_gfx950(1, n, k, 1, x, k, w[i % nbuf], n, 0, y, n)
+
+    return dict(fn=step, bytes=k * n + k + 4 * n, ops=2 * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
+                name="int8 GEMV 1x4096x11008 (row-major W, beta=0)", kernel="gemv_i8_rowmajor_kernel")
+
+
+def _dense(lib, rng, name, fn_name, m, n, k, abytes, gen_a, gen_b, alpha, beta, ctype, dkey, col_major_a=False):
+    a = DeviceBuffer.from_array(gen_a(m * k))
+    b = DeviceBuffer.from_array(gen_b(k * n))
+    c = DeviceBuffer.from_array(np.zeros(m * n, ctype) if beta == 0 else rng.normal(size=m * n).astype(ctype))
+    f = getattr(lib, fn_name)
+    lda = m if col_major_a else k
+
+    def step(i):
+        f(m, n, k, alpha, a, lda, b, n, beta, c, n)
+
+    return dict(fn=step, bytes=abytes * (m * k + k * n) + 4 * m * n * (2 if beta != 0 else 1), ops=2 * m * n * k,
+                bound="mfma", dtype=dkey, keep=(a, b, c), name=name, kernel="gemm_mfma_kernel")
+
+
+def wl_gemm_i8_8192(lib, rng):
+    return _dense(lib, rng, "int8 GEMM 8192^3 (row-major, alpha=1, beta=0)", "skl_gemm_i8_i8_i32_gfx950", 8192, 8192,
+                  8192, 1, lambda n: rand_i8(rng, n), lambda n: rand_i8(rng, n), 1, 0, np.int32, "i8")
+
+
+def wl_gemm_i8_512(lib, rng):
+    return _dense(lib, rng, "int8 GEMM 512^3 (row-major, alpha=1, beta=0)", "skl_gemm_i8_i8_i32_gfx950", 512, 512, 512,
+                  1, lambda n: rand_i8(rng, n), lambda n: rand_i8(rng, n), 1, 0, np.int32, "i8")
+
+
+def _fp8_operand(lib, rng, n, fmt):
+    """fp32 ~ N(0,1) converted on the GPU with the saturating cvt (scale 1)."""
+    src = DeviceBuffer.from_array(rng.normal(size=n).astype(np.float32))
+    dst = DeviceBuffer(n)
+    getattr(lib, f"skl_cvt_sat_f32_{fmt}_gfx950")(dst, src, 1.0, n)
+    lib.skl_hip_synchronize()
+    src.free()
+    return dst
+
+
+def wl_gemm_f8_8192(lib, rng, fmt_b="f8e4m3"):
+    m = n = k = 8192
+    a = _fp8_operand(lib, rng, m * k, "f8e4m3")   # stored column-major (k x m row-major = A^T)
+    b = _fp8_operand(lib, rng, k * n, fmt_b)
+    c = DeviceBuffer.from_array(np.zeros(m * n, np.float32))
+    if fmt_b == "f8e4m3":
+        def step(i):
+            lib.skl_gemm_f8e4m3c_f8e4m3_f32_gfx950(m, n, k, 1.0, a, m, b, n, 0.0, c, n)
+        name = "fp8 E4M3xE4M3 GEMM 8192^3 (column-major A, alpha=1, beta=0)"
+    else:
+        def step(i):
+            lib.skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950(m, n, k, 1.0, a, 1, m, b, n, 1, 0.0, c, n, 1)
+        name = "fp8 E4M3xE5M2 GEMM 8192^3 (column-major A, alpha=1, beta=0)"
+    return dict(fn=step, bytes=m * k + k * n + 8 * m * n, ops=2 * m * n * k, bound="mfma", dtype="f8", keep=(a, b, c),
+                name=name, kernel="gemm_mfma_kernel")
+
+
+def wl_gemm_bf16(lib, rng):
+    m, n, k = 2048, 4096, 4096
+    return _dense(lib, rng, "bf16 GEMM 2048x4096x4096 (row-major, alpha=1, beta=1)", "skl_gemm_bf16_bf16_f32_gfx950",
+                  m, n, k, 2, lambda c: bf16_bits(rng.normal(size=c)), lambda c: bf16_bits(rng.normal(size=c) * 0.02),
+                  1.0, 1.0, np.float32, "bf16")
+
+
+def wl_f16_pipeline(lib, rng):
+    """BASELINE config 5: pack A, pack B, panel GEMM, unpack C - one step is the whole pipeline."""
+    te, m, k, n = 64, 4096, 4096, 14336
+    a = DeviceBuffer.from_array(rng.uniform(-1, 1, m * k).astype(np.float16).view(np.uint16))
+    b = DeviceBuffer.from_array(rng.uniform(-1, 1, k * n).astype(np.float16).view(np.uint16))
+    ap, bp = DeviceBuffer(2 * m * k), DeviceBuffer(2 * k * n)
+    cp, c = DeviceBuffer(4 * m * n), DeviceBuffer(4 * m * n)
+    lib.skl_hip_memset(cp, 0, 4 * m * n)
+    m1, n1 = m // te, n // te
+
+    def step(i):
+        lib.skl_pack_e16_e16rcptex1c_gfx950(m, k, a, k, ap, k * te, te, 0)
+        lib.skl_pack_e16rc_e16rcprc_gfx950(k, n, b, n, 1, 1, te, bp, te, 1, te, k * te, 0)
+        lib.skl_gemm_f16rcptex1c_f16rcp1xte_f32rcptexterc_gfx950(m1, n1, k, 1.0, ap, k * te, te, bp, te, k * te, 0.0, cp,
+                                                                  te, 1, n1 * te * te, te * te)
+        lib.skl_unpack_e32rcprc_e32rc_gfx950(te, te, cp, te, 1, n1 * te * te, te * te, m, n, c, n, 1)
+
+    moved = 2 * (2 * m * k) + 2 * (2 * k * n) + 2 * (4 * m * n)
+    return dict(fn=step, bytes=moved, ops=2 * m * n * k, bound="mfma", dtype="f16", keep=(a, b, ap, bp, cp, c),
+                name="f16 pack->GEMM->unpack 4096x4096x14336 (TE=64 panels)", kernel="gemm_mfma_kernel")
+
+
+def wl_cvt(lib, rng):
+    n = 8192 * 8192
+    src = DeviceBuffer.from_array(rng.normal(size=n).astype(np.float32))
+    dst = DeviceBuffer(n)
+
+    def step(i):
+        lib.skl_cvt_sat_f32_f8e4m3_gfx950(dst, src, 1.0, n)
+
+    return dict(fn=step, bytes=5 * n, ops=n, bound="hbm", dtype="f32", keep=(src, dst),
+                name="cvt sat f32->E4M3, 8192^2 elements", kernel="cvt_f32_f8_kernel")
+
+
+def wl_pack_a(lib, rng):
+    te, m, k = 64, 4096, 4096
+    a = DeviceBuffer.from_array(rng.integers(0, 1 << 16, m * k, dtype=np.uint16))
+    ap = DeviceBuffer(2 * m * k)
+
+    def step(i):
+        lib.skl_pack_e16_e16rcptex1c_gfx950(m, k, a, k, ap, k * te, te, 0)
+
+    return dict(fn=step, bytes=4 * m * k, ops=m * k, bound="hbm", dtype="u16", keep=(a, ap),
+                name="pack e16 4096x4096 -> TEx1 column panels", kernel="pack_tile_kernel")
+
+
+WORKLOADS = {
+    "gemv_i8": (wl_gemv, 2000, 100),
+    "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
+    "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2),
+    "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2),
+    "gemm_bf16_2048x4096x4096": (wl_gemm_bf16, 20, 3),
+    "pipeline_f16_4096x4096x14336": (wl_f16_pipeline, 5, 1),
+    "gemm_i8_512": (wl_gemm_i8_512, 200, 20),
+    "cvt_f32_f8e4m3_8192sq": (wl_cvt, 20, 3),
+    "pack_e16_4096sq": (wl_pack_a, 20, 3),
+}
+HEADLINE = "gemv_i8"
+
+
+def measure(lib, key, steps=None, warmup=None, seed=0x5EED0000):
+    builder, dsteps, dwarm = WORKLOADS[key]
+    steps = steps or dsteps
+    warmup = dwarm if warmup is None else warmup
+    rng = np.random.default_rng(seed)
+    wl = builder(lib, rng)
+    wall_ms, ev_ms = Timer(lib).run(wl["fn"], steps, warmup)
+    out = dict(workload=key, name=wl["name"], steps=steps, warmup=warmup, ms_per_step=wall_ms, event_ms_per_step=ev_ms,
+               dtype=wl["dtype"])
+    sec = ev_ms * 1e-3
+    if wl["bound"] == "hbm":
+        gbs = wl["bytes"] / sec / 1e9
+        out.update(value=wl["bytes"] / (wall_ms * 1e-3) / 1e9, unit="GB/s",
+                   roofline=dict(bound="hbm", achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=gbs / HBM_PEAK_GBS,
+                                 traffic=None, kernel=wl["kernel"], algorithmic_bytes=wl["bytes"]))
+    else:
+        tops = wl["ops"] / sec / 1e12
+        peak = MFMA_PEAK_TOPS[wl["dtype"]]
+        unit = "TOP/s" if wl["dtype"] == "i8" else "TFLOP/s"
+        out.update(value=wl["ops"] / (wall_ms * 1e-3) / 1e12, unit=unit,
+                   roofline=dict(bound="mfma", achieved=tops, peak=peak, unit=unit, frac=tops / peak, traffic=None,
+                                 kernel=wl["kernel"], ops=wl["ops"]))
+    for buf in _flatten(wl["keep"]):
+        buf.free()
+    return out
+
+
+def _flatten(x):
+    for item in x:
+        if isinstance(item, (list, tuple)):
+            yield from _flatten(item)
+        else:
+            yield item
+
+
+def cpu_baseline(budget_s=12.0):
+    """The reference's scalar int8 GEMM (ref/gemm/gemm_i8rc_i8rc_i32rc.c) on the
+    headline shape, one thread, repeated until about `budget_s` seconds are spent."""
+    from oracle import loader
+    ref = loader.load_ref()
+    kind = "reference"
+    if ref is None:
+        ref, kind = loader.load_oracle(), "port"
+    fn = ref.skl_gemm_i8rc_i8rc_i32rc_ref if kind == "reference" else ref.skl_gemm_i8rc_i8rc_i32rc_oracle
+    k, n = 4096, 11008
+    rng = np.random.default_rng(0x5EED0021)
+    x, w, y = rand_i8(rng, k), rand_i8(rng, k * n), np.zeros(n, np.int32)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn(1, n, k, 1, x, k, 1, w, n, 1, 0, y, n, 1)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= 4096:
+            break
+    byts = k * n + k + 4 * n
+    return dict(value=byts * reps / el / 1e9, unit="GB/s", cores=1, kind=kind,
+                sample=f"{reps} full calls of the 1x4096x11008 int8 GEMV ({el:.1f} s, one thread)",
+                host_cpus=os.cpu_count())
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this library runs on one GPU; --gpus must be 1 (no multi-GPU path exists)")
+
+    lib = skl_amd.load()
+    if lib.skl_hip_init(0) != 0:
+        sys.exit("bench.py: no GPU: " + lib.skl_hip_last_error_string().decode())
+    lib.skl_hip_set_pointer_mode(1)  # device pointers only: no per-call pointer queries
+
+    head = measure(lib, args.workload, args.steps, args.warmup)
+    result = {
+        "metric": METRIC,
+        "value": head["value"],
+        "unit": head["unit"],
+        "n_gpus": 1,
+        "steps": head["steps"],
+        "warmup": head["warmup"],
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": head["dtype"],
+        "data": "synthetic",
+        "config": {"workload": head["name"], "key": head["workload"], "resident": "HBM",
+                   "weight_buffers_rotated": 8 if args.workload == "gemv_i8" else 1},
+        "roofline": head["roofline"],
+    }
+    if not args.no_extra:
+        extra = []
+        for key in WORKLOADS:
+            if key == args.workload:
+                continue
+            try:
+                r = measure(lib, key)
+                extra.append({"workload": r["workload"], "name": r["name"], "value": r["value"], "unit": r["unit"],
+                              "ms_per_step": r["ms_per_step"], "steps": r["steps"], "dtype": r["dtype"],
+                              "roofline": r["roofline"]})
+            except Exception as e:  # a failing extra must not hide the headline
+                extra.append({"workload": key, "error": str(e)})
+        result["extra"] = extra
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    name = (lambda b: (lib.skl_hip_device_info(b, 128, None, None), b.value.decode())[1])(
+        __import__("ctypes").create_string_buffer(128))
+    result["device"] = name
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

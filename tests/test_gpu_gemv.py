@@ -1,0 +1,82 @@
+"""GPU parity of the M == 1 streaming path with the CPU checker (bit-exact:
+integer sums are order-independent), at the BASELINE config-2 shape and around
+the kernel's tiling edges, including back-to-back calls that share the
+library's zero-initialised reduction scratch."""
+import numpy as np
+import pytest
+
+import skl_amd
+import support
+from gpu_support import run_gemm
+from support import GemmCase, colmajor_a_case, rowmajor_case, run_oracle_gemm
+
+pytestmark = pytest.mark.gpu
+
+
+def test_config2_decode_shape_bit_exact(gpu):
+    """1 x 4096 times 4096 x 11008, int8 -> int32, beta = 0."""
+    case = rowmajor_case("i8", 1, 11008, 4096, 1, 0)
+    a, b, c = case.make_inputs(0x5EED0020)
+    want = run_oracle_gemm(case, a, b, c)
+    for mode in ("device", "host"):
+        got = run_gemm(gpu, "rowmajor", case, a, b, c, mode)
+        assert np.array_equal(got, want)
+    # independent of the checker: exact integer matmul in numpy
+    ref = a.astype(np.int64)[None, :] @ b.reshape(4096, 11008).astype(np.int64)
+    assert np.array_equal(want, ref.ravel().astype(np.int32))
+
+
+def test_back_to_back_calls_reuse_scratch(gpu):
+    """Three calls in a row, shrinking shapes, accumulating into the same y: the
+    scratch accumulators and tickets must be back at zero after every call."""
+    rng = np.random.default_rng(3)
+    y = rng.integers(-1000, 1000, size=11008).astype(np.int32)
+    dy = skl_amd.DeviceBuffer.from_array(y)
+    want = y.copy()
+    for (n, k, alpha, beta) in ((11008, 4096, 1, 1), (4096, 1000, -3, 2), (1024, 128, 7, -1), (16, 4, 1, 0)):
+        case = rowmajor_case("i8", 1, n, k, alpha, beta)
+        a, b, _ = case.make_inputs(n + k)
+        da, db = skl_amd.DeviceBuffer.from_array(a), skl_amd.DeviceBuffer.from_array(b)
+        gpu.skl_gemm_i8_i8_i32_gfx950(1, n, k, alpha, da, k, db, n, beta, dy, n)
+        gpu.skl_hip_synchronize()
+        skl_amd.check_error()
+        want = run_oracle_gemm(case, a, b, want)
+        assert np.array_equal(dy.download(np.int32), want), (n, k)
+        da.free(), db.free()
+
+
+@pytest.mark.parametrize("n,k", ((16, 1), (1024, 127), (1040, 129), (2048, 4), (33 * 16, 1000), (11008, 4095)))
+def test_tiling_edges(gpu, n, k):
+    case = rowmajor_case("i8", 1, n, k, alpha=0x01010101, beta=-77, rsb=n + 32, rsc=n)
+    a, b, c = case.make_inputs(n * 7 + k)
+    c[:] = np.random.default_rng(k).integers(-2 ** 31, 2 ** 31, size=c.size)
+    assert np.array_equal(run_gemm(gpu, "rowmajor", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
+
+
+def test_strided_x_and_y(gpu):
+    """x read with a stride (column-major A with m = 1) and y written with a
+    stride (column-major-like C): gaps in y must be preserved."""
+    n, k = 2048, 300
+    case = GemmCase("i8", None, 2, 3, m0=1, n0=1, k0=1, m1=1, n1=n, k1=k, rsa0=0, csa0=0, rsa1=1, csa1=5,
+                    rsb0=0, csb0=0, rsb1=n, csb1=1, rsc0=0, csc0=0, rsc1=1, csc1=3)
+    a, b, c = case.make_inputs(99)
+    assert np.array_equal(run_gemm(gpu, "rc", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
+
+
+def test_panel_packed_weights(gpu):
+    """B in 1 x TE row panels (B_p[j/64][k][j%64]) with one block row of A."""
+    te = support.TE
+    k, n1 = 200, 5
+    case = GemmCase("i8", None, 1, 0, m0=1, n0=te, k0=1, m1=1, n1=n1, k1=k, rsa0=0, csa0=0, rsa1=k, csa1=1,
+                    rsb0=0, csb0=1, rsb1=te, csb1=k * te, rsc0=0, csc0=1, rsc1=n1 * te, csc1=te)
+    a, b, c = case.make_inputs(5)
+    assert np.array_equal(run_gemm(gpu, "rcprc", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
+
+
+def test_m1_shapes_outside_the_streaming_kernel(gpu):
+    """N not a multiple of 16 or a misaligned row stride: served by another
+    kernel, same answer (test/gemm/rvv/skl_gemm_i8_i8_i32_zve32x_x390.c:64)."""
+    for (n, k, rsb) in ((33, 31, 33), (255, 12, 255), (256, 31, 257)):
+        case = rowmajor_case("i8", 1, n, k, 1, 1, rsb=rsb)
+        a, b, c = case.make_inputs(n + k)
+        assert np.array_equal(run_gemm(gpu, "rowmajor", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
