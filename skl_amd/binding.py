@@ -30,7 +30,8 @@ class _Lib:
         self.cdll = ctypes.CDLL(path)
         self.names = []
         for name, (restype, sig) in signatures.RUNTIME.items():
-            setattr(self, name, signatures.bind(self.cdll, name, sig, restype))
+            raw = signatures.bind(self.cdll, name, sig, restype)
+            setattr(self, name, _wrap(raw, sig) if "p" in sig else raw)
         for table in (signatures.reference_shared(), signatures.gfx950_only()):
             for stem, sig in table.items():
                 cname = stem + _SUFFIX

@@ -1,4 +1,478 @@
-// placeholder until the matrix-core kernels land
+// skl_gemm_mfma.hip - the dense contractions on the gfx950 matrix cores:
+// int8 x int8 -> int32 (v_mfma_i32_32x32x32_i8), bf16 / f16 -> f32
+// (v_mfma_f32_32x32x16_{bf16,f16}) and OCP fp8 E4M3 / E5M2, in any pairing,
+// -> f32 (v_mfma_f32_32x32x64_f8f6f4).
+//
+// Semantics: C = alpha*A*B + beta*C of ref/gemm/gemm_i8rcprc_i8rcprc_i32rcprc.c:10-37
+// and its typed twins, for the layouts the optimized SKL entry points use
+// (src/gemm/gemm_i8_i8_i32_zve32x.h:38-48 row-major, src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:38-48
+// column-major A, :85-95 TE x 1 / 1 x TE panels with TE x TE blocks of C). The
+// integer result is exact; the fp result accumulates exact products in fp32
+// in an order that differs from the reference's k-ascending loop.
+//
+// One kernel template serves every layout pair. Each operand is either
+// "K-contiguous" (row-major A, column-major B) or "MN-contiguous" (column-major
+// A, row-major B, and both panel formats); blocks of 64 along M / N may sit
+// anywhere (block stride), which is what the panel formats need. A workgroup of
+// eight waves owns a BM x BN tile of C; per 128-byte slice of K it copies the
+// A and B tiles global -> registers -> LDS in their native orientation with
+// 128-bit accesses (double-buffered: the next slice is in flight while the
+// current one is multiplied) and the waves read MFMA operands straight from
+// LDS: ds_read_b128 for a K-contiguous tile (row pitch padded to 144 bytes),
+// ds_read_b64_tr_b8 / _tr_b16 - the LDS transpose loads - for an
+// MN-contiguous one (row pitch padded so the eight/four rows of one transpose
+// land in distinct banks). No data is transposed by VALU work. The k order
+// inside an MFMA is the same for both operands whichever way they were read, so
+// any layout pair multiplies matching k. alpha / beta are applied per wave on
+// the accumulator registers in the epilogue.
+#include <hip/hip_runtime.h>
+
 #include "skl_device.hpp"
-extern "C" int skl_hip_gemm_mfma_supported(const skl_gemm_canon *) { return 0; }
-extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *) { return -2; }
+
+namespace {
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T *)(p))
+
+constexpr int kThreads = 512;       // 8 waves: 2 along M x 4 along N
+constexpr int kSliceBytes = 128;    // bytes of K per LDS stage and operand row
+constexpr int kPitchKC = 144;       // LDS row pitch of a K-contiguous tile
+
+struct MfmaArgs {
+  const char *a;
+  const char *b;
+  char *c;
+  size_t m, n, k;
+  size_t a_s1, a_s0, a_sk;  // elements
+  size_t b_s1, b_s0, b_sk;
+  size_t rsc0, csc0, rsc1, csc1;
+  skl_scalar alpha, beta;
+  unsigned tiles_m, tiles_n;
+};
+
+// Operand kinds of the MFMA: element size, accumulator type, k per instruction.
+template <int DT>
+struct Kind;
+template <>
+struct Kind<SKL_DT_I8> {
+  static constexpr int ES = 1, KB = 32;  // KB: bytes of K consumed per MFMA per operand row
+  using Acc = v16i;
+};
+template <>
+struct Kind<SKL_DT_BF16> {
+  static constexpr int ES = 2, KB = 32;
+  using Acc = v16f;
+};
+template <>
+struct Kind<SKL_DT_F16> {
+  static constexpr int ES = 2, KB = 32;
+  using Acc = v16f;
+};
+template <>
+struct Kind<SKL_DT_F8E4M3> {
+  static constexpr int ES = 1, KB = 64;
+  using Acc = v16f;
+};
+template <>
+struct Kind<SKL_DT_F8E5M2> {
+  static constexpr int ES = 1, KB = 64;
+  using Acc = v16f;
+};
+
+// One MFMA: FR = bytes per lane / 4 registers of each operand fragment.
+template <int TA, int TB>
+struct Mma;
+template <>
+struct Mma<SKL_DT_I8, SKL_DT_I8> {
+  using Frag = v4i;
+  __device__ static v16i run(v4i a, v4i b, v16i c) { return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0); }
+};
+template <>
+struct Mma<SKL_DT_BF16, SKL_DT_BF16> {
+  using Frag = v4i;
+  __device__ static v16f run(v4i a, v4i b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<SKL_DT_F16, SKL_DT_F16> {
+  using Frag = v4i;
+  __device__ static v16f run(v4i a, v4i b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+// f8f6f4 format codes: 0 = E4M3, 1 = E5M2. Scales 0/0 select the unscaled instruction.
+#define SKL_F8_MMA(TA_, TB_, FA_, FB_)                                                                   \
+  template <>                                                                                            \
+  struct Mma<TA_, TB_> {                                                                                 \
+    using Frag = v8i;                                                                                    \
+    __device__ static v16f run(v8i a, v8i b, v16f c) {                                                   \
+      return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, FA_, FB_, 0, 0, 0, 0);             \
+    }                                                                                                    \
+  };
+SKL_F8_MMA(SKL_DT_F8E4M3, SKL_DT_F8E4M3, 0, 0)
+SKL_F8_MMA(SKL_DT_F8E5M2, SKL_DT_F8E5M2, 1, 1)
+SKL_F8_MMA(SKL_DT_F8E4M3, SKL_DT_F8E5M2, 0, 1)
+SKL_F8_MMA(SKL_DT_F8E5M2, SKL_DT_F8E4M3, 1, 0)
+
+// ---------------------------------------------------------------------------
+// LDS tile geometry of one operand: ROWS along M or N, 128 bytes of K.
+// ---------------------------------------------------------------------------
+template <int ES, int ROWS, bool KC>
+struct Tile {
+  static constexpr int CE = 16 / ES;                 // elements per 16-byte chunk
+  static constexpr int KE = kSliceBytes / ES;        // k elements per slice
+  // MN-contiguous tile: KE rows of ROWS*ES bytes, padded so that the rows one
+  // transpose load touches (8 rows x 16 B, or 4 rows x 32 B) hit distinct banks.
+  static constexpr int kPitchMC = ROWS * ES + (ES == 1 ? 16 : 32);
+  static constexpr int kBytes = KC ? ROWS * kPitchKC : KE * kPitchMC;
+  static constexpr int kChunks = ROWS * 8;           // 16-byte chunks per slice
+  static constexpr int kPerThread = kChunks / kThreads;
+  static constexpr int kMnChunks = ROWS * ES / 16;   // chunks along MN of an MN-contiguous row
+};
+
+// 16 bytes from global memory with `valid` (<= CE) leading elements in range.
+template <int ES>
+__device__ __forceinline__ uint4 load_chunk(const char *p, long valid) {
+  constexpr int CE = 16 / ES;
+  if (valid >= CE) return *reinterpret_cast<const uint4 *>(p);
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (valid > 0) {
+    unsigned w[4] = {0, 0, 0, 0};
+    for (int e = 0; e < CE; ++e) {
+      if (e < valid) {
+        unsigned x = ES == 1 ? (unsigned)*reinterpret_cast<const uint8_t *>(p + e)
+                             : (unsigned)*reinterpret_cast<const uint16_t *>(p + 2 * e);
+        w[(e * ES) / 4] |= x << (8 * ((e * ES) % 4));
+      }
+    }
+    v = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  return v;
+}
+
+// Per-thread source bookkeeping for one operand: byte pointer of each chunk at
+// k = 0, how many elements along the contiguous direction are in range, and
+// where the chunk goes in the LDS tile.
+template <int ES, int ROWS, bool KC>
+struct Loader {
+  using T = Tile<ES, ROWS, KC>;
+  const char *src[T::kPerThread];
+  long mn_valid[T::kPerThread];  // KC: 1/0 row in range; MC: elements in range along MN
+  int k_off[T::kPerThread];      // KC: k element offset of the chunk; MC: k row
+  unsigned lds_off[T::kPerThread];
+  size_t k_step;                 // bytes per slice along K
+  size_t sk_bytes;
+
+  __device__ void init(const char *base, size_t mn0, size_t mn_dim, size_t s1, size_t s0, size_t sk) {
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < T::kPerThread; ++i) {
+      const int q = t + kThreads * i;
+      if (KC) {
+        const int row = q >> 3, c = q & 7;
+        const size_t r = mn0 + row;
+        src[i] = base + ((r >> 6) * s1 + (r & 63) * s0 + (size_t)c * T::CE) * ES;
+        mn_valid[i] = r < mn_dim ? 1 : 0;
+        k_off[i] = c * T::CE;
+        lds_off[i] = row * kPitchKC + c * 16;
+      } else {
+        const int mc = q % T::kMnChunks, kr = q / T::kMnChunks;
+        const size_t r = mn0 + (size_t)mc * T::CE;
+        src[i] = base + ((r >> 6) * s1 + (r & 63) + (size_t)kr * sk) * ES;
+        mn_valid[i] = (long)mn_dim - (long)r;
+        k_off[i] = kr;
+        lds_off[i] = kr * T::kPitchMC + mc * 16;
+      }
+    }
+    sk_bytes = sk * ES;
+    k_step = KC ? (size_t)kSliceBytes : (size_t)T::KE * sk * ES;
+  }
+
+  __device__ __forceinline__ void fetch(uint4 (&regs)[T::kPerThread], size_t slice, size_t k_dim) const {
+    const long k0 = (long)(slice * T::KE);
+#pragma unroll
+    for (int i = 0; i < T::kPerThread; ++i) {
+      const char *p = src[i] + slice * k_step;
+      long valid;
+      if (KC)
+        valid = mn_valid[i] ? (long)k_dim - (k0 + k_off[i]) : 0;
+      else
+        valid = (k0 + k_off[i] < (long)k_dim) ? mn_valid[i] : 0;
+      regs[i] = load_chunk<ES>(p, valid);
+    }
+  }
+
+  __device__ __forceinline__ void stash(char *tile, const uint4 (&regs)[T::kPerThread]) const {
+#pragma unroll
+    for (int i = 0; i < T::kPerThread; ++i) *reinterpret_cast<uint4 *>(tile + lds_off[i]) = regs[i];
+  }
+};
+
+// Reads the MFMA operand fragment of 32 rows starting at `row0` for the k-step
+// that starts `kb` bytes into the slice. FRB = bytes per lane (16 or 32).
+template <int ES, int ROWS, bool KC, int FRB>
+__device__ __forceinline__ auto read_frag(const char *tile, int row0, int kb) {
+  using T = Tile<ES, ROWS, KC>;
+  const int lane = threadIdx.x & 63;
+  const int h = lane >> 5;  // which half of the k-step this lane feeds
+  if constexpr (KC) {
+    const char *p = tile + (row0 + (lane & 31)) * kPitchKC + kb + h * FRB;
+    if constexpr (FRB == 16) {
+      return *reinterpret_cast<const v4i *>(p);
+    } else {
+      const v4i lo = *reinterpret_cast<const v4i *>(p), hi = *reinterpret_cast<const v4i *>(p + 16);
+      return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+  } else if constexpr (ES == 1) {
+    // ds_read_b64_tr_b8: 16 lanes read an 8 (k) x 16 (mn) byte block; lane j receives column j.
+    const int g16 = (lane >> 4) & 1, j = lane & 15;
+    const int kfirst = kb + h * FRB + (j >> 1);
+    const char *p = tile + kfirst * T::kPitchMC + row0 + g16 * 16 + (j & 1) * 8;
+    v2i r[FRB / 8];
+#pragma unroll
+    for (int s = 0; s < FRB / 8; ++s) r[s] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, p + s * 8 * T::kPitchMC));
+    if constexpr (FRB == 16) {
+      return v4i{r[0].x, r[0].y, r[1].x, r[1].y};
+    } else {
+      return v8i{r[0].x, r[0].y, r[1].x, r[1].y, r[2].x, r[2].y, r[3].x, r[3].y};
+    }
+  } else {
+    // ds_read_b64_tr_b16: 16 lanes read a 4 (k) x 16 (mn) block of 16-bit elements.
+    static_assert(FRB == 16, "16-bit fragments are 16 bytes");
+    const int g16 = (lane >> 4) & 1, j = lane & 15;
+    const int kfirst = kb / 2 + h * 8 + (j >> 2);
+    const char *p = tile + kfirst * T::kPitchMC + (row0 + g16 * 16 + (j & 3) * 4) * 2;
+    const v4s r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(v4s, p));
+    const v4s r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(v4s, p + 4 * T::kPitchMC));
+    const v2i a = __builtin_bit_cast(v2i, r0), b = __builtin_bit_cast(v2i, r1);
+    return v4i{a.x, a.y, b.x, b.y};
+  }
+}
+
+__device__ __forceinline__ int epilogue(int acc, int c, skl_scalar alpha, skl_scalar beta) {
+  return (int)((unsigned)beta.i * (unsigned)c + (unsigned)alpha.i * (unsigned)acc);
+}
+__device__ __forceinline__ float epilogue(float acc, float c, skl_scalar alpha, skl_scalar beta) {
+  return __fadd_rn(__fmul_rn(beta.f, c), __fmul_rn(alpha.f, acc));
+}
+
+// Tile index of a workgroup. Consecutive workgroup ids go to different XCDs
+// (eight of them, each with its own L2), so ids are first regrouped per XCD into
+// contiguous ranges, then walked in column-major groups of kGroupM tile rows so
+// that the tiles resident on one XCD at a time share A and B panels.
+__device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, unsigned tiles_n, unsigned &tm,
+                                              unsigned &tn) {
+  constexpr unsigned kXcd = 8, kGroupM = 8;
+  const unsigned total = tiles_m * tiles_n;
+  unsigned t = bid;
+  if (total % kXcd == 0) t = (bid % kXcd) * (total / kXcd) + bid / kXcd;
+  const unsigned per_group = kGroupM * tiles_n;
+  const unsigned group = t / per_group, first_m = group * kGroupM;
+  const unsigned rows = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
+  const unsigned in_group = t % per_group;
+  tm = first_m + in_group % rows;
+  tn = in_group / rows;
+}
+
+template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN>
+__global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(MfmaArgs p) {
+  using KA = Kind<TA>;
+  using M = Mma<TA, TB>;
+  using Acc = typename KA::Acc;
+  using AccElem = decltype(Acc{}.x);
+  constexpr int ES = KA::ES;
+  constexpr int KB = KA::KB;                    // bytes of K per MFMA
+  constexpr int FRB = KB / 2;                   // fragment bytes per lane
+  constexpr int WM = BM / 2, WN = BN / 4;       // wave tile
+  constexpr int MI = WM / 32, NI = WN / 32;     // MFMA blocks per wave
+  using TileA = Tile<ES, BM, A_KC>;
+  using TileB = Tile<ES, BN, B_KC>;
+  constexpr int kStage = TileA::kBytes + TileB::kBytes;
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  unsigned tm, tn;
+  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave >> 2) * WM, wn = (wave & 3) * WN;
+
+  Loader<ES, BM, A_KC> la;
+  Loader<ES, BN, B_KC> lb;
+  la.init(p.a, m0, p.m, p.a_s1, p.a_s0, p.a_sk);
+  lb.init(p.b, n0, p.n, p.b_s1, p.b_s0, p.b_sk);
+
+  Acc acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  const size_t slices = (p.k * ES + kSliceBytes - 1) / kSliceBytes;
+  uint4 ra[TileA::kPerThread], rb[TileB::kPerThread];
+  la.fetch(ra, 0, p.k);
+  lb.fetch(rb, 0, p.k);
+  la.stash(smem, ra);
+  lb.stash(smem + TileA::kBytes, rb);
+  __syncthreads();
+
+  for (size_t s = 0; s < slices; ++s) {
+    const char *ta = smem + (s & 1) * kStage;
+    const char *tb = ta + TileA::kBytes;
+    const bool more = s + 1 < slices;
+    if (more) {  // next slice: global -> registers while this one is multiplied
+      la.fetch(ra, s + 1, p.k);
+      lb.fetch(rb, s + 1, p.k);
+    }
+#pragma unroll
+    for (int kb = 0; kb < kSliceBytes; kb += KB) {
+      typename M::Frag fa[MI], fb[NI];
+#pragma unroll
+      for (int i = 0; i < MI; ++i) fa[i] = read_frag<ES, BM, A_KC, FRB>(ta, wm + i * 32, kb);
+#pragma unroll
+      for (int j = 0; j < NI; ++j) fb[j] = read_frag<ES, BN, B_KC, FRB>(tb, wn + j * 32, kb);
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = M::run(fa[i], fb[j], acc[i][j]);
+    }
+    if (more) {
+      char *na = smem + ((s + 1) & 1) * kStage;
+      la.stash(na, ra);
+      lb.stash(na + TileA::kBytes, rb);
+    }
+    __syncthreads();
+  }
+
+  // Epilogue: lane l of a 32x32 block holds column l%32 and rows 8*(r/4) + 4*(l/32) + r%4.
+  AccElem *c = reinterpret_cast<AccElem *>(p.c);
+  const bool read_c = !(TA == SKL_DT_I8 && p.beta.i == 0);  // 0*c == 0 only for integers
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const size_t col = n0 + wn + j * 32 + (lane & 31);
+    if (col >= p.n) continue;
+    const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const size_t row = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (row < p.m) {
+          AccElem *out = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
+          const AccElem old = read_c ? *out : (AccElem)0;
+          *out = epilogue(acc[i][j][r], old, p.alpha, p.beta);
+        }
+      }
+    }
+  }
+}
+
+template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN>
+int launch_one(const MfmaArgs &args) {
+  constexpr int ES = Kind<TA>::ES;
+  constexpr int lds = 2 * (Tile<ES, BM, A_KC>::kBytes + Tile<ES, BN, B_KC>::kBytes);
+  auto kernel = gemm_mfma_kernel<TA, TB, A_KC, B_KC, BM, BN>;
+  static bool configured = false;  // per instantiation; racing threads would set the same value
+  if (!configured) {
+    int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "gemm_mfma: LDS size");
+    if (rc != 0) return rc;
+    configured = true;
+  }
+  MfmaArgs p = args;
+  p.tiles_m = skl_div_up(p.m, BM);
+  p.tiles_n = skl_div_up(p.n, BN);
+  const size_t grid = (size_t)p.tiles_m * p.tiles_n;
+  if (grid > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemm_mfma: grid too large");
+    return -2;
+  }
+  kernel<<<(unsigned)grid, kThreads, lds, skl_current_stream()>>>(p);
+  return skl_check_launch("gemm_mfma");
+}
+
+template <int TA, int TB, bool A_KC, bool B_KC>
+int launch_tile(const MfmaArgs &p) {
+  // Large tiles once they alone can fill the 256 compute units, small ones otherwise.
+  const size_t big_tiles = ((p.m + 255) / 256) * ((p.n + 255) / 256);
+  if (big_tiles >= 192) return launch_one<TA, TB, A_KC, B_KC, 256, 256>(p);
+  return launch_one<TA, TB, A_KC, B_KC, 128, 128>(p);
+}
+
+template <int TA, int TB>
+int launch_layout(const MfmaArgs &p) {
+  const bool a_kc = p.a_sk == 1, b_kc = p.b_sk == 1;
+  if (a_kc && b_kc) return launch_tile<TA, TB, true, true>(p);
+  if (a_kc) return launch_tile<TA, TB, true, false>(p);
+  if (b_kc) return launch_tile<TA, TB, false, true>(p);
+  return launch_tile<TA, TB, false, false>(p);
+}
+
+inline bool mult16(size_t bytes) { return (bytes & 15) == 0; }
+
+// One operand: exactly one unit stride; the other strides and the base 16-byte aligned.
+bool operand_ok(const void *base, size_t es, size_t s1, size_t s0, size_t sk, size_t mn, size_t k) {
+  if (((uintptr_t)base & 15) != 0) return false;
+  if (sk == 1) {  // K-contiguous: rows anywhere on 16-byte boundaries
+    return (mn <= 1 || mult16(s0 * es)) && (mn <= 64 || mult16(s1 * es));
+  }
+  if (s0 == 1) {  // MN-contiguous in runs of 64 elements
+    return (k <= 1 || mult16(sk * es)) && (mn <= 64 || mult16(s1 * es));
+  }
+  return false;
+}
+
+}  // namespace
+
+extern "C" int skl_hip_gemm_mfma_supported(const skl_gemm_canon *g) {
+  if (g->m == 0 || g->n == 0 || g->k == 0) return 0;
+  const bool fp8a = g->ta == SKL_DT_F8E4M3 || g->ta == SKL_DT_F8E5M2;
+  const bool fp8b = g->tb == SKL_DT_F8E4M3 || g->tb == SKL_DT_F8E5M2;
+  if (!(g->ta == g->tb || (fp8a && fp8b))) return 0;
+  const size_t es = (g->ta == SKL_DT_BF16 || g->ta == SKL_DT_F16) ? 2 : 1;
+  if (!operand_ok(g->a, es, g->a_s1, g->a_s0, g->a_sk, g->m, g->k)) return 0;
+  if (!operand_ok(g->b, es, g->b_s1, g->b_s0, g->b_sk, g->n, g->k)) return 0;
+  if (((uintptr_t)g->c & 3) != 0) return 0;
+  return 1;
+}
+
+extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
+  if (!skl_hip_gemm_mfma_supported(g)) {
+    skl_hip_record_error(-2, "gemm_mfma: unsupported problem");
+    return -2;
+  }
+  MfmaArgs p;
+  p.a = (const char *)g->a;
+  p.b = (const char *)g->b;
+  p.c = (char *)g->c;
+  p.m = g->m, p.n = g->n, p.k = g->k;
+  p.a_s1 = g->a_s1, p.a_s0 = g->a_s0, p.a_sk = g->a_sk;
+  p.b_s1 = g->b_s1, p.b_s0 = g->b_s0, p.b_sk = g->b_sk;
+  p.rsc0 = g->rsc0, p.csc0 = g->csc0, p.rsc1 = g->rsc1, p.csc1 = g->csc1;
+  p.alpha = g->alpha, p.beta = g->beta;
+  p.tiles_m = p.tiles_n = 0;
+  switch (g->ta * 8 + g->tb) {
+    case SKL_DT_I8 * 8 + SKL_DT_I8: return launch_layout<SKL_DT_I8, SKL_DT_I8>(p);
+    case SKL_DT_BF16 * 8 + SKL_DT_BF16: return launch_layout<SKL_DT_BF16, SKL_DT_BF16>(p);
+    case SKL_DT_F16 * 8 + SKL_DT_F16: return launch_layout<SKL_DT_F16, SKL_DT_F16>(p);
+    case SKL_DT_F8E4M3 * 8 + SKL_DT_F8E4M3: return launch_layout<SKL_DT_F8E4M3, SKL_DT_F8E4M3>(p);
+    case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E5M2: return launch_layout<SKL_DT_F8E5M2, SKL_DT_F8E5M2>(p);
+    case SKL_DT_F8E4M3 * 8 + SKL_DT_F8E5M2: return launch_layout<SKL_DT_F8E4M3, SKL_DT_F8E5M2>(p);
+    case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E4M3: return launch_layout<SKL_DT_F8E5M2, SKL_DT_F8E4M3>(p);
+    default:
+      skl_hip_record_error(-2, "gemm_mfma: operand type pair");
+      return -2;
+  }
+}
