@@ -13,8 +13,10 @@
 // One kernel template serves every layout pair. Each operand is either
 // "K-contiguous" (row-major A, column-major B) or "MN-contiguous" (column-major
 // A, row-major B, and both panel formats); blocks of 64 along M / N may sit
-// anywhere (block stride), which is what the panel formats need. A workgroup of
-// eight waves owns a BM x BN tile of C; per 128-byte slice of K it copies the
+// anywhere (block stride), which is what the panel formats need. A workgroup
+// owns a BM x BN tile of C (256 x 256 on four waves of 128 x 128 each - the
+// largest accumulator block a wave's 512 registers hold, which minimises LDS
+// reads per MFMA - or 128 x 128 on eight waves for small or ragged problems); per 128-byte slice of K it copies the
 // A and B tiles global -> registers -> LDS in their native orientation with
 // 128-bit accesses (double-buffered: the next slice is in flight while the
 // current one is multiplied) and the waves read MFMA operands straight from
@@ -42,7 +44,6 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T *)(p))
 
-constexpr int kThreads = 512;       // 8 waves: 2 along M x 4 along N
 constexpr int kSliceBytes = 128;    // bytes of K per LDS stage and operand row
 constexpr int kPitchKC = 144;       // LDS row pitch of a K-contiguous tile
 
@@ -126,25 +127,27 @@ SKL_F8_MMA(SKL_DT_F8E5M2, SKL_DT_F8E4M3, 1, 0)
 // ---------------------------------------------------------------------------
 // LDS tile geometry of one operand: ROWS along M or N, 128 bytes of K.
 // ---------------------------------------------------------------------------
-template <int ES, int ROWS, bool KC>
+template <int ES, int ROWS, bool KC, int NT>
 struct Tile {
   static constexpr int CE = 16 / ES;                 // elements per 16-byte chunk
   static constexpr int KE = kSliceBytes / ES;        // k elements per slice
-  // MN-contiguous tile: KE rows of ROWS*ES bytes, padded so that the rows one
-  // transpose load touches (8 rows x 16 B, or 4 rows x 32 B) hit distinct banks.
-  static constexpr int kPitchMC = ROWS * ES + (ES == 1 ? 16 : 32);
+  // MN-contiguous tile: KE rows of ROWS*ES bytes. A transpose load is served 32
+  // lanes at a time: 8 rows x 32 B (8-bit) or 4 rows x 64 B (16-bit). Skewing
+  // consecutive rows by that width spreads them over all 64 banks (measured:
+  // zero bank conflicts with 32 / 64 bytes of padding, conflicts with 16 / 32).
+  static constexpr int kPitchMC = ROWS * ES + (ES == 1 ? 32 : 64);
   static constexpr int kBytes = KC ? ROWS * kPitchKC : KE * kPitchMC;
   static constexpr int kChunks = ROWS * 8;           // 16-byte chunks per slice
-  static constexpr int kPerThread = kChunks / kThreads;
+  static constexpr int kPerThread = kChunks / NT;    // chunks each of the NT threads moves
   static constexpr int kMnChunks = ROWS * ES / 16;   // chunks along MN of an MN-contiguous row
 };
 
 // 16 bytes from global memory with `valid` (<= CE) leading elements in range.
 template <int ES>
-__device__ __forceinline__ uint4 load_chunk(const char *p, long valid) {
+__device__ __forceinline__ v4i load_chunk(const char *p, long valid) {
   constexpr int CE = 16 / ES;
-  if (valid >= CE) return *reinterpret_cast<const uint4 *>(p);
-  uint4 v = make_uint4(0, 0, 0, 0);
+  if (valid >= CE) return *reinterpret_cast<const v4i *>(p);
+  v4i v = {0, 0, 0, 0};
   if (valid > 0) {
     unsigned w[4] = {0, 0, 0, 0};
     for (int e = 0; e < CE; ++e) {
@@ -154,66 +157,83 @@ __device__ __forceinline__ uint4 load_chunk(const char *p, long valid) {
         w[(e * ES) / 4] |= x << (8 * ((e * ES) % 4));
       }
     }
-    v = make_uint4(w[0], w[1], w[2], w[3]);
+    v = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
   }
   return v;
 }
 
-// Per-thread source bookkeeping for one operand: byte pointer of each chunk at
-// k = 0, how many elements along the contiguous direction are in range, and
-// where the chunk goes in the LDS tile.
-template <int ES, int ROWS, bool KC>
+// Per-thread source bookkeeping for one operand. A chunk's address is a
+// workgroup-uniform 64-bit tile base (advanced by one slice per iteration) plus
+// a 32-bit per-thread offset, so the loop carries one scalar pointer instead of
+// a vector pointer per chunk.
+template <int ES, int ROWS, bool KC, int NT>
 struct Loader {
-  using T = Tile<ES, ROWS, KC>;
-  const char *src[T::kPerThread];
-  long mn_valid[T::kPerThread];  // KC: 1/0 row in range; MC: elements in range along MN
-  int k_off[T::kPerThread];      // KC: k element offset of the chunk; MC: k row
+  using T = Tile<ES, ROWS, KC, NT>;
+  const char *tile_base;         // uniform: first byte of the tile's first 64-block at k = 0
+  size_t k_step;                 // bytes between consecutive slices
+  unsigned off[T::kPerThread];   // byte offset of each chunk from tile_base
   unsigned lds_off[T::kPerThread];
-  size_t k_step;                 // bytes per slice along K
-  size_t sk_bytes;
+  long mn_valid[T::kPerThread];  // guarded path - KC: row in range (1/0); MC: elements in range along MN
+  int k_off[T::kPerThread];      // guarded path - KC: k element offset of the chunk; MC: k row
 
   __device__ void init(const char *base, size_t mn0, size_t mn_dim, size_t s1, size_t s0, size_t sk) {
     const int t = threadIdx.x;
+    tile_base = base + (mn0 >> 6) * s1 * ES;  // mn0 is a multiple of 64
 #pragma unroll
     for (int i = 0; i < T::kPerThread; ++i) {
-      const int q = t + kThreads * i;
+      const int q = t + NT * i;
       if (KC) {
         const int row = q >> 3, c = q & 7;
-        const size_t r = mn0 + row;
-        src[i] = base + ((r >> 6) * s1 + (r & 63) * s0 + (size_t)c * T::CE) * ES;
-        mn_valid[i] = r < mn_dim ? 1 : 0;
+        off[i] = (unsigned)(((size_t)(row >> 6) * s1 + (size_t)(row & 63) * s0 + (size_t)c * T::CE) * ES);
+        mn_valid[i] = mn0 + row < mn_dim ? 1 : 0;
         k_off[i] = c * T::CE;
         lds_off[i] = row * kPitchKC + c * 16;
       } else {
         const int mc = q % T::kMnChunks, kr = q / T::kMnChunks;
-        const size_t r = mn0 + (size_t)mc * T::CE;
-        src[i] = base + ((r >> 6) * s1 + (r & 63) + (size_t)kr * sk) * ES;
-        mn_valid[i] = (long)mn_dim - (long)r;
+        const int r = mc * T::CE;
+        off[i] = (unsigned)(((size_t)(r >> 6) * s1 + (size_t)(r & 63) + (size_t)kr * sk) * ES);
+        mn_valid[i] = (long)mn_dim - (long)(mn0 + r);
         k_off[i] = kr;
         lds_off[i] = kr * T::kPitchMC + mc * 16;
       }
     }
-    sk_bytes = sk * ES;
     k_step = KC ? (size_t)kSliceBytes : (size_t)T::KE * sk * ES;
   }
 
-  __device__ __forceinline__ void fetch(uint4 (&regs)[T::kPerThread], size_t slice, size_t k_dim) const {
+  // Interior tiles of problems whose extents are multiples of the tile: every chunk is whole.
+  __device__ __forceinline__ void fetch_whole(v4i (&regs)[T::kPerThread], size_t slice) const {
+    const char *b = tile_base + slice * k_step;
+#pragma unroll
+    for (int i = 0; i < T::kPerThread; ++i) regs[i] = *reinterpret_cast<const v4i *>(b + off[i]);
+  }
+
+  // Any extents: chunks that stick out of the matrix are zero-filled (zeros along
+  // K add nothing; rows/columns beyond M/N are never stored).
+  __device__ __forceinline__ void fetch_guarded(v4i (&regs)[T::kPerThread], size_t slice, size_t k_dim) const {
     const long k0 = (long)(slice * T::KE);
+    const char *b = tile_base + slice * k_step;
 #pragma unroll
     for (int i = 0; i < T::kPerThread; ++i) {
-      const char *p = src[i] + slice * k_step;
       long valid;
       if (KC)
         valid = mn_valid[i] ? (long)k_dim - (k0 + k_off[i]) : 0;
       else
         valid = (k0 + k_off[i] < (long)k_dim) ? mn_valid[i] : 0;
-      regs[i] = load_chunk<ES>(p, valid);
+      regs[i] = load_chunk<ES>(b + off[i], valid);
     }
   }
 
-  __device__ __forceinline__ void stash(char *tile, const uint4 (&regs)[T::kPerThread]) const {
+  template <bool GUARDED>
+  __device__ __forceinline__ void fetch(v4i (&regs)[T::kPerThread], size_t slice, size_t k_dim) const {
+    if constexpr (GUARDED)
+      fetch_guarded(regs, slice, k_dim);
+    else
+      fetch_whole(regs, slice);
+  }
+
+  __device__ __forceinline__ void stash(char *tile, const v4i (&regs)[T::kPerThread]) const {
 #pragma unroll
-    for (int i = 0; i < T::kPerThread; ++i) *reinterpret_cast<uint4 *>(tile + lds_off[i]) = regs[i];
+    for (int i = 0; i < T::kPerThread; ++i) *reinterpret_cast<v4i *>(tile + lds_off[i]) = regs[i];
   }
 };
 
@@ -221,7 +241,7 @@ struct Loader {
 // that starts `kb` bytes into the slice. FRB = bytes per lane (16 or 32).
 template <int ES, int ROWS, bool KC, int FRB>
 __device__ __forceinline__ auto read_frag(const char *tile, int row0, int kb) {
-  using T = Tile<ES, ROWS, KC>;
+  using T = Tile<ES, ROWS, KC, 64>;
   const int lane = threadIdx.x & 63;
   const int h = lane >> 5;  // which half of the k-step this lane feeds
   if constexpr (KC) {
@@ -283,8 +303,9 @@ __device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, un
   tn = in_group / rows;
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN>
-__global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(MfmaArgs p) {
+template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED>
+__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaArgs p) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
   using KA = Kind<TA>;
   using M = Mma<TA, TB>;
   using Acc = typename KA::Acc;
@@ -292,10 +313,10 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(MfmaArgs p) {
   constexpr int ES = KA::ES;
   constexpr int KB = KA::KB;                    // bytes of K per MFMA
   constexpr int FRB = KB / 2;                   // fragment bytes per lane
-  constexpr int WM = BM / 2, WN = BN / 4;       // wave tile
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
   constexpr int MI = WM / 32, NI = WN / 32;     // MFMA blocks per wave
-  using TileA = Tile<ES, BM, A_KC>;
-  using TileB = Tile<ES, BN, B_KC>;
+  using TileA = Tile<ES, BM, A_KC, NT>;
+  using TileB = Tile<ES, BN, B_KC, NT>;
   constexpr int kStage = TileA::kBytes + TileB::kBytes;
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -304,10 +325,10 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(MfmaArgs p) {
   tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
   const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = (wave >> 2) * WM, wn = (wave & 3) * WN;
+  const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
 
-  Loader<ES, BM, A_KC> la;
-  Loader<ES, BN, B_KC> lb;
+  Loader<ES, BM, A_KC, NT> la;
+  Loader<ES, BN, B_KC, NT> lb;
   la.init(p.a, m0, p.m, p.a_s1, p.a_s0, p.a_sk);
   lb.init(p.b, n0, p.n, p.b_s1, p.b_s0, p.b_sk);
 
@@ -320,39 +341,55 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(MfmaArgs p) {
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
   const size_t slices = (p.k * ES + kSliceBytes - 1) / kSliceBytes;
-  uint4 ra[TileA::kPerThread], rb[TileB::kPerThread];
-  la.fetch(ra, 0, p.k);
-  lb.fetch(rb, 0, p.k);
+  v4i ra[TileA::kPerThread], rb[TileB::kPerThread];
+  la.template fetch<GUARDED>(ra, 0, p.k);
+  lb.template fetch<GUARDED>(rb, 0, p.k);
   la.stash(smem, ra);
   lb.stash(smem + TileA::kBytes, rb);
   __syncthreads();
 
+  constexpr int kSteps = kSliceBytes / KB;  // MFMA k-steps per slice
+  typename M::Frag fa[2][MI], fb[2][NI];    // operand fragments, double-buffered across k-steps
+#pragma unroll
+  for (int i = 0; i < MI; ++i) fa[0][i] = read_frag<ES, BM, A_KC, FRB>(smem, wm + i * 32, 0);
+#pragma unroll
+  for (int j = 0; j < NI; ++j) fb[0][j] = read_frag<ES, BN, B_KC, FRB>(smem + TileA::kBytes, wn + j * 32, 0);
+
   for (size_t s = 0; s < slices; ++s) {
     const char *ta = smem + (s & 1) * kStage;
     const char *tb = ta + TileA::kBytes;
-    const bool more = s + 1 < slices;
-    if (more) {  // next slice: global -> registers while this one is multiplied
-      la.fetch(ra, s + 1, p.k);
-      lb.fetch(rb, s + 1, p.k);
-    }
+    char *na = smem + ((s + 1) & 1) * kStage;
+    // Next slice: global -> registers while this one is multiplied. The last
+    // iteration fetches its own slice again (in range, never consumed) so that
+    // the loop body has no branch around the loads.
+    const size_t nxt = s + 1 < slices ? s + 1 : s;
+    la.template fetch<GUARDED>(ra, nxt, p.k);
+    lb.template fetch<GUARDED>(rb, nxt, p.k);
+    // Keep the loads up here: left alone, the scheduler sinks them to just before
+    // the LDS stores below and the whole memory latency lands on every slice.
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int kb = 0; kb < kSliceBytes; kb += KB) {
-      typename M::Frag fa[MI], fb[NI];
+    for (int ks = 0; ks < kSteps; ++ks) {
+      const int cur = ks & 1, nx = cur ^ 1;
+      if (ks + 1 < kSteps) {  // fragments of the next k-step are requested before this step's MFMAs
 #pragma unroll
-      for (int i = 0; i < MI; ++i) fa[i] = read_frag<ES, BM, A_KC, FRB>(ta, wm + i * 32, kb);
+        for (int i = 0; i < MI; ++i) fa[nx][i] = read_frag<ES, BM, A_KC, FRB>(ta, wm + i * 32, (ks + 1) * KB);
 #pragma unroll
-      for (int j = 0; j < NI; ++j) fb[j] = read_frag<ES, BN, B_KC, FRB>(tb, wn + j * 32, kb);
+        for (int j = 0; j < NI; ++j) fb[nx][j] = read_frag<ES, BN, B_KC, FRB>(tb, wn + j * 32, (ks + 1) * KB);
+      }
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = M::run(fa[i], fb[j], acc[i][j]);
+        for (int j = 0; j < NI; ++j) acc[i][j] = M::run(fa[cur][i], fb[cur][j], acc[i][j]);
     }
-    if (more) {
-      char *na = smem + ((s + 1) & 1) * kStage;
-      la.stash(na, ra);
-      lb.stash(na + TileA::kBytes, rb);
-    }
+    la.stash(na, ra);
+    lb.stash(na + TileA::kBytes, rb);
     __syncthreads();
+    // First fragments of the next slice (kSteps is even, so they land in buffer 0 again).
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[0][i] = read_frag<ES, BM, A_KC, FRB>(na, wm + i * 32, 0);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) fb[0][j] = read_frag<ES, BN, B_KC, FRB>(na + TileA::kBytes, wn + j * 32, 0);
   }
 
   // Epilogue: lane l of a 32x32 block holds column l%32 and rows 8*(r/4) + 4*(l/32) + r%4.
@@ -361,14 +398,14 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(MfmaArgs p) {
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
-    if (col >= p.n) continue;
+    if (GUARDED && col >= p.n) continue;
     const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const size_t row = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        if (row < p.m) {
+        if (!GUARDED || row < p.m) {
           AccElem *out = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
           const AccElem old = read_c ? *out : (AccElem)0;
           *out = epilogue(acc[i][j][r], old, p.alpha, p.beta);
@@ -378,11 +415,12 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(MfmaArgs p) {
   }
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN>
+template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED>
 int launch_one(const MfmaArgs &args) {
   constexpr int ES = Kind<TA>::ES;
-  constexpr int lds = 2 * (Tile<ES, BM, A_KC>::kBytes + Tile<ES, BN, B_KC>::kBytes);
-  auto kernel = gemm_mfma_kernel<TA, TB, A_KC, B_KC, BM, BN>;
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int lds = 2 * (Tile<ES, BM, A_KC, NT>::kBytes + Tile<ES, BN, B_KC, NT>::kBytes);
+  auto kernel = gemm_mfma_kernel<TA, TB, A_KC, B_KC, BM, BN, WAVES_M, WAVES_N, GUARDED>;
   static bool configured = false;  // per instantiation; racing threads would set the same value
   if (!configured) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -399,16 +437,19 @@ int launch_one(const MfmaArgs &args) {
     skl_hip_record_error(-2, "gemm_mfma: grid too large");
     return -2;
   }
-  kernel<<<(unsigned)grid, kThreads, lds, skl_current_stream()>>>(p);
+  kernel<<<(unsigned)grid, NT, lds, skl_current_stream()>>>(p);
   return skl_check_launch("gemm_mfma");
 }
 
 template <int TA, int TB, bool A_KC, bool B_KC>
 int launch_tile(const MfmaArgs &p) {
-  // Large tiles once they alone can fill the 256 compute units, small ones otherwise.
-  const size_t big_tiles = ((p.m + 255) / 256) * ((p.n + 255) / 256);
-  if (big_tiles >= 192) return launch_one<TA, TB, A_KC, B_KC, 256, 256>(p);
-  return launch_one<TA, TB, A_KC, B_KC, 128, 128>(p);
+  constexpr int ES = Kind<TA>::ES;
+  // The large tile takes problems that it divides evenly and that can fill the
+  // 256 compute units with it; everything else runs on the small, bounds-checked one.
+  const bool whole = p.m % 256 == 0 && p.n % 256 == 0 && (p.k * ES) % kSliceBytes == 0;
+  const size_t big_tiles = (p.m / 256) * (p.n / 256);
+  if (whole && big_tiles >= 200) return launch_one<TA, TB, A_KC, B_KC, 256, 256, 2, 2, false>(p);
+  return launch_one<TA, TB, A_KC, B_KC, 128, 128, 2, 4, true>(p);
 }
 
 template <int TA, int TB>
@@ -425,10 +466,14 @@ inline bool mult16(size_t bytes) { return (bytes & 15) == 0; }
 // One operand: exactly one unit stride; the other strides and the base 16-byte aligned.
 bool operand_ok(const void *base, size_t es, size_t s1, size_t s0, size_t sk, size_t mn, size_t k) {
   if (((uintptr_t)base & 15) != 0) return false;
+  // Offsets inside one tile (up to four 64-blocks, 64 rows, 128 k-rows) are kept in 32 bits.
+  const size_t limit = size_t(1) << 31;
   if (sk == 1) {  // K-contiguous: rows anywhere on 16-byte boundaries
+    if (s1 * es * 4 >= limit || s0 * es * 64 >= limit) return false;
     return (mn <= 1 || mult16(s0 * es)) && (mn <= 64 || mult16(s1 * es));
   }
   if (s0 == 1) {  // MN-contiguous in runs of 64 elements
+    if (s1 * es * 4 >= limit || sk * es * 128 >= limit) return false;
     return (k <= 1 || mult16(sk * es)) && (mn <= 64 || mult16(s1 * es));
   }
   return false;
