@@ -29,6 +29,9 @@
 // the accumulator registers in the epilogue.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+#include <utility>
+
 #include "skl_device.hpp"
 
 namespace {
@@ -377,10 +380,16 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
 #pragma unroll
         for (int j = 0; j < NI; ++j) fb[nx][j] = read_frag<ES, BN, B_KC, FRB>(tb, wn + j * 32, (ks + 1) * KB);
       }
+      // The LDS reads above are all issued before the first MFMA below and are
+      // not needed until the next k-step: the scheduler must not pull them
+      // down next to their uses (with one wave per SIMD nothing else would
+      // hide their latency).
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < NI; ++j) acc[i][j] = M::run(fa[cur][i], fb[cur][j], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
     }
     la.stash(na, ra);
     lb.stash(na + TileA::kBytes, rb);
@@ -413,6 +422,262 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
       }
     }
   }
+}
+
+// ===========================================================================
+// Streaming variant for whole 256 x 256 tiles: global -> LDS without passing
+// through registers (global_load_lds_dwordx4). Each wave-level load deposits
+// 64 x 16 bytes as one contiguous KiB of LDS, so the tiles are stored without
+// padding and bank conflicts are avoided by an XOR swizzle of the 16-byte
+// chunk index instead; the swizzle is applied on the global side (which chunk
+// a lane fetches) and again by the fragment reads. Four waves, one per SIMD,
+// each own a 128 x 128 block of C (256 accumulator registers): half the LDS
+// bytes per MFMA of a 128 x 64 block, and the registers and LDS-store
+// instructions of the staged copy are gone, which matters because a wave's
+// instruction stream is serial - every load or LDS store it issues is a slot
+// in which it issues no MFMA.
+// ===========================================================================
+template <int ES, bool KC>
+struct STile {
+  static constexpr int kBytes = 256 * kSliceBytes;  // 256 rows x 128 bytes of K, 32 KiB
+  // Byte offset of 16-byte chunk `c` of line `r`. A line is an M/N row holding
+  // 128 bytes of K (KC), or a k-row holding 256 elements along M/N (MC).
+  __device__ static __forceinline__ int chunk(int r, int c) {
+    if constexpr (KC)
+      return r * 128 + ((c ^ ((r >> 1) & 7)) << 4);   // 8 chunks; b128 reads take 16 consecutive rows
+    else if constexpr (ES == 1)
+      return r * 256 + ((c ^ ((r & 7) << 1)) << 4);   // 16 chunks; tr8 reads take 8 k-rows x 32 B
+    else
+      return r * 512 + ((c ^ ((r & 3) << 2)) << 4);   // 32 chunks; tr16 reads take 4 k-rows x 64 B
+  }
+};
+
+template <int ES, bool KC, int WAVES>
+struct SLoader {
+  static constexpr int kBlocks = 32 / WAVES;  // KiB blocks per wave, operand and slice
+  const char *tile_base;
+  size_t k_step;
+  unsigned off[kBlocks];
+  unsigned lds_block;  // byte offset of this wave's first block inside the operand tile
+
+  __device__ void init(const char *base, size_t mn0, size_t s1, size_t s0, size_t sk) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    tile_base = base + (mn0 >> 6) * s1 * ES;
+    lds_block = wave * kBlocks * 1024;
+#pragma unroll
+    for (int i = 0; i < kBlocks; ++i) {
+      const int b = wave * kBlocks + i;
+      if constexpr (KC) {
+        const int row = 8 * b + (lane >> 3), pos = lane & 7;
+        const int c = pos ^ ((row >> 1) & 7);
+        off[i] = (unsigned)(((size_t)(row >> 6) * s1 + (size_t)(row & 63) * s0 + (size_t)c * (16 / ES)) * ES);
+      } else if constexpr (ES == 1) {
+        const int kr = 4 * b + (lane >> 4), pos = lane & 15;
+        const int mn = (pos ^ ((kr & 7) << 1)) * 16;
+        off[i] = (unsigned)((size_t)(mn >> 6) * s1 + (size_t)(mn & 63) + (size_t)kr * sk);
+      } else {
+        const int kr = 2 * b + (lane >> 5), pos = lane & 31;
+        const int mn = (pos ^ ((kr & 3) << 2)) * 8;
+        off[i] = (unsigned)(((size_t)(mn >> 6) * s1 + (size_t)(mn & 63) + (size_t)kr * sk) * 2);
+      }
+    }
+    k_step = KC ? (size_t)kSliceBytes : (size_t)(kSliceBytes / ES) * sk * ES;
+  }
+
+  // Requests this wave's eight blocks of `slice`; the data lands in `tile` (LDS).
+  __device__ __forceinline__ void issue(char *tile, size_t slice) const {
+    const char *g = tile_base + slice * k_step;
+#pragma unroll
+    for (int i = 0; i < kBlocks; ++i) {
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(g + off[i]),
+                                       (__attribute__((address_space(3))) void *)(tile + lds_block + i * 1024), 16, 0, 0);
+    }
+  }
+};
+
+template <int ES, bool KC, int FRB>
+__device__ __forceinline__ auto read_frag_s(const char *tile, int row0, int kb) {
+  using T = STile<ES, KC>;
+  const int lane = threadIdx.x & 63;
+  const int h = lane >> 5;
+  if constexpr (KC) {
+    const int row = row0 + (lane & 31), c0 = (kb + h * FRB) >> 4;
+    if constexpr (FRB == 16) {
+      return *reinterpret_cast<const v4i *>(tile + T::chunk(row, c0));
+    } else {
+      const v4i lo = *reinterpret_cast<const v4i *>(tile + T::chunk(row, c0));
+      const v4i hi = *reinterpret_cast<const v4i *>(tile + T::chunk(row, c0 + 1));
+      return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+  } else if constexpr (ES == 1) {
+    const int g16 = (lane >> 4) & 1, j = lane & 15;
+    const int kfirst = kb + h * FRB + (j >> 1), c = (row0 >> 4) + g16, sub = (j & 1) * 8;
+    v2i r[FRB / 8];
+#pragma unroll
+    for (int s = 0; s < FRB / 8; ++s)
+      r[s] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, tile + T::chunk(kfirst + 8 * s, c) + sub));
+    if constexpr (FRB == 16) {
+      return v4i{r[0].x, r[0].y, r[1].x, r[1].y};
+    } else {
+      return v8i{r[0].x, r[0].y, r[1].x, r[1].y, r[2].x, r[2].y, r[3].x, r[3].y};
+    }
+  } else {
+    static_assert(FRB == 16, "16-bit fragments are 16 bytes");
+    const int g16 = (lane >> 4) & 1, j = lane & 15;
+    const int kfirst = kb / 2 + h * 8 + (j >> 2);
+    const int c = (row0 >> 3) + g16 * 2 + ((j & 3) >> 1), sub = (j & 1) * 8;
+    const v4s r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(v4s, tile + T::chunk(kfirst, c) + sub));
+    const v4s r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(v4s, tile + T::chunk(kfirst + 4, c) + sub));
+    const v2i a = __builtin_bit_cast(v2i, r0), b = __builtin_bit_cast(v2i, r1);
+    return v4i{a.x, a.y, b.x, b.y};
+  }
+}
+
+// Scheduling recipe for one k-step of the streaming kernel: after each of the
+// MFMAs place this step's share of LDS reads (ND in total) and of global
+// loads (NV in total), evenly spread. A wave issues in order, so a burst of 16
+// loads or 12 LDS reads in front of the MFMAs is a stretch in which the matrix
+// pipe of its SIMD has nothing to do; one memory instruction in the shadow of
+// each MFMA costs nothing.
+template <int NM, int ND, int NV, int M>
+__device__ __forceinline__ void sched_slot() {
+  constexpr int d = (M + 1) * ND / NM - M * ND / NM;
+  constexpr int v = (M + 1) * NV / NM - M * NV / NM;
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // one MFMA
+  if constexpr (d > 0) __builtin_amdgcn_sched_group_barrier(0x100, d, 0);  // LDS reads
+  if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);  // global loads
+}
+template <int ND, int NV, int... Ms>
+__device__ __forceinline__ void sched_kstep(std::integer_sequence<int, Ms...>) {
+  (sched_slot<(int)sizeof...(Ms), ND, NV, Ms>(), ...);
+}
+
+template <int TA, int TB, bool A_KC, bool B_KC, int WAVES_N>
+__global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_stream_kernel(MfmaArgs p) {
+  using KA = Kind<TA>;
+  using M = Mma<TA, TB>;
+  using Acc = typename KA::Acc;
+  using AccElem = decltype(Acc{}.x);
+  constexpr int ES = KA::ES, KB = KA::KB, FRB = KB / 2;
+  constexpr int BM = 256, BN = 256, WM = 128, WN = BN / WAVES_N, MI = 4, NI = WN / 32, WAVES = 2 * WAVES_N;
+  constexpr int kTile = STile<ES, true>::kBytes, kStage = 2 * kTile;
+  constexpr int kSteps = kSliceBytes / KB;
+  // LDS read instructions per k-step: b128 per 16 fragment bytes of a K-contiguous
+  // operand, one transpose load per 8 fragment bytes of an MN-contiguous one.
+  constexpr int kReadsA = MI * (A_KC ? FRB / 16 : FRB / 8), kReadsB = NI * (B_KC ? FRB / 16 : FRB / 8);
+  constexpr int kLoadsPerStep = 2 * (32 / WAVES) / kSteps;
+  constexpr int kMfmas = MI * NI;
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  unsigned tm, tn;
+  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
+
+  SLoader<ES, A_KC, WAVES> la;
+  SLoader<ES, B_KC, WAVES> lb;
+  la.init(p.a, m0, p.a_s1, p.a_s0, p.a_sk);
+  lb.init(p.b, n0, p.b_s1, p.b_s0, p.b_sk);
+
+  Acc acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  const size_t slices = p.k * ES / kSliceBytes;
+  la.issue(smem, 0);
+  lb.issue(smem + kTile, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  typename M::Frag fa[2][MI], fb[2][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i) fa[0][i] = read_frag_s<ES, A_KC, FRB>(smem, wm + i * 32, 0);
+#pragma unroll
+  for (int j = 0; j < NI; ++j) fb[0][j] = read_frag_s<ES, B_KC, FRB>(smem + kTile, wn + j * 32, 0);
+
+  for (size_t s = 0; s < slices; ++s) {
+    const char *ta = smem + (s & 1) * kStage;
+    const char *tb = ta + kTile;
+    char *na = smem + ((s + 1) & 1) * kStage;
+    // The other stage was last read before the barrier that ended the previous
+    // iteration: the next slice streams into it while this one is multiplied.
+    // (The last iteration requests its own slice again: in range, never read.)
+    const size_t nxt = s + 1 < slices ? s + 1 : s;
+    la.issue(na, nxt);
+    lb.issue(na + kTile, nxt);
+#pragma unroll
+    for (int ks = 0; ks < kSteps; ++ks) {
+      const int cur = ks & 1, nx = cur ^ 1;
+      if (ks + 1 < kSteps) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fa[nx][i] = read_frag_s<ES, A_KC, FRB>(ta, wm + i * 32, (ks + 1) * KB);
+#pragma unroll
+        for (int j = 0; j < NI; ++j) fb[nx][j] = read_frag_s<ES, B_KC, FRB>(tb, wn + j * 32, (ks + 1) * KB);
+      }
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = M::run(fa[cur][i], fb[cur][j], acc[i][j]);
+      if (ks + 1 < kSteps)
+        sched_kstep<kReadsA + kReadsB, kLoadsPerStep>(std::make_integer_sequence<int, kMfmas>{});
+      else
+        sched_kstep<0, kLoadsPerStep>(std::make_integer_sequence<int, kMfmas>{});
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[0][i] = read_frag_s<ES, A_KC, FRB>(na, wm + i * 32, 0);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) fb[0][j] = read_frag_s<ES, B_KC, FRB>(na + kTile, wn + j * 32, 0);
+  }
+
+  AccElem *c = reinterpret_cast<AccElem *>(p.c);
+  const bool read_c = !(TA == SKL_DT_I8 && p.beta.i == 0);
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const size_t col = n0 + wn + j * 32 + (lane & 31);
+    const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const size_t row = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        AccElem *out = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
+        const AccElem old = read_c ? *out : (AccElem)0;
+        *out = epilogue(acc[i][j][r], old, p.alpha, p.beta);
+      }
+    }
+  }
+}
+
+template <int TA, int TB, bool A_KC, bool B_KC, int WAVES_N>
+int launch_stream(const MfmaArgs &args) {
+  constexpr int lds = 4 * STile<1, true>::kBytes;  // two stages of two 32 KiB tiles
+  auto kernel = gemm_mfma_stream_kernel<TA, TB, A_KC, B_KC, WAVES_N>;
+  static bool configured = false;
+  if (!configured) {
+    int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "gemm_mfma_stream: LDS size");
+    if (rc != 0) return rc;
+    configured = true;
+  }
+  MfmaArgs p = args;
+  p.tiles_m = (unsigned)(p.m / 256);
+  p.tiles_n = (unsigned)(p.n / 256);
+  const size_t grid = (size_t)p.tiles_m * p.tiles_n;
+  if (grid > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemm_mfma: grid too large");
+    return -2;
+  }
+  kernel<<<(unsigned)grid, 128 * WAVES_N, lds, skl_current_stream()>>>(p);
+  return skl_check_launch("gemm_mfma_stream");
 }
 
 template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED>
@@ -448,7 +713,11 @@ int launch_tile(const MfmaArgs &p) {
   // 256 compute units with it; everything else runs on the small, bounds-checked one.
   const bool whole = p.m % 256 == 0 && p.n % 256 == 0 && (p.k * ES) % kSliceBytes == 0;
   const size_t big_tiles = (p.m / 256) * (p.n / 256);
-  if (whole && big_tiles >= 200) return launch_one<TA, TB, A_KC, B_KC, 256, 256, 2, 2, false>(p);
+  if (whole && big_tiles >= 200) {
+    static const int waves_n = getenv("SKL_STREAM_WAVES_N") ? atoi(getenv("SKL_STREAM_WAVES_N")) : 4;
+    if (waves_n == 2) return launch_stream<TA, TB, A_KC, B_KC, 2>(p);
+    return launch_stream<TA, TB, A_KC, B_KC, 4>(p);
+  }
   return launch_one<TA, TB, A_KC, B_KC, 128, 128, 2, 4, true>(p);
 }
 

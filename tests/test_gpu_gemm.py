@@ -140,3 +140,45 @@ def test_zero_m_or_n_touches_nothing(gpu):
     gpu.skl_gemm_i8_i8_i32_gfx950(8, 0, 8, 1, a, 8, a, 8, 0, c, 8)
     skl_amd.check_error()
     assert np.all(c == 7)
+
+
+def _dense_case(ta, m, n, k, a_kc, b_kc, alpha, beta, tb=None):
+    """A (m x k) row-major if a_kc else column-major; B (k x n) column-major if b_kc else row-major."""
+    return support.GemmCase(ta, tb, alpha, beta, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0,
+                            rsa1=k if a_kc else 1, csa1=1 if a_kc else m, rsb0=0, csb0=0,
+                            rsb1=1 if b_kc else n, csb1=k if b_kc else 1, rsc0=0, csc0=0, rsc1=n, csc1=1)
+
+
+@pytest.mark.parametrize("a_kc,b_kc", ((True, False), (False, False), (True, True), (False, True)))
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f16", "f8e4m3", "f8e5m2", "mixed"))
+def test_whole_tile_streaming_kernel(gpu, ta, a_kc, b_kc):
+    """4096 x 4096 outputs (256 tiles of 256 x 256: the streaming matrix-core
+    kernel) for every operand orientation. Too large for the scalar checker: the
+    expected result is numpy's fp64 product, which is exact for the integer case
+    (|sum| < 2^53) and the fp64-accumulated reference for the others."""
+    m = n = 4096
+    k = 384 if ta == "i8" else 256
+    tb = None
+    if ta == "mixed":
+        ta, tb = "f8e4m3", "f8e5m2"
+    alpha, beta = (3, -2) if ta == "i8" else (1.5, 0.5)
+    case = _dense_case(ta, m, n, k, a_kc, b_kc, alpha, beta, tb)
+    rng = np.random.default_rng(hash((ta, a_kc, b_kc)) % (1 << 31))
+    a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+    if ta.startswith("f8"):   # N(0,1)-like spread instead of log-uniform bytes: the config-4 distribution
+        a = rng.integers(0x28, 0x48, size=a.size, dtype=np.uint8) | (rng.integers(0, 2, size=a.size, dtype=np.uint8) << 7)
+        b = rng.integers(0x28, 0x48, size=b.size, dtype=np.uint8) | (rng.integers(0, 2, size=b.size, dtype=np.uint8) << 7)
+    got = run_gemm(gpu, "rc", case, a, b, c, "device")
+    A, B, C, oc = case.dense(a, b, c)
+    exact = alpha * (A @ B) + beta * C
+    if case.is_int:
+        want = (exact.astype(np.int64) & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
+        assert np.array_equal(got[oc], want)
+    else:
+        rel = np.linalg.norm(got[oc] - exact) / np.linalg.norm(exact)
+        assert rel <= 1e-3, rel
+        gamma = 2.0 * ((1.0 + 2.0 ** -24) ** (k + 2) - 1.0)
+        extra = support.FP8_MFMA_REL if ta.startswith("f8") else 0.0
+        bound = (gamma + extra) * abs(alpha) * (np.abs(A) @ np.abs(B)) + gamma * abs(beta) * np.abs(C)
+        err = np.abs(got[oc] - exact)
+        assert np.all(err <= bound + np.abs(exact) * 2.0 ** -22), float((err / (bound + 1e-30)).max())
