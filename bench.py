@@ -93,7 +93,7 @@ def _dense(lib, rng, name, fn_name, m, n, k, abytes, gen_a, gen_b, alpha, beta, 
         f(m, n, k, alpha, a, lda, b, n, beta, c, n)
 
     return dict(fn=step, bytes=abytes * (m * k + k * n) + 4 * m * n * (2 if beta != 0 else 1), ops=2 * m * n * k,
-                bound="mfma", dtype=dkey, keep=(a, b, c), name=name, kernel="gemm_mfma_kernel")
+                bound="mfma", dtype=dkey, keep=(a, b, c), name=name, kernel="gemm_mfma_stream_kernel")
 
 
 def wl_gemm_i8_8192(lib, rng):
@@ -130,7 +130,7 @@ def wl_gemm_f8_8192(lib, rng, fmt_b="f8e4m3"):
             lib.skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950(m, n, k, 1.0, a, 1, m, b, n, 1, 0.0, c, n, 1)
         name = "fp8 E4M3xE5M2 GEMM 8192^3 (column-major A, alpha=1, beta=0)"
     return dict(fn=step, bytes=m * k + k * n + 8 * m * n, ops=2 * m * n * k, bound="mfma", dtype="f8", keep=(a, b, c),
-                name=name, kernel="gemm_mfma_kernel")
+                name=name, kernel="gemm_mfma_stream_kernel")
 
 
 def wl_gemm_bf16(lib, rng):
@@ -159,7 +159,7 @@ def wl_f16_pipeline(lib, rng):
 
     moved = 2 * (2 * m * k) + 2 * (2 * k * n) + 2 * (4 * m * n)
     return dict(fn=step, bytes=moved, ops=2 * m * n * k, bound="mfma", dtype="f16", keep=(a, b, ap, bp, cp, c),
-                name="f16 pack->GEMM->unpack 4096x4096x14336 (TE=64 panels)", kernel="gemm_mfma_kernel")
+                name="f16 pack->GEMM->unpack 4096x4096x14336 (TE=64 panels)", kernel="gemm_mfma_stream_kernel")
 
 
 def wl_cvt(lib, rng):
@@ -186,6 +186,20 @@ def wl_pack_a(lib, rng):
                 name="pack e16 4096x4096 -> TEx1 column panels", kernel="pack_tile_kernel")
 
 
+def wl_copy(lib, rng):
+    """Plain copy through the pack kernel (one block = the whole matrix): the
+    known-size stream the HBM traffic counters are calibrated against."""
+    m = n = 4096
+    src = DeviceBuffer.from_array(rng.integers(0, 1 << 32, m * n, dtype=np.uint32))
+    dst = DeviceBuffer(4 * m * n)
+
+    def step(i):
+        lib.skl_pack_e32rc_e32rcprc_gfx950(m, n, src, n, 1, m, n, dst, n, 1, 0, 0, 0)
+
+    return dict(fn=step, bytes=8 * m * n, ops=m * n, bound="hbm", dtype="u32", keep=(src, dst),
+                name="copy 4096x4096 u32 (64 MiB read + 64 MiB write)", kernel="pack_tile_kernel")
+
+
 WORKLOADS = {
     "gemv_i8": (wl_gemv, 2000, 100),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
@@ -196,8 +210,19 @@ WORKLOADS = {
     "gemm_i8_512": (wl_gemm_i8_512, 200, 20),
     "cvt_f32_f8e4m3_8192sq": (wl_cvt, 20, 3),
     "pack_e16_4096sq": (wl_pack_a, 20, 3),
+    "copy_u32_4096sq": (wl_copy, 20, 3),
 }
 HEADLINE = "gemv_i8"
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
+# dispatch), FETCH_SIZE scaled by 1.998 (what it under-reads on a 64 MiB copy), WRITE_SIZE by 1.000;
+# the runs are summarised in profiles/gemv_cvt_gemm_hbm_traffic.pmc.txt.
+MEASURED_TRAFFIC_BYTES = {
+    "gemv_i8": int((22099.6 * 1.998 + 454.2) * 1024),
+    "cvt_f32_f8e4m3_8192sq": int((131110 * 1.998 + 65536) * 1024),
+    "gemm_i8_8192": int((393986 * 1.998 + 262144) * 1024),
+    "copy_u32_4096sq": int((32799.3 * 1.998 + 65536) * 1024),
+}
 
 
 def measure(lib, key, steps=None, warmup=None, seed=0x5EED0000):
@@ -222,6 +247,7 @@ def measure(lib, key, steps=None, warmup=None, seed=0x5EED0000):
         out.update(value=wl["ops"] / (wall_ms * 1e-3) / 1e12, unit=unit,
                    roofline=dict(bound="mfma", achieved=tops, peak=peak, unit=unit, frac=tops / peak, traffic=None,
                                  kernel=wl["kernel"], ops=wl["ops"]))
+    out["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get(key)
     for buf in _flatten(wl["keep"]):
         buf.free()
     return out
