@@ -484,14 +484,15 @@ struct SLoader {
     k_step = KC ? (size_t)kSliceBytes : (size_t)(kSliceBytes / ES) * sk * ES;
   }
 
-  // Requests this wave's eight blocks of `slice`; the data lands in `tile` (LDS).
-  __device__ __forceinline__ void issue(char *tile, size_t slice) const {
+  // Requests block `i` of this wave's share of `slice`; the data lands in `tile` (LDS).
+  __device__ __forceinline__ void issue_one(char *tile, size_t slice, int i) const {
     const char *g = tile_base + slice * k_step;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(g + off[i]),
+                                     (__attribute__((address_space(3))) void *)(tile + lds_block + i * 1024), 16, 0, 0);
+  }
+  __device__ __forceinline__ void issue(char *tile, size_t slice) const {
 #pragma unroll
-    for (int i = 0; i < kBlocks; ++i) {
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(g + off[i]),
-                                       (__attribute__((address_space(3))) void *)(tile + lds_block + i * 1024), 16, 0, 0);
-    }
+    for (int i = 0; i < kBlocks; ++i) issue_one(tile, slice, i);
   }
 };
 
@@ -562,10 +563,6 @@ __global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_stream_kernel(MfmaArg
   constexpr int BM = 256, BN = 256, WM = 128, WN = BN / WAVES_N, MI = 4, NI = WN / 32, WAVES = 2 * WAVES_N;
   constexpr int kTile = STile<ES, true>::kBytes, kStage = 2 * kTile;
   constexpr int kSteps = kSliceBytes / KB;
-  // LDS read instructions per k-step: b128 per 16 fragment bytes of a K-contiguous
-  // operand, one transpose load per 8 fragment bytes of an MN-contiguous one.
-  constexpr int kReadsA = MI * (A_KC ? FRB / 16 : FRB / 8), kReadsB = NI * (B_KC ? FRB / 16 : FRB / 8);
-  constexpr int kLoadsPerStep = 2 * (32 / WAVES) / kSteps;
   constexpr int kMfmas = MI * NI;
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -609,32 +606,66 @@ __global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_stream_kernel(MfmaArg
     // iteration: the next slice streams into it while this one is multiplied.
     // (The last iteration requests its own slice again: in range, never read.)
     const size_t nxt = s + 1 < slices ? s + 1 : s;
-    la.issue(na, nxt);
-    lb.issue(na + kTile, nxt);
-#pragma unroll
-    for (int ks = 0; ks < kSteps; ++ks) {
-      const int cur = ks & 1, nx = cur ^ 1;
-      if (ks + 1 < kSteps) {
-#pragma unroll
-        for (int i = 0; i < MI; ++i) fa[nx][i] = read_frag_s<ES, A_KC, FRB>(ta, wm + i * 32, (ks + 1) * KB);
-#pragma unroll
-        for (int j = 0; j < NI; ++j) fb[nx][j] = read_frag_s<ES, B_KC, FRB>(tb, wn + j * 32, (ks + 1) * KB);
+    // A wave issues in order and the compute unit has one load path, so the
+    // loads of the next slice are dealt out between the MFMAs (one load per
+    // kGap MFMAs) instead of being issued in a burst, and the LDS reads of the
+    // next k-step go out ahead of this step's MFMAs. The scheduling fences pin
+    // that order: left alone the compiler bunches loads and sinks reads.
+    // The last k-step of the slice is multiplied AFTER the barrier, from
+    // fragments already in registers, so that its MFMAs cover the latency of the
+    // first fragment reads of the next slice.
+    constexpr int kLoads = 2 * (32 / WAVES);        // this wave's loads per slice (A then B)
+    constexpr int kItems = kLoads;
+    constexpr int kSlots = (kSteps - 1) * kMfmas;   // MFMAs before the barrier
+    static_assert(kSteps % 2 == 0, "fragment buffers alternate per k-step");
+    int issued = 0;
+    auto deal = [&](int item) {
+      if (item < kLoads / 2) {
+        la.issue_one(na, nxt, item);
+      } else {
+        lb.issue_one(na + kTile, nxt, item - kLoads / 2);
       }
+    };
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
+    for (int ks = 0; ks < kSteps - 1; ++ks) {
+      const int cur = ks & 1, nx = cur ^ 1;
 #pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = M::run(fa[cur][i], fb[cur][j], acc[i][j]);
-      if (ks + 1 < kSteps)
-        sched_kstep<kReadsA + kReadsB, kLoadsPerStep>(std::make_integer_sequence<int, kMfmas>{});
-      else
-        sched_kstep<0, kLoadsPerStep>(std::make_integer_sequence<int, kMfmas>{});
+      for (int i = 0; i < MI; ++i) fa[nx][i] = read_frag_s<ES, A_KC, FRB>(ta, wm + i * 32, (ks + 1) * KB);
+#pragma unroll
+      for (int j = 0; j < NI; ++j) fb[nx][j] = read_frag_s<ES, B_KC, FRB>(tb, wn + j * 32, (ks + 1) * KB);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 0; q < kMfmas; ++q) {
+        const int slot = ks * kMfmas + q;
+#pragma unroll
+        for (int it = 0; it < kItems; ++it)  // items due by this slot (spread evenly over the slots)
+          if (it == issued && it * kSlots <= slot * kItems) {
+            deal(it);
+            ++issued;
+          }
+        const int i = q / NI, j = q % NI;
+        acc[i][j] = M::run(fa[cur][i], fb[cur][j], acc[i][j]);
+        if ((q & 1) == 1) __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kItems; ++it)
+      if (it >= issued) deal(it);
+    // Every LDS read of this stage has been issued; wait for them and for the
+    // next slice's data, then let the other waves overwrite this stage.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 #pragma unroll
     for (int i = 0; i < MI; ++i) fa[0][i] = read_frag_s<ES, A_KC, FRB>(na, wm + i * 32, 0);
 #pragma unroll
     for (int j = 0; j < NI; ++j) fb[0][j] = read_frag_s<ES, B_KC, FRB>(na + kTile, wn + j * 32, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NI; ++j) acc[i][j] = M::run(fa[1][i], fb[1][j], acc[i][j]);
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
@@ -779,12 +810,14 @@ extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
   p.tiles_m = p.tiles_n = 0;
   switch (g->ta * 8 + g->tb) {
     case SKL_DT_I8 * 8 + SKL_DT_I8: return launch_layout<SKL_DT_I8, SKL_DT_I8>(p);
+#ifndef SKL_MFMA_INT8_ONLY  // kernel-development builds compile one operand kind only
     case SKL_DT_BF16 * 8 + SKL_DT_BF16: return launch_layout<SKL_DT_BF16, SKL_DT_BF16>(p);
     case SKL_DT_F16 * 8 + SKL_DT_F16: return launch_layout<SKL_DT_F16, SKL_DT_F16>(p);
     case SKL_DT_F8E4M3 * 8 + SKL_DT_F8E4M3: return launch_layout<SKL_DT_F8E4M3, SKL_DT_F8E4M3>(p);
     case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E5M2: return launch_layout<SKL_DT_F8E5M2, SKL_DT_F8E5M2>(p);
     case SKL_DT_F8E4M3 * 8 + SKL_DT_F8E5M2: return launch_layout<SKL_DT_F8E4M3, SKL_DT_F8E5M2>(p);
     case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E4M3: return launch_layout<SKL_DT_F8E5M2, SKL_DT_F8E4M3>(p);
+#endif
     default:
       skl_hip_record_error(-2, "gemm_mfma: operand type pair");
       return -2;
