@@ -25,6 +25,13 @@
 // write-back: a wait for the workgroup's outstanding atomics before the ticket
 // is taken is enough (a device-scope fence would flush the whole L2 and costs
 // ten times the kernel).
+//
+// The same skeleton serves three more operand kinds: bf16 and f16 weights
+// (a lane owns 8 columns, fp32 accumulation with v_fma, fp32 atomics between
+// workgroups - the summation order then varies from run to run, within the
+// reference's tolerance) and the K-packed int8 layout of the dot4 entry point
+// (B(4P+p, j) at P*rsb1 + 4j + p: a 128-bit load holds four columns times four
+// k, which v_dot4_i32_i8 consumes without any byte shuffling).
 #include <hip/hip_runtime.h>
 
 #include <mutex>
@@ -33,20 +40,31 @@
 
 namespace {
 
-constexpr int kColsPerLane = 16;
-constexpr int kColLanes = 8;                           // lanes side by side along a row
-constexpr int kRowLanes = 64 / kColLanes;              // lane groups taking different rows
-constexpr int kTileCols = kColLanes * kColsPerLane;    // 128 columns = one 128-byte line per row
-constexpr int kRowsPerLane = 16;
-constexpr int kWaves = 4;
-constexpr int kPartials = kWaves * kRowLanes;          // partial sums per column in a workgroup
-constexpr int kRowsPerGroup = kPartials * kRowsPerLane;  // 512 rows (k) per workgroup
+// Kernel modes.
+enum { kI8RowMajor = 0, kI8K4 = 1, kBF16 = 2, kF16 = 3 };
 
-// Zero-initialised per-device scratch: int32/float accumulators + tickets.
+constexpr int kColLanes = 8;                 // lanes side by side along a row: 8 x 16 B = one 128-byte line
+constexpr int kRowLanes = 64 / kColLanes;    // lane groups taking different rows
+constexpr int kLoadsPerLane = 16;            // 128-bit loads in flight per lane
+constexpr int kWaves = 4;
+constexpr int kPartials = kWaves * kRowLanes;  // partial sums per column in a workgroup
+
+template <int MODE>
+struct Mode {
+  static constexpr int kCols = MODE == kI8RowMajor ? 16 : MODE == kI8K4 ? 4 : 8;  // columns per lane
+  static constexpr int kTileCols = kColLanes * kCols;                              // columns per workgroup
+  static constexpr int kKPerLoad = MODE == kI8K4 ? 4 : 1;                          // k values per 128-bit load
+  static constexpr int kKPerLane = kLoadsPerLane * kKPerLoad;
+  static constexpr int kKPerGroup = kPartials * kKPerLane;                         // k per workgroup
+  static constexpr int kES = (MODE == kBF16 || MODE == kF16) ? 2 : 1;
+  using Acc = typename std::conditional<(MODE == kBF16 || MODE == kF16), float, int>::type;
+};
+
+// Zero-initialised per-device scratch: 32-bit accumulators + tickets.
 constexpr size_t kMaxCols = size_t(1) << 22;  // 4 Mi columns
-constexpr size_t kMaxTiles = kMaxCols / kTileCols;
+constexpr size_t kMaxTiles = kMaxCols / 32;
 struct Reduction {
-  void *acc = nullptr;      // kMaxCols 32-bit accumulators
+  void *acc = nullptr;          // kMaxCols 32-bit accumulators
   unsigned *tickets = nullptr;  // kMaxTiles counters
 };
 std::mutex g_mutex;
@@ -70,17 +88,17 @@ bool reduction_scratch(Reduction *out) {
 }
 
 struct GemvArgs {
-  const int8_t *x;
-  size_t x_sk;
-  int x_vec;  // x is contiguous and 16-byte aligned
-  const int8_t *b;
-  size_t b_sk;  // stride between k rows (bytes = elements)
-  size_t b_s1;  // stride between 64-column blocks
-  int32_t *y;
-  size_t y_s;
+  const char *x;
+  size_t x_sk;  // elements
+  int x_vec;    // x is contiguous and 16-byte aligned
+  const char *b;
+  size_t b_sk;  // bytes between consecutive k rows (K4 layout: between groups of four k)
+  size_t b_s1;  // bytes between 64-column blocks (row-major modes)
+  char *y;
+  size_t y_s;   // elements
   size_t n, k;
-  int32_t alpha, beta;
-  int32_t *acc;
+  skl_scalar alpha, beta;
+  void *acc;
   unsigned *tickets;
   unsigned tiles, slabs;
 };
@@ -99,90 +117,140 @@ __device__ __forceinline__ void transpose4x4(unsigned r0, unsigned r1, unsigned 
   t3 = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
 }
 
-__global__ void __launch_bounds__(kWaves * 64) gemv_i8_rowmajor_kernel(GemvArgs p) {
-  __shared__ int red[kPartials][kTileCols + 4];
+__device__ __forceinline__ float widen16(unsigned bits16, bool is_bf16) {
+  if (is_bf16) return __uint_as_float(bits16 << 16);
+  _Float16 h = __builtin_bit_cast(_Float16, (unsigned short)bits16);
+  return (float)h;
+}
+
+__device__ __forceinline__ int finish(int total, int old, skl_scalar alpha, skl_scalar beta) {
+  return (int)((unsigned)beta.i * (unsigned)old + (unsigned)alpha.i * (unsigned)total);
+}
+__device__ __forceinline__ float finish(float total, float old, skl_scalar alpha, skl_scalar beta) {
+  return __fadd_rn(__fmul_rn(beta.f, old), __fmul_rn(alpha.f, total));
+}
+
+template <int MODE>
+__global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
+  using Md = Mode<MODE>;
+  using Acc = typename Md::Acc;
+  constexpr int kCols = Md::kCols;
+  __shared__ Acc red[kPartials][Md::kTileCols + 4];
   __shared__ unsigned ticket_s;
 
   const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int cl = lane % kColLanes, rl = lane / kColLanes;
   const int part = wave * kRowLanes + rl;
-  const size_t k0 = (size_t)slab * kRowsPerGroup + (size_t)part * kRowsPerLane;
-  const size_t col = (size_t)tile * kTileCols + (size_t)cl * kColsPerLane;
+  const size_t k0 = (size_t)slab * Md::kKPerGroup + (size_t)part * Md::kKPerLane;
+  const size_t col = (size_t)tile * Md::kTileCols + (size_t)cl * kCols;
 
-  int acc[kColsPerLane];
+  Acc acc[kCols];
 #pragma unroll
-  for (int j = 0; j < kColsPerLane; ++j) acc[j] = 0;
+  for (int j = 0; j < kCols; ++j) acc[j] = 0;
 
   if (col < p.n && k0 < p.k) {
-    // All of the lane's rows are requested before anything is consumed.
-    const int8_t *wp = p.b + (col >> 6) * p.b_s1 + (col & 63) + k0 * p.b_sk;
-    uint4 rows[kRowsPerLane];
+    // All of the lane's loads are requested before anything is consumed.
+    const char *wp;
+    if constexpr (MODE == kI8K4)
+      wp = p.b + (k0 / 4) * p.b_sk + col * 4;
+    else
+      wp = p.b + (col >> 6) * p.b_s1 + (col & 63) * Md::kES + k0 * p.b_sk;
+    uint4 rows[kLoadsPerLane];
 #pragma unroll
-    for (int r = 0; r < kRowsPerLane; ++r) {
-      if (k0 + r < p.k)
+    for (int r = 0; r < kLoadsPerLane; ++r) {
+      if (k0 + (size_t)r * Md::kKPerLoad < p.k)
         rows[r] = *reinterpret_cast<const uint4 *>(wp + (size_t)r * p.b_sk);
       else
         rows[r] = make_uint4(0, 0, 0, 0);
     }
-    // Four x bytes per group of four rows; rows at or beyond K were loaded as zero.
-    int xw[kRowsPerLane / 4];
-    if (p.x_vec && k0 + kRowsPerLane <= p.k) {
-      const int4 *xp = reinterpret_cast<const int4 *>(p.x + k0);
+    if constexpr (MODE == kI8RowMajor || MODE == kI8K4) {
+      // x as packed bytes, four k per dword; k at or beyond K contributes zero.
+      constexpr int kWords = Md::kKPerLane / 4;
+      int xw[kWords];
+      const int8_t *x = reinterpret_cast<const int8_t *>(p.x);
+      if (p.x_vec && k0 + Md::kKPerLane <= p.k) {
+        const int4 *xp = reinterpret_cast<const int4 *>(x + k0);
 #pragma unroll
-      for (int q = 0; q < kRowsPerLane / 16; ++q) {
-        const int4 v = xp[q];
-        xw[4 * q] = v.x, xw[4 * q + 1] = v.y, xw[4 * q + 2] = v.z, xw[4 * q + 3] = v.w;
+        for (int q = 0; q < kWords / 4; ++q) {
+          const int4 v = xp[q];
+          xw[4 * q] = v.x, xw[4 * q + 1] = v.y, xw[4 * q + 2] = v.z, xw[4 * q + 3] = v.w;
+        }
+      } else {
+#pragma unroll
+        for (int g = 0; g < kWords; ++g) {
+          unsigned w = 0;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const size_t k = k0 + 4 * g + i;
+            const unsigned byte = k < p.k ? (unsigned)(uint8_t)x[k * p.x_sk] : 0u;
+            w |= byte << (8 * i);
+          }
+          xw[g] = (int)w;
+        }
+      }
+      if constexpr (MODE == kI8RowMajor) {
+#pragma unroll
+        for (int g = 0; g < kLoadsPerLane / 4; ++g) {
+          const uint4 r0 = rows[4 * g], r1 = rows[4 * g + 1], r2 = rows[4 * g + 2], r3 = rows[4 * g + 3];
+          const unsigned a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
+          const unsigned a2[4] = {r2.x, r2.y, r2.z, r2.w}, a3[4] = {r3.x, r3.y, r3.z, r3.w};
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            unsigned t0, t1, t2, t3;
+            transpose4x4(a0[d], a1[d], a2[d], a3[d], t0, t1, t2, t3);
+            acc[4 * d + 0] = __builtin_amdgcn_sdot4((int)t0, xw[g], acc[4 * d + 0], false);
+            acc[4 * d + 1] = __builtin_amdgcn_sdot4((int)t1, xw[g], acc[4 * d + 1], false);
+            acc[4 * d + 2] = __builtin_amdgcn_sdot4((int)t2, xw[g], acc[4 * d + 2], false);
+            acc[4 * d + 3] = __builtin_amdgcn_sdot4((int)t3, xw[g], acc[4 * d + 3], false);
+          }
+        }
+      } else {  // K4: each dword already holds four k of one column
+#pragma unroll
+        for (int r = 0; r < kLoadsPerLane; ++r) {
+          acc[0] = __builtin_amdgcn_sdot4((int)rows[r].x, xw[r], acc[0], false);
+          acc[1] = __builtin_amdgcn_sdot4((int)rows[r].y, xw[r], acc[1], false);
+          acc[2] = __builtin_amdgcn_sdot4((int)rows[r].z, xw[r], acc[2], false);
+          acc[3] = __builtin_amdgcn_sdot4((int)rows[r].w, xw[r], acc[3], false);
+        }
       }
     } else {
+      constexpr bool bf = MODE == kBF16;
+      const unsigned short *x = reinterpret_cast<const unsigned short *>(p.x);
 #pragma unroll
-      for (int g = 0; g < kRowsPerLane / 4; ++g) {
-        unsigned w = 0;
+      for (int r = 0; r < kLoadsPerLane; ++r) {
+        const size_t k = k0 + r;
+        const float xv = k < p.k ? widen16(x[k * p.x_sk], bf) : 0.0f;
+        const unsigned w[4] = {rows[r].x, rows[r].y, rows[r].z, rows[r].w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const size_t k = k0 + 4 * g + i;
-          const unsigned byte = k < p.k ? (unsigned)(uint8_t)p.x[k * p.x_sk] : 0u;
-          w |= byte << (8 * i);
+        for (int d = 0; d < 4; ++d) {
+          acc[2 * d] = __fmaf_rn(xv, widen16(w[d] & 0xFFFFu, bf), acc[2 * d]);
+          acc[2 * d + 1] = __fmaf_rn(xv, widen16(w[d] >> 16, bf), acc[2 * d + 1]);
         }
-        xw[g] = (int)w;
-      }
-    }
-#pragma unroll
-    for (int g = 0; g < kRowsPerLane / 4; ++g) {
-      const uint4 r0 = rows[4 * g], r1 = rows[4 * g + 1], r2 = rows[4 * g + 2], r3 = rows[4 * g + 3];
-      const unsigned a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
-      const unsigned a2[4] = {r2.x, r2.y, r2.z, r2.w}, a3[4] = {r3.x, r3.y, r3.z, r3.w};
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        unsigned t0, t1, t2, t3;
-        transpose4x4(a0[d], a1[d], a2[d], a3[d], t0, t1, t2, t3);
-        acc[4 * d + 0] = __builtin_amdgcn_sdot4((int)t0, xw[g], acc[4 * d + 0], false);
-        acc[4 * d + 1] = __builtin_amdgcn_sdot4((int)t1, xw[g], acc[4 * d + 1], false);
-        acc[4 * d + 2] = __builtin_amdgcn_sdot4((int)t2, xw[g], acc[4 * d + 2], false);
-        acc[4 * d + 3] = __builtin_amdgcn_sdot4((int)t3, xw[g], acc[4 * d + 3], false);
       }
     }
   }
   // The workgroup's partial sums meet in LDS.
 #pragma unroll
-  for (int j = 0; j < kColsPerLane; j += 4)
-    *reinterpret_cast<int4 *>(&red[part][cl * kColsPerLane + j]) = make_int4(acc[j], acc[j + 1], acc[j + 2], acc[j + 3]);
+  for (int j = 0; j < kCols; ++j) red[part][cl * kCols + j] = acc[j];
   __syncthreads();
-  const size_t tile_col0 = (size_t)tile * kTileCols;
-  const bool owner = threadIdx.x < kTileCols && tile_col0 + threadIdx.x < p.n;
-  int sum = 0;
+  const size_t tile_col0 = (size_t)tile * Md::kTileCols;
+  const bool owner = threadIdx.x < Md::kTileCols && tile_col0 + threadIdx.x < p.n;
+  Acc sum = 0;
   if (owner) {
 #pragma unroll
     for (int w = 0; w < kPartials; ++w) sum += red[w][threadIdx.x];
   }
+  Acc *yv = reinterpret_cast<Acc *>(p.y);
   if (p.slabs == 1) {  // the strip is complete inside this workgroup
     if (owner) {
-      int32_t *y = p.y + (tile_col0 + threadIdx.x) * p.y_s;
-      *y = (int32_t)((uint32_t)p.beta * (uint32_t)*y + (uint32_t)p.alpha * (uint32_t)sum);
+      Acc *y = yv + (tile_col0 + threadIdx.x) * p.y_s;
+      *y = finish(sum, *y, p.alpha, p.beta);
     }
     return;
   }
-  if (owner) atomicAdd(&p.acc[tile_col0 + threadIdx.x], sum);
+  Acc *scratch = reinterpret_cast<Acc *>(p.acc);
+  if (owner) atomicAdd(&scratch[tile_col0 + threadIdx.x], sum);
   // Wait until this wave's atomics have been performed, then take a ticket.
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_waitcnt(0);
@@ -192,23 +260,65 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_i8_rowmajor_kernel(GemvArgs 
   if (ticket_s != p.slabs - 1) return;
   if (owner) {
     const size_t j = tile_col0 + threadIdx.x;
-    const int total = atomicExch(&p.acc[j], 0);  // read the total and leave zero behind
-    int32_t *y = p.y + j * p.y_s;
-    *y = (int32_t)((uint32_t)p.beta * (uint32_t)*y + (uint32_t)p.alpha * (uint32_t)total);
+    const Acc total = atomicExch(&scratch[j], (Acc)0);  // read the total and leave zero behind
+    Acc *y = yv + j * p.y_s;
+    *y = finish(total, *y, p.alpha, p.beta);
   }
   if (threadIdx.x == 0) atomicExch(&p.tickets[tile], 0u);
 }
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
+int mode_of(const skl_gemm_canon *g, int layout) {
+  if (g->ta != g->tb) return -1;
+  if (layout == 1) return g->ta == SKL_DT_I8 ? kI8K4 : -1;
+  switch (g->ta) {
+    case SKL_DT_I8: return kI8RowMajor;
+    case SKL_DT_BF16: return kBF16;
+    case SKL_DT_F16: return kF16;
+    default: return -1;  // fp8 M = 1 goes to the matrix-core kernel
+  }
+}
+
+template <int MODE>
+int launch(const skl_gemm_canon *g, const Reduction &red) {
+  using Md = Mode<MODE>;
+  GemvArgs p;
+  p.x = (const char *)g->a;
+  p.x_sk = g->a_sk;
+  p.x_vec = (g->a_sk == 1 && aligned16(g->a)) ? 1 : 0;
+  p.b = (const char *)g->b;
+  p.b_sk = g->b_sk * Md::kES;
+  p.b_s1 = g->b_s1 * Md::kES;
+  p.y = (char *)g->c;
+  p.y_s = g->csc0;
+  p.n = g->n;
+  p.k = g->k;
+  p.alpha = g->alpha;
+  p.beta = g->beta;
+  p.acc = red.acc;
+  p.tickets = red.tickets;
+  p.tiles = skl_div_up(g->n, Md::kTileCols);
+  p.slabs = skl_div_up(g->k, Md::kKPerGroup);
+  const size_t grid = (size_t)p.tiles * p.slabs;
+  if (grid > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemv: grid too large");
+    return -2;
+  }
+  gemv_kernel<MODE><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
+  return skl_check_launch("gemv");
+}
+
 }  // namespace
 
 extern "C" int skl_hip_gemv_supported(const skl_gemm_canon *g, int layout) {
-  if (layout != 0) return 0;
-  if (g->ta != SKL_DT_I8 || g->tb != SKL_DT_I8) return 0;
-  if (g->m != 1 || g->k == 0 || g->n == 0) return 0;
-  if (g->b_s0 != 1 || (g->n % kColsPerLane) != 0 || g->n > kMaxCols) return 0;
-  if (!aligned16(g->b) || (g->b_sk % 16) != 0 || (g->b_s1 % 16) != 0) return 0;
+  const int mode = mode_of(g, layout);
+  if (mode < 0) return 0;
+  if (g->m != 1 || g->k == 0 || g->n == 0 || g->n > kMaxCols) return 0;
+  const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1;
+  const size_t cols = mode == kI8RowMajor ? 16 : mode == kI8K4 ? 4 : 8;
+  if ((g->n % cols) != 0 || !aligned16(g->b) || ((g->b_sk * es) % 16) != 0) return 0;
+  if (mode != kI8K4 && (g->b_s0 != 1 || ((g->b_s1 * es) % 16) != 0)) return 0;
   if (g->csc1 != 64 * g->csc0) return 0;  // y must be a flat strided vector
   return 1;
 }
@@ -220,28 +330,10 @@ extern "C" int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout) {
   }
   Reduction red;
   if (!reduction_scratch(&red)) return -4;
-  GemvArgs p;
-  p.x = (const int8_t *)g->a;
-  p.x_sk = g->a_sk;
-  p.x_vec = (g->a_sk == 1 && aligned16(g->a)) ? 1 : 0;
-  p.b = (const int8_t *)g->b;
-  p.b_sk = g->b_sk;
-  p.b_s1 = g->b_s1;
-  p.y = (int32_t *)g->c;
-  p.y_s = g->csc0;
-  p.n = g->n;
-  p.k = g->k;
-  p.alpha = g->alpha.i;
-  p.beta = g->beta.i;
-  p.acc = (int32_t *)red.acc;
-  p.tickets = red.tickets;
-  p.tiles = skl_div_up(g->n, kTileCols);
-  p.slabs = skl_div_up(g->k, kRowsPerGroup);
-  const size_t grid = (size_t)p.tiles * p.slabs;
-  if (grid > 0x7FFFFFFFu) {
-    skl_hip_record_error(-2, "gemv: grid too large");
-    return -2;
+  switch (mode_of(g, layout)) {
+    case kI8RowMajor: return launch<kI8RowMajor>(g, red);
+    case kI8K4: return launch<kI8K4>(g, red);
+    case kBF16: return launch<kBF16>(g, red);
+    default: return launch<kF16>(g, red);
   }
-  gemv_i8_rowmajor_kernel<<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
-  return skl_check_launch("gemv_i8_rowmajor");
 }

@@ -80,3 +80,27 @@ def test_m1_shapes_outside_the_streaming_kernel(gpu):
         case = rowmajor_case("i8", 1, n, k, 1, 1, rsb=rsb)
         a, b, c = case.make_inputs(n + k)
         assert np.array_equal(run_gemm(gpu, "rowmajor", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
+
+
+@pytest.mark.parametrize("ta", ("bf16", "f16"))
+@pytest.mark.parametrize("n,k", ((256, 12), (256, 31), (1024, 1000), (11008, 4096)))
+def test_16bit_decode_shapes(gpu, ta, n, k):
+    """bf16 / f16 weights, fp32 accumulation: the M = 1 rows of the reference's suites
+    (test/gemm/rvv/skl_gemm_f16_f16_f32_zvfh_x390.c:66-72) and the decode shape. The
+    split-K order differs from the reference's k-ascending loop and varies between runs
+    (fp32 atomics): compared through the reference's elementwise bound."""
+    case = rowmajor_case(ta, 1, n, k, 1.5, -0.5)
+    a, b, c = case.make_inputs(n + k)
+    for _ in range(2):   # twice: the reduction scratch must come back clean
+        got = run_gemm(gpu, "rowmajor", case, a, b, c, "device")
+        support.assert_fp_gemm_close(case, a, b, c, got)
+
+
+@pytest.mark.parametrize("n,k1", ((64, 1), (128, 4), (192, 3), (256, 17), (11008, 1024)))
+def test_k_packed_int8_decode(gpu, n, k1):
+    """The dot4 layout with M = 1 (src/gemm/gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.c:645-660
+    dispatches this case to its own GEMV kernels): A 1 x 4 K-blocks, B 4 x 1 K-blocks."""
+    case = support.dot4_case(1, n, k1, alpha=-3, beta=5)
+    a, b, c = case.make_inputs(n * 3 + k1)
+    for mode in ("device", "host"):
+        assert np.array_equal(run_gemm(gpu, "dot4", case, a, b, c, mode), run_oracle_gemm(case, a, b, c))
