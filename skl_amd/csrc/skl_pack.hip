@@ -13,6 +13,8 @@
 // are coalesced even when the copy transposes.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "skl_device.hpp"
 
 namespace {
@@ -83,6 +85,150 @@ __global__ void __launch_bounds__(kThreads) pack_tile_kernel(const T *__restrict
   }
 }
 
+// ---- 16-byte vector variants -------------------------------------------------------------------
+// When each side has a unit-stride direction whose runs are whole 16-byte vectors, a lane moves a
+// vector instead of an element. If both sides are dense along the same direction the tile is a
+// straight vector copy with table-driven addresses; if they are dense along different directions
+// (the TE x 1 panel packer of a row-major matrix, transposes) the tile goes through LDS: written
+// as vectors along the source's direction, gathered element by element into vectors along the
+// destination's. The 16-byte chunks of an LDS line are XOR-swizzled by (line / V) so that the
+// gather (lanes V lines apart) and the vector writes are both free of bank conflicts.
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+// Development switch: SKL_PACK_ELEMENTWISE=1 forces the element kernel.
+bool skl_pack_vectorise() {
+  static const bool on = [] {
+    const char *e = getenv("SKL_PACK_ELEMENTWISE");
+    return !(e && e[0] == '1');
+  }();
+  return on;
+}
+
+template <int ES>
+struct VecShape {
+  static constexpr int V = 16 / ES;            // elements per vector
+  static constexpr int T = ES == 1 ? 128 : 64;  // tile edge in elements
+  static constexpr int NV = T / V;              // vectors per tile line
+};
+
+template <int ES> struct ElemOf;
+template <> struct ElemOf<1> { typedef uint8_t type; };
+template <> struct ElemOf<2> { typedef uint16_t type; };
+template <> struct ElemOf<4> { typedef uint32_t type; };
+
+template <int ES, bool PACK, bool TRANSPOSE>
+__global__ void __launch_bounds__(kThreads) pack_vec_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                            PackArgs p) {
+  typedef typename ElemOf<ES>::type E;
+  constexpr int V = VecShape<ES>::V, T = VecShape<ES>::T, NV = VecShape<ES>::NV;
+  constexpr int kIters = T * NV / kThreads;
+  __shared__ size_t plain_r[T], plain_c[T], blk_r[T], blk_c[T];
+  __shared__ v4i stage[TRANSPOSE ? T * NV : 1];
+
+  const size_t r0 = (size_t)(blockIdx.x / p.tiles_x) * T, c0 = (size_t)(blockIdx.x % p.tiles_x) * T;
+  const int t = threadIdx.x;
+  for (int i = t; i < 2 * T; i += kThreads) {
+    if (i < T) {
+      const size_t r = r0 + i;
+      plain_r[i] = r * p.rs;
+      blk_r[i] = (r / p.m0) * p.rs1 + (r % p.m0) * p.rs0;
+    } else {
+      const size_t c = c0 + (i - T);
+      plain_c[i - T] = c * p.cs;
+      blk_c[i - T] = (c / p.n0) * p.cs1 + (c % p.n0) * p.cs0;
+    }
+  }
+  __syncthreads();
+
+  const bool in_along_c = PACK ? p.plain_along_c : p.blocked_along_c;
+  v4i padv;
+  {
+    unsigned w = p.pad;
+    if (ES == 1) w = (w & 0xFF) * 0x01010101u;
+    if (ES == 2) w = (w & 0xFFFF) * 0x00010001u;
+    padv = (v4i)((int)w);
+  }
+
+#pragma unroll
+  for (int it = 0; it < kIters; ++it) {
+    const int idx = it * kThreads + t;
+    const int wv = idx % NV, u = idx / NV;  // vector within the line, line
+    const int tr = in_along_c ? u : wv * V, tc = in_along_c ? wv * V : u;
+    const size_t r = r0 + tr, c = c0 + tc;
+    if (r < p.rows && c < p.cols) {
+      v4i v;
+      if (PACK)
+        v = (r < p.m && c < p.n) ? *(const v4i *)(src + (plain_r[tr] + plain_c[tc]) * ES) : padv;
+      else
+        v = *(const v4i *)(src + (blk_r[tr] + blk_c[tc]) * ES);
+      if (TRANSPOSE)
+        stage[u * NV + (wv ^ ((u / V) & (NV - 1)))] = v;
+      else
+        *(v4i *)(dst + (PACK ? blk_r[tr] + blk_c[tc] : plain_r[tr] + plain_c[tc]) * ES) = v;
+    }
+  }
+  if (!TRANSPOSE) return;
+  __syncthreads();
+
+  const uint8_t *bytes = (const uint8_t *)stage;
+#pragma unroll
+  for (int it = 0; it < kIters; ++it) {
+    const int idx = it * kThreads + t;
+    const int uv = idx % NV, w = idx / NV;  // vector of V source lines, position along the source's direction
+    const int tr = in_along_c ? uv * V : w, tc = in_along_c ? w : uv * V;
+    const size_t r = r0 + tr, c = c0 + tc;
+    if (r < p.rows && c < p.cols) {
+      const int chunk = (w * ES) >> 4, within = (w * ES) & 15;
+      const uint8_t *col = bytes + (size_t)(((uv * V) * NV + (chunk ^ uv)) * 16 + within);
+      E e[V];
+#pragma unroll
+      for (int i = 0; i < V; ++i) e[i] = *(const E *)(col + i * NV * 16);
+      v4i v;
+      __builtin_memcpy(&v, e, 16);
+      *(v4i *)(dst + (PACK ? blk_r[tr] + blk_c[tc] : plain_r[tr] + plain_c[tc]) * ES) = v;
+    }
+  }
+}
+
+// 0: element kernel; 1: vector copy; 2: vector transpose. Sets the lane directions for the vector kernels.
+int vector_plan(int es, const void *src, const void *dst, PackArgs &p) {
+  const size_t V = 16 / es;
+  if ((((uintptr_t)src | (uintptr_t)dst) & 15) != 0) return 0;
+  const bool use_rs0 = p.m0 > 1, use_cs0 = p.n0 > 1, use_rs1 = p.rows > p.m0, use_cs1 = p.cols > p.n0;
+  auto mult = [&](bool used, size_t s) { return !used || s % V == 0; };
+  const bool plain_c = p.cs == 1 && p.n % V == 0 && (p.m == 1 || p.rs % V == 0);
+  const bool plain_r = p.rs == 1 && p.m % V == 0 && (p.n == 1 || p.cs % V == 0);
+  const bool blk_c = use_cs0 && p.cs0 == 1 && p.n0 % V == 0 && mult(use_rs0, p.rs0) && mult(use_rs1, p.rs1) &&
+                     mult(use_cs1, p.cs1);
+  const bool blk_r = use_rs0 && p.rs0 == 1 && p.m0 % V == 0 && mult(use_cs0, p.cs0) && mult(use_rs1, p.rs1) &&
+                     mult(use_cs1, p.cs1);
+  if (plain_c && blk_c) { p.plain_along_c = 1; p.blocked_along_c = 1; return 1; }
+  if (plain_r && blk_r) { p.plain_along_c = 0; p.blocked_along_c = 0; return 1; }
+  if (plain_c && blk_r) { p.plain_along_c = 1; p.blocked_along_c = 0; return 2; }
+  if (plain_r && blk_c) { p.plain_along_c = 0; p.blocked_along_c = 1; return 2; }
+  return 0;
+}
+
+template <int ES>
+int launch_vec(bool pack, bool transpose, const void *src, void *dst, PackArgs p) {
+  constexpr int T = VecShape<ES>::T;
+  const size_t gx = (p.cols + T - 1) / T, gy = (p.rows + T - 1) / T;
+  if (gx * gy > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "pack: matrix too large for one launch");
+    return -2;
+  }
+  p.tiles_x = (unsigned)gx;
+  const unsigned grid = (unsigned)(gx * gy);
+  hipStream_t st = skl_current_stream();
+  const uint8_t *s = (const uint8_t *)src;
+  uint8_t *d = (uint8_t *)dst;
+  if (pack && transpose) pack_vec_kernel<ES, true, true><<<grid, kThreads, 0, st>>>(s, d, p);
+  else if (pack) pack_vec_kernel<ES, true, false><<<grid, kThreads, 0, st>>>(s, d, p);
+  else if (transpose) pack_vec_kernel<ES, false, true><<<grid, kThreads, 0, st>>>(s, d, p);
+  else pack_vec_kernel<ES, false, false><<<grid, kThreads, 0, st>>>(s, d, p);
+  return skl_check_launch(pack ? "pack" : "unpack");
+}
+
 template <typename T>
 int launch(bool pack, const void *src, void *dst, PackArgs p) {
   if (p.rows == 0 || p.cols == 0) return 0;
@@ -100,7 +246,18 @@ int launch(bool pack, const void *src, void *dst, PackArgs p) {
   return skl_check_launch(pack ? "pack" : "unpack");
 }
 
-int dispatch(int esize, bool pack, const void *src, void *dst, const PackArgs &p) {
+int dispatch(int esize, bool pack, const void *src, void *dst, PackArgs p) {
+  if (p.rows == 0 || p.cols == 0) return 0;
+  if (esize == 1 || esize == 2 || esize == 4) {
+    const int plan = skl_pack_vectorise() ? vector_plan(esize, src, dst, p) : 0;
+    if (plan) {
+      switch (esize) {
+        case 1: return launch_vec<1>(pack, plan == 2, src, dst, p);
+        case 2: return launch_vec<2>(pack, plan == 2, src, dst, p);
+        default: return launch_vec<4>(pack, plan == 2, src, dst, p);
+      }
+    }
+  }
   switch (esize) {
     case 1: return launch<uint8_t>(pack, src, dst, p);
     case 2: return launch<uint16_t>(pack, src, dst, p);

@@ -130,3 +130,59 @@ def test_config5_pipeline_shapes(gpu):
     want = c.reshape(m // te, n // te, te, te).transpose(0, 2, 1, 3).reshape(m, n)
     assert np.array_equal(got, want)
     dc.free(), dcu.free()
+
+
+def _vector_layouts(w):
+    """Layouts whose unit-stride runs are whole 16-byte vectors on both sides: dense along the same
+    direction (vector copy) and along different directions (vector transpose through LDS). Extents cross
+    tile edges, rows and columns are padded, and every leading dimension leaves a gap."""
+    v = 128 // w
+    out = []
+    # plain dense along c, blocks dense along c
+    m, n, m0, n0 = 203, 21 * v, 5, 4 * v
+    n1 = -(-n // n0)
+    rs0, cs1 = n0 + v, m0 * (n0 + v) + v
+    out.append(dict(m=m, n=n, rs=n + v, cs=1, m0=m0, n0=n0, rs0=rs0, cs0=1, cs1=cs1, rs1=n1 * cs1 + v))
+    # plain dense along r, blocks dense along r
+    m, n, m0, n0 = 19 * v, 150, 2 * v, 3
+    m1 = -(-m // m0)
+    cs0, rs1 = m0 + v, n0 * (m0 + v)
+    out.append(dict(m=m, n=n, rs=1, cs=m + v, m0=m0, n0=n0, rs0=1, cs0=cs0, rs1=rs1, cs1=m1 * rs1 + v))
+    # plain dense along c, blocks dense along r: the TE x 1 panel packer's shape (n0 = 1) and a 3-wide one
+    for n0 in (1, 3):
+        m, n, m0 = 200, 19 * v, 64
+        cs0 = m0 + v
+        cs1 = n0 * cs0
+        n1 = -(-n // n0)
+        out.append(dict(m=m, n=n, rs=n + 2 * v, cs=1, m0=m0, n0=n0, rs0=1, cs0=cs0, cs1=cs1, rs1=n1 * cs1 + v))
+    # plain dense along r, blocks dense along c
+    m, n, m0, n0 = 18 * v, 170, 3, 2 * v
+    rs0 = n0 + v
+    rs1 = m0 * rs0
+    m1 = -(-m // m0)
+    out.append(dict(m=m, n=n, rs=1, cs=m + v, m0=m0, n0=n0, rs0=rs0, cs0=1, rs1=rs1, cs1=m1 * rs1 + 2 * v))
+    return out
+
+
+@pytest.mark.parametrize("w", (8, 16, 32))
+def test_vector_paths_pack_and_unpack(gpu, w):
+    for i, row in enumerate(_vector_layouts(w)):
+        src, dst = pack_case_buffers(row, w, 900 + i)
+        tail = (row["m0"], row["n0"])
+        bs = (row["rs0"], row["cs0"], row["rs1"], row["cs1"])
+        want = dst.copy()
+        getattr(oracle(), f"skl_pack_e{w}rc_e{w}rcprc_oracle")(row["m"], row["n"], src, row["rs"], row["cs"], *tail,
+                                                                want, *bs, PAD[w] ^ 0x5A)
+        got = run_inout(gpu, f"skl_pack_e{w}rc_e{w}rcprc_gfx950",
+                        lambda s, d: (row["m"], row["n"], s, row["rs"], row["cs"], *tail, d, *bs, PAD[w] ^ 0x5A),
+                        src, dst, "device")
+        assert np.array_equal(got, want), ("pack", row)
+        packed, plain = want, src.copy()
+        plain[:] = np.arange(plain.size).astype(plain.dtype)
+        want_u = plain.copy()
+        getattr(oracle(), f"skl_unpack_e{w}rcprc_e{w}rc_oracle")(*tail, packed, *bs, row["m"], row["n"], want_u,
+                                                                  row["rs"], row["cs"])
+        got_u = run_inout(gpu, f"skl_unpack_e{w}rcprc_e{w}rc_gfx950",
+                          lambda s, d: (*tail, s, *bs, row["m"], row["n"], d, row["rs"], row["cs"]),
+                          packed, plain, "device")
+        assert np.array_equal(got_u, want_u), ("unpack", row)
