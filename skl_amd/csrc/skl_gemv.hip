@@ -19,12 +19,16 @@
 // column of a workgroup meet in LDS; the few workgroups that share a column
 // strip (K / kRowsPerGroup of them) meet in a zero-initialised int32 accumulator
 // in device memory through relaxed device-scope atomics (integer adds: exact in
-// any order). A ticket counter per strip tells the workgroup that arrives last
-// to apply alpha and beta, write y and put accumulator and ticket back to zero.
-// Only atomics carry data between workgroups, so ordering needs no cache
-// write-back: a wait for the workgroup's outstanding atomics before the ticket
-// is taken is enough (a device-scope fence would flush the whole L2 and costs
-// ten times the kernel).
+// any order). The slot is 64 bits wide: the sum lives in the high word and an
+// arrival count in the low word, one atomic add carries both and returns the
+// previous value, so the lane whose add completes the count knows the total,
+// applies alpha and beta, writes y and puts the slot back to zero - one round
+// trip to memory after the last byte of B has arrived. (The floating-point
+// modes cannot fold a count into the sum: there a ticket counter per strip
+// tells the workgroup that arrives last to read the totals back. Only atomics
+// carry data between workgroups, so ordering needs no cache write-back: a wait
+// for the workgroup's outstanding atomics before the ticket is taken is enough;
+// a device-scope fence would flush the whole L2 and costs ten times the kernel.)
 //
 // The same skeleton serves three more operand kinds: bf16 and f16 weights
 // (a lane owns 8 columns, fp32 accumulation with v_fma, fp32 atomics between
@@ -35,6 +39,7 @@
 #include <hip/hip_runtime.h>
 
 #include <mutex>
+#include <type_traits>
 
 #include "skl_device.hpp"
 
@@ -45,8 +50,8 @@ enum { kI8RowMajor = 0, kI8K4 = 1, kBF16 = 2, kF16 = 3 };
 
 constexpr int kColLanes = 8;                 // lanes side by side along a row: 8 x 16 B = one 128-byte line
 constexpr int kRowLanes = 64 / kColLanes;    // lane groups taking different rows
-constexpr int kLoadsPerLane = 16;            // 128-bit loads in flight per lane
-constexpr int kWaves = 4;
+constexpr int kLoadsPerLane = 8;             // 128-bit loads in flight per lane
+constexpr int kWaves = 8;
 constexpr int kPartials = kWaves * kRowLanes;  // partial sums per column in a workgroup
 
 template <int MODE>
@@ -60,11 +65,12 @@ struct Mode {
   using Acc = typename std::conditional<(MODE == kBF16 || MODE == kF16), float, int>::type;
 };
 
-// Zero-initialised per-device scratch: 32-bit accumulators + tickets.
+// Zero-initialised per-device scratch: one 64-bit slot per column (the floating-point modes use the
+// first 32 bits of the region as an fp32 array) + tickets.
 constexpr size_t kMaxCols = size_t(1) << 22;  // 4 Mi columns
 constexpr size_t kMaxTiles = kMaxCols / 32;
 struct Reduction {
-  void *acc = nullptr;          // kMaxCols 32-bit accumulators
+  void *acc = nullptr;          // kMaxCols 64-bit slots
   unsigned *tickets = nullptr;  // kMaxTiles counters
 };
 std::mutex g_mutex;
@@ -76,12 +82,12 @@ bool reduction_scratch(Reduction *out) {
   std::lock_guard<std::mutex> lock(g_mutex);
   Reduction &r = g_reduction[dev];
   if (!r.acc) {
-    const size_t bytes = kMaxCols * 4 + kMaxTiles * sizeof(unsigned);
+    const size_t bytes = kMaxCols * 8 + kMaxTiles * sizeof(unsigned);
     void *p = nullptr;
     if (skl_check_hip(hipMalloc(&p, bytes), "gemv scratch") != 0) return false;
     if (skl_check_hip(hipMemset(p, 0, bytes), "gemv scratch clear") != 0) return false;
     r.acc = p;
-    r.tickets = (unsigned *)((char *)p + kMaxCols * 4);
+    r.tickets = (unsigned *)((char *)p + kMaxCols * 8);
   }
   *out = r;
   return true;
@@ -102,6 +108,13 @@ struct GemvArgs {
   unsigned *tickets;
   unsigned tiles, slabs;
 };
+
+// B is read once: a non-temporal 128-bit load.
+typedef unsigned u4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 stream_load(const char *p) {
+  const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v *>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
 
 // 4x4 byte transpose: in r[j] byte i  ->  out t[i] byte j.
 __device__ __forceinline__ void transpose4x4(unsigned r0, unsigned r1, unsigned r2, unsigned r3, unsigned &t0,
@@ -160,7 +173,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
 #pragma unroll
     for (int r = 0; r < kLoadsPerLane; ++r) {
       if (k0 + (size_t)r * Md::kKPerLoad < p.k)
-        rows[r] = *reinterpret_cast<const uint4 *>(wp + (size_t)r * p.b_sk);
+        rows[r] = stream_load(wp + (size_t)r * p.b_sk);
       else
         rows[r] = make_uint4(0, 0, 0, 0);
     }
@@ -170,12 +183,9 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
       int xw[kWords];
       const int8_t *x = reinterpret_cast<const int8_t *>(p.x);
       if (p.x_vec && k0 + Md::kKPerLane <= p.k) {
-        const int4 *xp = reinterpret_cast<const int4 *>(x + k0);
+        const int *xp = reinterpret_cast<const int *>(x + k0);  // k0 is a multiple of kKPerLane: aligned
 #pragma unroll
-        for (int q = 0; q < kWords / 4; ++q) {
-          const int4 v = xp[q];
-          xw[4 * q] = v.x, xw[4 * q + 1] = v.y, xw[4 * q + 2] = v.z, xw[4 * q + 3] = v.w;
-        }
+        for (int q = 0; q < kWords; ++q) xw[q] = xp[q];
       } else {
 #pragma unroll
         for (int g = 0; g < kWords; ++g) {
@@ -249,22 +259,39 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
     }
     return;
   }
-  Acc *scratch = reinterpret_cast<Acc *>(p.acc);
-  if (owner) atomicAdd(&scratch[tile_col0 + threadIdx.x], sum);
-  // Wait until this wave's atomics have been performed, then take a ticket.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  if (threadIdx.x == 0) ticket_s = atomicAdd(&p.tickets[tile], 1u);
-  __syncthreads();
-  if (ticket_s != p.slabs - 1) return;
-  if (owner) {
-    const size_t j = tile_col0 + threadIdx.x;
-    const Acc total = atomicExch(&scratch[j], (Acc)0);  // read the total and leave zero behind
-    Acc *y = yv + j * p.y_s;
-    *y = finish(total, *y, p.alpha, p.beta);
+  if constexpr (std::is_same<Acc, int>::value) {
+    // Integer strips: sum and arrival count travel in one 64-bit atomic (sum in the high word, where
+    // it wraps like int32; count in the low word). The add returns the previous value, so the lane
+    // whose add completes the count holds the total: no ticket, no read-back.
+    if (owner) {
+      const size_t j = tile_col0 + threadIdx.x;
+      unsigned long long *slot = reinterpret_cast<unsigned long long *>(p.acc) + j;
+      const unsigned long long mine = ((unsigned long long)(unsigned)sum << 32) | 1ull;
+      const unsigned long long now = atomicAdd(slot, mine) + mine;
+      if ((unsigned)now == p.slabs) {
+        __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
+        Acc *y = yv + j * p.y_s;
+        *y = finish((int)(unsigned)(now >> 32), *y, p.alpha, p.beta);
+      }
+    }
+  } else {
+    Acc *scratch = reinterpret_cast<Acc *>(p.acc);
+    if (owner) atomicAdd(&scratch[tile_col0 + threadIdx.x], sum);
+    // Wait until this wave's atomics have been performed, then take a ticket.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) ticket_s = atomicAdd(&p.tickets[tile], 1u);
+    __syncthreads();
+    if (ticket_s != p.slabs - 1) return;
+    if (owner) {
+      const size_t j = tile_col0 + threadIdx.x;
+      const Acc total = atomicExch(&scratch[j], (Acc)0);  // read the total and leave zero behind
+      Acc *y = yv + j * p.y_s;
+      *y = finish(total, *y, p.alpha, p.beta);
+    }
+    if (threadIdx.x == 0) atomicExch(&p.tickets[tile], 0u);
   }
-  if (threadIdx.x == 0) atomicExch(&p.tickets[tile], 0u);
 }
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
