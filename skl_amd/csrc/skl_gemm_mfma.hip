@@ -425,26 +425,24 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
 }
 
 // ===========================================================================
-// Streaming variant for whole 256 x 256 tiles: global -> LDS without passing
+// Streaming kernel for whole 256 x 256 tiles: global -> LDS without passing
 // through registers (global_load_lds_dwordx4). Each wave-level load deposits
 // 64 x 16 bytes as one contiguous KiB of LDS, so the tiles are stored without
 // padding and bank conflicts are avoided by an XOR swizzle of the 16-byte
 // chunk index instead; the swizzle is applied on the global side (which chunk
-// a lane fetches) and again by the fragment reads. Four waves, one per SIMD,
-// each own a 128 x 128 block of C (256 accumulator registers): half the LDS
-// bytes per MFMA of a 128 x 64 block, and the registers and LDS-store
-// instructions of the staged copy are gone, which matters because a wave's
-// instruction stream is serial - every load or LDS store it issues is a slot
-// in which it issues no MFMA.
+// a lane fetches) and again by the fragment reads. Eight waves, two per SIMD,
+// each own a 128 x 64 block of C.
 // ===========================================================================
-template <int ES, bool KC>
+template <int ES, bool KC, int SB = kSliceBytes>
 struct STile {
-  static constexpr int kBytes = 256 * kSliceBytes;  // 256 rows x 128 bytes of K, 32 KiB
+  static constexpr int kBytes = 256 * SB;  // 256 rows x SB bytes of K
   // Byte offset of 16-byte chunk `c` of line `r`. A line is an M/N row holding
   // 128 bytes of K (KC), or a k-row holding 256 elements along M/N (MC).
   __device__ static __forceinline__ int chunk(int r, int c) {
-    if constexpr (KC)
+    if constexpr (KC && SB == 128)
       return r * 128 + ((c ^ ((r >> 1) & 7)) << 4);   // 8 chunks; b128 reads take 16 consecutive rows
+    else if constexpr (KC)
+      return r * 64 + ((c ^ ((r >> 2) & 3)) << 4);    // 4 chunks: rows r and r+4 share banks, the XOR parts them
     else if constexpr (ES == 1)
       return r * 256 + ((c ^ ((r & 7) << 1)) << 4);   // 16 chunks; tr8 reads take 8 k-rows x 32 B
     else
@@ -452,9 +450,9 @@ struct STile {
   }
 };
 
-template <int ES, bool KC, int WAVES>
+template <int ES, bool KC, int WAVES, int SB = kSliceBytes>
 struct SLoader {
-  static constexpr int kBlocks = 32 / WAVES;  // KiB blocks per wave, operand and slice
+  static constexpr int kBlocks = SB / 4 / WAVES;  // KiB blocks per wave, operand and slice
   const char *tile_base;
   size_t k_step;
   unsigned off[kBlocks];
@@ -467,9 +465,13 @@ struct SLoader {
 #pragma unroll
     for (int i = 0; i < kBlocks; ++i) {
       const int b = wave * kBlocks + i;
-      if constexpr (KC) {
+      if constexpr (KC && SB == 128) {
         const int row = 8 * b + (lane >> 3), pos = lane & 7;
         const int c = pos ^ ((row >> 1) & 7);
+        off[i] = (unsigned)(((size_t)(row >> 6) * s1 + (size_t)(row & 63) * s0 + (size_t)c * (16 / ES)) * ES);
+      } else if constexpr (KC) {
+        const int row = 16 * b + (lane >> 2), pos = lane & 3;
+        const int c = pos ^ ((row >> 2) & 3);
         off[i] = (unsigned)(((size_t)(row >> 6) * s1 + (size_t)(row & 63) * s0 + (size_t)c * (16 / ES)) * ES);
       } else if constexpr (ES == 1) {
         const int kr = 4 * b + (lane >> 4), pos = lane & 15;
@@ -481,7 +483,7 @@ struct SLoader {
         off[i] = (unsigned)(((size_t)(mn >> 6) * s1 + (size_t)(mn & 63) + (size_t)kr * sk) * 2);
       }
     }
-    k_step = KC ? (size_t)kSliceBytes : (size_t)(kSliceBytes / ES) * sk * ES;
+    k_step = KC ? (size_t)SB : (size_t)(SB / ES) * sk * ES;
   }
 
   // Requests block `i` of this wave's share of `slice`; the data lands in `tile` (LDS).
@@ -496,76 +498,139 @@ struct SLoader {
   }
 };
 
-template <int ES, bool KC, int FRB>
-__device__ __forceinline__ auto read_frag_s(const char *tile, int row0, int kb) {
-  using T = STile<ES, KC>;
-  const int lane = threadIdx.x & 63;
-  const int h = lane >> 5;
-  if constexpr (KC) {
-    const int row = row0 + (lane & 31), c0 = (kb + h * FRB) >> 4;
-    if constexpr (FRB == 16) {
-      return *reinterpret_cast<const v4i *>(tile + T::chunk(row, c0));
-    } else {
-      const v4i lo = *reinterpret_cast<const v4i *>(tile + T::chunk(row, c0));
-      const v4i hi = *reinterpret_cast<const v4i *>(tile + T::chunk(row, c0 + 1));
-      return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    }
-  } else if constexpr (ES == 1) {
-    const int g16 = (lane >> 4) & 1, j = lane & 15;
-    const int kfirst = kb + h * FRB + (j >> 1), c = (row0 >> 4) + g16, sub = (j & 1) * 8;
-    v2i r[FRB / 8];
+// ---------------------------------------------------------------------------
+// The kernel: slices of SB bytes of K in a ring of LDS stages, loads running
+// AHEAD slices ahead (64 bytes, four stages, three ahead as launched), and a
+// software pipeline written out by hand:
+//   * Fragment reads are inline assembly. The compiler cannot tell an LDS read
+//     from the LDS writes of outstanding global->LDS loads apart and makes every
+//     ds_read_tr wait for ALL loads in flight (vmcnt(0)), and it waits for reads
+//     it has only just issued (lgkmcnt(0) in front of every k-step) - either
+//     one exposes a memory latency per k-step. Here the kernel does its own
+//     counting: one lgkmcnt(0) at the top of a k-step, when the only reads in
+//     flight are the ones issued during the previous k-step; one vmcnt(n) per
+//     slice in front of the barrier.
+//   * Reads and loads are dealt out one at a time behind the MFMAs instead of
+//     going out in bursts: a wave issues in order, and a burst that finds the
+//     LDS or the load path busy is a stretch in which it issues no MFMA. The
+//     reads sit behind the first half of a k-step's MFMAs, which leaves the
+//     second half for them to land.
+// ---------------------------------------------------------------------------
+template <int N>
+__device__ __forceinline__ void wait_loads_upto() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int OFF>
+__device__ __forceinline__ v4i lds_read_b128(unsigned addr) {
+  v4i r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+  return r;
+}
+template <int OFF>
+__device__ __forceinline__ v2i lds_read_tr8(unsigned addr) {
+  v2i r;
+  asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+  return r;
+}
+template <int OFF>
+__device__ __forceinline__ v2i lds_read_tr16(unsigned addr) {
+  v2i r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+  return r;
+}
+
+// The fragments of one operand for one wave: NFRAG blocks of 32 rows, read from a tile in pieces of one
+// LDS instruction each. Offsets inside the tile are per lane and computed once; what changes from k-step to
+// k-step and from fragment to fragment is, wherever the swizzle allows, an immediate offset.
+template <int ES, bool KC, int FRB, int KB, int SB, int NFRAG>
+struct FragReader {
+  using T = STile<ES, KC, SB>;
+  using Piece = typename std::conditional<KC, v4i, v2i>::type;
+  static constexpr int kPieceBytes = KC ? 16 : 8;
+  static constexpr int kPieces = FRB / kPieceBytes;  // LDS instructions per fragment
+  static constexpr int kSteps = SB / KB;
+  static constexpr int kBases = KC ? kSteps * kPieces : NFRAG;
+  unsigned base[kBases];
+
+  __device__ void init(int row0) {
+    const int lane = threadIdx.x & 63, h = lane >> 5;
+    if constexpr (KC) {
 #pragma unroll
-    for (int s = 0; s < FRB / 8; ++s)
-      r[s] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, tile + T::chunk(kfirst + 8 * s, c) + sub));
-    if constexpr (FRB == 16) {
-      return v4i{r[0].x, r[0].y, r[1].x, r[1].y};
+      for (int ks = 0; ks < kSteps; ++ks)
+#pragma unroll
+        for (int pc = 0; pc < kPieces; ++pc)
+          base[ks * kPieces + pc] = (unsigned)T::chunk(row0 + (lane & 31), ((ks * KB + h * FRB) >> 4) + pc);
+    } else if constexpr (ES == 1) {
+      const int g16 = (lane >> 4) & 1, j = lane & 15;
+#pragma unroll
+      for (int f = 0; f < NFRAG; ++f)
+        base[f] = (unsigned)(T::chunk(h * FRB + (j >> 1), ((row0 + 32 * f) >> 4) + g16) + (j & 1) * 8);
     } else {
-      return v8i{r[0].x, r[0].y, r[1].x, r[1].y, r[2].x, r[2].y, r[3].x, r[3].y};
+      const int g16 = (lane >> 4) & 1, j = lane & 15;
+#pragma unroll
+      for (int f = 0; f < NFRAG; ++f)
+        base[f] = (unsigned)(T::chunk(h * 8 + (j >> 2), ((row0 + 32 * f) >> 3) + g16 * 2 + ((j & 3) >> 1)) + (j & 1) * 8);
     }
+  }
+  // Piece PC of fragment F for k-step KS of the tile at LDS address `tile`.
+  template <int F, int KS, int PC>
+  __device__ __forceinline__ Piece read(unsigned tile) const {
+    if constexpr (KC)
+      return lds_read_b128<F * 32 * SB>(tile + base[KS * kPieces + PC]);
+    else if constexpr (ES == 1)
+      return lds_read_tr8<KS * KB * 256 + PC * 2048>(tile + base[F]);
+    else
+      return lds_read_tr16<KS * (KB / 2) * 512 + PC * 2048>(tile + base[F]);
+  }
+};
+
+template <typename Frag, typename Piece, int N>
+__device__ __forceinline__ Frag join_pieces(const Piece (&pc)[N]) {
+  if constexpr (sizeof(Piece) == sizeof(Frag)) {
+    return pc[0];
+  } else if constexpr (sizeof(Piece) == 16) {  // two 128-bit pieces
+    return Frag{pc[0].x, pc[0].y, pc[0].z, pc[0].w, pc[1].x, pc[1].y, pc[1].z, pc[1].w};
+  } else if constexpr (N == 2) {
+    return Frag{pc[0].x, pc[0].y, pc[1].x, pc[1].y};
   } else {
-    static_assert(FRB == 16, "16-bit fragments are 16 bytes");
-    const int g16 = (lane >> 4) & 1, j = lane & 15;
-    const int kfirst = kb / 2 + h * 8 + (j >> 2);
-    const int c = (row0 >> 3) + g16 * 2 + ((j & 3) >> 1), sub = (j & 1) * 8;
-    const v4s r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(v4s, tile + T::chunk(kfirst, c) + sub));
-    const v4s r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(v4s, tile + T::chunk(kfirst + 4, c) + sub));
-    const v2i a = __builtin_bit_cast(v2i, r0), b = __builtin_bit_cast(v2i, r1);
-    return v4i{a.x, a.y, b.x, b.y};
+    return Frag{pc[0].x, pc[0].y, pc[1].x, pc[1].y, pc[2].x, pc[2].y, pc[3].x, pc[3].y};
   }
 }
 
-// Scheduling recipe for one k-step of the streaming kernel: after each of the
-// MFMAs place this step's share of LDS reads (ND in total) and of global
-// loads (NV in total), evenly spread. A wave issues in order, so a burst of 16
-// loads or 12 LDS reads in front of the MFMAs is a stretch in which the matrix
-// pipe of its SIMD has nothing to do; one memory instruction in the shadow of
-// each MFMA costs nothing.
-template <int NM, int ND, int NV, int M>
-__device__ __forceinline__ void sched_slot() {
-  constexpr int d = (M + 1) * ND / NM - M * ND / NM;
-  constexpr int v = (M + 1) * NV / NM - M * NV / NM;
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // one MFMA
-  if constexpr (d > 0) __builtin_amdgcn_sched_group_barrier(0x100, d, 0);  // LDS reads
-  if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);  // global loads
-}
-template <int ND, int NV, int... Ms>
-__device__ __forceinline__ void sched_kstep(std::integer_sequence<int, Ms...>) {
-  (sched_slot<(int)sizeof...(Ms), ND, NV, Ms>(), ...);
-}
-
-template <int TA, int TB, bool A_KC, bool B_KC, int WAVES_N>
-__global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_stream_kernel(MfmaArgs p) {
+template <int TA, int TB, bool A_KC, bool B_KC, int WAVES_N, int SB, int STAGES, int AHEAD>
+__global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_ring_kernel(MfmaArgs p) {
   using KA = Kind<TA>;
   using M = Mma<TA, TB>;
+  using Frag = typename M::Frag;
   using Acc = typename KA::Acc;
   using AccElem = decltype(Acc{}.x);
+  static_assert(AHEAD >= 1 && AHEAD < STAGES, "the stage being filled must not be one being read");
   constexpr int ES = KA::ES, KB = KA::KB, FRB = KB / 2;
   constexpr int BM = 256, BN = 256, WM = 128, WN = BN / WAVES_N, MI = 4, NI = WN / 32, WAVES = 2 * WAVES_N;
-  constexpr int kTile = STile<ES, true>::kBytes, kStage = 2 * kTile;
-  constexpr int kSteps = kSliceBytes / KB;
+  constexpr int kTile = STile<ES, true, SB>::kBytes, kStage = 2 * kTile;
+  constexpr int kSteps = SB / KB;
+  constexpr int kUnroll = (kSteps & 1) ? 2 : 1;  // fragment buffers alternate per k-step
   constexpr int kMfmas = MI * NI;
+  constexpr int kLoads = 2 * (SB / 4 / WAVES);   // this wave's loads per slice (A then B)
+  constexpr int kSlots = kSteps * kMfmas;        // MFMA slots per slice
+  constexpr int kPre = (kSteps - 1) * kMfmas;    // slots before the slice's barrier
+  // With one slice of lookahead the next slice is read right after this slice's barrier, so all of
+  // its loads go out before the barrier; with more, they are spread over the whole slice.
+  constexpr int kWindow = AHEAD == 1 ? kPre : kSlots;
+  constexpr int kPeriod = kWindow / kLoads;      // one load every kPeriod slots
+  static_assert(kPeriod >= 1 && kWindow % kLoads == 0 && kPre % kPeriod == 0, "loads must divide the MFMA slots evenly");
+  constexpr int kLoadsPre = kPre / kPeriod;      // loads of an iteration issued before its barrier
+  constexpr int kInFlight = (AHEAD - 2) * kLoads + kLoadsPre;  // loads younger than the next slice's at the barrier
+
+  using RA = FragReader<ES, A_KC, FRB, KB, SB, MI>;
+  using RB = FragReader<ES, B_KC, FRB, KB, SB, NI>;
+  constexpr int PA = RA::kPieces, PB = RB::kPieces;
+  constexpr int kReads = MI * PA + NI * PB;      // LDS instructions per k-step
+  constexpr int kReadSlots = kMfmas / 2;         // ... issued behind the first half of its MFMAs, the rest is time to land
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  const unsigned smem_addr = (unsigned)(size_t)LDS_PTR(char, smem);
 
   unsigned tm, tn;
   tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
@@ -573,10 +638,14 @@ __global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_stream_kernel(MfmaArg
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
 
-  SLoader<ES, A_KC, WAVES> la;
-  SLoader<ES, B_KC, WAVES> lb;
+  SLoader<ES, A_KC, WAVES, SB> la;
+  SLoader<ES, B_KC, WAVES, SB> lb;
   la.init(p.a, m0, p.a_s1, p.a_s0, p.a_sk);
   lb.init(p.b, n0, p.b_s1, p.b_s0, p.b_sk);
+  RA ra;
+  RB rb;
+  ra.init(wm);
+  rb.init(wn);
 
   Acc acc[MI][NI];
 #pragma unroll
@@ -586,87 +655,125 @@ __global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_stream_kernel(MfmaArg
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-  const size_t slices = p.k * ES / kSliceBytes;
-  la.issue(smem, 0);
-  lb.issue(smem + kTile, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  const size_t slices = p.k * ES / SB;
+  // Slices beyond the end are requested as the last slice again: in range, and
+  // the stage they land in is never read, which keeps the load counts static.
+#pragma unroll
+  for (int i = 0; i < AHEAD; ++i) {
+    const size_t sl = (size_t)i < slices ? (size_t)i : slices - 1;
+    la.issue(smem + i * kStage, sl);
+    lb.issue(smem + i * kStage + kTile, sl);
+  }
+  wait_loads_upto<(AHEAD - 1) * kLoads>();
   __syncthreads();
 
-  typename M::Frag fa[2][MI], fb[2][NI];
-#pragma unroll
-  for (int i = 0; i < MI; ++i) fa[0][i] = read_frag_s<ES, A_KC, FRB>(smem, wm + i * 32, 0);
-#pragma unroll
-  for (int j = 0; j < NI; ++j) fb[0][j] = read_frag_s<ES, B_KC, FRB>(smem + kTile, wn + j * 32, 0);
+  typename RA::Piece pa[2][MI][PA];
+  typename RB::Piece pb[2][NI][PB];
 
-  for (size_t s = 0; s < slices; ++s) {
-    const char *ta = smem + (s & 1) * kStage;
-    const char *tb = ta + kTile;
-    char *na = smem + ((s + 1) & 1) * kStage;
-    // The other stage was last read before the barrier that ended the previous
-    // iteration: the next slice streams into it while this one is multiplied.
-    // (The last iteration requests its own slice again: in range, never read.)
-    const size_t nxt = s + 1 < slices ? s + 1 : s;
-    // A wave issues in order and the compute unit has one load path, so the
-    // loads of the next slice are dealt out between the MFMAs (one load per
-    // kGap MFMAs) instead of being issued in a burst, and the LDS reads of the
-    // next k-step go out ahead of this step's MFMAs. The scheduling fences pin
-    // that order: left alone the compiler bunches loads and sinks reads.
-    // The last k-step of the slice is multiplied AFTER the barrier, from
-    // fragments already in registers, so that its MFMAs cover the latency of the
-    // first fragment reads of the next slice.
-    constexpr int kLoads = 2 * (32 / WAVES);        // this wave's loads per slice (A then B)
-    constexpr int kItems = kLoads;
-    constexpr int kSlots = (kSteps - 1) * kMfmas;   // MFMAs before the barrier
-    static_assert(kSteps % 2 == 0, "fragment buffers alternate per k-step");
-    int issued = 0;
-    auto deal = [&](int item) {
-      if (item < kLoads / 2) {
-        la.issue_one(na, nxt, item);
-      } else {
-        lb.issue_one(na + kTile, nxt, item - kLoads / 2);
-      }
-    };
-#pragma unroll
-    for (int ks = 0; ks < kSteps - 1; ++ks) {
-      const int cur = ks & 1, nx = cur ^ 1;
-#pragma unroll
-      for (int i = 0; i < MI; ++i) fa[nx][i] = read_frag_s<ES, A_KC, FRB>(ta, wm + i * 32, (ks + 1) * KB);
-#pragma unroll
-      for (int j = 0; j < NI; ++j) fb[nx][j] = read_frag_s<ES, B_KC, FRB>(tb, wn + j * 32, (ks + 1) * KB);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int q = 0; q < kMfmas; ++q) {
-        const int slot = ks * kMfmas + q;
-#pragma unroll
-        for (int it = 0; it < kItems; ++it)  // items due by this slot (spread evenly over the slots)
-          if (it == issued && it * kSlots <= slot * kItems) {
-            deal(it);
-            ++issued;
-          }
-        const int i = q / NI, j = q % NI;
-        acc[i][j] = M::run(fa[cur][i], fb[cur][j], acc[i][j]);
-        if ((q & 1) == 1) __builtin_amdgcn_sched_barrier(0);
-      }
+  // Read item R of a k-step: fragment by fragment, A and B alternating, so that
+  // what the next k-step's first MFMAs need is requested first.
+  auto read_item = [&](auto rc, auto ksc, int buf, unsigned tile_a, unsigned tile_b) {
+    constexpr int R = decltype(rc)::value, KS = decltype(ksc)::value;
+    constexpr int kPair = PA + PB, kBoth = (MI < NI ? MI : NI) * kPair;
+    if constexpr (R < kBoth) {
+      constexpr int F = R / kPair, W = R % kPair;
+      if constexpr (W < PA)
+        pa[buf][F][W] = ra.template read<F, KS, W>(tile_a);
+      else
+        pb[buf][F][W - PA] = rb.template read<F, KS, W - PA>(tile_b);
+    } else if constexpr (MI > NI) {
+      constexpr int X = R - kBoth, F = NI + X / PA, W = X % PA;
+      pa[buf][F][W] = ra.template read<F, KS, W>(tile_a);
+    } else {
+      constexpr int X = R - kBoth, F = MI + X / PB, W = X % PB;
+      pb[buf][F][W] = rb.template read<F, KS, W>(tile_b);
     }
-#pragma unroll
-    for (int it = 0; it < kItems; ++it)
-      if (it >= issued) deal(it);
-    // Every LDS read of this stage has been issued; wait for them and for the
-    // next slice's data, then let the other waves overwrite this stage.
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-#pragma unroll
-    for (int i = 0; i < MI; ++i) fa[0][i] = read_frag_s<ES, A_KC, FRB>(na, wm + i * 32, 0);
-#pragma unroll
-    for (int j = 0; j < NI; ++j) fb[0][j] = read_frag_s<ES, B_KC, FRB>(na + kTile, wn + j * 32, 0);
-    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto read_all = [&](auto ksc, int buf, unsigned tile_a, unsigned tile_b, auto seq) {
+    [&]<int... Rs>(std::integer_sequence<int, Rs...>) {
+      (read_item(std::integral_constant<int, Rs>{}, ksc, buf, tile_a, tile_b), ...);
+    }(seq);
+  };
+  // All reads in flight have landed; from here on the compiler may use buffer `buf`.
+  auto landed = [&](int buf) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int j = 0; j < NI; ++j) acc[i][j] = M::run(fa[1][i], fb[1][j], acc[i][j]);
-    __builtin_amdgcn_sched_barrier(0);
+      for (int w = 0; w < PA; ++w) asm volatile("" : "+v"(pa[buf][i][w]));
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int w = 0; w < PB; ++w) asm volatile("" : "+v"(pb[buf][j][w]));
+  };
+
+  read_all(std::integral_constant<int, 0>{}, 0, smem_addr, smem_addr + kTile, std::make_integer_sequence<int, kReads>{});
+
+  for (size_t s0 = 0; s0 < slices; s0 += kUnroll) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const size_t s = s0 + u;
+      const unsigned cur_a = smem_addr + (unsigned)(s % STAGES) * kStage;
+      const unsigned nxt_a = smem_addr + (unsigned)((s + 1) % STAGES) * kStage;
+      char *fill = smem + ((s + AHEAD) % STAGES) * kStage;
+      const size_t fill_slice = s + AHEAD < slices ? s + AHEAD : slices - 1;
+      [&]<int... KSs>(std::integer_sequence<int, KSs...>) {
+        (
+            [&](auto ksc) {
+              constexpr int KS = decltype(ksc)::value;
+              constexpr bool kLast = KS == kSteps - 1;
+              constexpr int KSN = kLast ? 0 : KS + 1;       // k-step whose fragments are read during this one
+              const int cur = (u * kSteps + KS) & 1, nx = cur ^ 1;
+              if constexpr (kLast) {
+                // The reads below cross into the next slice: its data must have landed for every wave.
+                // (The loads issued after it - a slice and a bit - may stay in flight.)
+                // Own reads first, so that nobody's read of the stage refilled next is still in flight.
+                wait_loads_upto<kInFlight>();
+                landed(cur);
+                __builtin_amdgcn_s_barrier();
+              } else {
+                landed(cur);
+              }
+              Frag fa[MI], fb[NI];
+#pragma unroll
+              for (int i = 0; i < MI; ++i) fa[i] = join_pieces<Frag>(pa[cur][i]);
+#pragma unroll
+              for (int j = 0; j < NI; ++j) fb[j] = join_pieces<Frag>(pb[cur][j]);
+              const unsigned ta = kLast ? nxt_a : cur_a, tb = ta + kTile;
+              __builtin_amdgcn_sched_barrier(0);
+              [&]<int... Qs>(std::integer_sequence<int, Qs...>) {
+                (
+                    [&](auto qc) {
+                      constexpr int Q = decltype(qc)::value, kSlot = KS * kMfmas + Q;
+                      constexpr int i = Q / NI, j = Q % NI;
+                      acc[i][j] = M::run(fa[i], fb[j], acc[i][j]);
+                      // this slot's share of the next k-step's reads
+                      [&]<int... Rs>(std::integer_sequence<int, Rs...>) {
+                        (
+                            [&](auto rc) {
+                              constexpr int R = decltype(rc)::value;
+                              if constexpr (R * kReadSlots / kReads == Q) read_item(rc, std::integral_constant<int, KSN>{}, nx, ta, tb);
+                            }(std::integral_constant<int, Rs>{}),
+                            ...);
+                      }(std::make_integer_sequence<int, kReads>{});
+                      // and, every kPeriod slots, one load of the slice that is AHEAD slices ahead
+                      if constexpr (kSlot < kWindow && kSlot % kPeriod == 0) {
+                        constexpr int item = kSlot / kPeriod;
+                        if constexpr (item < kLoads / 2)
+                          la.issue_one(fill, fill_slice, item);
+                        else
+                          lb.issue_one(fill + kTile, fill_slice, item - kLoads / 2);
+                      }
+                      __builtin_amdgcn_sched_barrier(0);
+                    }(std::integral_constant<int, Qs>{}),
+                    ...);
+              }(std::make_integer_sequence<int, kMfmas>{});
+            }(std::integral_constant<int, KSs>{}),
+            ...);
+      }(std::make_integer_sequence<int, kSteps>{});
+    }
   }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
   const bool read_c = !(TA == SKL_DT_I8 && p.beta.i == 0);
@@ -687,15 +794,15 @@ __global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_stream_kernel(MfmaArg
   }
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int WAVES_N>
-int launch_stream(const MfmaArgs &args) {
-  constexpr int lds = 4 * STile<1, true>::kBytes;  // two stages of two 32 KiB tiles
-  auto kernel = gemm_mfma_stream_kernel<TA, TB, A_KC, B_KC, WAVES_N>;
+template <int TA, int TB, bool A_KC, bool B_KC, int WAVES_N, int SB, int STAGES, int AHEAD>
+int launch_ring(const MfmaArgs &args) {
+  constexpr int lds = STAGES * 2 * STile<1, true, SB>::kBytes;
+  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, WAVES_N, SB, STAGES, AHEAD>;
   static bool configured = false;
   if (!configured) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                           "gemm_mfma_stream: LDS size");
+                           "gemm_mfma_ring: LDS size");
     if (rc != 0) return rc;
     configured = true;
   }
@@ -708,7 +815,7 @@ int launch_stream(const MfmaArgs &args) {
     return -2;
   }
   kernel<<<(unsigned)grid, 128 * WAVES_N, lds, skl_current_stream()>>>(p);
-  return skl_check_launch("gemm_mfma_stream");
+  return skl_check_launch("gemm_mfma_ring");
 }
 
 template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED>
@@ -744,11 +851,7 @@ int launch_tile(const MfmaArgs &p) {
   // 256 compute units with it; everything else runs on the small, bounds-checked one.
   const bool whole = p.m % 256 == 0 && p.n % 256 == 0 && (p.k * ES) % kSliceBytes == 0;
   const size_t big_tiles = (p.m / 256) * (p.n / 256);
-  if (whole && big_tiles >= 200) {
-    static const int waves_n = getenv("SKL_STREAM_WAVES_N") ? atoi(getenv("SKL_STREAM_WAVES_N")) : 4;
-    if (waves_n == 2) return launch_stream<TA, TB, A_KC, B_KC, 2>(p);
-    return launch_stream<TA, TB, A_KC, B_KC, 4>(p);
-  }
+  if (whole && big_tiles >= 200) return launch_ring<TA, TB, A_KC, B_KC, 4, 64, 4, 3>(p);
   return launch_one<TA, TB, A_KC, B_KC, 128, 128, 2, 4, true>(p);
 }
 
