@@ -433,26 +433,30 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
 // a lane fetches) and again by the fragment reads. Eight waves, two per SIMD,
 // each own a 128 x 64 block of C.
 // ===========================================================================
-template <int ES, bool KC, int SB = kSliceBytes>
+template <int ES, bool KC, int SB, int ROWS>
 struct STile {
-  static constexpr int kBytes = 256 * SB;  // 256 rows x SB bytes of K
+  static constexpr int kBytes = ROWS * SB;   // ROWS rows x SB bytes of K
+  static constexpr int kRowBytes = ROWS * ES;  // a k-row of an MN-contiguous tile
   // Byte offset of 16-byte chunk `c` of line `r`. A line is an M/N row holding
-  // 128 bytes of K (KC), or a k-row holding 256 elements along M/N (MC).
+  // SB bytes of K (KC), or a k-row holding ROWS elements along M/N (MC).
   __device__ static __forceinline__ int chunk(int r, int c) {
     if constexpr (KC && SB == 128)
       return r * 128 + ((c ^ ((r >> 1) & 7)) << 4);   // 8 chunks; b128 reads take 16 consecutive rows
     else if constexpr (KC)
       return r * 64 + ((c ^ ((r >> 2) & 3)) << 4);    // 4 chunks: rows r and r+4 share banks, the XOR parts them
-    else if constexpr (ES == 1)
+    else if constexpr (ES == 1 && kRowBytes == 256)
       return r * 256 + ((c ^ ((r & 7) << 1)) << 4);   // 16 chunks; tr8 reads take 8 k-rows x 32 B
+    else if constexpr (ES == 1)
+      return r * 128 + ((c ^ (((r >> 1) & 3) << 1)) << 4);  // 8 chunks: two k-rows fill the banks once
     else
-      return r * 512 + ((c ^ ((r & 3) << 2)) << 4);   // 32 chunks; tr16 reads take 4 k-rows x 64 B
+      return r * kRowBytes + ((c ^ ((r & 3) << 2)) << 4);   // 32 or 16 chunks; tr16 reads take 4 k-rows x 64 B
   }
 };
 
-template <int ES, bool KC, int WAVES, int SB = kSliceBytes>
+template <int ES, bool KC, int WAVES, int SB, int ROWS>
 struct SLoader {
-  static constexpr int kBlocks = SB / 4 / WAVES;  // KiB blocks per wave, operand and slice
+  static constexpr int kBlocks = ROWS * SB / 1024 / WAVES;  // KiB blocks per wave, operand and slice
+  static_assert(kBlocks >= 1, "every wave loads at least one block per slice");
   const char *tile_base;
   size_t k_step;
   unsigned off[kBlocks];
@@ -473,14 +477,12 @@ struct SLoader {
         const int row = 16 * b + (lane >> 2), pos = lane & 3;
         const int c = pos ^ ((row >> 2) & 3);
         off[i] = (unsigned)(((size_t)(row >> 6) * s1 + (size_t)(row & 63) * s0 + (size_t)c * (16 / ES)) * ES);
-      } else if constexpr (ES == 1) {
-        const int kr = 4 * b + (lane >> 4), pos = lane & 15;
-        const int mn = (pos ^ ((kr & 7) << 1)) * 16;
-        off[i] = (unsigned)((size_t)(mn >> 6) * s1 + (size_t)(mn & 63) + (size_t)kr * sk);
       } else {
-        const int kr = 2 * b + (lane >> 5), pos = lane & 31;
-        const int mn = (pos ^ ((kr & 3) << 2)) * 8;
-        off[i] = (unsigned)(((size_t)(mn >> 6) * s1 + (size_t)(mn & 63) + (size_t)kr * sk) * 2);
+        using T = STile<ES, false, SB, ROWS>;
+        constexpr int kLanesPerRow = T::kRowBytes / 16, kRowsPerBlock = 1024 / T::kRowBytes;
+        const int kr = kRowsPerBlock * b + lane / kLanesPerRow, pos = lane % kLanesPerRow;
+        const int mn = ((T::chunk(kr, pos) - kr * T::kRowBytes) >> 4) * (16 / ES);  // the chunk stored at position `pos`
+        off[i] = (unsigned)(((size_t)(mn >> 6) * s1 + (size_t)(mn & 63) + (size_t)kr * sk) * ES);
       }
     }
     k_step = KC ? (size_t)SB : (size_t)(SB / ES) * sk * ES;
@@ -543,9 +545,10 @@ __device__ __forceinline__ v2i lds_read_tr16(unsigned addr) {
 // The fragments of one operand for one wave: NFRAG blocks of 32 rows, read from a tile in pieces of one
 // LDS instruction each. Offsets inside the tile are per lane and computed once; what changes from k-step to
 // k-step and from fragment to fragment is, wherever the swizzle allows, an immediate offset.
-template <int ES, bool KC, int FRB, int KB, int SB, int NFRAG>
+template <int ES, bool KC, int FRB, int KB, int SB, int ROWS, int NFRAG>
 struct FragReader {
-  using T = STile<ES, KC, SB>;
+  using T = STile<ES, KC, SB, ROWS>;
+  static constexpr int RB = T::kRowBytes;
   using Piece = typename std::conditional<KC, v4i, v2i>::type;
   static constexpr int kPieceBytes = KC ? 16 : 8;
   static constexpr int kPieces = FRB / kPieceBytes;  // LDS instructions per fragment
@@ -579,9 +582,9 @@ struct FragReader {
     if constexpr (KC)
       return lds_read_b128<F * 32 * SB>(tile + base[KS * kPieces + PC]);
     else if constexpr (ES == 1)
-      return lds_read_tr8<KS * KB * 256 + PC * 2048>(tile + base[F]);
+      return lds_read_tr8<KS * KB * RB + PC * 8 * RB>(tile + base[F]);
     else
-      return lds_read_tr16<KS * (KB / 2) * 512 + PC * 2048>(tile + base[F]);
+      return lds_read_tr16<KS * (KB / 2) * RB + PC * 4 * RB>(tile + base[F]);
   }
 };
 
@@ -598,8 +601,8 @@ __device__ __forceinline__ Frag join_pieces(const Piece (&pc)[N]) {
   }
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int WAVES_N, int SB, int STAGES, int AHEAD>
-__global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_ring_kernel(MfmaArgs p) {
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, int SB, int STAGES, int AHEAD>
+__global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   using KA = Kind<TA>;
   using M = Mma<TA, TB>;
   using Frag = typename M::Frag;
@@ -607,24 +610,28 @@ __global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_ring_kernel(MfmaArgs 
   using AccElem = decltype(Acc{}.x);
   static_assert(AHEAD >= 1 && AHEAD < STAGES, "the stage being filled must not be one being read");
   constexpr int ES = KA::ES, KB = KA::KB, FRB = KB / 2;
-  constexpr int BM = 256, BN = 256, WM = 128, WN = BN / WAVES_N, MI = 4, NI = WN / 32, WAVES = 2 * WAVES_N;
-  constexpr int kTile = STile<ES, true, SB>::kBytes, kStage = 2 * kTile;
+  // Eight waves: 2 x 4 blocks of 128 x 64 on a 256 x 256 tile, 4 x 2 blocks of 64 x 64 on a 256 x 128 one.
+  constexpr int BM = 256, WAVES = 8, WAVES_N = BN == 256 ? 4 : 2, WAVES_M = WAVES / WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MI = WM / 32, NI = WN / 32;
+  constexpr int kTile = BM * SB, kTileB = BN * SB, kStage = kTile + kTileB;  // a stage: A's tile, then B's
   constexpr int kSteps = SB / KB;
   constexpr int kUnroll = (kSteps & 1) ? 2 : 1;  // fragment buffers alternate per k-step
   constexpr int kMfmas = MI * NI;
-  constexpr int kLoads = 2 * (SB / 4 / WAVES);   // this wave's loads per slice (A then B)
+  using LA = SLoader<ES, A_KC, WAVES, SB, BM>;
+  using LB = SLoader<ES, B_KC, WAVES, SB, BN>;
+  constexpr int kLoadsA = LA::kBlocks, kLoads = kLoadsA + LB::kBlocks;  // this wave's loads per slice (A then B)
   constexpr int kSlots = kSteps * kMfmas;        // MFMA slots per slice
   constexpr int kPre = (kSteps - 1) * kMfmas;    // slots before the slice's barrier
   // With one slice of lookahead the next slice is read right after this slice's barrier, so all of
   // its loads go out before the barrier; with more, they are spread over the whole slice.
   constexpr int kWindow = AHEAD == 1 ? kPre : kSlots;
-  constexpr int kPeriod = kWindow / kLoads;      // one load every kPeriod slots
-  static_assert(kPeriod >= 1 && kWindow % kLoads == 0 && kPre % kPeriod == 0, "loads must divide the MFMA slots evenly");
-  constexpr int kLoadsPre = kPre / kPeriod;      // loads of an iteration issued before its barrier
+  static_assert(kWindow >= 1, "one slice of lookahead needs a k-step in front of the barrier");
+  // Load `it` goes out behind MFMA slot it * kWindow / kLoads.
+  constexpr int kLoadsPre = AHEAD == 1 ? kLoads : (kPre * kLoads + kWindow - 1) / kWindow;  // issued before the barrier
   constexpr int kInFlight = (AHEAD - 2) * kLoads + kLoadsPre;  // loads younger than the next slice's at the barrier
 
-  using RA = FragReader<ES, A_KC, FRB, KB, SB, MI>;
-  using RB = FragReader<ES, B_KC, FRB, KB, SB, NI>;
+  using RA = FragReader<ES, A_KC, FRB, KB, SB, BM, MI>;
+  using RB = FragReader<ES, B_KC, FRB, KB, SB, BN, NI>;
   constexpr int PA = RA::kPieces, PB = RB::kPieces;
   constexpr int kReads = MI * PA + NI * PB;      // LDS instructions per k-step
   constexpr int kReadSlots = kMfmas / 2;         // ... issued behind the first half of its MFMAs, the rest is time to land
@@ -638,8 +645,8 @@ __global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_ring_kernel(MfmaArgs 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
 
-  SLoader<ES, A_KC, WAVES, SB> la;
-  SLoader<ES, B_KC, WAVES, SB> lb;
+  LA la;
+  LB lb;
   la.init(p.a, m0, p.a_s1, p.a_s0, p.a_sk);
   lb.init(p.b, n0, p.b_s1, p.b_s0, p.b_sk);
   RA ra;
@@ -756,14 +763,20 @@ __global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_ring_kernel(MfmaArgs 
                             }(std::integral_constant<int, Rs>{}),
                             ...);
                       }(std::make_integer_sequence<int, kReads>{});
-                      // and, every kPeriod slots, one load of the slice that is AHEAD slices ahead
-                      if constexpr (kSlot < kWindow && kSlot % kPeriod == 0) {
-                        constexpr int item = kSlot / kPeriod;
-                        if constexpr (item < kLoads / 2)
-                          la.issue_one(fill, fill_slice, item);
-                        else
-                          lb.issue_one(fill + kTile, fill_slice, item - kLoads / 2);
-                      }
+                      // and this slot's share of the loads of the slice that is AHEAD slices ahead
+                      [&]<int... Ls>(std::integer_sequence<int, Ls...>) {
+                        (
+                            [&](auto lc) {
+                              constexpr int L = decltype(lc)::value;
+                              if constexpr (L * kWindow / kLoads == kSlot) {
+                                if constexpr (L < kLoadsA)
+                                  la.issue_one(fill, fill_slice, L);
+                                else
+                                  lb.issue_one(fill + kTile, fill_slice, L - kLoadsA);
+                              }
+                            }(std::integral_constant<int, Ls>{}),
+                            ...);
+                      }(std::make_integer_sequence<int, kLoads>{});
                       __builtin_amdgcn_sched_barrier(0);
                     }(std::integral_constant<int, Qs>{}),
                     ...);
@@ -794,10 +807,10 @@ __global__ void __launch_bounds__(128 * WAVES_N) gemm_mfma_ring_kernel(MfmaArgs 
   }
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int WAVES_N, int SB, int STAGES, int AHEAD>
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, int SB, int STAGES, int AHEAD>
 int launch_ring(const MfmaArgs &args) {
-  constexpr int lds = STAGES * 2 * STile<1, true, SB>::kBytes;
-  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, WAVES_N, SB, STAGES, AHEAD>;
+  constexpr int lds = STAGES * (256 + BN) * SB;
+  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, SB, STAGES, AHEAD>;
   static bool configured = false;
   if (!configured) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -808,13 +821,13 @@ int launch_ring(const MfmaArgs &args) {
   }
   MfmaArgs p = args;
   p.tiles_m = (unsigned)(p.m / 256);
-  p.tiles_n = (unsigned)(p.n / 256);
+  p.tiles_n = (unsigned)(p.n / BN);
   const size_t grid = (size_t)p.tiles_m * p.tiles_n;
   if (grid > 0x7FFFFFFFu) {
     skl_hip_record_error(-2, "gemm_mfma: grid too large");
     return -2;
   }
-  kernel<<<(unsigned)grid, 128 * WAVES_N, lds, skl_current_stream()>>>(p);
+  kernel<<<(unsigned)grid, 512, lds, skl_current_stream()>>>(p);
   return skl_check_launch("gemm_mfma_ring");
 }
 
@@ -847,11 +860,14 @@ int launch_one(const MfmaArgs &args) {
 template <int TA, int TB, bool A_KC, bool B_KC>
 int launch_tile(const MfmaArgs &p) {
   constexpr int ES = Kind<TA>::ES;
-  // The large tile takes problems that it divides evenly and that can fill the
-  // 256 compute units with it; everything else runs on the small, bounds-checked one.
-  const bool whole = p.m % 256 == 0 && p.n % 256 == 0 && (p.k * ES) % kSliceBytes == 0;
-  const size_t big_tiles = (p.m / 256) * (p.n / 256);
-  if (whole && big_tiles >= 200) return launch_ring<TA, TB, A_KC, B_KC, 4, 64, 4, 3>(p);
+  // The streaming kernel takes problems that its tiles divide evenly: 256 x 256 tiles when those
+  // can fill the 256 compute units, 256 x 128 tiles for the sizes below that; everything else runs
+  // on the small, bounds-checked kernel.
+  if (p.m % 256 == 0 && (p.k * ES) % 128 == 0) {
+    const size_t tiles_m = p.m / 256;
+    if (p.n % 256 == 0 && tiles_m * (p.n / 256) >= 200) return launch_ring<TA, TB, A_KC, B_KC, 256, 64, 4, 3>(p);
+    if (p.n % 128 == 0 && tiles_m * (p.n / 128) >= 96) return launch_ring<TA, TB, A_KC, B_KC, 128, 64, 4, 3>(p);
+  }
   return launch_one<TA, TB, A_KC, B_KC, 128, 128, 2, 4, true>(p);
 }
 

@@ -149,21 +149,22 @@ def _dense_case(ta, m, n, k, a_kc, b_kc, alpha, beta, tb=None):
                             rsb1=1 if b_kc else n, csb1=k if b_kc else 1, rsc0=0, csc0=0, rsc1=n, csc1=1)
 
 
+@pytest.mark.parametrize("m,n", ((4096, 4096), (2048, 1664)))
 @pytest.mark.parametrize("a_kc,b_kc", ((True, False), (False, False), (True, True), (False, True)))
 @pytest.mark.parametrize("ta", ("i8", "bf16", "f16", "f8e4m3", "f8e5m2", "mixed"))
-def test_whole_tile_streaming_kernel(gpu, ta, a_kc, b_kc):
-    """4096 x 4096 outputs (256 tiles of 256 x 256: the streaming matrix-core
-    kernel) for every operand orientation. Too large for the scalar checker: the
+def test_whole_tile_streaming_kernel(gpu, ta, a_kc, b_kc, m, n):
+    """4096 x 4096 outputs (256 tiles of 256 x 256) and 2048 x 1664 outputs (104
+    tiles of 256 x 128): the two tile shapes of the streaming matrix-core kernel,
+    for every operand orientation. Too large for the scalar checker: the
     expected result is numpy's fp64 product, which is exact for the integer case
     (|sum| < 2^53) and the fp64-accumulated reference for the others."""
-    m = n = 4096
     k = 384 if ta == "i8" else 256
     tb = None
     if ta == "mixed":
         ta, tb = "f8e4m3", "f8e5m2"
     alpha, beta = (3, -2) if ta == "i8" else (1.5, 0.5)
     case = _dense_case(ta, m, n, k, a_kc, b_kc, alpha, beta, tb)
-    rng = np.random.default_rng(hash((ta, a_kc, b_kc)) % (1 << 31))
+    rng = np.random.default_rng((sum(map(ord, ta + str(tb))) * 4 + a_kc * 2 + b_kc + n) % (1 << 31))
     a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
     if ta.startswith("f8"):   # N(0,1)-like spread instead of log-uniform bytes: the config-4 distribution
         a = rng.integers(0x28, 0x48, size=a.size, dtype=np.uint8) | (rng.integers(0, 2, size=a.size, dtype=np.uint8) << 7)
