@@ -425,25 +425,39 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
 }
 
 // ===========================================================================
-// Streaming kernel for whole 256 x 256 tiles: global -> LDS without passing
-// through registers (global_load_lds_dwordx4). Each wave-level load deposits
-// 64 x 16 bytes as one contiguous KiB of LDS, so the tiles are stored without
+// Streaming kernel for whole tiles (256 x 256 or 256 x 128): global -> LDS
+// without passing through registers (global_load_lds_dwordx4), K in slices of
+// 64 bytes held in a ring of four LDS stages. Each wave-level load deposits
+// 64 x 16 bytes as one contiguous KiB of LDS, so tiles are stored without
 // padding and bank conflicts are avoided by an XOR swizzle of the 16-byte
 // chunk index instead; the swizzle is applied on the global side (which chunk
-// a lane fetches) and again by the fragment reads. Eight waves, two per SIMD,
-// each own a 128 x 64 block of C.
+// a lane fetches) and again by the fragment reads. Eight waves, two per SIMD.
+//
+// An MN-contiguous operand (k-rows of ROWS elements) is loaded a slice at a
+// time: a load covers whole k-rows, i.e. whole 128-byte lines. A K-contiguous
+// operand is different: a 64-byte slice is HALF a line of each row, and loads
+// made of half lines run at less than half the rate of loads made of whole
+// ones. So its loads cover 8 rows x 128 bytes - two slices at once - and the
+// four stages of such an operand are interleaved in LDS at 512-byte granularity
+// (8 rows x 64 bytes of stage 0, then of stage 1, ...), which puts the two
+// halves of such a load next to each other: one KiB, as the load writes it.
 // ===========================================================================
-template <int ES, bool KC, int SB, int ROWS>
+constexpr int kRingSlice = 64;   // bytes of K per stage
+constexpr int kRingStages = 4;
+
+template <int ES, bool KC, int ROWS, int NS = kRingStages>
 struct STile {
-  static constexpr int kBytes = ROWS * SB;   // ROWS rows x SB bytes of K
-  static constexpr int kRowBytes = ROWS * ES;  // a k-row of an MN-contiguous tile
-  // Byte offset of 16-byte chunk `c` of line `r`. A line is an M/N row holding
-  // SB bytes of K (KC), or a k-row holding ROWS elements along M/N (MC).
+  static constexpr int kStages = NS;
+  static constexpr int kBytes = ROWS * kRingSlice;            // one stage
+  static constexpr int kRegion = kBytes * NS;                 // all stages of the operand
+  static constexpr int kRowBytes = ROWS * ES;                 // a k-row of an MN-contiguous tile
+  static constexpr int kStageStep = KC ? 512 : kBytes;        // from one stage to the next
+  static constexpr int kGroup = NS * 512;                     // K-contiguous: from 8 rows to the next 8
+  // Byte offset (inside stage 0) of 16-byte chunk `c` of line `r`. A line is an M/N row
+  // holding 64 bytes of K (KC), or a k-row holding ROWS elements along M/N (MC).
   __device__ static __forceinline__ int chunk(int r, int c) {
-    if constexpr (KC && SB == 128)
-      return r * 128 + ((c ^ ((r >> 1) & 7)) << 4);   // 8 chunks; b128 reads take 16 consecutive rows
-    else if constexpr (KC)
-      return r * 64 + ((c ^ ((r >> 2) & 3)) << 4);    // 4 chunks: rows r and r+4 share banks, the XOR parts them
+    if constexpr (KC)  // 4 chunks: rows r and r+4 share banks, the XOR parts them; 16 rows fill the banks once
+      return (r >> 3) * kGroup + (r & 7) * 64 + ((c ^ ((r >> 2) & 3)) << 4);
     else if constexpr (ES == 1 && kRowBytes == 256)
       return r * 256 + ((c ^ ((r & 7) << 1)) << 4);   // 16 chunks; tr8 reads take 8 k-rows x 32 B
     else if constexpr (ES == 1)
@@ -453,57 +467,56 @@ struct STile {
   }
 };
 
-template <int ES, bool KC, int WAVES, int SB, int ROWS>
+// Global -> LDS loads of one operand, this wave's share. `unit` below is a slice
+// for an MN-contiguous operand and a pair of slices for a K-contiguous one.
+template <int ES, bool KC, int WAVES, int ROWS, int NS>
 struct SLoader {
-  static constexpr int kBlocks = ROWS * SB / 1024 / WAVES;  // KiB blocks per wave, operand and slice
-  static_assert(kBlocks >= 1, "every wave loads at least one block per slice");
+  using T = STile<ES, KC, ROWS, NS>;
+  static constexpr int kUnitBytes = KC ? 2 * T::kBytes : T::kBytes;
+  static constexpr int kBlocks = kUnitBytes / 1024 / WAVES;  // KiB blocks per wave and unit
+  static_assert(kBlocks >= 1, "every wave loads at least one block per unit");
   const char *tile_base;
-  size_t k_step;
-  unsigned off[kBlocks];
-  unsigned lds_block;  // byte offset of this wave's first block inside the operand tile
+  size_t k_step;           // bytes from one unit to the next
+  unsigned off[kBlocks];   // global byte offsets of this lane
+  unsigned lds[kBlocks];   // LDS byte offsets (inside the operand's region, stage 0) of the blocks
 
   __device__ void init(const char *base, size_t mn0, size_t s1, size_t s0, size_t sk) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     tile_base = base + (mn0 >> 6) * s1 * ES;
-    lds_block = wave * kBlocks * 1024;
 #pragma unroll
     for (int i = 0; i < kBlocks; ++i) {
       const int b = wave * kBlocks + i;
-      if constexpr (KC && SB == 128) {
-        const int row = 8 * b + (lane >> 3), pos = lane & 7;
-        const int c = pos ^ ((row >> 1) & 7);
-        off[i] = (unsigned)(((size_t)(row >> 6) * s1 + (size_t)(row & 63) * s0 + (size_t)c * (16 / ES)) * ES);
-      } else if constexpr (KC) {
-        const int row = 16 * b + (lane >> 2), pos = lane & 3;
+      if constexpr (KC) {  // block = 8 rows x (64 bytes of the even slice, then 64 bytes of the odd one)
+        const int half = lane >> 5, row = 8 * b + ((lane & 31) >> 2), pos = lane & 3;
         const int c = pos ^ ((row >> 2) & 3);
-        off[i] = (unsigned)(((size_t)(row >> 6) * s1 + (size_t)(row & 63) * s0 + (size_t)c * (16 / ES)) * ES);
+        off[i] = (unsigned)(((size_t)(row >> 6) * s1 + (size_t)(row & 63) * s0) * ES + half * 64 + c * 16);
+        lds[i] = b * T::kGroup;
       } else {
-        using T = STile<ES, false, SB, ROWS>;
         constexpr int kLanesPerRow = T::kRowBytes / 16, kRowsPerBlock = 1024 / T::kRowBytes;
         const int kr = kRowsPerBlock * b + lane / kLanesPerRow, pos = lane % kLanesPerRow;
         const int mn = ((T::chunk(kr, pos) - kr * T::kRowBytes) >> 4) * (16 / ES);  // the chunk stored at position `pos`
         off[i] = (unsigned)(((size_t)(mn >> 6) * s1 + (size_t)(mn & 63) + (size_t)kr * sk) * ES);
+        lds[i] = b * 1024;
       }
     }
-    k_step = KC ? (size_t)SB : (size_t)(SB / ES) * sk * ES;
+    k_step = KC ? (size_t)(2 * kRingSlice) : (size_t)(kRingSlice / ES) * sk * ES;
   }
 
-  // Requests block `i` of this wave's share of `slice`; the data lands in `tile` (LDS).
-  __device__ __forceinline__ void issue_one(char *tile, size_t slice, int i) const {
-    const char *g = tile_base + slice * k_step;
+  // Requests block `i` of `unit`; it lands in stage `stage` (the even one of the pair for KC) of `region`.
+  __device__ __forceinline__ void issue_one(char *region, int stage, size_t unit, int i) const {
+    const char *g = tile_base + unit * k_step;
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(g + off[i]),
-                                     (__attribute__((address_space(3))) void *)(tile + lds_block + i * 1024), 16, 0, 0);
+                                     (__attribute__((address_space(3))) void *)(region + stage * T::kStageStep + lds[i]),
+                                     16, 0, 0);
   }
-  __device__ __forceinline__ void issue(char *tile, size_t slice) const {
+  __device__ __forceinline__ void issue(char *region, int stage, size_t unit) const {
 #pragma unroll
-    for (int i = 0; i < kBlocks; ++i) issue_one(tile, slice, i);
+    for (int i = 0; i < kBlocks; ++i) issue_one(region, stage, unit, i);
   }
 };
 
 // ---------------------------------------------------------------------------
-// The kernel: slices of SB bytes of K in a ring of LDS stages, loads running
-// AHEAD slices ahead (64 bytes, four stages, three ahead as launched), and a
-// software pipeline written out by hand:
+// The software pipeline is written out by hand:
 //   * Fragment reads are inline assembly. The compiler cannot tell an LDS read
 //     from the LDS writes of outstanding global->LDS loads apart and makes every
 //     ds_read_tr wait for ALL loads in flight (vmcnt(0)), and it waits for reads
@@ -542,17 +555,17 @@ __device__ __forceinline__ v2i lds_read_tr16(unsigned addr) {
   return r;
 }
 
-// The fragments of one operand for one wave: NFRAG blocks of 32 rows, read from a tile in pieces of one
-// LDS instruction each. Offsets inside the tile are per lane and computed once; what changes from k-step to
+// The fragments of one operand for one wave: NFRAG blocks of 32 rows, read from a stage in pieces of one
+// LDS instruction each. Offsets inside the stage are per lane and computed once; what changes from k-step to
 // k-step and from fragment to fragment is, wherever the swizzle allows, an immediate offset.
-template <int ES, bool KC, int FRB, int KB, int SB, int ROWS, int NFRAG>
+template <int ES, bool KC, int FRB, int KB, int ROWS, int NS, int NFRAG>
 struct FragReader {
-  using T = STile<ES, KC, SB, ROWS>;
-  static constexpr int RB = T::kRowBytes;
+  using T = STile<ES, KC, ROWS, NS>;
   using Piece = typename std::conditional<KC, v4i, v2i>::type;
+  static constexpr int RB = T::kRowBytes;
   static constexpr int kPieceBytes = KC ? 16 : 8;
   static constexpr int kPieces = FRB / kPieceBytes;  // LDS instructions per fragment
-  static constexpr int kSteps = SB / KB;
+  static constexpr int kSteps = kRingSlice / KB;
   static constexpr int kBases = KC ? kSteps * kPieces : NFRAG;
   unsigned base[kBases];
 
@@ -576,15 +589,15 @@ struct FragReader {
         base[f] = (unsigned)(T::chunk(h * 8 + (j >> 2), ((row0 + 32 * f) >> 3) + g16 * 2 + ((j & 3) >> 1)) + (j & 1) * 8);
     }
   }
-  // Piece PC of fragment F for k-step KS of the tile at LDS address `tile`.
+  // Piece PC of fragment F for k-step KS of the stage at LDS address `stage`.
   template <int F, int KS, int PC>
-  __device__ __forceinline__ Piece read(unsigned tile) const {
+  __device__ __forceinline__ Piece read(unsigned stage) const {
     if constexpr (KC)
-      return lds_read_b128<F * 32 * SB>(tile + base[KS * kPieces + PC]);
+      return lds_read_b128<F * 4 * T::kGroup>(stage + base[KS * kPieces + PC]);  // 32 rows = four groups of 8
     else if constexpr (ES == 1)
-      return lds_read_tr8<KS * KB * RB + PC * 8 * RB>(tile + base[F]);
+      return lds_read_tr8<KS * KB * RB + PC * 8 * RB>(stage + base[F]);
     else
-      return lds_read_tr16<KS * (KB / 2) * RB + PC * 4 * RB>(tile + base[F]);
+      return lds_read_tr16<KS * (KB / 2) * RB + PC * 4 * RB>(stage + base[F]);
   }
 };
 
@@ -601,43 +614,57 @@ __device__ __forceinline__ Frag join_pieces(const Piece (&pc)[N]) {
   }
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BN, int SB, int STAGES, int AHEAD>
+constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+template <int TA, int TB, bool A_KC, bool B_KC, int BN>
 __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   using KA = Kind<TA>;
   using M = Mma<TA, TB>;
   using Frag = typename M::Frag;
   using Acc = typename KA::Acc;
   using AccElem = decltype(Acc{}.x);
-  static_assert(AHEAD >= 1 && AHEAD < STAGES, "the stage being filled must not be one being read");
+  constexpr int SB = kRingSlice, STAGES = kRingStages;
   constexpr int ES = KA::ES, KB = KA::KB, FRB = KB / 2;
   // Eight waves: 2 x 4 blocks of 128 x 64 on a 256 x 256 tile, 4 x 2 blocks of 64 x 64 on a 256 x 128 one.
   constexpr int BM = 256, WAVES = 8, WAVES_N = BN == 256 ? 4 : 2, WAVES_M = WAVES / WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MI = WM / 32, NI = WN / 32;
-  constexpr int kTile = BM * SB, kTileB = BN * SB, kStage = kTile + kTileB;  // a stage: A's tile, then B's
   constexpr int kSteps = SB / KB;
-  constexpr int kUnroll = (kSteps & 1) ? 2 : 1;  // fragment buffers alternate per k-step
   constexpr int kMfmas = MI * NI;
-  using LA = SLoader<ES, A_KC, WAVES, SB, BM>;
-  using LB = SLoader<ES, B_KC, WAVES, SB, BN>;
-  constexpr int kLoadsA = LA::kBlocks, kLoads = kLoadsA + LB::kBlocks;  // this wave's loads per slice (A then B)
   constexpr int kSlots = kSteps * kMfmas;        // MFMA slots per slice
   constexpr int kPre = (kSteps - 1) * kMfmas;    // slots before the slice's barrier
-  // With one slice of lookahead the next slice is read right after this slice's barrier, so all of
-  // its loads go out before the barrier; with more, they are spread over the whole slice.
-  constexpr int kWindow = AHEAD == 1 ? kPre : kSlots;
-  static_assert(kWindow >= 1, "one slice of lookahead needs a k-step in front of the barrier");
-  // Load `it` goes out behind MFMA slot it * kWindow / kLoads.
-  constexpr int kLoadsPre = AHEAD == 1 ? kLoads : (kPre * kLoads + kWindow - 1) / kWindow;  // issued before the barrier
-  constexpr int kInFlight = (AHEAD - 2) * kLoads + kLoadsPre;  // loads younger than the next slice's at the barrier
+  // Four stages per operand; pair loads run two slices ahead. (Six stages for a K-contiguous operand
+  // and pairs four slices ahead fit the 160 KiB of LDS next to an MN-contiguous partner, and measured slower.)
+  constexpr int NSA = STAGES, NSB = STAGES;
+  constexpr int kPairAhead = 2;
+  using LA = SLoader<ES, A_KC, WAVES, BM, NSA>;
+  using LB = SLoader<ES, B_KC, WAVES, BN, NSB>;
+  using TileA = STile<ES, A_KC, BM, NSA>;
+  using TileB = STile<ES, B_KC, BN, NSB>;
+  // An even slice issues the pair loads of the K-contiguous operands (slices s+2 and s+3) and, like
+  // every slice, the loads of slice s+3 of the MN-contiguous ones. Load `it` of the kLoads<even/odd>
+  // goes out behind MFMA slot it * kSlots / kLoads, K-contiguous operands first.
+  constexpr int kPairA = A_KC ? LA::kBlocks : 0, kPairB = B_KC ? LB::kBlocks : 0;
+  constexpr int kEachA = A_KC ? 0 : LA::kBlocks, kEachB = B_KC ? 0 : LB::kBlocks;
+  constexpr int kEach = kEachA + kEachB;
+  constexpr int kLoadsEven = kPairA + kPairB + kEach, kLoadsOdd = kEach;
+  // At the barrier of slice s the data of slice s+1 must have landed. With pair loads two slices ahead
+  // it was requested two slices ago, or - K-contiguous operand, s odd - by the previous slice and then
+  // first in line: younger than it are at most the every-slice loads of the slice before this one and
+  // what this slice has issued in front of its barrier. With pair loads four slices ahead the youngest
+  // request is the every-slice one of two slices ago: all of the previous slice's loads are younger.
+  constexpr int kPreEven = ceil_div(kPre * kLoadsEven, kSlots), kPreOdd = ceil_div(kPre * kLoadsOdd, kSlots);
+  constexpr int kInFlightEven = (kPairAhead == 4 ? kLoadsOdd : kEach) + kPreEven;
+  constexpr int kInFlightOdd = (kPairAhead == 4 ? kLoadsEven : kEach) + kPreOdd;
 
-  using RA = FragReader<ES, A_KC, FRB, KB, SB, BM, MI>;
-  using RB = FragReader<ES, B_KC, FRB, KB, SB, BN, NI>;
+  using RA = FragReader<ES, A_KC, FRB, KB, BM, NSA, MI>;
+  using RB = FragReader<ES, B_KC, FRB, KB, BN, NSB, NI>;
   constexpr int PA = RA::kPieces, PB = RB::kPieces;
   constexpr int kReads = MI * PA + NI * PB;      // LDS instructions per k-step
   constexpr int kReadSlots = kMfmas / 2;         // ... issued behind the first half of its MFMAs, the rest is time to land
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  const unsigned smem_addr = (unsigned)(size_t)LDS_PTR(char, smem);
+  char *region_a = smem, *region_b = smem + TileA::kRegion;
+  const unsigned addr_a = (unsigned)(size_t)LDS_PTR(char, smem), addr_b = addr_a + TileA::kRegion;
 
   unsigned tm, tn;
   tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
@@ -662,16 +689,24 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-  const size_t slices = p.k * ES / SB;
-  // Slices beyond the end are requested as the last slice again: in range, and
-  // the stage they land in is never read, which keeps the load counts static.
+  // K is a whole number of slice pairs. Units beyond the end are requested as the last unit
+  // again: in range, and the stage they land in is never read, which keeps the load counts static.
+  const size_t slices = p.k * ES / SB, pairs = slices / 2;
+  if constexpr (A_KC) {
 #pragma unroll
-  for (int i = 0; i < AHEAD; ++i) {
-    const size_t sl = (size_t)i < slices ? (size_t)i : slices - 1;
-    la.issue(smem + i * kStage, sl);
-    lb.issue(smem + i * kStage + kTile, sl);
+    for (int i = 0; i < kPairAhead / 2; ++i) la.issue(region_a, 2 * i, (size_t)i < pairs ? (size_t)i : pairs - 1);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) la.issue(region_a, i, (size_t)i < slices ? (size_t)i : slices - 1);
   }
-  wait_loads_upto<(AHEAD - 1) * kLoads>();
+  if constexpr (B_KC) {
+#pragma unroll
+    for (int i = 0; i < kPairAhead / 2; ++i) lb.issue(region_b, 2 * i, (size_t)i < pairs ? (size_t)i : pairs - 1);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) lb.issue(region_b, i, (size_t)i < slices ? (size_t)i : slices - 1);
+  }
+  wait_loads_upto<0>();
   __syncthreads();
 
   typename RA::Piece pa[2][MI][PA];
@@ -679,27 +714,22 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 
   // Read item R of a k-step: fragment by fragment, A and B alternating, so that
   // what the next k-step's first MFMAs need is requested first.
-  auto read_item = [&](auto rc, auto ksc, int buf, unsigned tile_a, unsigned tile_b) {
+  auto read_item = [&](auto rc, auto ksc, int buf, unsigned stage_a, unsigned stage_b) {
     constexpr int R = decltype(rc)::value, KS = decltype(ksc)::value;
     constexpr int kPair = PA + PB, kBoth = (MI < NI ? MI : NI) * kPair;
     if constexpr (R < kBoth) {
       constexpr int F = R / kPair, W = R % kPair;
       if constexpr (W < PA)
-        pa[buf][F][W] = ra.template read<F, KS, W>(tile_a);
+        pa[buf][F][W] = ra.template read<F, KS, W>(stage_a);
       else
-        pb[buf][F][W - PA] = rb.template read<F, KS, W - PA>(tile_b);
+        pb[buf][F][W - PA] = rb.template read<F, KS, W - PA>(stage_b);
     } else if constexpr (MI > NI) {
       constexpr int X = R - kBoth, F = NI + X / PA, W = X % PA;
-      pa[buf][F][W] = ra.template read<F, KS, W>(tile_a);
+      pa[buf][F][W] = ra.template read<F, KS, W>(stage_a);
     } else {
       constexpr int X = R - kBoth, F = MI + X / PB, W = X % PB;
-      pb[buf][F][W] = rb.template read<F, KS, W>(tile_b);
+      pb[buf][F][W] = rb.template read<F, KS, W>(stage_b);
     }
-  };
-  auto read_all = [&](auto ksc, int buf, unsigned tile_a, unsigned tile_b, auto seq) {
-    [&]<int... Rs>(std::integer_sequence<int, Rs...>) {
-      (read_item(std::integral_constant<int, Rs>{}, ksc, buf, tile_a, tile_b), ...);
-    }(seq);
   };
   // All reads in flight have landed; from here on the compiler may use buffer `buf`.
   auto landed = [&](int buf) {
@@ -714,77 +744,94 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
       for (int w = 0; w < PB; ++w) asm volatile("" : "+v"(pb[buf][j][w]));
   };
 
-  read_all(std::integral_constant<int, 0>{}, 0, smem_addr, smem_addr + kTile, std::make_integer_sequence<int, kReads>{});
+  [&]<int... Rs>(std::integer_sequence<int, Rs...>) {
+    (read_item(std::integral_constant<int, Rs>{}, std::integral_constant<int, 0>{}, 0, addr_a, addr_b), ...);
+  }(std::make_integer_sequence<int, kReads>{});
 
-  for (size_t s0 = 0; s0 < slices; s0 += kUnroll) {
+  // Two slices per trip: the parity of the slice decides which loads it issues, and (for the
+  // operand kinds with one k-step per slice) which fragment buffer a k-step uses.
+  for (size_t s0 = 0; s0 < slices; s0 += 2) {
+    [&]<int... Us>(std::integer_sequence<int, Us...>) {
+      (
+          [&](auto uc) {
+            constexpr int U = decltype(uc)::value;
+            constexpr int kLoads = U == 0 ? kLoadsEven : kLoadsOdd;
+            const size_t s = s0 + U;
+            const size_t fill_slice = s + 3 < slices ? s + 3 : slices - 1;  // every-slice operands
+            const size_t fill_pair = (s + kPairAhead) / 2 < pairs ? (s + kPairAhead) / 2 : pairs - 1;  // pair operands (s even)
+            const int cur_a = (int)(s % NSA), nxt_a = (int)((s + 1) % NSA), cur_b = (int)(s % NSB), nxt_b = (int)((s + 1) % NSB);
+            const int fill_a = (int)((s + (A_KC ? kPairAhead : 3)) % NSA), fill_b = (int)((s + (B_KC ? kPairAhead : 3)) % NSB);
+            [&]<int... KSs>(std::integer_sequence<int, KSs...>) {
+              (
+                  [&](auto ksc) {
+                    constexpr int KS = decltype(ksc)::value;
+                    constexpr bool kLast = KS == kSteps - 1;
+                    constexpr int KSN = kLast ? 0 : KS + 1;  // k-step whose fragments are read during this one
+                    constexpr int cur = (U * kSteps + KS) & 1, nx = cur ^ 1;
+                    if constexpr (kLast) {
+                      // The reads below cross into the next slice: its data must have landed for every wave.
+                      // Own reads first, so that nobody's read of the stage refilled next is still in flight.
+                      wait_loads_upto<U == 0 ? kInFlightEven : kInFlightOdd>();
+                      landed(cur);
+                      __builtin_amdgcn_s_barrier();
+                    } else {
+                      landed(cur);
+                    }
+                    Frag fa[MI], fb[NI];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const size_t s = s0 + u;
-      const unsigned cur_a = smem_addr + (unsigned)(s % STAGES) * kStage;
-      const unsigned nxt_a = smem_addr + (unsigned)((s + 1) % STAGES) * kStage;
-      char *fill = smem + ((s + AHEAD) % STAGES) * kStage;
-      const size_t fill_slice = s + AHEAD < slices ? s + AHEAD : slices - 1;
-      [&]<int... KSs>(std::integer_sequence<int, KSs...>) {
-        (
-            [&](auto ksc) {
-              constexpr int KS = decltype(ksc)::value;
-              constexpr bool kLast = KS == kSteps - 1;
-              constexpr int KSN = kLast ? 0 : KS + 1;       // k-step whose fragments are read during this one
-              const int cur = (u * kSteps + KS) & 1, nx = cur ^ 1;
-              if constexpr (kLast) {
-                // The reads below cross into the next slice: its data must have landed for every wave.
-                // (The loads issued after it - a slice and a bit - may stay in flight.)
-                // Own reads first, so that nobody's read of the stage refilled next is still in flight.
-                wait_loads_upto<kInFlight>();
-                landed(cur);
-                __builtin_amdgcn_s_barrier();
-              } else {
-                landed(cur);
-              }
-              Frag fa[MI], fb[NI];
+                    for (int i = 0; i < MI; ++i) fa[i] = join_pieces<Frag>(pa[cur][i]);
 #pragma unroll
-              for (int i = 0; i < MI; ++i) fa[i] = join_pieces<Frag>(pa[cur][i]);
-#pragma unroll
-              for (int j = 0; j < NI; ++j) fb[j] = join_pieces<Frag>(pb[cur][j]);
-              const unsigned ta = kLast ? nxt_a : cur_a, tb = ta + kTile;
-              __builtin_amdgcn_sched_barrier(0);
-              [&]<int... Qs>(std::integer_sequence<int, Qs...>) {
-                (
-                    [&](auto qc) {
-                      constexpr int Q = decltype(qc)::value, kSlot = KS * kMfmas + Q;
-                      constexpr int i = Q / NI, j = Q % NI;
-                      acc[i][j] = M::run(fa[i], fb[j], acc[i][j]);
-                      // this slot's share of the next k-step's reads
-                      [&]<int... Rs>(std::integer_sequence<int, Rs...>) {
-                        (
-                            [&](auto rc) {
-                              constexpr int R = decltype(rc)::value;
-                              if constexpr (R * kReadSlots / kReads == Q) read_item(rc, std::integral_constant<int, KSN>{}, nx, ta, tb);
-                            }(std::integral_constant<int, Rs>{}),
-                            ...);
-                      }(std::make_integer_sequence<int, kReads>{});
-                      // and this slot's share of the loads of the slice that is AHEAD slices ahead
-                      [&]<int... Ls>(std::integer_sequence<int, Ls...>) {
-                        (
-                            [&](auto lc) {
-                              constexpr int L = decltype(lc)::value;
-                              if constexpr (L * kWindow / kLoads == kSlot) {
-                                if constexpr (L < kLoadsA)
-                                  la.issue_one(fill, fill_slice, L);
-                                else
-                                  lb.issue_one(fill + kTile, fill_slice, L - kLoadsA);
-                              }
-                            }(std::integral_constant<int, Ls>{}),
-                            ...);
-                      }(std::make_integer_sequence<int, kLoads>{});
-                      __builtin_amdgcn_sched_barrier(0);
-                    }(std::integral_constant<int, Qs>{}),
-                    ...);
-              }(std::make_integer_sequence<int, kMfmas>{});
-            }(std::integral_constant<int, KSs>{}),
-            ...);
-      }(std::make_integer_sequence<int, kSteps>{});
-    }
+                    for (int j = 0; j < NI; ++j) fb[j] = join_pieces<Frag>(pb[cur][j]);
+                    const unsigned sa = addr_a + (kLast ? nxt_a : cur_a) * TileA::kStageStep;
+                    const unsigned sb = addr_b + (kLast ? nxt_b : cur_b) * TileB::kStageStep;
+                    __builtin_amdgcn_sched_barrier(0);
+                    [&]<int... Qs>(std::integer_sequence<int, Qs...>) {
+                      (
+                          [&](auto qc) {
+                            constexpr int Q = decltype(qc)::value, kSlot = KS * kMfmas + Q;
+                            constexpr int i = Q / NI, j = Q % NI;
+                            acc[i][j] = M::run(fa[i], fb[j], acc[i][j]);
+                            // this slot's share of the next k-step's reads
+                            [&]<int... Rs>(std::integer_sequence<int, Rs...>) {
+                              (
+                                  [&](auto rc) {
+                                    constexpr int R = decltype(rc)::value;
+                                    if constexpr (R * kReadSlots / kReads == Q)
+                                      read_item(rc, std::integral_constant<int, KSN>{}, nx, sa, sb);
+                                  }(std::integral_constant<int, Rs>{}),
+                                  ...);
+                            }(std::make_integer_sequence<int, kReads>{});
+                            // and this slot's share of the slice's loads
+                            [&]<int... Ls>(std::integer_sequence<int, Ls...>) {
+                              (
+                                  [&](auto lc) {
+                                    constexpr int L = decltype(lc)::value;
+                                    if constexpr (L * kSlots / kLoads == kSlot) {
+                                      constexpr int kPairs = U == 0 ? kPairA + kPairB : 0;
+                                      if constexpr (L < kPairs) {
+                                        if constexpr (L < kPairA && U == 0)
+                                          la.issue_one(region_a, fill_a, fill_pair, L);
+                                        else
+                                          lb.issue_one(region_b, fill_b, fill_pair, L - (U == 0 ? kPairA : 0));
+                                      } else if constexpr (L - kPairs < kEachA) {
+                                        la.issue_one(region_a, fill_a, fill_slice, L - kPairs);
+                                      } else {
+                                        lb.issue_one(region_b, fill_b, fill_slice, L - kPairs - kEachA);
+                                      }
+                                    }
+                                  }(std::integral_constant<int, Ls>{}),
+                                  ...);
+                            }(std::make_integer_sequence<int, kLoads>{});
+                            __builtin_amdgcn_sched_barrier(0);
+                          }(std::integral_constant<int, Qs>{}),
+                          ...);
+                    }(std::make_integer_sequence<int, kMfmas>{});
+                  }(std::integral_constant<int, KSs>{}),
+                  ...);
+            }(std::make_integer_sequence<int, kSteps>{});
+          }(std::integral_constant<int, Us>{}),
+          ...);
+    }(std::make_integer_sequence<int, 2>{});
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
@@ -807,10 +854,10 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   }
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BN, int SB, int STAGES, int AHEAD>
+template <int TA, int TB, bool A_KC, bool B_KC, int BN>
 int launch_ring(const MfmaArgs &args) {
-  constexpr int lds = STAGES * (256 + BN) * SB;
-  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, SB, STAGES, AHEAD>;
+  constexpr int lds = kRingStages * (256 + BN) * kRingSlice;
+  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN>;
   static bool configured = false;
   if (!configured) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -865,8 +912,8 @@ int launch_tile(const MfmaArgs &p) {
   // on the small, bounds-checked kernel.
   if (p.m % 256 == 0 && (p.k * ES) % 128 == 0) {
     const size_t tiles_m = p.m / 256;
-    if (p.n % 256 == 0 && tiles_m * (p.n / 256) >= 200) return launch_ring<TA, TB, A_KC, B_KC, 256, 64, 4, 3>(p);
-    if (p.n % 128 == 0 && tiles_m * (p.n / 128) >= 96) return launch_ring<TA, TB, A_KC, B_KC, 128, 64, 4, 3>(p);
+    if (p.n % 256 == 0 && tiles_m * (p.n / 256) >= 200) return launch_ring<TA, TB, A_KC, B_KC, 256>(p);
+    if (p.n % 128 == 0 && tiles_m * (p.n / 128) >= 96) return launch_ring<TA, TB, A_KC, B_KC, 128>(p);
   }
   return launch_one<TA, TB, A_KC, B_KC, 128, 128, 2, 4, true>(p);
 }
