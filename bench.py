@@ -79,7 +79,35 @@ def wl_gemv(lib, rng):
         lib.skl_gemm_i8_i8_i32_gfx950(1, n, k, 1, x, k, w[i % nbuf], n, 0, y, n)
 
     return dict(fn=step, bytes=k * n + k + 4 * n, ops=2 * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
-                name="int8 GEMV 1x4096x11008 (row-major W, beta=0)", kernel="gemv_i8_rowmajor_kernel")
+                name="int8 GEMV 1x4096x11008 (row-major W, beta=0)", kernel="gemv_kernel<int8 row-major>")
+
+
+def wl_gemv_p4x1c(lib, rng):
+    """Config 2 with W prepacked in the K-packed dot4 layout (B(4P+p, j) at P*rsb1 + 4j + p): same bytes."""
+    k, n, nbuf = 4096, 11008, 8
+    w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(rand_i8(rng, k))
+    y = DeviceBuffer(4 * n)
+
+    def step(i):
+        lib.skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(1, n, k // 4, 1, x, k, 4, w[i % nbuf], 4 * n, 0, y, n)
+
+    return dict(fn=step, bytes=k * n + k + 4 * n, ops=2 * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
+                name="int8 GEMV 1x4096x11008 (W in the p4x1c K-packed layout, beta=0)", kernel="gemv_kernel<int8 K-packed>")
+
+
+def wl_gemv_bf16(lib, rng):
+    k, n, nbuf = 4096, 11008, 4
+    w = [DeviceBuffer.from_array(bf16_bits(rng.normal(size=k * n) * 0.02)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(bf16_bits(rng.normal(size=k)))
+    y = DeviceBuffer(4 * n)
+    lib.skl_hip_memset(y, 0, 4 * n)
+
+    def step(i):
+        lib.skl_gemm_bf16_bf16_f32_gfx950(1, n, k, 1.0, x, k, w[i % nbuf], n, 0.0, y, n)
+
+    return dict(fn=step, bytes=2 * k * n + 2 * k + 8 * n, ops=2 * k * n, bound="hbm", dtype="bf16", keep=(w, x, y),
+                name="bf16 GEMV 1x4096x11008 (row-major W, beta=0)", kernel="gemv_kernel<bf16>")
 
 
 def _dense(lib, rng, name, fn_name, m, n, k, abytes, gen_a, gen_b, alpha, beta, ctype, dkey, col_major_a=False):
@@ -93,7 +121,7 @@ def _dense(lib, rng, name, fn_name, m, n, k, abytes, gen_a, gen_b, alpha, beta, 
         f(m, n, k, alpha, a, lda, b, n, beta, c, n)
 
     return dict(fn=step, bytes=abytes * (m * k + k * n) + 4 * m * n * (2 if beta != 0 else 1), ops=2 * m * n * k,
-                bound="mfma", dtype=dkey, keep=(a, b, c), name=name, kernel="gemm_mfma_stream_kernel")
+                bound="mfma", dtype=dkey, keep=(a, b, c), name=name, kernel="gemm_mfma_ring_kernel")
 
 
 def wl_gemm_i8_8192(lib, rng):
@@ -130,7 +158,7 @@ def wl_gemm_f8_8192(lib, rng, fmt_b="f8e4m3"):
             lib.skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950(m, n, k, 1.0, a, 1, m, b, n, 1, 0.0, c, n, 1)
         name = "fp8 E4M3xE5M2 GEMM 8192^3 (column-major A, alpha=1, beta=0)"
     return dict(fn=step, bytes=m * k + k * n + 8 * m * n, ops=2 * m * n * k, bound="mfma", dtype="f8", keep=(a, b, c),
-                name=name, kernel="gemm_mfma_stream_kernel")
+                name=name, kernel="gemm_mfma_ring_kernel")
 
 
 def wl_gemm_bf16(lib, rng):
@@ -159,7 +187,7 @@ def wl_f16_pipeline(lib, rng):
 
     moved = 2 * (2 * m * k) + 2 * (2 * k * n) + 2 * (4 * m * n)
     return dict(fn=step, bytes=moved, ops=2 * m * n * k, bound="mfma", dtype="f16", keep=(a, b, ap, bp, cp, c),
-                name="f16 pack->GEMM->unpack 4096x4096x14336 (TE=64 panels)", kernel="gemm_mfma_stream_kernel")
+                name="f16 pack->GEMM->unpack 4096x4096x14336 (TE=64 panels)", kernel="gemm_mfma_ring_kernel")
 
 
 def wl_cvt(lib, rng):
@@ -183,7 +211,7 @@ def wl_pack_a(lib, rng):
         lib.skl_pack_e16_e16rcptex1c_gfx950(m, k, a, k, ap, k * te, te, 0)
 
     return dict(fn=step, bytes=4 * m * k, ops=m * k, bound="hbm", dtype="u16", keep=(a, ap),
-                name="pack e16 4096x4096 -> TEx1 column panels", kernel="pack_tile_kernel")
+                name="pack e16 4096x4096 -> TEx1 column panels", kernel="pack_vec_kernel (transposing)")
 
 
 def wl_copy(lib, rng):
@@ -197,11 +225,13 @@ def wl_copy(lib, rng):
         lib.skl_pack_e32rc_e32rcprc_gfx950(m, n, src, n, 1, m, n, dst, n, 1, 0, 0, 0)
 
     return dict(fn=step, bytes=8 * m * n, ops=m * n, bound="hbm", dtype="u32", keep=(src, dst),
-                name="copy 4096x4096 u32 (64 MiB read + 64 MiB write)", kernel="pack_tile_kernel")
+                name="copy 4096x4096 u32 (64 MiB read + 64 MiB write)", kernel="pack_vec_kernel (copy)")
 
 
 WORKLOADS = {
     "gemv_i8": (wl_gemv, 2000, 100),
+    "gemv_i8_p4x1c": (wl_gemv_p4x1c, 1000, 50),
+    "gemv_bf16": (wl_gemv_bf16, 500, 50),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2),
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2),

@@ -23,24 +23,32 @@ __device__ __forceinline__ unsigned scaled_bits(float x, float scale) {
   return __float_as_uint(__fmul_rn(x, scale));
 }
 
+// A workgroup converts 4096 consecutive elements: four rounds in which the 256 threads read 256
+// consecutive float4 (every load instruction of a wave covers one contiguous KiB) and write 256
+// consecutive dwords; the four loads of a thread are all requested before the first is used.
+constexpr int kCvtRounds = 4;
 template <class F>
 __global__ void __launch_bounds__(256) cvt_f32_f8_kernel(uint8_t *__restrict__ dst, const float *__restrict__ src,
                                                          float scale, size_t n, bool sat, bool vec) {
-  const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const size_t base = t * 8;
-  if (base >= n) return;
-  if (vec && base + 8 <= n) {
-    const float4 x0 = reinterpret_cast<const float4 *>(src + base)[0];
-    const float4 x1 = reinterpret_cast<const float4 *>(src + base)[1];
-    uint2 out;
-    out.x = encode_ofp8<F>(scaled_bits(x0.x, scale), sat) | (encode_ofp8<F>(scaled_bits(x0.y, scale), sat) << 8) |
-            (encode_ofp8<F>(scaled_bits(x0.z, scale), sat) << 16) | (encode_ofp8<F>(scaled_bits(x0.w, scale), sat) << 24);
-    out.y = encode_ofp8<F>(scaled_bits(x1.x, scale), sat) | (encode_ofp8<F>(scaled_bits(x1.y, scale), sat) << 8) |
-            (encode_ofp8<F>(scaled_bits(x1.z, scale), sat) << 16) | (encode_ofp8<F>(scaled_bits(x1.w, scale), sat) << 24);
-    *reinterpret_cast<uint2 *>(dst + base) = out;
+  const size_t block0 = (size_t)blockIdx.x * (256 * 4 * kCvtRounds);
+  if (vec && block0 + 256 * 4 * kCvtRounds <= n) {
+    typedef float f4v __attribute__((ext_vector_type(4)));
+    f4v x[kCvtRounds];
+#pragma unroll
+    for (int j = 0; j < kCvtRounds; ++j)
+      x[j] = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(src + block0) + j * 256 + threadIdx.x);
+#pragma unroll
+    for (int j = 0; j < kCvtRounds; ++j) {
+      const unsigned out = encode_ofp8<F>(scaled_bits(x[j].x, scale), sat) | (encode_ofp8<F>(scaled_bits(x[j].y, scale), sat) << 8) |
+                           (encode_ofp8<F>(scaled_bits(x[j].z, scale), sat) << 16) |
+                           (encode_ofp8<F>(scaled_bits(x[j].w, scale), sat) << 24);
+      __builtin_nontemporal_store(out, reinterpret_cast<unsigned *>(dst + block0) + j * 256 + threadIdx.x);
+    }
   } else {
-    const size_t end = base + 8 < n ? base + 8 : n;
-    for (size_t i = base; i < end; ++i) dst[i] = (uint8_t)encode_ofp8<F>(scaled_bits(src[i], scale), sat);
+    for (int j = 0; j < kCvtRounds; ++j) {
+      const size_t base = block0 + ((size_t)j * 256 + threadIdx.x) * 4;
+      for (size_t i = base; i < base + 4 && i < n; ++i) dst[i] = (uint8_t)encode_ofp8<F>(scaled_bits(src[i], scale), sat);
+    }
   }
 }
 
@@ -132,8 +140,8 @@ extern "C" {
 
 int skl_hip_launch_cvt_f32_f8(int fmt, int saturate, uint8_t *dst, const float *src, float scale, size_t n) {
   if (n == 0) return 0;
-  const bool vec = aligned(src, 16) && aligned(dst, 8);
-  const unsigned blocks = skl_div_up(skl_div_up(n, 8), 256);
+  const bool vec = aligned(src, 16) && aligned(dst, 4);
+  const unsigned blocks = skl_div_up(n, 256 * 4 * kCvtRounds);
   hipStream_t s = skl_current_stream();
   if (fmt == SKL_DT_F8E4M3)
     cvt_f32_f8_kernel<E4M3><<<blocks, 256, 0, s>>>(dst, src, scale, n, saturate != 0, vec);
