@@ -67,6 +67,14 @@ void skl_gemm_f8e5m2rc_f8e5m2rc_f32rc_gfx950(size_t m, size_t n, size_t k, float
 void skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
                                              size_t rsa, size_t csa, const uint8_t *b, size_t rsb,
                                              size_t csb, float beta, float *c, size_t rsc, size_t csc);
+/* ref/gemm/gemm_f32rc_f32rc_f32rc.h:44. Served by the any-stride kernel (no matrix-core path). */
+void skl_gemm_f32rc_f32rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const float *a, size_t rsa,
+                                       size_t csa, const float *b, size_t rsb, size_t csb, float beta,
+                                       float *c, size_t rsc, size_t csc);
+/* ref/gemm/gemm_f64rc_f64rc_f64rc.h:44. Served by the any-stride kernel. */
+void skl_gemm_f64rc_f64rc_f64rc_gfx950(size_t m, size_t n, size_t k, double alpha, const double *a,
+                                       size_t rsa, size_t csa, const double *b, size_t rsb, size_t csb,
+                                       double beta, double *c, size_t rsc, size_t csc);
 
 /* Blocked ("rcprc") forms: element (I,i ; P,p) of A is at
  * a[I*rsa1 + P*csa1 + i*rsa0 + p*csa0], likewise B (rows k) and C. */
@@ -85,6 +93,10 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f32rcprc_gfx950, skl_f16_t, 
 SKL_GFX950_DECLARE_RCPRC(skl_gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950, uint8_t, float);
 /* ref/gemm/gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc.h:53 */
 SKL_GFX950_DECLARE_RCPRC(skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, float);
+/* ref/gemm/gemm_f32rcprc_f32rcprc_f32rcprc.h:49 */
+SKL_GFX950_DECLARE_RCPRC(skl_gemm_f32rcprc_f32rcprc_f32rcprc_gfx950, float, float);
+/* ref/gemm/gemm_f64rcprc_f64rcprc_f64rcprc.h:49 */
+SKL_GFX950_DECLARE_RCPRC(skl_gemm_f64rcprc_f64rcprc_f64rcprc_gfx950, double, double);
 
 /* ======================================================================== */
 /* GEMM - the optimized entry points of skl.h                                */
@@ -101,6 +113,12 @@ void skl_gemm_bf16_bf16_f32_gfx950(size_t m, size_t n, size_t k, float alpha, co
 /* src/gemm/gemm_f16_f16_f32_zvfh.h:49, src/gemm/gemm_f16_f16_f32_zvfh_x390.h:49 */
 void skl_gemm_f16_f16_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const skl_f16_t *a, size_t rsa,
                                  const skl_f16_t *b, size_t rsb, float beta, float *c, size_t rsc);
+/* src/gemm/gemm_f32_f32_f32_zve32f.h:48, src/gemm/gemm_f32_f32_f32_zve32f_x390.h */
+void skl_gemm_f32_f32_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const float *a, size_t rsa,
+                                 const float *b, size_t rsb, float beta, float *c, size_t rsc);
+/* src/gemm/gemm_f64_f64_f64_zve64d.h:48, src/gemm/gemm_f64_f64_f64_zve64d_x390.h */
+void skl_gemm_f64_f64_f64_gfx950(size_t m, size_t n, size_t k, double alpha, const double *a, size_t rsa,
+                                 const double *b, size_t rsb, double beta, double *c, size_t rsc);
 
 /* Column-major A (= A^T stored row-major with row stride csa), row-major B, C.
  * src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:57 */
@@ -121,6 +139,9 @@ void skl_gemm_f8e4m3c_f8e4m3_f32_gfx950(size_t m, size_t n, size_t k, float alph
 void skl_gemm_f8e5m2c_f8e5m2_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
                                         size_t csa, const uint8_t *b, size_t rsb, float beta, float *c,
                                         size_t rsc);
+/* src/gemm/gemm_f32c_f32_f32_xsfmm32a32f.h:56 */
+void skl_gemm_f32c_f32_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const float *a, size_t csa,
+                                  const float *b, size_t rsb, float beta, float *c, size_t rsc);
 
 /* Panel-packed operands, TE = skl_hip_te() = 64: A in TE x 1 column panels
  * (m0 = TE, k0 = 1, rsa0 = 1), B in 1 x TE row panels (n0 = TE, csb0 = 1), C in
@@ -139,6 +160,8 @@ SKL_GFX950_DECLARE_PANEL(skl_gemm_f16rcptex1c_f16rcp1xte_f32rcptexterc_gfx950, s
 SKL_GFX950_DECLARE_PANEL(skl_gemm_f8e4m3rcptex1c_f8e4m3rcp1xte_f32rcptexterc_gfx950, uint8_t, float);
 /* src/gemm/gemm_f8e5m2c_f8e5m2_f32_xsfmm32a8f.h:98 */
 SKL_GFX950_DECLARE_PANEL(skl_gemm_f8e5m2rcptex1c_f8e5m2rcp1xte_f32rcptexterc_gfx950, uint8_t, float);
+/* src/gemm/gemm_f32c_f32_f32_xsfmm32a32f.h:96 */
+SKL_GFX950_DECLARE_PANEL(skl_gemm_f32rcptex1c_f32rcp1xte_f32rcptexterc_gfx950, float, float);
 
 /* K-packed int8 ("dot4") layout: A in 1 x 4 K-blocks (A(i, 4P+p) at i*rsa1 +
  * P*csa1 + p), B in 4 x 1 K-blocks (B(4P+p, j) at P*rsb1 + 4*j + p), C row-major.

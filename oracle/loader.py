@@ -32,12 +32,7 @@ _EXTRA_ORACLE = {
 
 _RC = "zzz{s}pzzpzz{s}pzz"
 _RCPRC = "zzzzzz{s}pzzzzpzzzz{s}pzzzz"
-#: helper GEMMs (f32, f64) present in both the checker and the reference library
-_HELPER_GEMMS = {
-    "skl_gemm_f32rc_f32rc_f32rc": _RC.format(s="f"),
-    "skl_gemm_f64rc_f64rc_f64rc": _RC.format(s="d"),
-    "skl_gemm_f64rcprc_f64rcprc_f64rcprc": _RCPRC.format(s="d"),
-}
+_HELPER_GEMMS = {}  # the f32 / f64 routines are part of the shared list
 #: scalar routines of the reference library
 _REF_SCALARS = {
     "skl_cvt_f8e4m3_f32": (ctypes.c_float, "b"),

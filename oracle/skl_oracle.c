@@ -333,6 +333,8 @@ GEMM_RCPRC(f8e4m3rcprc_f8e4m3rcprc_f32rcprc, uint8_t, uint8_t, float,
            skl_oracle_f8e4m3_to_f32, skl_oracle_f8e4m3_to_f32)
 GEMM_RCPRC(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, uint8_t, float,
            skl_oracle_f8e5m2_to_f32, skl_oracle_f8e5m2_to_f32)
+/* ref/gemm/gemm_f32rcprc_f32rcprc_f32rcprc.c:9-36 */
+GEMM_RCPRC(f32rcprc_f32rcprc_f32rcprc, float, float, float, LOAD_ID, LOAD_ID)
 GEMM_RCPRC(f64rcprc_f64rcprc_f64rcprc, double, double, double, LOAD_ID, LOAD_ID)
 
 /* ======================================================================== */

@@ -92,6 +92,7 @@ SKL_ORACLE_PGEMM_DECL(bf16rcprc_bf16rcprc_f32rcprc, uint16_t, uint16_t, float)
 SKL_ORACLE_PGEMM_DECL(f16rcprc_f16rcprc_f32rcprc, uint16_t, uint16_t, float)
 SKL_ORACLE_PGEMM_DECL(f8e4m3rcprc_f8e4m3rcprc_f32rcprc, uint8_t, uint8_t, float)
 SKL_ORACLE_PGEMM_DECL(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, uint8_t, float)
+SKL_ORACLE_PGEMM_DECL(f32rcprc_f32rcprc_f32rcprc, float, float, float)
 SKL_ORACLE_PGEMM_DECL(f64rcprc_f64rcprc_f64rcprc, double, double, double)
 
 /* Widening helpers used to build fp64 comparison operands on the host. */

@@ -25,7 +25,16 @@
 /* helpers                                                                   */
 /* ------------------------------------------------------------------------ */
 
-static size_t elem_size(int dt) { return (dt == SKL_DT_BF16 || dt == SKL_DT_F16) ? 2u : 1u; }
+static size_t elem_size(int dt) {
+  switch (dt) {
+    case SKL_DT_BF16:
+    case SKL_DT_F16: return 2u;
+    case SKL_DT_F32: return 4u;
+    case SKL_DT_F64: return 8u;
+    default: return 1u;
+  }
+}
+static size_t c_elem_size(int dt) { return dt == SKL_DT_F64 ? 8u : 4u; }
 
 /* Number of elements between the first and one past the last addressed element
  * of a 4-level strided array; 0 if any extent is 0. */
@@ -140,7 +149,7 @@ static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g) {
 
 static void gemm_on_device(const skl_gemm_desc *d) {
   skl_gemm_canon g;
-  if (d->k0 * d->k1 != 0) {
+  if (d->k0 * d->k1 != 0 && d->ta <= SKL_DT_F8E5M2) {
     if (canonicalize_k4(d, &g) && skl_hip_gemv_supported(&g, 1)) {
       skl_hip_launch_gemv(&g, 1);
       return;
@@ -177,7 +186,7 @@ static void gemm_run(const skl_gemm_desc *d, const char *who) {
     const size_t nb = K ? span4(d->k1, d->rsb1, d->n1, d->csb1, d->k0, d->rsb0, d->n0, d->csb0) : 0;
     const size_t nc = span4(d->m1, d->rsc1, d->n1, d->csc1, d->m0, d->rsc0, d->n0, d->csc0);
     skl_gemm_desc dd = *d;
-    void *da = stage_in(d->a, na * esa), *db = stage_in(d->b, nb * esb), *dc = stage_in(d->c, nc * 4);
+    void *da = stage_in(d->a, na * esa), *db = stage_in(d->b, nb * esb), *dc = stage_in(d->c, nc * c_elem_size(d->ta));
     if ((na && !da) || (nb && !db) || !dc) {
       skl_hip_free(da);
       skl_hip_free(db);
@@ -188,7 +197,7 @@ static void gemm_run(const skl_gemm_desc *d, const char *who) {
     dd.b = db;
     dd.c = dc;
     gemm_on_device(&dd);
-    skl_hip_memcpy_d2h(d->c, dc, nc * 4);
+    skl_hip_memcpy_d2h(d->c, dc, nc * c_elem_size(d->ta));
     skl_hip_free(da);
     skl_hip_free(db);
     skl_hip_free(dc);
@@ -197,6 +206,7 @@ static void gemm_run(const skl_gemm_desc *d, const char *who) {
 
 #define SCALAR_i32(x) .i = (x)
 #define SCALAR_f32(x) .f = (x)
+#define SCALAR_f64(x) .d = (x)
 
 /* strided (rc) form: one element per block */
 #define DEFINE_GEMM_RC(NAME, TA_T, TC_T, DTA, DTB, SC)                                             \
@@ -213,6 +223,8 @@ DEFINE_GEMM_RC(skl_gemm_f16rc_f16rc_f32rc_gfx950, skl_f16_t, float, SKL_DT_F16, 
 DEFINE_GEMM_RC(skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950, uint8_t, float, SKL_DT_F8E4M3, SKL_DT_F8E4M3, SCALAR_f32)
 DEFINE_GEMM_RC(skl_gemm_f8e5m2rc_f8e5m2rc_f32rc_gfx950, uint8_t, float, SKL_DT_F8E5M2, SKL_DT_F8E5M2, SCALAR_f32)
 DEFINE_GEMM_RC(skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950, uint8_t, float, SKL_DT_F8E4M3, SKL_DT_F8E5M2, SCALAR_f32)
+DEFINE_GEMM_RC(skl_gemm_f32rc_f32rc_f32rc_gfx950, float, float, SKL_DT_F32, SKL_DT_F32, SCALAR_f32)
+DEFINE_GEMM_RC(skl_gemm_f64rc_f64rc_f64rc_gfx950, double, double, SKL_DT_F64, SKL_DT_F64, SCALAR_f64)
 
 /* blocked (rcprc) form */
 #define DEFINE_GEMM_RCPRC(NAME, TA_T, TC_T, DT, SC)                                                \
@@ -231,6 +243,8 @@ DEFINE_GEMM_RCPRC(skl_gemm_bf16rcprc_bf16rcprc_f32rcprc_gfx950, skl_bf16_t, floa
 DEFINE_GEMM_RCPRC(skl_gemm_f16rcprc_f16rcprc_f32rcprc_gfx950, skl_f16_t, float, SKL_DT_F16, SCALAR_f32)
 DEFINE_GEMM_RCPRC(skl_gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950, uint8_t, float, SKL_DT_F8E4M3, SCALAR_f32)
 DEFINE_GEMM_RCPRC(skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, float, SKL_DT_F8E5M2, SCALAR_f32)
+DEFINE_GEMM_RCPRC(skl_gemm_f32rcprc_f32rcprc_f32rcprc_gfx950, float, float, SKL_DT_F32, SCALAR_f32)
+DEFINE_GEMM_RCPRC(skl_gemm_f64rcprc_f64rcprc_f64rcprc_gfx950, double, double, SKL_DT_F64, SCALAR_f64)
 
 /* row-major A, B, C: the rc form with csa = csb = csc = 1
  * (src/gemm/gemm_i8_i8_i32_zve32x.h:38-48) */
@@ -242,6 +256,8 @@ DEFINE_GEMM_RCPRC(skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, flo
 DEFINE_GEMM_ROWMAJOR(skl_gemm_i8_i8_i32_gfx950, skl_gemm_i8rc_i8rc_i32rc_gfx950, int8_t, int32_t)
 DEFINE_GEMM_ROWMAJOR(skl_gemm_bf16_bf16_f32_gfx950, skl_gemm_bf16rc_bf16rc_f32rc_gfx950, skl_bf16_t, float)
 DEFINE_GEMM_ROWMAJOR(skl_gemm_f16_f16_f32_gfx950, skl_gemm_f16rc_f16rc_f32rc_gfx950, skl_f16_t, float)
+DEFINE_GEMM_ROWMAJOR(skl_gemm_f32_f32_f32_gfx950, skl_gemm_f32rc_f32rc_f32rc_gfx950, float, float)
+DEFINE_GEMM_ROWMAJOR(skl_gemm_f64_f64_f64_gfx950, skl_gemm_f64rc_f64rc_f64rc_gfx950, double, double)
 
 /* column-major A: the rc form with rsa = 1
  * (src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:38-48) */
@@ -255,6 +271,7 @@ DEFINE_GEMM_COLMAJOR_A(skl_gemm_bf16c_bf16_f32_gfx950, skl_gemm_bf16rc_bf16rc_f3
 DEFINE_GEMM_COLMAJOR_A(skl_gemm_f16c_f16_f32_gfx950, skl_gemm_f16rc_f16rc_f32rc_gfx950, skl_f16_t, float)
 DEFINE_GEMM_COLMAJOR_A(skl_gemm_f8e4m3c_f8e4m3_f32_gfx950, skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950, uint8_t, float)
 DEFINE_GEMM_COLMAJOR_A(skl_gemm_f8e5m2c_f8e5m2_f32_gfx950, skl_gemm_f8e5m2rc_f8e5m2rc_f32rc_gfx950, uint8_t, float)
+DEFINE_GEMM_COLMAJOR_A(skl_gemm_f32c_f32_f32_gfx950, skl_gemm_f32rc_f32rc_f32rc_gfx950, float, float)
 
 /* panel-packed: the rcprc form with (m0, n0, k0) = (TE, TE, 1), rsa0 = 1, csb0 = 1
  * (src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:85-95) */
@@ -270,6 +287,7 @@ DEFINE_GEMM_PANEL(skl_gemm_bf16rcptex1c_bf16rcp1xte_f32rcptexterc_gfx950, skl_ge
 DEFINE_GEMM_PANEL(skl_gemm_f16rcptex1c_f16rcp1xte_f32rcptexterc_gfx950, skl_gemm_f16rcprc_f16rcprc_f32rcprc_gfx950, skl_f16_t, float)
 DEFINE_GEMM_PANEL(skl_gemm_f8e4m3rcptex1c_f8e4m3rcp1xte_f32rcptexterc_gfx950, skl_gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950, uint8_t, float)
 DEFINE_GEMM_PANEL(skl_gemm_f8e5m2rcptex1c_f8e5m2rcp1xte_f32rcptexterc_gfx950, skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, float)
+DEFINE_GEMM_PANEL(skl_gemm_f32rcptex1c_f32rcp1xte_f32rcptexterc_gfx950, skl_gemm_f32rcprc_f32rcprc_f32rcprc_gfx950, float, float)
 
 /* K-packed int8: the rcprc form with (m0, n0, k0) = (1, 1, 4)
  * (src/gemm/gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.h:43-53) */

@@ -10,7 +10,11 @@
 // fused multiply-add used for the accumulation rounds exactly like the
 // reference's separate multiply and add, and the epilogue is kept as two
 // roundings, so for finite data the fp results are bit-identical to the
-// reference's, not merely within tolerance.
+// reference's, not merely within tolerance. The f32 and f64 contractions
+// (ref/gemm/gemm_f32rc_f32rc_f32rc.c:9-24, gemm_f64rc_f64rc_f64rc.c:9-24 and
+// the blocked twins) run here only; their products are not exact, so they are
+// accumulated with a separately rounded multiply and add, as the reference's C
+// source spells it.
 #include <hip/hip_runtime.h>
 
 #include "skl_device.hpp"
@@ -51,11 +55,28 @@ struct Elem<SKL_DT_F8E5M2> {
   __device__ static acc widen(type v) { return __uint_as_float(skl_fp8::decode_ofp8_bits<skl_fp8::E5M2>(v)); }
 };
 
+template <>
+struct Elem<SKL_DT_F32> {
+  using type = float;
+  using acc = float;
+  __device__ static acc widen(type v) { return v; }
+};
+template <>
+struct Elem<SKL_DT_F64> {
+  using type = double;
+  using acc = double;
+  __device__ static acc widen(type v) { return v; }
+};
+
 __device__ __forceinline__ int32_t axpby(int32_t alpha, int32_t acc, int32_t beta, int32_t c) {
   return (int32_t)((uint32_t)beta * (uint32_t)c + (uint32_t)alpha * (uint32_t)acc);  // wraps like -fwrapv
 }
 __device__ __forceinline__ float axpby(float alpha, float acc, float beta, float c) {
   return __fadd_rn(__fmul_rn(beta, c), __fmul_rn(alpha, acc));
+}
+
+__device__ __forceinline__ double axpby(double alpha, double acc, double beta, double c) {
+  return __dadd_rn(__dmul_rn(beta, c), __dmul_rn(alpha, acc));
 }
 
 template <int TA, int TB>
@@ -79,6 +100,10 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(skl_gemm_desc d, unsi
       const Acc bv = EB::widen(bp[p * d.rsb0]);
       if constexpr (TA == SKL_DT_I8)
         acc = (Acc)((uint32_t)acc + (uint32_t)av * (uint32_t)bv);
+      else if constexpr (TA == SKL_DT_F32)  // products are not exact here: multiply, then add, as the reference's C does
+        acc = __fadd_rn(acc, __fmul_rn(av, bv));
+      else if constexpr (TA == SKL_DT_F64)
+        acc = __dadd_rn(acc, __dmul_rn(av, bv));
       else
         acc = __fmaf_rn(av, bv, acc);
     }
@@ -86,6 +111,8 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(skl_gemm_desc d, unsi
   Acc *c = (Acc *)d.c + I * d.rsc1 + J * d.csc1 + i0 * d.rsc0 + j0 * d.csc0;
   if constexpr (TA == SKL_DT_I8)
     *c = axpby(d.alpha.i, acc, d.beta.i, *c);
+  else if constexpr (TA == SKL_DT_F64)
+    *c = axpby(d.alpha.d, acc, d.beta.d, *c);
   else
     *c = axpby(d.alpha.f, acc, d.beta.f, *c);
 }
@@ -115,6 +142,8 @@ extern "C" int skl_hip_launch_gemm_generic(const skl_gemm_desc *d) {
     case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E5M2: return launch<SKL_DT_F8E5M2, SKL_DT_F8E5M2>(*d);
     case SKL_DT_F8E4M3 * 8 + SKL_DT_F8E5M2: return launch<SKL_DT_F8E4M3, SKL_DT_F8E5M2>(*d);
     case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E4M3: return launch<SKL_DT_F8E5M2, SKL_DT_F8E4M3>(*d);
+    case SKL_DT_F32 * 8 + SKL_DT_F32: return launch<SKL_DT_F32, SKL_DT_F32>(*d);
+    case SKL_DT_F64 * 8 + SKL_DT_F64: return launch<SKL_DT_F64, SKL_DT_F64>(*d);
     default:
       skl_hip_record_error(-2, "gemm: operand type pair");
       return -2;

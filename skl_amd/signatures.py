@@ -44,6 +44,8 @@ GEMM_RC = {
     "skl_gemm_f8e4m3rc_f8e4m3rc_f32rc": "f",
     "skl_gemm_f8e5m2rc_f8e5m2rc_f32rc": "f",
     "skl_gemm_f8e4m3rc_f8e5m2rc_f32rc": "f",
+    "skl_gemm_f32rc_f32rc_f32rc": "f",
+    "skl_gemm_f64rc_f64rc_f64rc": "d",
 }
 GEMM_RCPRC = {
     "skl_gemm_i8rcprc_i8rcprc_i32rcprc": "i",
@@ -51,11 +53,15 @@ GEMM_RCPRC = {
     "skl_gemm_f16rcprc_f16rcprc_f32rcprc": "f",
     "skl_gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc": "f",
     "skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc": "f",
+    "skl_gemm_f32rcprc_f32rcprc_f32rcprc": "f",
+    "skl_gemm_f64rcprc_f64rcprc_f64rcprc": "d",
 }
 GEMM_ROWMAJOR = {
     "skl_gemm_i8_i8_i32": "i",
     "skl_gemm_bf16_bf16_f32": "f",
     "skl_gemm_f16_f16_f32": "f",
+    "skl_gemm_f32_f32_f32": "f",
+    "skl_gemm_f64_f64_f64": "d",
 }
 GEMM_COLMAJOR_A = {
     "skl_gemm_i8c_i8_i32": "i",
@@ -63,6 +69,7 @@ GEMM_COLMAJOR_A = {
     "skl_gemm_f16c_f16_f32": "f",
     "skl_gemm_f8e4m3c_f8e4m3_f32": "f",
     "skl_gemm_f8e5m2c_f8e5m2_f32": "f",
+    "skl_gemm_f32c_f32_f32": "f",
 }
 GEMM_PANEL = {
     "skl_gemm_i8rcptex1c_i8rcp1xte_i32rcptexterc": "i",
@@ -70,6 +77,7 @@ GEMM_PANEL = {
     "skl_gemm_f16rcptex1c_f16rcp1xte_f32rcptexterc": "f",
     "skl_gemm_f8e4m3rcptex1c_f8e4m3rcp1xte_f32rcptexterc": "f",
     "skl_gemm_f8e5m2rcptex1c_f8e5m2rcp1xte_f32rcptexterc": "f",
+    "skl_gemm_f32rcptex1c_f32rcp1xte_f32rcptexterc": "f",
 }
 
 _PAD = {8: "b", 16: "h", 32: "w"}

@@ -19,16 +19,22 @@ SUITES = [
     "test/gemm/rvv/skl_gemm_bf16_bf16_f32_zvfbfwma_x390.c",
     "test/gemm/rvv/skl_gemm_f16_f16_f32_zvfh.c",
     "test/gemm/rvv/skl_gemm_f16_f16_f32_zvfh_x390.c",
+    "test/gemm/rvv/skl_gemm_f32_f32_f32_zve32f.c",
+    "test/gemm/rvv/skl_gemm_f32_f32_f32_zve32f_x390.c",
+    "test/gemm/rvv/skl_gemm_f64_f64_f64_zve64d.c",
+    "test/gemm/rvv/skl_gemm_f64_f64_f64_zve64d_x390.c",
     "test/gemm/xsfmm/skl_gemm_i8c_i8_i32_xsfmm32a8i.c",
     "test/gemm/xsfmm/skl_gemm_bf16c_bf16_f32_xsfmm32a16f.c",
     "test/gemm/xsfmm/skl_gemm_f16c_f16_f32_xsfmm32a16f.c",
     "test/gemm/xsfmm/skl_gemm_f8e4m3c_f8e4m3_f32_xsfmm32a8f.c",
     "test/gemm/xsfmm/skl_gemm_f8e5m2c_f8e5m2_f32_xsfmm32a8f.c",
+    "test/gemm/xsfmm/skl_gemm_f32c_f32_f32_xsfmm32a32f.c",
     "test/gemm/xsfmm/skl_gemm_i8rcptex1c_i8rcp1xte_i32rcptexterc_xsfmm32a8i.c",
     "test/gemm/xsfmm/skl_gemm_bf16rcptex1c_bf16rcp1xte_f32rcptexterc_xsfmm32a16f.c",
     "test/gemm/xsfmm/skl_gemm_f16rcptex1c_f16rcp1xte_f32rcptexterc_xsfmm32a16f.c",
     "test/gemm/xsfmm/skl_gemm_f8e4m3rcptex1c_f8e4m3rcp1xte_f32rcptexterc_xsfmm32a8f.c",
     "test/gemm/xsfmm/skl_gemm_f8e5m2rcptex1c_f8e5m2rcp1xte_f32rcptexterc_xsfmm32a8f.c",
+    "test/gemm/xsfmm/skl_gemm_f32rcptex1c_f32rcp1xte_f32rcptexterc_xsfmm32a32f.c",
     "test/gemm/xsfvqdotq/skl_gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.c",
     "test/pack/rvv/skl_pack_e8rc_e8rcprc_zve32x.c",
     "test/pack/rvv/skl_pack_e16rc_e16rcprc_zve32x.c",

@@ -19,7 +19,7 @@ def gemm_entry_args(kind, case, a, b, c):
     """(function name, argument tuple) of the entry point `kind` for a case that
     fits it; mirrors the execute() callbacks of the reference's suites."""
     t = case.ta
-    cty = "i32" if case.is_int else "f32"
+    cty = case.ctag
     if kind == "rcprc":
         return case.stem() + "_gfx950", case.rcprc_args(a, b, c)
     if kind == "rc":

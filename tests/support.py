@@ -118,7 +118,17 @@ def _gen_e5m2(rng, n):  # test/gemm/gemm_f8rcprc_f8rcprc_f32rcprc.h:80-86: bytes
     return rng.integers(4, 124, size=n, dtype=np.uint8)
 
 
+def _gen_f32(rng, n):  # test/gemm/gemm_f32rcprc_f32rcprc_f32rcprc.h:64-66: uniform in [-1, 1]
+    return rng.uniform(-1.0, 1.0, size=n).astype(np.float32)
+
+
+def _gen_f64(rng, n):
+    return rng.uniform(-1.0, 1.0, size=n)
+
+
 ETYPES = {
+    "f32": EType("f32", np.float32, _gen_f32, lambda a: a.astype(np.float64)),
+    "f64": EType("f64", np.float64, _gen_f64, lambda a: a.astype(np.float64)),
     "i8": EType("i8", np.int8, _gen_i8, lambda a: a.astype(np.float64)),
     "bf16": EType("bf16", np.uint16, _gen_bf16, lambda a: bf16_bits_to_f32(a).astype(np.float64)),
     "f16": EType("f16", np.uint16, _gen_f16, lambda a: f16_bits_to_f32(a).astype(np.float64)),
@@ -164,7 +174,17 @@ class GemmCase:
 
     @property
     def cdtype(self):
-        return np.int32 if self.is_int else np.float32
+        return np.int32 if self.is_int else np.float64 if self.ta == "f64" else np.float32
+
+    @property
+    def ctag(self):
+        """C's element type as the function names spell it."""
+        return "i32" if self.is_int else "f64" if self.ta == "f64" else "f32"
+
+    @property
+    def unit_roundoff_bits(self):
+        """P of the reference's bound: accumulator precision (test/gemm/gemm_f64rcprc_f64rcprc_f64rcprc.c:190)."""
+        return 53 if self.ta == "f64" else 24
 
     def spans(self):
         a = span((self.m1, self.k1, self.m0, self.k0), (self.rsa1, self.csa1, self.rsa0, self.csa0))
@@ -180,7 +200,7 @@ class GemmCase:
         if self.is_int:
             c = rng.integers(-128, 128, size=max(nc, 1)).astype(np.int32)
         else:
-            c = rng.uniform(-1.0, 1.0, size=max(nc, 1)).astype(np.float32)
+            c = rng.uniform(-1.0, 1.0, size=max(nc, 1)).astype(self.cdtype)
         return a, b, c
 
     def rcprc_args(self, a, b, c):
@@ -190,9 +210,7 @@ class GemmCase:
                 self.beta, c, self.rsc0, self.csc0, self.rsc1, self.csc1)
 
     def stem(self):
-        t = {"i8": "i8", "bf16": "bf16", "f16": "f16", "f8e4m3": "f8e4m3", "f8e5m2": "f8e5m2"}
-        cty = "i32" if self.is_int else "f32"
-        return f"skl_gemm_{t[self.ta]}rcprc_{t[self.tb]}rcprc_{cty}rcprc"
+        return f"skl_gemm_{self.ta}rcprc_{self.tb}rcprc_{self.ctag}rcprc"
 
     def dense(self, a, b, c):
         """Logical (M x K), (K x N), (M x N) views gathered from the buffers, widened to fp64."""
@@ -209,7 +227,7 @@ class GemmCase:
         (test/gemm/gemm_bf16rcprc_bf16rcprc_f32rcprc.c:131-168)."""
         A, B, C, oc = self.dense(a, b, c_before)
         K = self.k0 * self.k1
-        gamma = 2.0 * ((1.0 + 2.0 ** -24) ** (K + 2) - 1.0)
+        gamma = 2.0 * np.expm1((K + 2) * np.log1p(2.0 ** -self.unit_roundoff_bits))
         bound = gamma * (abs(self.alpha) * (np.abs(A) @ np.abs(B)) + abs(self.beta) * np.abs(C))
         exact = self.alpha * (A @ B) + self.beta * C
         return exact, bound, oc
@@ -303,7 +321,7 @@ def assert_fp_gemm_close(case, a, b, c_before, c_after, frob_tol=1e-3, extra_rel
     got = c_after[oc].astype(np.float64) if oc.size else exact
     err = np.abs(got - exact)
     # a few ulps of slack on top of the bound for the final rounding of tiny results
-    slack = np.abs(exact) * 2.0 ** -22 + 1e-30
+    slack = np.abs(exact) * 2.0 ** -(case.unit_roundoff_bits - 2) + 1e-30
     bad = err > bound + slack
     assert not bad.any(), (f"{int(bad.sum())} elements exceed the reference bound; worst ratio "
                            f"{float((err / (bound + slack)).max()):.3g}")

@@ -120,6 +120,9 @@ FP_SUITES = {
                "test/gemm/xsfmm/skl_gemm_f8e4m3rcptex1c_f8e4m3rcp1xte_f32rcptexterc_xsfmm32a8f.c"),
     "f8e5m2": (None, "test/gemm/xsfmm/skl_gemm_f8e5m2c_f8e5m2_f32_xsfmm32a8f.c",
                "test/gemm/xsfmm/skl_gemm_f8e5m2rcptex1c_f8e5m2rcp1xte_f32rcptexterc_xsfmm32a8f.c"),
+    "f32": ("test/gemm/rvv/skl_gemm_f32_f32_f32_zve32f_x390.c", "test/gemm/xsfmm/skl_gemm_f32c_f32_f32_xsfmm32a32f.c",
+            "test/gemm/xsfmm/skl_gemm_f32rcptex1c_f32rcp1xte_f32rcptexterc_xsfmm32a32f.c"),
+    "f64": ("test/gemm/rvv/skl_gemm_f64_f64_f64_zve64d_x390.c", None, None),
 }
 
 
@@ -128,8 +131,10 @@ def fp_cases(ta, panel_stride=17):
     cases = []
     if rvv:
         cases += rvv_cases(rvv, ta)
-    cases += xsfmm_c_cases(xc, ta)
-    cases += panel_cases(xp, ta, stride=panel_stride)
+    if xc:
+        cases += xsfmm_c_cases(xc, ta)
+    if xp:
+        cases += panel_cases(xp, ta, stride=panel_stride)
     return cases
 
 
@@ -141,7 +146,7 @@ def test_fp_within_reference_bound_and_equal_to_reference(ta):
         support.assert_fp_gemm_close(case, a, b, c, got)
         if ref() is not None:
             want = ref_gemm(case, a, b, c)
-            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), vars(case)
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), vars(case)
 
 
 @pytest.mark.parametrize("ta", list(FP_SUITES))
@@ -161,14 +166,16 @@ def test_fp_exactly_summable_inputs(ta):
             return support.f32_to_bf16_bits(x32)
         if ta == "f16":
             return x32.astype(np.float16).view(np.uint16)
+        if ta in ("f32", "f64"):
+            return x.astype(support.ETYPES[ta].dtype)
         out = np.zeros(x32.size, np.uint8)
         getattr(oracle(), f"skl_cvt_f32_{ta}_oracle")(out, x32.ravel(), 1.0, x32.size)
         return out.reshape(x.shape)
 
     case = rowmajor_case(ta, m, n, k, alpha=2.0, beta=-3.0)
-    a, b, c = enc(A).ravel(), enc(B).ravel(), C.astype(np.float32).ravel()
+    a, b, c = enc(A).ravel(), enc(B).ravel(), C.astype(case.cdtype).ravel()
     got = run_oracle_gemm(case, a, b, c).reshape(m, n)
-    assert np.array_equal(got, (2.0 * (A @ B) - 3.0 * C).astype(np.float32))
+    assert np.array_equal(got, (2.0 * (A @ B) - 3.0 * C).astype(case.cdtype))
 
 
 def test_mixed_fp8_equals_decode_then_f32_gemm():
