@@ -248,10 +248,10 @@ HEADLINE = "gemv_i8"
 # dispatch), FETCH_SIZE scaled by 1.998 (what it under-reads on a 64 MiB copy), WRITE_SIZE by 1.000;
 # the runs are summarised in profiles/gemv_cvt_gemm_hbm_traffic.pmc.txt.
 MEASURED_TRAFFIC_BYTES = {
-    "gemv_i8": int((22099.6 * 1.998 + 454.2) * 1024),
-    "cvt_f32_f8e4m3_8192sq": int((131110 * 1.998 + 65536) * 1024),
-    "gemm_i8_8192": int((393986 * 1.998 + 262144) * 1024),
-    "copy_u32_4096sq": int((32799.3 * 1.998 + 65536) * 1024),
+    "gemv_i8": int((22088.7 * 1.998 + 817) * 1024),
+    "cvt_f32_f8e4m3_8192sq": int((131135 * 1.998 + 65536) * 1024),
+    "gemm_i8_8192": int((393396 * 1.998 + 262144) * 1024),
+    "copy_u32_4096sq": int((32800.3 * 1.998 + 65536) * 1024),
 }
 
 
