@@ -912,7 +912,22 @@ int launch_tile(const MfmaArgs &p) {
   // on the small, bounds-checked kernel.
   if (p.m % 256 == 0 && (p.k * ES) % 128 == 0) {
     const size_t tiles_m = p.m / 256;
-    if (p.n % 256 == 0 && tiles_m * (p.n / 256) >= 200) return launch_ring<TA, TB, A_KC, B_KC, 256>(p);
+    if (p.n % 256 == 0 && tiles_m * (p.n / 256) >= 200) {
+      // A last round that would fill at most half of the 256 compute units is run as 256 x 128 tiles
+      // instead (a second launch on the trailing columns): twice the workgroups at half the length.
+      const size_t tiles = tiles_m * (p.n / 256), rest = tiles % 256;
+      if (rest != 0 && rest <= 128 && rest % tiles_m == 0) {
+        const size_t tail_cols = rest / tiles_m * 256, head_cols = p.n - tail_cols;
+        MfmaArgs head = p, tail = p;
+        head.n = head_cols;
+        tail.n = tail_cols;
+        tail.b = p.b + (head_cols / 64) * p.b_s1 * ES;
+        tail.c = p.c + (head_cols / 64) * p.csc1 * sizeof(float);  // C elements are 4 bytes for every kind
+        const int rc = launch_ring<TA, TB, A_KC, B_KC, 256>(head);
+        return rc != 0 ? rc : launch_ring<TA, TB, A_KC, B_KC, 128>(tail);
+      }
+      return launch_ring<TA, TB, A_KC, B_KC, 256>(p);
+    }
     if (p.n % 128 == 0 && tiles_m * (p.n / 128) >= 96) return launch_ring<TA, TB, A_KC, B_KC, 128>(p);
   }
   return launch_one<TA, TB, A_KC, B_KC, 128, 128, 2, 4, true>(p);

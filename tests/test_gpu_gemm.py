@@ -165,13 +165,14 @@ def _dense_case(ta, m, n, k, a_kc, b_kc, alpha, beta, tb=None):
                             rsb1=1 if b_kc else n, csb1=k if b_kc else 1, rsc0=0, csc0=0, rsc1=n, csc1=1)
 
 
-@pytest.mark.parametrize("m,n", ((4096, 4096), (2048, 1664)))
+@pytest.mark.parametrize("m,n", ((4096, 4096), (2048, 1664), (2048, 8704)))
 @pytest.mark.parametrize("a_kc,b_kc", ((True, False), (False, False), (True, True), (False, True)))
 @pytest.mark.parametrize("ta", ("i8", "bf16", "f16", "f8e4m3", "f8e5m2", "mixed"))
 def test_whole_tile_streaming_kernel(gpu, ta, a_kc, b_kc, m, n):
-    """4096 x 4096 outputs (256 tiles of 256 x 256) and 2048 x 1664 outputs (104
-    tiles of 256 x 128): the two tile shapes of the streaming matrix-core kernel,
-    for every operand orientation. Too large for the scalar checker: the
+    """4096 x 4096 outputs (256 tiles of 256 x 256), 2048 x 1664 outputs (104
+    tiles of 256 x 128) and 2048 x 8704 outputs (272 tiles: one full round of
+    256 x 256 tiles and a short last round that runs as 256 x 128 tiles): the
+    tile shapes of the streaming matrix-core kernel, for every operand orientation. Too large for the scalar checker: the
     expected result is numpy's fp64 product, which is exact for the integer case
     (|sum| < 2^53) and the fp64-accumulated reference for the others."""
     k = 384 if ta == "i8" else 256
