@@ -191,7 +191,7 @@ __global__ void __launch_bounds__(kThreads) pack_vec_kernel(const uint8_t *__res
 }
 
 // 0: element kernel; 1: vector copy; 2: vector transpose. Sets the lane directions for the vector kernels.
-int vector_plan(int es, const void *src, const void *dst, PackArgs &p) {
+int vector_plan(int es, bool pack, const void *src, const void *dst, PackArgs &p) {
   const size_t V = 16 / es;
   if ((((uintptr_t)src | (uintptr_t)dst) & 15) != 0) return 0;
   const bool use_rs0 = p.m0 > 1, use_cs0 = p.n0 > 1, use_rs1 = p.rows > p.m0, use_cs1 = p.cols > p.n0;
@@ -204,8 +204,10 @@ int vector_plan(int es, const void *src, const void *dst, PackArgs &p) {
                      mult(use_cs1, p.cs1);
   if (plain_c && blk_c) { p.plain_along_c = 1; p.blocked_along_c = 1; return 1; }
   if (plain_r && blk_r) { p.plain_along_c = 0; p.blocked_along_c = 0; return 1; }
-  if (plain_c && blk_r) { p.plain_along_c = 1; p.blocked_along_c = 0; return 2; }
-  if (plain_r && blk_c) { p.plain_along_c = 0; p.blocked_along_c = 1; return 2; }
+  // Unpack reads only in-range elements (the caller's last block may be cut short), so the source
+  // vectors of a transposing unpack - V rows (columns) of a block - must lie inside m (n) as well.
+  if (plain_c && blk_r && (pack || p.m % V == 0)) { p.plain_along_c = 1; p.blocked_along_c = 0; return 2; }
+  if (plain_r && blk_c && (pack || p.n % V == 0)) { p.plain_along_c = 0; p.blocked_along_c = 1; return 2; }
   return 0;
 }
 
@@ -249,7 +251,7 @@ int launch(bool pack, const void *src, void *dst, PackArgs p) {
 int dispatch(int esize, bool pack, const void *src, void *dst, PackArgs p) {
   if (p.rows == 0 || p.cols == 0) return 0;
   if (esize == 1 || esize == 2 || esize == 4) {
-    const int plan = skl_pack_vectorise() ? vector_plan(esize, src, dst, p) : 0;
+    const int plan = skl_pack_vectorise() ? vector_plan(esize, pack, src, dst, p) : 0;
     if (plan) {
       switch (esize) {
         case 1: return launch_vec<1>(pack, plan == 2, src, dst, p);
