@@ -417,7 +417,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
         if (!GUARDED || row < p.m) {
           AccElem *out = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
           const AccElem old = read_c ? *out : (AccElem)0;
-          *out = epilogue(acc[i][j][r], old, p.alpha, p.beta);
+          // C is written once and not read again by this kernel: keep it out of the caches the operands live in.
+          __builtin_nontemporal_store(epilogue(acc[i][j][r], old, p.alpha, p.beta), out);
         }
       }
     }
@@ -848,7 +849,8 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
         const size_t row = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
         AccElem *out = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
         const AccElem old = read_c ? *out : (AccElem)0;
-        *out = epilogue(acc[i][j][r], old, p.alpha, p.beta);
+        // C is written once and not read again by this kernel: keep it out of the caches the operands live in.
+        __builtin_nontemporal_store(epilogue(acc[i][j][r], old, p.alpha, p.beta), out);
       }
     }
   }
