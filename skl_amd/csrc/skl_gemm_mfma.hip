@@ -932,6 +932,8 @@ int launch_tile(const MfmaArgs &p) {
     }
     if (p.n % 128 == 0 && tiles_m * (p.n / 128) >= 96) return launch_ring<TA, TB, A_KC, B_KC, 128>(p);
   }
+  // Small problems: 64 x 64 tiles put four times as many workgroups on the chip.
+  if (skl_div_up(p.m, 128) * (size_t)skl_div_up(p.n, 128) < 64) return launch_one<TA, TB, A_KC, B_KC, 64, 64, 2, 2, true>(p);
   return launch_one<TA, TB, A_KC, B_KC, 128, 128, 2, 4, true>(p);
 }
 

@@ -100,6 +100,27 @@ def test_general_strides(gpu, kind):
         check(gpu, kind, case, int(rng.integers(1 << 30)), "host")
 
 
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f8e4m3"))
+def test_ragged_mid_size_bounds_checked_tiles(gpu, ta):
+    """1000 x 1100 x 333 with gapped leading dimensions: 72 tiles of 128 x 128, none of them whole in
+    every dimension (the small shapes of the tables run on 64 x 64 tiles, the aligned large ones on the
+    streaming kernel)."""
+    m, n, k = 1000, 1100, 336 if ta != "i8" else 333
+    for a_kc in (True, False):
+        case = (rowmajor_case(ta, m, n, k, 2, 1, rsa=k + 16 - k % 16 + 16, rsb=1104 + 16, rsc=1101) if a_kc else
+                colmajor_a_case(ta, m, n, k, 2, 1, csa=1008, rsb=1104, rsc=1100))
+        a, b, c = case.make_inputs(77 + a_kc)
+        got = run_gemm(gpu, "rc", case, a, b, c, "device")
+        A, B, C, oc = case.dense(a, b, c)
+        exact = case.alpha * (A @ B) + case.beta * C
+        if case.is_int:
+            assert np.array_equal(got, run_oracle_gemm(case, a, b, c))
+        else:
+            rel = np.linalg.norm(got[oc] - exact) / np.linalg.norm(exact)
+            assert rel <= 1e-3, rel
+            support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=support.FP8_MFMA_REL if ta.startswith("f8") else 0.0)
+
+
 def test_f32_f64_bit_identical_to_the_checker(gpu):
     """The f32 and f64 contractions run on the any-stride kernel, which evaluates the reference's loop
     with a separately rounded multiply and add: for finite data the result equals the checker's
