@@ -21,3 +21,52 @@ int skl_check_hip(hipError_t e, const char *what);
 static inline int skl_check_launch(const char *what) { return skl_check_hip(hipGetLastError(), what); }
 
 static inline unsigned skl_div_up(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+// ---------------------------------------------------------------------------
+// C = beta*C + alpha*acc for one element, as the reference's C computes it: two
+// products and a sum, each rounded on its own (the translation units are built
+// with -ffp-contract=off); int32 wraps.
+//
+// beta == 0 is the initialising call (src/gemm/README.md:43 of the reference:
+// "accumulation (beta=1) and initialization (beta=0)"). There beta*C is a zero
+// whose sign is all the old value contributes, and the sign matters only when
+// alpha*acc is itself a zero: the old value is read for exactly those
+// elements. Results are bit-identical to the reference's for every finite C;
+// an Inf or NaN in C, which the reference would turn into NaN, is overwritten.
+// ---------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ bool skl_beta_is_zero(skl_scalar beta);
+template <>
+__device__ __forceinline__ bool skl_beta_is_zero<int>(skl_scalar beta) { return beta.i == 0; }
+template <>
+__device__ __forceinline__ bool skl_beta_is_zero<float>(skl_scalar beta) { return beta.f == 0.0f; }
+template <>
+__device__ __forceinline__ bool skl_beta_is_zero<double>(skl_scalar beta) { return beta.d == 0.0; }
+
+__device__ __forceinline__ int skl_combine(int acc, int old, skl_scalar alpha, skl_scalar beta) {
+  return (int)((unsigned)beta.i * (unsigned)old + (unsigned)alpha.i * (unsigned)acc);
+}
+__device__ __forceinline__ float skl_combine(float acc, float old, skl_scalar alpha, skl_scalar beta) {
+  return __fadd_rn(__fmul_rn(beta.f, old), __fmul_rn(alpha.f, acc));
+}
+__device__ __forceinline__ double skl_combine(double acc, double old, skl_scalar alpha, skl_scalar beta) {
+  return __dadd_rn(__dmul_rn(beta.d, old), __dmul_rn(alpha.d, acc));
+}
+
+// The beta == 0 case; `c` is dereferenced only where alpha*acc is a zero.
+__device__ __forceinline__ int skl_initialise(int acc, const int *, skl_scalar alpha, skl_scalar) {
+  return (int)((unsigned)alpha.i * (unsigned)acc);
+}
+__device__ __forceinline__ float skl_initialise(float acc, const float *c, skl_scalar alpha, skl_scalar beta) {
+  const float x = __fmul_rn(alpha.f, acc);
+  return x == 0.0f ? __fadd_rn(__fmul_rn(beta.f, *c), x) : x;
+}
+__device__ __forceinline__ double skl_initialise(double acc, const double *c, skl_scalar alpha, skl_scalar beta) {
+  const double x = __dmul_rn(alpha.d, acc);
+  return x == 0.0 ? __dadd_rn(__dmul_rn(beta.d, *c), x) : x;
+}
+
+template <typename T>
+__device__ __forceinline__ void skl_update(T acc, T *c, skl_scalar alpha, skl_scalar beta) {
+  *c = skl_beta_is_zero<T>(beta) ? skl_initialise(acc, c, alpha, beta) : skl_combine(acc, *c, alpha, beta);
+}

@@ -68,17 +68,6 @@ struct Elem<SKL_DT_F64> {
   __device__ static acc widen(type v) { return v; }
 };
 
-__device__ __forceinline__ int32_t axpby(int32_t alpha, int32_t acc, int32_t beta, int32_t c) {
-  return (int32_t)((uint32_t)beta * (uint32_t)c + (uint32_t)alpha * (uint32_t)acc);  // wraps like -fwrapv
-}
-__device__ __forceinline__ float axpby(float alpha, float acc, float beta, float c) {
-  return __fadd_rn(__fmul_rn(beta, c), __fmul_rn(alpha, acc));
-}
-
-__device__ __forceinline__ double axpby(double alpha, double acc, double beta, double c) {
-  return __dadd_rn(__dmul_rn(beta, c), __dmul_rn(alpha, acc));
-}
-
 template <int TA, int TB>
 __global__ void __launch_bounds__(256) gemm_generic_kernel(skl_gemm_desc d, unsigned tiles_n) {
   using EA = Elem<TA>;
@@ -109,12 +98,7 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(skl_gemm_desc d, unsi
     }
   }
   Acc *c = (Acc *)d.c + I * d.rsc1 + J * d.csc1 + i0 * d.rsc0 + j0 * d.csc0;
-  if constexpr (TA == SKL_DT_I8)
-    *c = axpby(d.alpha.i, acc, d.beta.i, *c);
-  else if constexpr (TA == SKL_DT_F64)
-    *c = axpby(d.alpha.d, acc, d.beta.d, *c);
-  else
-    *c = axpby(d.alpha.f, acc, d.beta.f, *c);
+  skl_update(acc, c, d.alpha, d.beta);
 }
 
 template <int TA, int TB>

@@ -281,13 +281,6 @@ __device__ __forceinline__ auto read_frag(const char *tile, int row0, int kb) {
   }
 }
 
-__device__ __forceinline__ int epilogue(int acc, int c, skl_scalar alpha, skl_scalar beta) {
-  return (int)((unsigned)beta.i * (unsigned)c + (unsigned)alpha.i * (unsigned)acc);
-}
-__device__ __forceinline__ float epilogue(float acc, float c, skl_scalar alpha, skl_scalar beta) {
-  return __fadd_rn(__fmul_rn(beta.f, c), __fmul_rn(alpha.f, acc));
-}
-
 // Tile index of a workgroup. Consecutive workgroup ids go to different XCDs
 // (eight of them, each with its own L2), so ids are first regrouped per XCD into
 // contiguous ranges, then walked in column-major groups of kGroupM tile rows so
@@ -318,6 +311,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
   constexpr int FRB = KB / 2;                   // fragment bytes per lane
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
   constexpr int MI = WM / 32, NI = WN / 32;     // MFMA blocks per wave
+  constexpr int kEpilogueBatch = MI < 2 ? MI : 2;  // blocks whose old C values are requested together
   using TileA = Tile<ES, BM, A_KC, NT>;
   using TileB = Tile<ES, BN, B_KC, NT>;
   constexpr int kStage = TileA::kBytes + TileB::kBytes;
@@ -401,25 +395,51 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
     for (int j = 0; j < NI; ++j) fb[0][j] = read_frag<ES, BN, B_KC, FRB>(na + TileA::kBytes, wn + j * 32, 0);
   }
 
-  // Epilogue: lane l of a 32x32 block holds column l%32 and rows 8*(r/4) + 4*(l/32) + r%4.
+  // Epilogue: lane l of a 32x32 block holds column l%32 and rows 8*(r/4) + 4*(l/32) + r%4. When C is
+  // updated, the old values of kEpilogueBatch blocks are all requested before the first of them is used
+  // (a load behind a store that may alias it would wait for that store: one exposed memory latency per
+  // element). C is written once and not read again: non-temporal stores keep it out of the operands' caches.
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
-  const bool read_c = !(TA == SKL_DT_I8 && p.beta.i == 0);  // 0*c == 0 only for integers
+  const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
     if (GUARDED && col >= p.n) continue;
     const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
 #pragma unroll
-    for (int i = 0; i < MI; ++i) {
+    for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
+      AccElem *out[kEpilogueBatch][4];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const size_t row = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        if (!GUARDED || row < p.m) {
-          AccElem *out = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
-          const AccElem old = read_c ? *out : (AccElem)0;
-          // C is written once and not read again by this kernel: keep it out of the caches the operands live in.
-          __builtin_nontemporal_store(epilogue(acc[i][j][r], old, p.alpha, p.beta), out);
+      for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block of 64
+          out[i][g] = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
         }
+      auto in_range = [&](int i, int r) {
+        return !GUARDED || m0 + wm + (i0 + i) * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3) < p.m;
+      };
+      if (init) {
+#pragma unroll
+        for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (in_range(i, r)) {
+              AccElem *dst = out[i][r >> 2] + (r & 3) * p.rsc0;
+              __builtin_nontemporal_store(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst);
+            }
+      } else {
+        AccElem old[kEpilogueBatch][16];
+#pragma unroll
+        for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) old[i][r] = in_range(i, r) ? out[i][r >> 2][(r & 3) * p.rsc0] : (AccElem)0;
+#pragma unroll
+        for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (in_range(i, r))
+              __builtin_nontemporal_store(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][r >> 2] + (r & 3) * p.rsc0);
       }
     }
   }
@@ -629,33 +649,44 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   // Eight waves: 2 x 4 blocks of 128 x 64 on a 256 x 256 tile, 4 x 2 blocks of 64 x 64 on a 256 x 128 one.
   constexpr int BM = 256, WAVES = 8, WAVES_N = BN == 256 ? 4 : 2, WAVES_M = WAVES / WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MI = WM / 32, NI = WN / 32;
+  constexpr int kEpilogueBatch = 2;              // blocks whose old C values are requested together
   constexpr int kSteps = SB / KB;
   constexpr int kMfmas = MI * NI;
   constexpr int kSlots = kSteps * kMfmas;        // MFMA slots per slice
   constexpr int kPre = (kSteps - 1) * kMfmas;    // slots before the slice's barrier
-  // Four stages per operand; pair loads run two slices ahead. (Six stages for a K-contiguous operand
-  // and pairs four slices ahead fit the 160 KiB of LDS next to an MN-contiguous partner, and measured slower.)
+  // Four stages per operand. A slice's fragments are read from LDS while the k-step before them is
+  // multiplied; with one k-step per slice (64 bytes of K per MFMA) that is the slice before, and the
+  // stage of the slice being multiplied is free from its barrier on. So loads run kExtra = 1 slice
+  // further ahead there: every-slice loads fill the issuing slice's own stage with slice s+4, pair loads
+  // go out on odd slices for slices s+3 and s+4. Otherwise: slice s+3, and pairs on even slices for
+  // s+2 and s+3. (Six stages for a K-contiguous operand fit the 160 KiB of LDS next to an MN-contiguous
+  // partner, and measured slower.)
   constexpr int NSA = STAGES, NSB = STAGES;
-  constexpr int kPairAhead = 2;
+  constexpr int kExtra = kSteps == 1 ? 1 : 0;
+  constexpr int kEachAhead = 3 + kExtra, kPairAhead = 2 + kExtra;
+  constexpr int kPairU = kPairAhead & 1;             // parity of the slices that issue pair loads
+  constexpr int kPairsPrologue = (kPairU + kPairAhead) / 2;
   using LA = SLoader<ES, A_KC, WAVES, BM, NSA>;
   using LB = SLoader<ES, B_KC, WAVES, BN, NSB>;
   using TileA = STile<ES, A_KC, BM, NSA>;
   using TileB = STile<ES, B_KC, BN, NSB>;
-  // An even slice issues the pair loads of the K-contiguous operands (slices s+2 and s+3) and, like
-  // every slice, the loads of slice s+3 of the MN-contiguous ones. Load `it` of the kLoads<even/odd>
-  // goes out behind MFMA slot it * kSlots / kLoads, K-contiguous operands first.
+  // Load `it` of a slice's kLoads goes out behind MFMA slot it * kSlots / kLoads, pair loads first.
   constexpr int kPairA = A_KC ? LA::kBlocks : 0, kPairB = B_KC ? LB::kBlocks : 0;
   constexpr int kEachA = A_KC ? 0 : LA::kBlocks, kEachB = B_KC ? 0 : LB::kBlocks;
-  constexpr int kEach = kEachA + kEachB;
-  constexpr int kLoadsEven = kPairA + kPairB + kEach, kLoadsOdd = kEach;
-  // At the barrier of slice s the data of slice s+1 must have landed. With pair loads two slices ahead
-  // it was requested two slices ago, or - K-contiguous operand, s odd - by the previous slice and then
-  // first in line: younger than it are at most the every-slice loads of the slice before this one and
-  // what this slice has issued in front of its barrier. With pair loads four slices ahead the youngest
-  // request is the every-slice one of two slices ago: all of the previous slice's loads are younger.
-  constexpr int kPreEven = ceil_div(kPre * kLoadsEven, kSlots), kPreOdd = ceil_div(kPre * kLoadsOdd, kSlots);
-  constexpr int kInFlightEven = (kPairAhead == 4 ? kLoadsOdd : kEach) + kPreEven;
-  constexpr int kInFlightOdd = (kPairAhead == 4 ? kLoadsEven : kEach) + kPreOdd;
+  constexpr int kEach = kEachA + kEachB, kPairs = kPairA + kPairB;
+  constexpr int kLoadsOfU[2] = {(kPairU == 0 ? kPairs : 0) + kEach, (kPairU == 1 ? kPairs : 0) + kEach};
+  // At the barrier of slice s the data of slice s+1 must have landed; vmcnt may leave in flight what
+  // was requested after it. Every-slice loads: requested by slice s+1-kEachAhead. Pair loads: by the
+  // latest slice of parity kPairU not after s+1-kPairAhead, and first in that slice. Counted as younger
+  // (conservatively): the every-slice loads of that pair-issuing slice, all loads of the slices after
+  // the older of the two requesting slices, and what slice s itself has issued in front of its barrier.
+  //   kExtra = 0: s even -> both from s-2: slice s-1 (odd, kEach).  s odd -> pairs from s-1: its kEach.
+  //   kExtra = 1: s even -> both from s-3: slices s-2 (kEach) and s-1 (pairs + kEach).
+  //               s odd  -> pairs from s-2: its kEach, and slice s-1 (kEach).
+  constexpr int kPreOfU[2] = {ceil_div(kPre * kLoadsOfU[0], kSlots), ceil_div(kPre * kLoadsOfU[1], kSlots)};
+  constexpr int kInFlightOfU[2] = {(kExtra ? 2 * kEach + kPairs : kEach) + kPreOfU[0],
+                                   (kExtra ? 2 * kEach : kEach) + kPreOfU[1]};
+  static_assert(kInFlightOfU[0] < 64 && kInFlightOfU[1] < 64, "vmcnt is a 6-bit counter");
 
   using RA = FragReader<ES, A_KC, FRB, KB, BM, NSA, MI>;
   using RB = FragReader<ES, B_KC, FRB, KB, BN, NSB, NI>;
@@ -695,17 +726,17 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   const size_t slices = p.k * ES / SB, pairs = slices / 2;
   if constexpr (A_KC) {
 #pragma unroll
-    for (int i = 0; i < kPairAhead / 2; ++i) la.issue(region_a, 2 * i, (size_t)i < pairs ? (size_t)i : pairs - 1);
+    for (int i = 0; i < kPairsPrologue; ++i) la.issue(region_a, 2 * i, (size_t)i < pairs ? (size_t)i : pairs - 1);
   } else {
 #pragma unroll
-    for (int i = 0; i < 3; ++i) la.issue(region_a, i, (size_t)i < slices ? (size_t)i : slices - 1);
+    for (int i = 0; i < kEachAhead; ++i) la.issue(region_a, i, (size_t)i < slices ? (size_t)i : slices - 1);
   }
   if constexpr (B_KC) {
 #pragma unroll
-    for (int i = 0; i < kPairAhead / 2; ++i) lb.issue(region_b, 2 * i, (size_t)i < pairs ? (size_t)i : pairs - 1);
+    for (int i = 0; i < kPairsPrologue; ++i) lb.issue(region_b, 2 * i, (size_t)i < pairs ? (size_t)i : pairs - 1);
   } else {
 #pragma unroll
-    for (int i = 0; i < 3; ++i) lb.issue(region_b, i, (size_t)i < slices ? (size_t)i : slices - 1);
+    for (int i = 0; i < kEachAhead; ++i) lb.issue(region_b, i, (size_t)i < slices ? (size_t)i : slices - 1);
   }
   wait_loads_upto<0>();
   __syncthreads();
@@ -756,12 +787,12 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
       (
           [&](auto uc) {
             constexpr int U = decltype(uc)::value;
-            constexpr int kLoads = U == 0 ? kLoadsEven : kLoadsOdd;
+            constexpr int kLoads = kLoadsOfU[U];
             const size_t s = s0 + U;
-            const size_t fill_slice = s + 3 < slices ? s + 3 : slices - 1;  // every-slice operands
-            const size_t fill_pair = (s + kPairAhead) / 2 < pairs ? (s + kPairAhead) / 2 : pairs - 1;  // pair operands (s even)
+            const size_t fill_slice = s + kEachAhead < slices ? s + kEachAhead : slices - 1;  // every-slice operands
+            const size_t fill_pair = (s + kPairAhead) / 2 < pairs ? (s + kPairAhead) / 2 : pairs - 1;  // pair operands (s of parity kPairU)
             const int cur_a = (int)(s % NSA), nxt_a = (int)((s + 1) % NSA), cur_b = (int)(s % NSB), nxt_b = (int)((s + 1) % NSB);
-            const int fill_a = (int)((s + (A_KC ? kPairAhead : 3)) % NSA), fill_b = (int)((s + (B_KC ? kPairAhead : 3)) % NSB);
+            const int fill_a = (int)((s + (A_KC ? kPairAhead : kEachAhead)) % NSA), fill_b = (int)((s + (B_KC ? kPairAhead : kEachAhead)) % NSB);
             [&]<int... KSs>(std::integer_sequence<int, KSs...>) {
               (
                   [&](auto ksc) {
@@ -772,7 +803,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
                     if constexpr (kLast) {
                       // The reads below cross into the next slice: its data must have landed for every wave.
                       // Own reads first, so that nobody's read of the stage refilled next is still in flight.
-                      wait_loads_upto<U == 0 ? kInFlightEven : kInFlightOdd>();
+                      wait_loads_upto<kInFlightOfU[U]>();
                       landed(cur);
                       __builtin_amdgcn_s_barrier();
                     } else {
@@ -808,16 +839,16 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
                                   [&](auto lc) {
                                     constexpr int L = decltype(lc)::value;
                                     if constexpr (L * kSlots / kLoads == kSlot) {
-                                      constexpr int kPairs = U == 0 ? kPairA + kPairB : 0;
-                                      if constexpr (L < kPairs) {
-                                        if constexpr (L < kPairA && U == 0)
+                                      constexpr int kPairsNow = U == kPairU ? kPairs : 0;
+                                      if constexpr (L < kPairsNow) {
+                                        if constexpr (L < kPairA)
                                           la.issue_one(region_a, fill_a, fill_pair, L);
                                         else
-                                          lb.issue_one(region_b, fill_b, fill_pair, L - (U == 0 ? kPairA : 0));
-                                      } else if constexpr (L - kPairs < kEachA) {
-                                        la.issue_one(region_a, fill_a, fill_slice, L - kPairs);
+                                          lb.issue_one(region_b, fill_b, fill_pair, L - kPairA);
+                                      } else if constexpr (L - kPairsNow < kEachA) {
+                                        la.issue_one(region_a, fill_a, fill_slice, L - kPairsNow);
                                       } else {
-                                        lb.issue_one(region_b, fill_b, fill_slice, L - kPairs - kEachA);
+                                        lb.issue_one(region_b, fill_b, fill_slice, L - kPairsNow - kEachA);
                                       }
                                     }
                                   }(std::integral_constant<int, Ls>{}),
@@ -836,21 +867,42 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
+  // Epilogue, as in the kernel above: old values requested kEpilogueBatch blocks at a time, non-temporal stores.
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
-  const bool read_c = !(TA == SKL_DT_I8 && p.beta.i == 0);
+  const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
     const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
 #pragma unroll
-    for (int i = 0; i < MI; ++i) {
+    for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
+      AccElem *out[kEpilogueBatch][4];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const size_t row = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        AccElem *out = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
-        const AccElem old = read_c ? *out : (AccElem)0;
-        // C is written once and not read again by this kernel: keep it out of the caches the operands live in.
-        __builtin_nontemporal_store(epilogue(acc[i][j][r], old, p.alpha, p.beta), out);
+      for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block of 64
+          out[i][g] = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
+        }
+      if (init) {
+#pragma unroll
+        for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            AccElem *dst = out[i][r >> 2] + (r & 3) * p.rsc0;
+            __builtin_nontemporal_store(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst);
+          }
+      } else {
+        AccElem old[kEpilogueBatch][16];
+#pragma unroll
+        for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) old[i][r] = out[i][r >> 2][(r & 3) * p.rsc0];
+#pragma unroll
+        for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            __builtin_nontemporal_store(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][r >> 2] + (r & 3) * p.rsc0);
       }
     }
   }

@@ -136,12 +136,6 @@ __device__ __forceinline__ float widen16(unsigned bits16, bool is_bf16) {
   return (float)h;
 }
 
-__device__ __forceinline__ int finish(int total, int old, skl_scalar alpha, skl_scalar beta) {
-  return (int)((unsigned)beta.i * (unsigned)old + (unsigned)alpha.i * (unsigned)total);
-}
-__device__ __forceinline__ float finish(float total, float old, skl_scalar alpha, skl_scalar beta) {
-  return __fadd_rn(__fmul_rn(beta.f, old), __fmul_rn(alpha.f, total));
-}
 
 template <int MODE>
 __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
@@ -255,7 +249,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
   if (p.slabs == 1) {  // the strip is complete inside this workgroup
     if (owner) {
       Acc *y = yv + (tile_col0 + threadIdx.x) * p.y_s;
-      *y = finish(sum, *y, p.alpha, p.beta);
+      skl_update(sum, y, p.alpha, p.beta);
     }
     return;
   }
@@ -271,7 +265,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
       if ((unsigned)now == p.slabs) {
         __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
         Acc *y = yv + j * p.y_s;
-        *y = finish((int)(unsigned)(now >> 32), *y, p.alpha, p.beta);
+        skl_update((int)(unsigned)(now >> 32), y, p.alpha, p.beta);
       }
     }
   } else {
@@ -288,7 +282,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
       const size_t j = tile_col0 + threadIdx.x;
       const Acc total = atomicExch(&scratch[j], (Acc)0);  // read the total and leave zero behind
       Acc *y = yv + j * p.y_s;
-      *y = finish(total, *y, p.alpha, p.beta);
+      skl_update(total, y, p.alpha, p.beta);
     }
     if (threadIdx.x == 0) atomicExch(&p.tickets[tile], 0u);
   }

@@ -137,6 +137,43 @@ def test_f32_f64_bit_identical_to_the_checker(gpu):
                 assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (ta, mode)
 
 
+@pytest.mark.parametrize("ta,m,n,k", (("bf16", 130, 200, 64), ("f8e4m3", 256, 256, 128), ("f16", 512, 2048 + 128, 256),
+                                       ("f32", 33, 47, 17), ("f64", 20, 31, 9), ("bf16", 1, 4096, 512)))
+def test_beta_zero_initialises_c(gpu, ta, m, n, k):
+    """beta == 0 is the initialising call. The old C then contributes nothing but the sign of an exact
+    zero (beta*c is a signed zero, and it only shows when alpha*acc is a zero too), so the result must
+    equal the checker's bit for bit wherever it is a zero - rows of A are zeroed to make such elements,
+    C holds both signs - and an Inf or NaN in C must be overwritten exactly as a finite value is."""
+    rng = np.random.default_rng(77)
+    for alpha, beta in ((-1.5, 0.0), (2.0, -0.0)):
+        case = rowmajor_case(ta, m, n, k, alpha, beta)
+        a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+        zero_rows = sorted(set((0, m // 2, m - 1)))
+        for i in zero_rows:
+            a[i * k:(i + 1) * k] = 0
+        want = run_oracle_gemm(case, a, b, c)
+        spoiled = c.copy()
+        live = np.ones(m, dtype=bool)
+        live[zero_rows] = False
+        rows = np.flatnonzero(live)
+        if rows.size:
+            view = spoiled.reshape(m, n)
+            view[rows[::3], ::5] = np.nan
+            view[rows[1::3], 1::7] = np.inf
+            view[rows[2::3], 2::11] = -np.inf
+        for mode in MODES:
+            got = run_gemm(gpu, "rc", case, a, b, c, mode)
+            again = run_gemm(gpu, "rc", case, a, b, spoiled, mode)
+            for i in zero_rows:
+                row = slice(i * n, (i + 1) * n)
+                assert np.array_equal(got[row].view(np.uint8), want[row].view(np.uint8)), (ta, mode, alpha, i)
+            assert np.all(np.isfinite(again)), (ta, mode, alpha)
+            if m > 1:  # the M = 1 path sums with floating-point atomics: not the same bits from run to run
+                assert np.array_equal(got.view(np.uint8), again.view(np.uint8)), (ta, mode, alpha)
+            if ta in ("f32", "f64"):
+                assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (ta, mode, alpha)
+
+
 def test_mixed_e4m3_e5m2(gpu):
     for (m, n, k) in ((13, 21, 37), (128, 192, 256)):
         case = rowmajor_case("f8e4m3", m, n, k, 1.0, 0.0, tb="f8e5m2")
