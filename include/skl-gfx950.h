@@ -27,6 +27,7 @@
 #if defined(__clang__) || (defined(__GNUC__) && __GNUC__ >= 13)
 typedef __bf16 skl_bf16_t;
 typedef _Float16 skl_f16_t;
+#define SKL_GFX950_HAS_F16_SCALARS 1 /* `_Float16` can be passed by value: the f16 -> f16 GEMMs are declared */
 #else
 typedef uint16_t skl_bf16_t;
 typedef uint16_t skl_f16_t;
@@ -98,6 +99,21 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f32rcprc_f32rcprc_f32rcprc_gfx950, float, floa
 /* ref/gemm/gemm_f64rcprc_f64rcprc_f64rcprc.h:49 */
 SKL_GFX950_DECLARE_RCPRC(skl_gemm_f64rcprc_f64rcprc_f64rcprc_gfx950, double, double);
 
+#ifdef SKL_GFX950_HAS_F16_SCALARS
+/* f16 operands, f16 accumulator, f16 C; alpha and beta are `_Float16` by value, as in the reference.
+ * `_Float16` expressions are evaluated in float and rounded to half where they are assigned (what a C
+ * compiler does for a target without half arithmetic, i.e. how the reference's scalar library computes
+ * on a general-purpose host); hardware with native half arithmetic rounds the product as well and may
+ * differ in the last place, inside the reference's own bound (test/gemm/gemm_f16rcprc_f16rcprc_f16rcprc.c:157).
+ * Served by the any-stride kernel.
+ * ref/gemm/gemm_f16rc_f16rc_f16rc.h:44 */
+void skl_gemm_f16rc_f16rc_f16rc_gfx950(size_t m, size_t n, size_t k, skl_f16_t alpha, const skl_f16_t *a,
+                                       size_t rsa, size_t csa, const skl_f16_t *b, size_t rsb, size_t csb,
+                                       skl_f16_t beta, skl_f16_t *c, size_t rsc, size_t csc);
+/* ref/gemm/gemm_f16rcprc_f16rcprc_f16rcprc.h:49 */
+SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, skl_f16_t);
+#endif
+
 /* ======================================================================== */
 /* GEMM - the optimized entry points of skl.h                                */
 /* ======================================================================== */
@@ -119,6 +135,11 @@ void skl_gemm_f32_f32_f32_gfx950(size_t m, size_t n, size_t k, float alpha, cons
 /* src/gemm/gemm_f64_f64_f64_zve64d.h:48, src/gemm/gemm_f64_f64_f64_zve64d_x390.h */
 void skl_gemm_f64_f64_f64_gfx950(size_t m, size_t n, size_t k, double alpha, const double *a, size_t rsa,
                                  const double *b, size_t rsb, double beta, double *c, size_t rsc);
+#ifdef SKL_GFX950_HAS_F16_SCALARS
+/* src/gemm/gemm_f16_f16_f16_zvfh.h:48, src/gemm/gemm_f16_f16_f16_zvfh_x390.h */
+void skl_gemm_f16_f16_f16_gfx950(size_t m, size_t n, size_t k, skl_f16_t alpha, const skl_f16_t *a, size_t rsa,
+                                 const skl_f16_t *b, size_t rsb, skl_f16_t beta, skl_f16_t *c, size_t rsc);
+#endif
 
 /* Column-major A (= A^T stored row-major with row stride csa), row-major B, C.
  * src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:57 */

@@ -144,6 +144,30 @@ float skl_oracle_f16_to_f32(uint16_t h) {
   return bits_to_f32(s | ((e + 112u) << 23) | (m << 13));
 }
 
+/* f32 -> f16, round to nearest even, as the conversion `(_Float16)x` rounds: overflow goes to infinity,
+ * results below the smallest normal are subnormal halves, NaN keeps its sign and the top payload bits. */
+uint16_t skl_oracle_f32_to_f16(float x) {
+  const uint32_t u = f32_to_bits(x);
+  const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  const uint32_t mag = u & 0x7FFFFFFFu;
+  if (mag > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((mag >> 13) & 0x3FFu)); /* NaN, made quiet */
+  if (mag >= 0x47800000u) return (uint16_t)(sign | 0x7C00u);                         /* >= 65536, incl. infinity */
+  if (mag < 0x33000000u) return sign;                                                /* < 2^-25: to zero */
+  {
+    const int32_t e = (int32_t)(mag >> 23) - 127; /* unbiased exponent, -25 .. 15 */
+    const uint32_t sig = (mag & 0x7FFFFFu) | 0x800000u; /* 24-bit significand, value sig * 2^(e-23) */
+    /* target unit: 2^(e-10) for a normal half (e >= -14), 2^-24 for a subnormal */
+    const int shift = e >= -14 ? 13 : (-24) - (e - 23); /* bits dropped from sig */
+    const uint32_t kept = sig >> shift, rest = sig & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    uint32_t q = kept + ((rest > half || (rest == half && (kept & 1u))) ? 1u : 0u);
+    if (e >= -14) { /* q in [2^10, 2^11]; a carry to 2^11 bumps the exponent through the addition */
+      const uint32_t h = ((uint32_t)(e + 15) << 10) + (q - 0x400u);
+      return (uint16_t)(sign | (h >= 0x7C00u ? 0x7C00u : h));
+    }
+    return (uint16_t)(sign | q); /* q <= 2^10: 2^10 is the smallest normal, encoded by the same bits */
+  }
+}
+
 /* f32 -> bf16, round to nearest even; NaN becomes the quiet NaN with the
  * payload truncated (the C cast `(__bf16)x` the reference uses at
  * ref/cvt/cvt_ofp8.c:233,240). */
@@ -336,6 +360,55 @@ GEMM_RCPRC(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, uint8_t, float,
 /* ref/gemm/gemm_f32rcprc_f32rcprc_f32rcprc.c:9-36 */
 GEMM_RCPRC(f32rcprc_f32rcprc_f32rcprc, float, float, float, LOAD_ID, LOAD_ID)
 GEMM_RCPRC(f64rcprc_f64rcprc_f64rcprc, double, double, double, LOAD_ID, LOAD_ID)
+
+/*
+ * f16 operands, f16 accumulator, f16 C: ref/gemm/gemm_f16rc_f16rc_f16rc.c:9-24 and
+ * ref/gemm/gemm_f16rcprc_f16rcprc_f16rcprc.c. The reference writes `_Float16 acc; acc += a * b;` and
+ * `c = beta * c + alpha * acc`. A C compiler for a target without half arithmetic evaluates `_Float16`
+ * expressions in float and rounds to half where the value is assigned, so
+ *   acc = half(float(acc) + a*b)            the product of two halves is exact in float
+ *   c   = half(float(beta*c + alpha*acc))   both products exact, the sum rounded to float, then to half.
+ * alpha and beta arrive as floats holding half values.
+ */
+static uint16_t f16h_step(uint16_t acc, uint16_t a, uint16_t b) {
+  volatile float prod = skl_oracle_f16_to_f32(a) * skl_oracle_f16_to_f32(b);
+  volatile float sum = skl_oracle_f16_to_f32(acc) + prod;
+  return skl_oracle_f32_to_f16(sum);
+}
+static uint16_t f16h_finish(uint16_t acc, uint16_t c, float alpha, float beta) {
+  volatile float bc = beta * skl_oracle_f16_to_f32(c), aa = alpha * skl_oracle_f16_to_f32(acc);
+  volatile float sum = bc + aa;
+  return skl_oracle_f32_to_f16(sum);
+}
+void skl_gemm_f16rc_f16rc_f16rc_oracle(size_t m, size_t n, size_t k, float alpha, const uint16_t *a, size_t rsa,
+                                       size_t csa, const uint16_t *b, size_t rsb, size_t csb, float beta,
+                                       uint16_t *c, size_t rsc, size_t csc) {
+  for (size_t i = 0; i < m; ++i)
+    for (size_t j = 0; j < n; ++j) {
+      uint16_t acc = 0;
+      for (size_t p = 0; p < k; ++p) acc = f16h_step(acc, a[i * rsa + p * csa], b[p * rsb + j * csb]);
+      uint16_t *out = c + i * rsc + j * csc;
+      *out = f16h_finish(acc, *out, alpha, beta);
+    }
+}
+void skl_gemm_f16rcprc_f16rcprc_f16rcprc_oracle(size_t m0, size_t n0, size_t k0, size_t m1, size_t n1, size_t k1,
+                                                float alpha, const uint16_t *a, size_t rsa0, size_t csa0,
+                                                size_t rsa1, size_t csa1, const uint16_t *b, size_t rsb0,
+                                                size_t csb0, size_t rsb1, size_t csb1, float beta, uint16_t *c,
+                                                size_t rsc0, size_t csc0, size_t rsc1, size_t csc1) {
+  for (size_t I = 0; I < m1; ++I)
+    for (size_t J = 0; J < n1; ++J)
+      for (size_t i = 0; i < m0; ++i)
+        for (size_t j = 0; j < n0; ++j) {
+          uint16_t acc = 0;
+          for (size_t P = 0; P < k1; ++P)
+            for (size_t p = 0; p < k0; ++p)
+              acc = f16h_step(acc, a[I * rsa1 + P * csa1 + i * rsa0 + p * csa0],
+                              b[P * rsb1 + J * csb1 + p * rsb0 + j * csb0]);
+          uint16_t *out = c + I * rsc1 + J * csc1 + i * rsc0 + j * csc0;
+          *out = f16h_finish(acc, *out, alpha, beta);
+        }
+}
 
 /* ======================================================================== */
 /* Widening helpers                                                          */

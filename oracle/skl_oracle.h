@@ -35,6 +35,7 @@ uint8_t skl_oracle_f32_to_f8e5m2(float x, int saturate);
 float skl_oracle_bf16_to_f32(uint16_t bits);
 float skl_oracle_f16_to_f32(uint16_t bits);
 uint16_t skl_oracle_f32_to_bf16(float x);
+uint16_t skl_oracle_f32_to_f16(float x);
 
 /* ---- array conversions (dst, src, scale, n) ----------------------------- */
 void skl_cvt_f32_f8e4m3_oracle(uint8_t *dst, const float *src, float scale, size_t n);
@@ -94,6 +95,16 @@ SKL_ORACLE_PGEMM_DECL(f8e4m3rcprc_f8e4m3rcprc_f32rcprc, uint8_t, uint8_t, float)
 SKL_ORACLE_PGEMM_DECL(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, uint8_t, float)
 SKL_ORACLE_PGEMM_DECL(f32rcprc_f32rcprc_f32rcprc, float, float, float)
 SKL_ORACLE_PGEMM_DECL(f64rcprc_f64rcprc_f64rcprc, double, double, double)
+/* f16 accumulator and C (ref/gemm/gemm_f16rc_f16rc_f16rc.c:9-24 and the rcprc twin); alpha, beta: floats
+ * holding half values */
+void skl_gemm_f16rc_f16rc_f16rc_oracle(size_t m, size_t n, size_t k, float alpha, const uint16_t *a, size_t rsa,
+                                       size_t csa, const uint16_t *b, size_t rsb, size_t csb, float beta,
+                                       uint16_t *c, size_t rsc, size_t csc);
+void skl_gemm_f16rcprc_f16rcprc_f16rcprc_oracle(size_t m0, size_t n0, size_t k0, size_t m1, size_t n1, size_t k1,
+                                                float alpha, const uint16_t *a, size_t rsa0, size_t csa0,
+                                                size_t rsa1, size_t csa1, const uint16_t *b, size_t rsb0,
+                                                size_t csb0, size_t rsb1, size_t csb1, float beta, uint16_t *c,
+                                                size_t rsc0, size_t csc0, size_t rsc1, size_t csc1);
 
 /* Widening helpers used to build fp64 comparison operands on the host. */
 void skl_oracle_widen_bf16_f64(double *dst, const uint16_t *src, size_t n);

@@ -28,13 +28,14 @@
 static size_t elem_size(int dt) {
   switch (dt) {
     case SKL_DT_BF16:
-    case SKL_DT_F16: return 2u;
+    case SKL_DT_F16:
+    case SKL_DT_F16H: return 2u;
     case SKL_DT_F32: return 4u;
     case SKL_DT_F64: return 8u;
     default: return 1u;
   }
 }
-static size_t c_elem_size(int dt) { return dt == SKL_DT_F64 ? 8u : 4u; }
+static size_t c_elem_size(int dt) { return dt == SKL_DT_F64 ? 8u : dt == SKL_DT_F16H ? 2u : 4u; }
 
 /* Number of elements between the first and one past the last addressed element
  * of a 4-level strided array; 0 if any extent is 0. */
@@ -225,6 +226,8 @@ DEFINE_GEMM_RC(skl_gemm_f8e5m2rc_f8e5m2rc_f32rc_gfx950, uint8_t, float, SKL_DT_F
 DEFINE_GEMM_RC(skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950, uint8_t, float, SKL_DT_F8E4M3, SKL_DT_F8E5M2, SCALAR_f32)
 DEFINE_GEMM_RC(skl_gemm_f32rc_f32rc_f32rc_gfx950, float, float, SKL_DT_F32, SKL_DT_F32, SCALAR_f32)
 DEFINE_GEMM_RC(skl_gemm_f64rc_f64rc_f64rc_gfx950, double, double, SKL_DT_F64, SKL_DT_F64, SCALAR_f64)
+/* _Float16 scalars widen exactly */
+DEFINE_GEMM_RC(skl_gemm_f16rc_f16rc_f16rc_gfx950, skl_f16_t, skl_f16_t, SKL_DT_F16H, SKL_DT_F16H, SCALAR_f32)
 
 /* blocked (rcprc) form */
 #define DEFINE_GEMM_RCPRC(NAME, TA_T, TC_T, DT, SC)                                                \
@@ -245,6 +248,7 @@ DEFINE_GEMM_RCPRC(skl_gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950, uint8_t, flo
 DEFINE_GEMM_RCPRC(skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, float, SKL_DT_F8E5M2, SCALAR_f32)
 DEFINE_GEMM_RCPRC(skl_gemm_f32rcprc_f32rcprc_f32rcprc_gfx950, float, float, SKL_DT_F32, SCALAR_f32)
 DEFINE_GEMM_RCPRC(skl_gemm_f64rcprc_f64rcprc_f64rcprc_gfx950, double, double, SKL_DT_F64, SCALAR_f64)
+DEFINE_GEMM_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, skl_f16_t, SKL_DT_F16H, SCALAR_f32)
 
 /* row-major A, B, C: the rc form with csa = csb = csc = 1
  * (src/gemm/gemm_i8_i8_i32_zve32x.h:38-48) */
@@ -258,6 +262,7 @@ DEFINE_GEMM_ROWMAJOR(skl_gemm_bf16_bf16_f32_gfx950, skl_gemm_bf16rc_bf16rc_f32rc
 DEFINE_GEMM_ROWMAJOR(skl_gemm_f16_f16_f32_gfx950, skl_gemm_f16rc_f16rc_f32rc_gfx950, skl_f16_t, float)
 DEFINE_GEMM_ROWMAJOR(skl_gemm_f32_f32_f32_gfx950, skl_gemm_f32rc_f32rc_f32rc_gfx950, float, float)
 DEFINE_GEMM_ROWMAJOR(skl_gemm_f64_f64_f64_gfx950, skl_gemm_f64rc_f64rc_f64rc_gfx950, double, double)
+DEFINE_GEMM_ROWMAJOR(skl_gemm_f16_f16_f16_gfx950, skl_gemm_f16rc_f16rc_f16rc_gfx950, skl_f16_t, skl_f16_t)
 
 /* column-major A: the rc form with rsa = 1
  * (src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:38-48) */

@@ -61,6 +61,18 @@ struct Elem<SKL_DT_F32> {
   using acc = float;
   __device__ static acc widen(type v) { return v; }
 };
+// f16 operands with an f16 accumulator (ref/gemm/gemm_f16rc_f16rc_f16rc.c:9-24). `_Float16` arithmetic is
+// evaluated the way a C compiler evaluates it for a target without half-precision arithmetic, which is
+// how the reference's scalar library comes out when it is built for a general-purpose host: operands are
+// promoted to float, an expression is evaluated in float, and the value is rounded to half where it is
+// assigned. So acc = half(float(acc) + a*b) per step (the product of two halves is exact in float) and
+// C = half(beta*C + alpha*acc) with exact products, one float rounding of the sum and one to half.
+template <>
+struct Elem<SKL_DT_F16H> {
+  using type = _Float16;
+  using acc = _Float16;
+  __device__ static float widen(type v) { return (float)v; }
+};
 template <>
 struct Elem<SKL_DT_F64> {
   using type = double;
@@ -85,9 +97,11 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(skl_gemm_desc d, unsi
     const typename EA::type *ap = a + P * d.csa1;
     const typename EB::type *bp = b + P * d.rsb1;
     for (size_t p = 0; p < d.k0; ++p) {
-      const Acc av = EA::widen(ap[p * d.csa0]);
-      const Acc bv = EB::widen(bp[p * d.rsb0]);
-      if constexpr (TA == SKL_DT_I8)
+      const auto av = EA::widen(ap[p * d.csa0]);
+      const auto bv = EB::widen(bp[p * d.rsb0]);
+      if constexpr (TA == SKL_DT_F16H)
+        acc = (_Float16)__fadd_rn((float)acc, __fmul_rn(av, bv));
+      else if constexpr (TA == SKL_DT_I8)
         acc = (Acc)((uint32_t)acc + (uint32_t)av * (uint32_t)bv);
       else if constexpr (TA == SKL_DT_F32)  // products are not exact here: multiply, then add, as the reference's C does
         acc = __fadd_rn(acc, __fmul_rn(av, bv));
@@ -98,7 +112,14 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(skl_gemm_desc d, unsi
     }
   }
   Acc *c = (Acc *)d.c + I * d.rsc1 + J * d.csc1 + i0 * d.rsc0 + j0 * d.csc0;
-  skl_update(acc, c, d.alpha, d.beta);
+  if constexpr (TA == SKL_DT_F16H) {
+    float wide = (float)*c;
+    float *alias = &wide;
+    skl_update((float)acc, alias, d.alpha, d.beta);
+    *c = (_Float16)wide;
+  } else {
+    skl_update(acc, c, d.alpha, d.beta);
+  }
 }
 
 template <int TA, int TB>
@@ -128,6 +149,7 @@ extern "C" int skl_hip_launch_gemm_generic(const skl_gemm_desc *d) {
     case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E4M3: return launch<SKL_DT_F8E5M2, SKL_DT_F8E4M3>(*d);
     case SKL_DT_F32 * 8 + SKL_DT_F32: return launch<SKL_DT_F32, SKL_DT_F32>(*d);
     case SKL_DT_F64 * 8 + SKL_DT_F64: return launch<SKL_DT_F64, SKL_DT_F64>(*d);
+    case SKL_DT_F16H * 8 + SKL_DT_F16H: return launch<SKL_DT_F16H, SKL_DT_F16H>(*d);
     default:
       skl_hip_record_error(-2, "gemm: operand type pair");
       return -2;

@@ -26,7 +26,8 @@ enum {
   SKL_DT_F8E4M3 = 3,
   SKL_DT_F8E5M2 = 4,
   SKL_DT_F32 = 5, /* any-stride kernel only */
-  SKL_DT_F64 = 6  /* any-stride kernel only */
+  SKL_DT_F64 = 6, /* any-stride kernel only */
+  SKL_DT_F16H = 7 /* f16 operands with an f16 accumulator and an f16 C; any-stride kernel only */
 };
 
 typedef union {
@@ -39,7 +40,8 @@ typedef union {
  * (I,i ; P,p) of A is at a + I*rsa1 + P*csa1 + i*rsa0 + p*csa0, and likewise
  * for B (rows = k, columns = n) and C. Strides are in elements. */
 typedef struct {
-  int ta, tb; /* element kind of A and B; C is int32 for SKL_DT_I8, f64 for SKL_DT_F64, else f32 */
+  int ta, tb; /* element kind of A and B; C is int32 for SKL_DT_I8, f64 for SKL_DT_F64, f16 for SKL_DT_F16H,
+                 else f32. alpha and beta of SKL_DT_F16H travel widened in `.f` */
   size_t m0, n0, k0, m1, n1, k1;
   const void *a;
   size_t rsa0, csa0, rsa1, csa1;

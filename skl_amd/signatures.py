@@ -1,12 +1,29 @@
 """Argument signatures of the C entry points, one string per function.
 
 Each character is one C parameter: ``z`` size_t, ``p`` pointer, ``i`` int32_t,
-``f`` float, ``d`` double, ``b`` uint8_t, ``h`` uint16_t, ``w`` uint32_t.
+``f`` float, ``d`` double, ``b`` uint8_t, ``h`` uint16_t, ``w`` uint32_t,
+``H`` a ``_Float16`` passed by value.
 Names are given without the implementation suffix (``_gfx950`` for the GPU
 library); the parameter order is the reference's (include/skl-gfx950.h cites
 the prototype each one mirrors).
 """
 import ctypes
+import struct
+
+import numpy as np
+
+
+class HalfByValue:
+    """`_Float16` by value. The x86-64 System V ABI passes it in the low 16 bits of
+    an SSE register, the register a ``float`` argument in the same position would
+    use; ctypes has no half type, so a float whose low 16 bits are the half's
+    pattern is passed in its place."""
+
+    @classmethod
+    def from_param(cls, value):
+        bits = int(np.float16(value).view(np.uint16))
+        return ctypes.c_float(struct.unpack("<f", struct.pack("<I", bits))[0])
+
 
 CTYPES = {
     "z": ctypes.c_size_t,
@@ -17,6 +34,7 @@ CTYPES = {
     "b": ctypes.c_uint8,
     "h": ctypes.c_uint16,
     "w": ctypes.c_uint32,
+    "H": HalfByValue,
 }
 
 
@@ -46,6 +64,7 @@ GEMM_RC = {
     "skl_gemm_f8e4m3rc_f8e5m2rc_f32rc": "f",
     "skl_gemm_f32rc_f32rc_f32rc": "f",
     "skl_gemm_f64rc_f64rc_f64rc": "d",
+    "skl_gemm_f16rc_f16rc_f16rc": "H",
 }
 GEMM_RCPRC = {
     "skl_gemm_i8rcprc_i8rcprc_i32rcprc": "i",
@@ -55,6 +74,7 @@ GEMM_RCPRC = {
     "skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc": "f",
     "skl_gemm_f32rcprc_f32rcprc_f32rcprc": "f",
     "skl_gemm_f64rcprc_f64rcprc_f64rcprc": "d",
+    "skl_gemm_f16rcprc_f16rcprc_f16rcprc": "H",
 }
 GEMM_ROWMAJOR = {
     "skl_gemm_i8_i8_i32": "i",
@@ -62,6 +82,7 @@ GEMM_ROWMAJOR = {
     "skl_gemm_f16_f16_f32": "f",
     "skl_gemm_f32_f32_f32": "f",
     "skl_gemm_f64_f64_f64": "d",
+    "skl_gemm_f16_f16_f16": "H",
 }
 GEMM_COLMAJOR_A = {
     "skl_gemm_i8c_i8_i32": "i",

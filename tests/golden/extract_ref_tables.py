@@ -19,6 +19,8 @@ SUITES = [
     "test/gemm/rvv/skl_gemm_bf16_bf16_f32_zvfbfwma_x390.c",
     "test/gemm/rvv/skl_gemm_f16_f16_f32_zvfh.c",
     "test/gemm/rvv/skl_gemm_f16_f16_f32_zvfh_x390.c",
+    "test/gemm/rvv/skl_gemm_f16_f16_f16_zvfh.c",
+    "test/gemm/rvv/skl_gemm_f16_f16_f16_zvfh_x390.c",
     "test/gemm/rvv/skl_gemm_f32_f32_f32_zve32f.c",
     "test/gemm/rvv/skl_gemm_f32_f32_f32_zve32f_x390.c",
     "test/gemm/rvv/skl_gemm_f64_f64_f64_zve64d.c",
@@ -62,7 +64,7 @@ FIELD = re.compile(r"\.(\w+)\s*=\s*([^,}]+)")
 
 
 def evaluate(expr, unknown):
-    expr = expr.strip().replace("(size_t)", "")
+    expr = expr.strip().replace("(size_t)", "").replace("(_Float16)", "").strip()
     if re.fullmatch(r"[\d.]+[fFuUlL]*", expr):
         expr = expr.rstrip("fFuUlL")
     try:

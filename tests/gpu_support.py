@@ -18,12 +18,12 @@ def _finish(lib):
 def gemm_entry_args(kind, case, a, b, c):
     """(function name, argument tuple) of the entry point `kind` for a case that
     fits it; mirrors the execute() callbacks of the reference's suites."""
-    t = case.ta
+    t = case.atag
     cty = case.ctag
     if kind == "rcprc":
         return case.stem() + "_gfx950", case.rcprc_args(a, b, c)
     if kind == "rc":
-        tb = case.tb
+        tb = case.btag
         return (f"skl_gemm_{t}rc_{tb}rc_{cty}rc_gfx950",
                 (case.m1, case.n1, case.k1, case.alpha, a, case.rsa1, case.csa1, b, case.rsb1, case.csb1,
                  case.beta, c, case.rsc1, case.csc1))

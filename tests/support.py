@@ -132,6 +132,8 @@ ETYPES = {
     "i8": EType("i8", np.int8, _gen_i8, lambda a: a.astype(np.float64)),
     "bf16": EType("bf16", np.uint16, _gen_bf16, lambda a: bf16_bits_to_f32(a).astype(np.float64)),
     "f16": EType("f16", np.uint16, _gen_f16, lambda a: f16_bits_to_f32(a).astype(np.float64)),
+    # f16 operands with an f16 accumulator and an f16 C (the f16 -> f16 GEMMs)
+    "f16h": EType("f16h", np.uint16, _gen_f16, lambda a: f16_bits_to_f32(a).astype(np.float64)),
     "f8e4m3": EType("f8e4m3", np.uint8, _gen_e4m3, lambda a: decode_table("f8e4m3")[a]),
     "f8e5m2": EType("f8e5m2", np.uint8, _gen_e5m2, lambda a: decode_table("f8e5m2")[a]),
 }
@@ -174,17 +176,27 @@ class GemmCase:
 
     @property
     def cdtype(self):
-        return np.int32 if self.is_int else np.float64 if self.ta == "f64" else np.float32
+        return {"i8": np.int32, "f64": np.float64, "f16h": np.float16}.get(self.ta, np.float32)
 
     @property
     def ctag(self):
         """C's element type as the function names spell it."""
-        return "i32" if self.is_int else "f64" if self.ta == "f64" else "f32"
+        return {"i8": "i32", "f64": "f64", "f16h": "f16"}.get(self.ta, "f32")
+
+    @property
+    def atag(self):
+        """A's element type as the function names spell it."""
+        return "f16" if self.ta == "f16h" else self.ta
+
+    @property
+    def btag(self):
+        return "f16" if self.tb == "f16h" else self.tb
 
     @property
     def unit_roundoff_bits(self):
-        """P of the reference's bound: accumulator precision (test/gemm/gemm_f64rcprc_f64rcprc_f64rcprc.c:190)."""
-        return 53 if self.ta == "f64" else 24
+        """P of the reference's bound: accumulator precision (test/gemm/gemm_f64rcprc_f64rcprc_f64rcprc.c:190,
+        test/gemm/gemm_f16rcprc_f16rcprc_f16rcprc.c:157)."""
+        return {"f64": 53, "f16h": 11}.get(self.ta, 24)
 
     def spans(self):
         a = span((self.m1, self.k1, self.m0, self.k0), (self.rsa1, self.csa1, self.rsa0, self.csa0))
@@ -210,7 +222,7 @@ class GemmCase:
                 self.beta, c, self.rsc0, self.csc0, self.rsc1, self.csc1)
 
     def stem(self):
-        return f"skl_gemm_{self.ta}rcprc_{self.tb}rcprc_{self.ctag}rcprc"
+        return f"skl_gemm_{self.atag}rcprc_{self.btag}rcprc_{self.ctag}rcprc"
 
     def dense(self, a, b, c):
         """Logical (M x K), (K x N), (M x N) views gathered from the buffers, widened to fp64."""
@@ -326,12 +338,12 @@ def assert_fp_gemm_close(case, a, b, c_before, c_after, frob_tol=1e-3, extra_rel
     assert not bad.any(), (f"{int(bad.sum())} elements exceed the reference bound; worst ratio "
                            f"{float((err / (bound + slack)).max()):.3g}")
     denom = np.linalg.norm(exact)
-    if denom > 0:
+    if denom > 0 and frob_tol is not None:
         rel = np.linalg.norm(got - exact) / denom
         assert rel <= frob_tol, f"relative Frobenius error {rel:.3e} > {frob_tol}"
     mask = np.ones(c_after.shape, dtype=bool)
     if oc.size:
         mask[oc.ravel()] = False
-    assert np.array_equal(c_after[mask].view(np.uint32), c_before[mask].view(np.uint32)), \
+    assert np.array_equal(c_after[mask].view(np.uint8), c_before[mask].view(np.uint8)), \
         "elements outside the addressed C were modified"
     return float((err / (ref_bound + slack)).max()) if err.size else 0.0

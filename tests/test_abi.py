@@ -12,7 +12,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_functions(header):
-    text = subprocess.run(["gcc", "-E", "-P", "-I", os.path.join(ROOT, "include"), os.path.join(ROOT, "include", header)],
+    # a preprocessor that knows `_Float16`, so that the prototypes taking it by value are seen as well
+    clang = "/opt/rocm/lib/llvm/bin/clang"
+    text = subprocess.run([clang if os.path.exists(clang) else "gcc", "-E", "-P", "-I", os.path.join(ROOT, "include"), os.path.join(ROOT, "include", header)],
                           check=True, capture_output=True, text=True).stdout
     return set(re.findall(r"\b(skl_\w+)\s*\(", text))
 

@@ -27,9 +27,9 @@ pytestmark = pytest.mark.gpu
 def check(gpu, kind, case, seed, mode):
     a, b, c = case.make_inputs(seed)
     got = run_gemm(gpu, kind, case, a, b, c, mode)
-    if case.is_int:
+    if case.is_int or case.ta == "f16h":  # the half-accumulating GEMM is defined operation by operation
         want = run_oracle_gemm(case, a, b, c)
-        assert np.array_equal(got, want), (kind, vars(case))
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (kind, vars(case))
     else:
         fp8 = case.ta.startswith("f8")
         support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=support.FP8_MFMA_REL if fp8 else 0.0)
@@ -86,7 +86,7 @@ def test_general_strides(gpu, kind):
     """Column-major B and C, gapped strides, blocked layouts with k0 > 1: the
     layouts only the full-stride forms can express."""
     rng = np.random.default_rng(77)
-    for ta in ("i8", "bf16", "f16", "f8e4m3", "f8e5m2", "f32", "f64"):
+    for ta in ("i8", "bf16", "f16", "f8e4m3", "f8e5m2", "f32", "f64", "f16h"):
         m, n, k = 37, 29, 53
         if kind == "rc":
             case = support.GemmCase(ta, None, 2, 3, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0,
@@ -138,7 +138,8 @@ def test_f32_f64_bit_identical_to_the_checker(gpu):
 
 
 @pytest.mark.parametrize("ta,m,n,k", (("bf16", 130, 200, 64), ("f8e4m3", 256, 256, 128), ("f16", 512, 2048 + 128, 256),
-                                       ("f32", 33, 47, 17), ("f64", 20, 31, 9), ("bf16", 1, 4096, 512)))
+                                       ("f32", 33, 47, 17), ("f64", 20, 31, 9), ("f16h", 21, 30, 19),
+                                       ("bf16", 1, 4096, 512)))
 def test_beta_zero_initialises_c(gpu, ta, m, n, k):
     """beta == 0 is the initialising call. The old C then contributes nothing but the sign of an exact
     zero (beta*c is a signed zero, and it only shows when alpha*acc is a zero too), so the result must
@@ -170,7 +171,7 @@ def test_beta_zero_initialises_c(gpu, ta, m, n, k):
             assert np.all(np.isfinite(again)), (ta, mode, alpha)
             if m > 1:  # the M = 1 path sums with floating-point atomics: not the same bits from run to run
                 assert np.array_equal(got.view(np.uint8), again.view(np.uint8)), (ta, mode, alpha)
-            if ta in ("f32", "f64"):
+            if ta in ("f32", "f64", "f16h"):
                 assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (ta, mode, alpha)
 
 

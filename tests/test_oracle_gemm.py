@@ -123,6 +123,7 @@ FP_SUITES = {
     "f32": ("test/gemm/rvv/skl_gemm_f32_f32_f32_zve32f_x390.c", "test/gemm/xsfmm/skl_gemm_f32c_f32_f32_xsfmm32a32f.c",
             "test/gemm/xsfmm/skl_gemm_f32rcptex1c_f32rcp1xte_f32rcptexterc_xsfmm32a32f.c"),
     "f64": ("test/gemm/rvv/skl_gemm_f64_f64_f64_zve64d_x390.c", None, None),
+    "f16h": ("test/gemm/rvv/skl_gemm_f16_f16_f16_zvfh_x390.c", None, None),  # f16 accumulator and C
 }
 
 
@@ -143,7 +144,8 @@ def test_fp_within_reference_bound_and_equal_to_reference(ta):
     for idx, case in enumerate(fp_cases(ta)):
         a, b, c = case.make_inputs(500 + idx)
         got = run_oracle_gemm(case, a, b, c)
-        support.assert_fp_gemm_close(case, a, b, c, got)
+        # (the 1e-3 Frobenius target is stated for fp32 accumulation; a half accumulator has the bound only)
+        support.assert_fp_gemm_close(case, a, b, c, got, frob_tol=None if ta == "f16h" else 1e-3)
         if ref() is not None:
             want = ref_gemm(case, a, b, c)
             assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), vars(case)
@@ -156,6 +158,8 @@ def test_fp_exactly_summable_inputs(ta):
     rng = np.random.default_rng(21)
     m, n, k = 17, 19, 40
     vals = np.array([-2.0, -1.0, -0.5, 0.0, 0.5, 1.0, 2.0, 4.0])
+    if ta == "f16h":  # partial sums must be exact in half precision too
+        vals = np.array([-1.0, -0.5, 0.0, 0.5, 1.0, 2.0])
     A = rng.choice(vals, size=(m, k))
     B = rng.choice(vals, size=(k, n))
     C = rng.integers(-8, 9, size=(m, n)).astype(np.float64)
@@ -164,7 +168,7 @@ def test_fp_exactly_summable_inputs(ta):
         x32 = x.astype(np.float32)
         if ta == "bf16":
             return support.f32_to_bf16_bits(x32)
-        if ta == "f16":
+        if ta in ("f16", "f16h"):
             return x32.astype(np.float16).view(np.uint16)
         if ta in ("f32", "f64"):
             return x.astype(support.ETYPES[ta].dtype)
@@ -208,3 +212,25 @@ def test_f64_helper_matches_numpy_and_reference():
         want = C.copy().ravel()
         ref().skl_gemm_f64rc_f64rc_f64rc_ref(m, n, k, 1.25, A.ravel(), k, 1, B.ravel(), n, 1, -0.5, want, n, 1)
         assert np.array_equal(got, want)
+
+
+def test_f32_to_f16_rounding_matches_numpy():
+    """The half rounding the f16 -> f16 GEMM restatement is built on, against numpy's float16
+    conversion (round to nearest even, subnormals, overflow to infinity): random patterns plus every
+    pattern around the zero / subnormal, subnormal / normal and overflow thresholds."""
+    import ctypes
+    f = oracle().cdll.skl_oracle_f32_to_f16
+    f.argtypes, f.restype = [ctypes.c_float], ctypes.c_uint16
+    rng = np.random.default_rng(5)
+    bits = np.concatenate([rng.integers(0, 1 << 32, 60000, dtype=np.uint64).astype(np.uint32),
+                           np.arange(0x33000000 - 64, 0x33000000 + 64, dtype=np.uint32),
+                           np.arange(0x38800000 - 9000, 0x38800000 + 9000, dtype=np.uint32),
+                           np.arange(0x477FE000 - 9000, 0x477FE000 + 9000, dtype=np.uint32),
+                           np.arange(0x3F800000, 0x3F800000 + 20000, dtype=np.uint32)])
+    bits = np.concatenate([bits, bits | np.uint32(0x80000000)])
+    x = bits.view(np.float32)
+    x = x[~np.isnan(x)]
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    got = np.fromiter((f(float(v)) for v in x), dtype=np.uint16, count=x.size)
+    assert np.array_equal(got, want)
