@@ -115,6 +115,48 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, 
 #endif
 
 /* ======================================================================== */
+/* GEMM with a fused epilogue                                                */
+/* ======================================================================== */
+
+/* What the reference's per-tile fused kernels compute on the matrix engine's tile state
+ * (src/gemm/fused-kernel-API.md:85-216: alpha/beta scaling :104-125, adding a bias :159-178, a global
+ * maximum :186-207), applied here to the accumulators in registers before C is written - the fusion
+ * src/gemm/README.md:141-146 tells users to approximate by tiling the output. The reference keeps its
+ * fused kernels private (SKL_FUNC_PRIVATE), so these entry points have no public prototype to mirror;
+ * they take the argument list of the rc / rcprc form plus the descriptor.
+ * For every addressed element (i, j), j the logical column:
+ *     v = beta*C(i,j) + alpha*(A*B)(i,j)        as in the plain GEMM, beta == 0 included
+ *     v = v + bias[j]                            if bias != NULL (one rounded addition; int32 wraps)
+ *     C(i,j) = v
+ *     *max = v  if v > *max                      if max != NULL (a NaN never replaces the maximum;
+ *                                                the sign of a zero maximum is unspecified)
+ * bias points to n = n1*n0 values of C's type, max to one; both must be memory of the same kind as C
+ * (device or host), must not overlap C, and *max must not be NaN on entry. ep == NULL: the plain GEMM. */
+typedef struct skl_gfx950_epilogue {
+  const void *bias;
+  void *max;
+} skl_gfx950_epilogue_t;
+
+#define SKL_GFX950_DECLARE_FUSED_RC(NAME, TA, TC)                                                    \
+  void NAME(size_t m, size_t n, size_t k, TC alpha, const TA *a, size_t rsa, size_t csa, const TA *b, \
+            size_t rsb, size_t csb, TC beta, TC *c, size_t rsc, size_t csc, const skl_gfx950_epilogue_t *ep)
+#define SKL_GFX950_DECLARE_FUSED_RCPRC(NAME, TA, TC)                                                 \
+  void NAME(size_t m0, size_t n0, size_t k0, size_t m1, size_t n1, size_t k1, TC alpha, const TA *a, \
+            size_t rsa0, size_t csa0, size_t rsa1, size_t csa1, const TA *b, size_t rsb0,            \
+            size_t csb0, size_t rsb1, size_t csb1, TC beta, TC *c, size_t rsc0, size_t csc0,         \
+            size_t rsc1, size_t csc1, const skl_gfx950_epilogue_t *ep)
+SKL_GFX950_DECLARE_FUSED_RC(skl_gemm_fused_i8rc_i8rc_i32rc_gfx950, int8_t, int32_t);
+SKL_GFX950_DECLARE_FUSED_RC(skl_gemm_fused_bf16rc_bf16rc_f32rc_gfx950, skl_bf16_t, float);
+SKL_GFX950_DECLARE_FUSED_RC(skl_gemm_fused_f16rc_f16rc_f32rc_gfx950, skl_f16_t, float);
+SKL_GFX950_DECLARE_FUSED_RC(skl_gemm_fused_f8e4m3rc_f8e4m3rc_f32rc_gfx950, uint8_t, float);
+SKL_GFX950_DECLARE_FUSED_RC(skl_gemm_fused_f8e5m2rc_f8e5m2rc_f32rc_gfx950, uint8_t, float);
+SKL_GFX950_DECLARE_FUSED_RCPRC(skl_gemm_fused_i8rcprc_i8rcprc_i32rcprc_gfx950, int8_t, int32_t);
+SKL_GFX950_DECLARE_FUSED_RCPRC(skl_gemm_fused_bf16rcprc_bf16rcprc_f32rcprc_gfx950, skl_bf16_t, float);
+SKL_GFX950_DECLARE_FUSED_RCPRC(skl_gemm_fused_f16rcprc_f16rcprc_f32rcprc_gfx950, skl_f16_t, float);
+SKL_GFX950_DECLARE_FUSED_RCPRC(skl_gemm_fused_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950, uint8_t, float);
+SKL_GFX950_DECLARE_FUSED_RCPRC(skl_gemm_fused_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, float);
+
+/* ======================================================================== */
 /* GEMM - the optimized entry points of skl.h                                */
 /* ======================================================================== */
 

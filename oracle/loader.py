@@ -90,6 +90,9 @@ def load_oracle():
         setattr(f, name, _wrap(signatures.bind(cdll, name, sig), sig))
     for name, (restype, sig) in _EXTRA_ORACLE.items():
         setattr(f, name, _wrap(signatures.bind(cdll, name, sig, restype), sig))
+    for stem, sig in signatures.GEMM_FUSED.items():  # bias and max follow as two pointers
+        name, sig = stem + "_oracle", sig + "pp"
+        setattr(f, name, _wrap(signatures.bind(cdll, name, sig), sig))
     return f
 
 

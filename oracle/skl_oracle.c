@@ -410,6 +410,57 @@ void skl_gemm_f16rcprc_f16rcprc_f16rcprc_oracle(size_t m0, size_t n0, size_t k0,
         }
 }
 
+/*
+ * GEMM with the fused steps of the reference's per-tile fused kernels behind the alpha/beta step
+ * (src/gemm/fused-kernel-API.md:159-178, "adding a bias": c_block[i,j] = tile[i,j] + bias_block[j], the bias
+ * indexed by the logical column; :186-207, "computing a global maximum": if (tile[i,j] > *max) *max = tile[i,j],
+ * the tile value being what is written to C). Every element is independent, so running the plain GEMM first
+ * and the two steps over C afterwards computes what a fused kernel computes.
+ */
+#define FUSED_RC(NAME, TA, TC)                                                                     \
+  void skl_gemm_fused_##NAME##_oracle(size_t m, size_t n, size_t k, TC alpha, const TA *a, size_t rsa, \
+                                      size_t csa, const TA *b, size_t rsb, size_t csb, TC beta, TC *c, \
+                                      size_t rsc, size_t csc, const TC *bias, TC *max) {            \
+    skl_gemm_##NAME##_oracle(m, n, k, alpha, a, rsa, csa, b, rsb, csb, beta, c, rsc, csc);          \
+    for (size_t i = 0; i < m; ++i)                                                                  \
+      for (size_t j = 0; j < n; ++j) {                                                              \
+        TC *out = c + i * rsc + j * csc;                                                            \
+        TC v = *out;                                                                                \
+        if (bias) v = v + bias[j];                                                                  \
+        *out = v;                                                                                   \
+        if (max && v > *max) *max = v;                                                              \
+      }                                                                                             \
+  }
+#define FUSED_RCPRC(NAME, TA, TC)                                                                  \
+  void skl_gemm_fused_##NAME##_oracle(size_t m0, size_t n0, size_t k0, size_t m1, size_t n1, size_t k1, \
+                                      TC alpha, const TA *a, size_t rsa0, size_t csa0, size_t rsa1, \
+                                      size_t csa1, const TA *b, size_t rsb0, size_t csb0, size_t rsb1, \
+                                      size_t csb1, TC beta, TC *c, size_t rsc0, size_t csc0, size_t rsc1, \
+                                      size_t csc1, const TC *bias, TC *max) {                       \
+    skl_gemm_##NAME##_oracle(m0, n0, k0, m1, n1, k1, alpha, a, rsa0, csa0, rsa1, csa1, b, rsb0, csb0, rsb1, \
+                             csb1, beta, c, rsc0, csc0, rsc1, csc1);                                \
+    for (size_t I = 0; I < m1; ++I)                                                                 \
+      for (size_t J = 0; J < n1; ++J)                                                               \
+        for (size_t i = 0; i < m0; ++i)                                                             \
+          for (size_t j = 0; j < n0; ++j) {                                                         \
+            TC *out = c + I * rsc1 + J * csc1 + i * rsc0 + j * csc0;                                \
+            TC v = *out;                                                                            \
+            if (bias) v = v + bias[J * n0 + j];                                                     \
+            *out = v;                                                                               \
+            if (max && v > *max) *max = v;                                                          \
+          }                                                                                         \
+  }
+FUSED_RC(i8rc_i8rc_i32rc, int8_t, int32_t)
+FUSED_RC(bf16rc_bf16rc_f32rc, uint16_t, float)
+FUSED_RC(f16rc_f16rc_f32rc, uint16_t, float)
+FUSED_RC(f8e4m3rc_f8e4m3rc_f32rc, uint8_t, float)
+FUSED_RC(f8e5m2rc_f8e5m2rc_f32rc, uint8_t, float)
+FUSED_RCPRC(i8rcprc_i8rcprc_i32rcprc, int8_t, int32_t)
+FUSED_RCPRC(bf16rcprc_bf16rcprc_f32rcprc, uint16_t, float)
+FUSED_RCPRC(f16rcprc_f16rcprc_f32rcprc, uint16_t, float)
+FUSED_RCPRC(f8e4m3rcprc_f8e4m3rcprc_f32rcprc, uint8_t, float)
+FUSED_RCPRC(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, float)
+
 /* ======================================================================== */
 /* Widening helpers                                                          */
 /* ======================================================================== */

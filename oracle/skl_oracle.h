@@ -106,6 +106,28 @@ void skl_gemm_f16rcprc_f16rcprc_f16rcprc_oracle(size_t m0, size_t n0, size_t k0,
                                                 size_t csb0, size_t rsb1, size_t csb1, float beta, uint16_t *c,
                                                 size_t rsc0, size_t csc0, size_t rsc1, size_t csc1);
 
+/* GEMM + fused bias / maximum steps (src/gemm/fused-kernel-API.md:159-207); bias and max may be NULL. */
+#define SKL_ORACLE_FUSED_DECL(NAME, TA, TC)                                                        \
+  void skl_gemm_fused_##NAME##_oracle(size_t m, size_t n, size_t k, TC alpha, const TA *a, size_t rsa, \
+                                      size_t csa, const TA *b, size_t rsb, size_t csb, TC beta, TC *c, \
+                                      size_t rsc, size_t csc, const TC *bias, TC *max);
+#define SKL_ORACLE_PFUSED_DECL(NAME, TA, TC)                                                       \
+  void skl_gemm_fused_##NAME##_oracle(size_t m0, size_t n0, size_t k0, size_t m1, size_t n1, size_t k1, \
+                                      TC alpha, const TA *a, size_t rsa0, size_t csa0, size_t rsa1, \
+                                      size_t csa1, const TA *b, size_t rsb0, size_t csb0, size_t rsb1, \
+                                      size_t csb1, TC beta, TC *c, size_t rsc0, size_t csc0, size_t rsc1, \
+                                      size_t csc1, const TC *bias, TC *max);
+SKL_ORACLE_FUSED_DECL(i8rc_i8rc_i32rc, int8_t, int32_t)
+SKL_ORACLE_FUSED_DECL(bf16rc_bf16rc_f32rc, uint16_t, float)
+SKL_ORACLE_FUSED_DECL(f16rc_f16rc_f32rc, uint16_t, float)
+SKL_ORACLE_FUSED_DECL(f8e4m3rc_f8e4m3rc_f32rc, uint8_t, float)
+SKL_ORACLE_FUSED_DECL(f8e5m2rc_f8e5m2rc_f32rc, uint8_t, float)
+SKL_ORACLE_PFUSED_DECL(i8rcprc_i8rcprc_i32rcprc, int8_t, int32_t)
+SKL_ORACLE_PFUSED_DECL(bf16rcprc_bf16rcprc_f32rcprc, uint16_t, float)
+SKL_ORACLE_PFUSED_DECL(f16rcprc_f16rcprc_f32rcprc, uint16_t, float)
+SKL_ORACLE_PFUSED_DECL(f8e4m3rcprc_f8e4m3rcprc_f32rcprc, uint8_t, float)
+SKL_ORACLE_PFUSED_DECL(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, float)
+
 /* Widening helpers used to build fp64 comparison operands on the host. */
 void skl_oracle_widen_bf16_f64(double *dst, const uint16_t *src, size_t n);
 void skl_oracle_widen_f16_f64(double *dst, const uint16_t *src, size_t n);

@@ -7,4 +7,4 @@ may be numpy arrays (ordinary host memory: the library stages them) or
 :class:`DeviceBuffer` objects (device memory: asynchronous launch). There is no
 CPU fallback: if the library is not built, importing the entry points fails.
 """
-from .binding import (DeviceBuffer, LibraryNotBuilt, check_error, lib, library_path, load)  # noqa: F401
+from .binding import (DeviceBuffer, Epilogue, LibraryNotBuilt, check_error, lib, library_path, load)  # noqa: F401

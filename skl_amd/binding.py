@@ -50,8 +50,20 @@ def _as_pointer(x):
     return x  # integer address
 
 
+class Epilogue:
+    """Fused-epilogue operands of the `skl_gemm_fused_*` entry points: `bias` (n values of C's
+    type) and `max` (one value of C's type), each a DeviceBuffer, a numpy array or None."""
+
+    def __init__(self, bias=None, max=None):
+        self.bias, self.max = bias, max
+
+    def as_struct(self):
+        return signatures.EpilogueStruct(_as_pointer(self.bias), _as_pointer(self.max))
+
+
 def _wrap(raw, sig):
     ptr_positions = [i for i, ch in enumerate(sig) if ch == "p"]
+    epilogue_positions = [i for i, ch in enumerate(sig) if ch == "E"]
 
     def call(*args):
         if len(args) != len(sig):
@@ -59,6 +71,11 @@ def _wrap(raw, sig):
         args = list(args)
         for i in ptr_positions:
             args[i] = _as_pointer(args[i])
+        keep = []  # descriptors stay alive until the call returns
+        for i in epilogue_positions:
+            if args[i] is not None:
+                keep.append(args[i].as_struct())
+                args[i] = ctypes.addressof(keep[-1])
         return raw(*args)
 
     call.__name__ = raw.__name__

@@ -117,6 +117,8 @@ static int canonicalize(const skl_gemm_desc *d, skl_gemm_canon *g) {
   g->c = d->c;
   g->alpha = d->alpha;
   g->beta = d->beta;
+  g->bias = d->bias;
+  g->max = d->max;
   if (!flat_k(d->k0, d->k1, d->csa0, d->csa1, &g->a_sk)) return 0;
   if (!flat_k(d->k0, d->k1, d->rsb0, d->rsb1, &g->b_sk)) return 0;
   if (!block64(d->m0, d->m1, d->rsa0, d->rsa1, &g->a_s0, &g->a_s1)) return 0;
@@ -150,13 +152,14 @@ static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g) {
 
 static void gemm_on_device(const skl_gemm_desc *d) {
   skl_gemm_canon g;
+  const int fused = d->bias != NULL || d->max != NULL; /* the M = 1 kernels have no fused steps */
   if (d->k0 * d->k1 != 0 && d->ta <= SKL_DT_F8E5M2) {
-    if (canonicalize_k4(d, &g) && skl_hip_gemv_supported(&g, 1)) {
+    if (!fused && canonicalize_k4(d, &g) && skl_hip_gemv_supported(&g, 1)) {
       skl_hip_launch_gemv(&g, 1);
       return;
     }
     if (canonicalize(d, &g)) {
-      if (g.m == 1 && skl_hip_gemv_supported(&g, 0)) {
+      if (!fused && g.m == 1 && skl_hip_gemv_supported(&g, 0)) {
         skl_hip_launch_gemv(&g, 0);
         return;
       }
@@ -175,6 +178,14 @@ static void gemm_run(const skl_gemm_desc *d, const char *who) {
   if (M == 0 || N == 0) return; /* nothing is addressed */
   where = classify(K ? d->a : NULL, K ? d->b : NULL, d->c, who);
   if (where < 0) return;
+  if (d->bias || d->max) { /* the fused operands must be of the same kind as C */
+    const int extra = classify(d->bias, d->max, NULL, who);
+    if (extra < 0) return;
+    if (extra != where) {
+      skl_hip_record_error(SKL_HIP_ERR_MIXED_POINTERS, who);
+      return;
+    }
+  }
   if (where == 1) {
     gemm_on_device(d);
     return;
@@ -187,21 +198,30 @@ static void gemm_run(const skl_gemm_desc *d, const char *who) {
     const size_t nb = K ? span4(d->k1, d->rsb1, d->n1, d->csb1, d->k0, d->rsb0, d->n0, d->csb0) : 0;
     const size_t nc = span4(d->m1, d->rsc1, d->n1, d->csc1, d->m0, d->rsc0, d->n0, d->csc0);
     skl_gemm_desc dd = *d;
-    void *da = stage_in(d->a, na * esa), *db = stage_in(d->b, nb * esb), *dc = stage_in(d->c, nc * c_elem_size(d->ta));
-    if ((na && !da) || (nb && !db) || !dc) {
+    const size_t esc = c_elem_size(d->ta);
+    void *da = stage_in(d->a, na * esa), *db = stage_in(d->b, nb * esb), *dc = stage_in(d->c, nc * esc);
+    void *dbias = d->bias ? stage_in(d->bias, N * esc) : NULL, *dmax = d->max ? stage_in(d->max, esc) : NULL;
+    if ((na && !da) || (nb && !db) || !dc || (d->bias && !dbias) || (d->max && !dmax)) {
       skl_hip_free(da);
       skl_hip_free(db);
       skl_hip_free(dc);
+      skl_hip_free(dbias);
+      skl_hip_free(dmax);
       return;
     }
     dd.a = da;
     dd.b = db;
     dd.c = dc;
+    dd.bias = dbias;
+    dd.max = dmax;
     gemm_on_device(&dd);
-    skl_hip_memcpy_d2h(d->c, dc, nc * c_elem_size(d->ta));
+    skl_hip_memcpy_d2h(d->c, dc, nc * esc);
+    if (dmax) skl_hip_memcpy_d2h(d->max, dmax, esc);
     skl_hip_free(da);
     skl_hip_free(db);
     skl_hip_free(dc);
+    skl_hip_free(dbias);
+    skl_hip_free(dmax);
   }
 }
 
@@ -214,7 +234,8 @@ static void gemm_run(const skl_gemm_desc *d, const char *who) {
   void NAME(size_t m, size_t n, size_t k, TC_T alpha, const TA_T *a, size_t rsa, size_t csa,       \
             const TA_T *b, size_t rsb, size_t csb, TC_T beta, TC_T *c, size_t rsc, size_t csc) {   \
     skl_gemm_desc d = {DTA, DTB, 1,   1,   1,   m,    n,    k,   a,    0, 0, rsa, csa,             \
-                       b,   0,   0,   rsb, csb, c,    0,    0,   rsc,  csc, {SC(alpha)}, {SC(beta)}}; \
+                       b,   0,   0,   rsb, csb, c,    0,    0,   rsc,  csc, {SC(alpha)}, {SC(beta)}, \
+                       NULL, NULL};                                                                \
     gemm_run(&d, #NAME);                                                                           \
   }
 
@@ -237,7 +258,7 @@ DEFINE_GEMM_RC(skl_gemm_f16rc_f16rc_f16rc_gfx950, skl_f16_t, skl_f16_t, SKL_DT_F
             size_t csc0, size_t rsc1, size_t csc1) {                                               \
     skl_gemm_desc d = {DT,   DT,   m0,   n0,   k0,   m1,   n1,   k1,   a,    rsa0, csa0, rsa1, csa1, \
                        b,    rsb0, csb0, rsb1, csb1, c,    rsc0, csc0, rsc1, csc1, {SC(alpha)},    \
-                       {SC(beta)}};                                                                \
+                       {SC(beta)}, NULL, NULL};                                                    \
     gemm_run(&d, #NAME);                                                                           \
   }
 
@@ -249,6 +270,37 @@ DEFINE_GEMM_RCPRC(skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, flo
 DEFINE_GEMM_RCPRC(skl_gemm_f32rcprc_f32rcprc_f32rcprc_gfx950, float, float, SKL_DT_F32, SCALAR_f32)
 DEFINE_GEMM_RCPRC(skl_gemm_f64rcprc_f64rcprc_f64rcprc_gfx950, double, double, SKL_DT_F64, SCALAR_f64)
 DEFINE_GEMM_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, skl_f16_t, SKL_DT_F16H, SCALAR_f32)
+
+/* The same two forms with the fused steps of `ep` behind the alpha/beta step; ep == NULL is the plain GEMM. */
+#define DEFINE_GEMM_FUSED_RC(NAME, TA_T, TC_T, DT, SC)                                             \
+  void NAME(size_t m, size_t n, size_t k, TC_T alpha, const TA_T *a, size_t rsa, size_t csa,       \
+            const TA_T *b, size_t rsb, size_t csb, TC_T beta, TC_T *c, size_t rsc, size_t csc,     \
+            const skl_gfx950_epilogue_t *ep) {                                                     \
+    skl_gemm_desc d = {DT,  DT,  1,   1,   1,   m,    n,    k,   a,    0, 0, rsa, csa,             \
+                       b,   0,   0,   rsb, csb, c,    0,    0,   rsc,  csc, {SC(alpha)}, {SC(beta)}, \
+                       ep ? ep->bias : NULL, ep ? ep->max : NULL};                                 \
+    gemm_run(&d, #NAME);                                                                           \
+  }
+#define DEFINE_GEMM_FUSED_RCPRC(NAME, TA_T, TC_T, DT, SC)                                          \
+  void NAME(size_t m0, size_t n0, size_t k0, size_t m1, size_t n1, size_t k1, TC_T alpha,          \
+            const TA_T *a, size_t rsa0, size_t csa0, size_t rsa1, size_t csa1, const TA_T *b,      \
+            size_t rsb0, size_t csb0, size_t rsb1, size_t csb1, TC_T beta, TC_T *c, size_t rsc0,   \
+            size_t csc0, size_t rsc1, size_t csc1, const skl_gfx950_epilogue_t *ep) {              \
+    skl_gemm_desc d = {DT,   DT,   m0,   n0,   k0,   m1,   n1,   k1,   a,    rsa0, csa0, rsa1, csa1, \
+                       b,    rsb0, csb0, rsb1, csb1, c,    rsc0, csc0, rsc1, csc1, {SC(alpha)},    \
+                       {SC(beta)}, ep ? ep->bias : NULL, ep ? ep->max : NULL};                     \
+    gemm_run(&d, #NAME);                                                                           \
+  }
+DEFINE_GEMM_FUSED_RC(skl_gemm_fused_i8rc_i8rc_i32rc_gfx950, int8_t, int32_t, SKL_DT_I8, SCALAR_i32)
+DEFINE_GEMM_FUSED_RC(skl_gemm_fused_bf16rc_bf16rc_f32rc_gfx950, skl_bf16_t, float, SKL_DT_BF16, SCALAR_f32)
+DEFINE_GEMM_FUSED_RC(skl_gemm_fused_f16rc_f16rc_f32rc_gfx950, skl_f16_t, float, SKL_DT_F16, SCALAR_f32)
+DEFINE_GEMM_FUSED_RC(skl_gemm_fused_f8e4m3rc_f8e4m3rc_f32rc_gfx950, uint8_t, float, SKL_DT_F8E4M3, SCALAR_f32)
+DEFINE_GEMM_FUSED_RC(skl_gemm_fused_f8e5m2rc_f8e5m2rc_f32rc_gfx950, uint8_t, float, SKL_DT_F8E5M2, SCALAR_f32)
+DEFINE_GEMM_FUSED_RCPRC(skl_gemm_fused_i8rcprc_i8rcprc_i32rcprc_gfx950, int8_t, int32_t, SKL_DT_I8, SCALAR_i32)
+DEFINE_GEMM_FUSED_RCPRC(skl_gemm_fused_bf16rcprc_bf16rcprc_f32rcprc_gfx950, skl_bf16_t, float, SKL_DT_BF16, SCALAR_f32)
+DEFINE_GEMM_FUSED_RCPRC(skl_gemm_fused_f16rcprc_f16rcprc_f32rcprc_gfx950, skl_f16_t, float, SKL_DT_F16, SCALAR_f32)
+DEFINE_GEMM_FUSED_RCPRC(skl_gemm_fused_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950, uint8_t, float, SKL_DT_F8E4M3, SCALAR_f32)
+DEFINE_GEMM_FUSED_RCPRC(skl_gemm_fused_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950, uint8_t, float, SKL_DT_F8E5M2, SCALAR_f32)
 
 /* row-major A, B, C: the rc form with csa = csb = csc = 1
  * (src/gemm/gemm_i8_i8_i32_zve32x.h:38-48) */

@@ -70,3 +70,38 @@ template <typename T>
 __device__ __forceinline__ void skl_update(T acc, T *c, skl_scalar alpha, skl_scalar beta) {
   *c = skl_beta_is_zero<T>(beta) ? skl_initialise(acc, c, alpha, beta) : skl_combine(acc, *c, alpha, beta);
 }
+
+// ---------------------------------------------------------------------------
+// Fused epilogue steps after the alpha/beta step (the GPU form of the reference's per-tile fused
+// kernels, src/gemm/fused-kernel-API.md:159-178 "adding a bias", :186-207 "computing a global maximum").
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ int skl_add_bias(int v, int b) { return (int)((unsigned)v + (unsigned)b); }
+__device__ __forceinline__ float skl_add_bias(float v, float b) { return __fadd_rn(v, b); }
+
+template <typename T>
+__device__ __forceinline__ T skl_lowest();
+template <>
+__device__ __forceinline__ int skl_lowest<int>() { return (int)0x80000000; }
+template <>
+__device__ __forceinline__ float skl_lowest<float>() { return -__builtin_inff(); }
+
+// Largest value over the 64 lanes of a wave (all lanes must take part); NaN never wins, as in `if (x > max)`.
+template <typename T>
+__device__ __forceinline__ T skl_wave_max(T v) {
+#pragma unroll
+  for (int step = 32; step > 0; step >>= 1) {
+    const T other = __shfl_xor(v, step, 64);
+    if (other > v) v = other;
+  }
+  return v;
+}
+
+// *p = max(*p, v) for a v that is not NaN. Floats order like sign-magnitude integers: non-negative ones
+// ascend as signed ints, negative ones descend as unsigned ints, so one integer atomic does it.
+__device__ __forceinline__ void skl_atomic_max(int *p, int v) { atomicMax(p, v); }
+__device__ __forceinline__ void skl_atomic_max(float *p, float v) {
+  if (!(v < 0.0f) && !__builtin_signbit(v))
+    atomicMax(reinterpret_cast<int *>(p), __float_as_int(v));
+  else
+    atomicMin(reinterpret_cast<unsigned *>(p), __float_as_uint(v));
+}

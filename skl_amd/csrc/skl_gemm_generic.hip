@@ -17,6 +17,8 @@
 // source spells it.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "skl_device.hpp"
 #include "skl_fp8.hpp"
 
@@ -119,6 +121,16 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(skl_gemm_desc d, unsi
     *c = (_Float16)wide;
   } else {
     skl_update(acc, c, d.alpha, d.beta);
+    if constexpr (std::is_same<Acc, int32_t>::value || std::is_same<Acc, float>::value) {
+      if (d.bias || d.max) {  // fused steps behind the alpha/beta step
+        Acc v = *c;
+        if (d.bias) {
+          v = skl_add_bias(v, reinterpret_cast<const Acc *>(d.bias)[j]);
+          *c = v;
+        }
+        if (d.max && v > skl_lowest<Acc>()) skl_atomic_max(reinterpret_cast<Acc *>(d.max), v);
+      }
+    }
   }
 }
 

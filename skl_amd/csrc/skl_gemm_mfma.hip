@@ -59,7 +59,33 @@ struct MfmaArgs {
   size_t b_s1, b_s0, b_sk;
   size_t rsc0, csc0, rsc1, csc1;
   skl_scalar alpha, beta;
+  const char *bias;  // fused epilogue: per-column addend and running maximum of C's type, or null
+  char *max;
   unsigned tiles_m, tiles_n;
+};
+
+// The fused steps behind the alpha/beta step, for one lane: bias of the lane's column, running maximum.
+template <typename T>
+struct FusedSteps {
+  const T *bias;
+  T *max;
+  T bias_j, running;
+  __device__ explicit FusedSteps(const MfmaArgs &p)
+      : bias(reinterpret_cast<const T *>(p.bias)), max(reinterpret_cast<T *>(p.max)), bias_j(0), running(skl_lowest<T>()) {}
+  __device__ __forceinline__ void column(size_t col) {
+    if (bias) bias_j = bias[col];
+  }
+  __device__ __forceinline__ T apply(T v) {
+    if (bias) v = skl_add_bias(v, bias_j);
+    if (max && v > running) running = v;
+    return v;
+  }
+  // Every lane of the wave calls this once, after its last element.
+  __device__ __forceinline__ void finish() {
+    if (!max) return;
+    const T best = skl_wave_max(running);
+    if ((threadIdx.x & 63) == 0 && best > skl_lowest<T>()) skl_atomic_max(max, best);
+  }
 };
 
 // Operand kinds of the MFMA: element size, accumulator type, k per instruction.
@@ -401,10 +427,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
   // element). C is written once and not read again: non-temporal stores keep it out of the operands' caches.
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
   const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
+  FusedSteps<AccElem> fused(p);
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
     if (GUARDED && col >= p.n) continue;
+    fused.column(col);
     const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
 #pragma unroll
     for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
@@ -426,7 +454,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
           for (int r = 0; r < 16; ++r)
             if (in_range(i, r)) {
               AccElem *dst = out[i][r >> 2] + (r & 3) * p.rsc0;
-              __builtin_nontemporal_store(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst);
+              __builtin_nontemporal_store(fused.apply(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta)), dst);
             }
       } else {
         AccElem old[kEpilogueBatch][16];
@@ -439,10 +467,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
 #pragma unroll
           for (int r = 0; r < 16; ++r)
             if (in_range(i, r))
-              __builtin_nontemporal_store(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][r >> 2] + (r & 3) * p.rsc0);
+              __builtin_nontemporal_store(fused.apply(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta)), out[i][r >> 2] + (r & 3) * p.rsc0);
       }
     }
   }
+  fused.finish();
 }
 
 // ===========================================================================
@@ -870,9 +899,11 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   // Epilogue, as in the kernel above: old values requested kEpilogueBatch blocks at a time, non-temporal stores.
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
   const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
+  FusedSteps<AccElem> fused(p);
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
+    fused.column(col);
     const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
 #pragma unroll
     for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
@@ -890,7 +921,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             AccElem *dst = out[i][r >> 2] + (r & 3) * p.rsc0;
-            __builtin_nontemporal_store(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst);
+            __builtin_nontemporal_store(fused.apply(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta)), dst);
           }
       } else {
         AccElem old[kEpilogueBatch][16];
@@ -902,10 +933,11 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
         for (int i = 0; i < kEpilogueBatch; ++i)
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            __builtin_nontemporal_store(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][r >> 2] + (r & 3) * p.rsc0);
+            __builtin_nontemporal_store(fused.apply(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta)), out[i][r >> 2] + (r & 3) * p.rsc0);
       }
     }
   }
+  fused.finish();
 }
 
 template <int TA, int TB, bool A_KC, bool B_KC, int BN>
@@ -977,6 +1009,7 @@ int launch_tile(const MfmaArgs &p) {
         tail.n = tail_cols;
         tail.b = p.b + (head_cols / 64) * p.b_s1 * ES;
         tail.c = p.c + (head_cols / 64) * p.csc1 * sizeof(float);  // C elements are 4 bytes for every kind
+        if (p.bias) tail.bias = p.bias + head_cols * sizeof(float);
         const int rc = launch_ring<TA, TB, A_KC, B_KC, 256>(head);
         return rc != 0 ? rc : launch_ring<TA, TB, A_KC, B_KC, 128>(tail);
       }
@@ -1044,6 +1077,7 @@ extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
   p.b_s1 = g->b_s1, p.b_s0 = g->b_s0, p.b_sk = g->b_sk;
   p.rsc0 = g->rsc0, p.csc0 = g->csc0, p.rsc1 = g->rsc1, p.csc1 = g->csc1;
   p.alpha = g->alpha, p.beta = g->beta;
+  p.bias = (const char *)g->bias, p.max = (char *)g->max;
   p.tiles_m = p.tiles_n = 0;
   switch (g->ta * 8 + g->tb) {
     case SKL_DT_I8 * 8 + SKL_DT_I8: return launch_layout<SKL_DT_I8, SKL_DT_I8>(p);

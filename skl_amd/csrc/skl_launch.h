@@ -50,6 +50,10 @@ typedef struct {
   void *c;
   size_t rsc0, csc0, rsc1, csc1;
   skl_scalar alpha, beta;
+  /* Fused epilogue (both may be NULL): bias[j] of C's type is added to every element of logical column j after
+   * the alpha/beta step; *max of C's type is raised to the largest element written. */
+  const void *bias;
+  void *max;
 } skl_gemm_desc;
 
 /* Canonical form served by the matrix-core kernels: flat in K, blocked by 64
@@ -66,6 +70,8 @@ typedef struct {
   void *c;
   size_t rsc0, csc0, rsc1, csc1;
   skl_scalar alpha, beta;
+  const void *bias; /* as in skl_gemm_desc */
+  void *max;
 } skl_gemm_canon;
 
 int skl_hip_launch_gemm_generic(const skl_gemm_desc *d);

@@ -2,7 +2,7 @@
 
 Each character is one C parameter: ``z`` size_t, ``p`` pointer, ``i`` int32_t,
 ``f`` float, ``d`` double, ``b`` uint8_t, ``h`` uint16_t, ``w`` uint32_t,
-``H`` a ``_Float16`` passed by value.
+``H`` a ``_Float16`` passed by value, ``E`` a pointer to a ``skl_gfx950_epilogue_t``.
 Names are given without the implementation suffix (``_gfx950`` for the GPU
 library); the parameter order is the reference's (include/skl-gfx950.h cites
 the prototype each one mirrors).
@@ -35,7 +35,13 @@ CTYPES = {
     "h": ctypes.c_uint16,
     "w": ctypes.c_uint32,
     "H": HalfByValue,
+    "E": ctypes.c_void_p,
 }
+
+
+class EpilogueStruct(ctypes.Structure):
+    """``skl_gfx950_epilogue_t`` (include/skl-gfx950.h)."""
+    _fields_ = [("bias", ctypes.c_void_p), ("max", ctypes.c_void_p)]
 
 
 def _rc(s):      # m n k alpha a rsa csa b rsb csb beta c rsc csc
@@ -101,6 +107,21 @@ GEMM_PANEL = {
     "skl_gemm_f32rcptex1c_f32rcp1xte_f32rcptexterc": "f",
 }
 
+#: GEMMs with a fused epilogue: the rc / rcprc argument list followed by the fused operands
+#: (GPU library: one pointer to the descriptor; CPU checker: bias pointer, max pointer).
+GEMM_FUSED = {
+    "skl_gemm_fused_i8rc_i8rc_i32rc": _rc("i"),
+    "skl_gemm_fused_bf16rc_bf16rc_f32rc": _rc("f"),
+    "skl_gemm_fused_f16rc_f16rc_f32rc": _rc("f"),
+    "skl_gemm_fused_f8e4m3rc_f8e4m3rc_f32rc": _rc("f"),
+    "skl_gemm_fused_f8e5m2rc_f8e5m2rc_f32rc": _rc("f"),
+    "skl_gemm_fused_i8rcprc_i8rcprc_i32rcprc": _rcprc("i"),
+    "skl_gemm_fused_bf16rcprc_bf16rcprc_f32rcprc": _rcprc("f"),
+    "skl_gemm_fused_f16rcprc_f16rcprc_f32rcprc": _rcprc("f"),
+    "skl_gemm_fused_f8e4m3rcprc_f8e4m3rcprc_f32rcprc": _rcprc("f"),
+    "skl_gemm_fused_f8e5m2rcprc_f8e5m2rcprc_f32rcprc": _rcprc("f"),
+}
+
 _PAD = {8: "b", 16: "h", 32: "w"}
 
 
@@ -138,6 +159,8 @@ def gfx950_only():
     for name, s in GEMM_PANEL.items():
         sigs[name] = _panel(s)
     sigs["skl_gemm_i8rcp1x4_i8p4x1c_i32"] = "zzzipzzpzipz"
+    for name, sig in GEMM_FUSED.items():
+        sigs[name] = sig + "E"
     for w, pad in _PAD.items():
         sigs[f"skl_pack_e{w}_e{w}rcptex1c"] = "zzpzpzz" + pad
     return sigs

@@ -62,6 +62,30 @@ def run_gemm(lib, kind, case, a, b, c, mode):
     return out
 
 
+def run_fused_gemm(lib, kind, case, a, b, c, bias, mx, mode):
+    """Runs `skl_gemm_fused_*` (kind "rc" or "rcprc"); returns (C's whole buffer, *max) afterwards.
+    `bias` / `mx` are arrays of C's type (n values / one value) or None."""
+    def call(a_, b_, c_, bias_, mx_):
+        name, args = gemm_entry_args(kind, case, a_, b_, c_)
+        fused = name.replace("skl_gemm_", "skl_gemm_fused_")
+        getattr(lib, fused)(*args, skl_amd.Epilogue(bias_, mx_))
+
+    if mode == "host":
+        out, mo = c.copy(), None if mx is None else mx.copy()
+        call(a, b, out, bias, mo)
+        skl_amd.check_error()
+        return out, mo
+    bufs = [DeviceBuffer.from_array(x) if x is not None else None for x in (a, b, c, bias, mx)]
+    call(*bufs)
+    _finish(lib)
+    out = bufs[2].download(c.dtype, c.size)
+    mo = None if mx is None else bufs[4].download(mx.dtype, mx.size)
+    for d in bufs:
+        if d is not None:
+            d.free()
+    return out, mo
+
+
 def run_inout(lib, name, build_args, src, dst, mode):
     """Runs an entry point with one input and one in/out buffer. `build_args(src, dst)`
     returns the C argument tuple."""

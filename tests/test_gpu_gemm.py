@@ -17,9 +17,9 @@ import pytest
 
 import skl_amd
 import support
-from gpu_support import MODES, run_gemm
+from gpu_support import MODES, run_fused_gemm, run_gemm
 from support import colmajor_a_case, rowmajor_case, run_oracle_gemm
-from test_oracle_gemm import FP_SUITES, dot4_cases, panel_cases, rvv_cases, xsfmm_c_cases
+from test_oracle_gemm import FP_SUITES, dot4_cases, fused_expectation, panel_cases, rvv_cases, xsfmm_c_cases
 
 pytestmark = pytest.mark.gpu
 
@@ -173,6 +173,86 @@ def test_beta_zero_initialises_c(gpu, ta, m, n, k):
                 assert np.array_equal(got.view(np.uint8), again.view(np.uint8)), (ta, mode, alpha)
             if ta in ("f32", "f64", "f16h"):
                 assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (ta, mode, alpha)
+
+
+FUSED_SHAPES = (
+    # m, n, k, what serves it
+    (130, 200, 64, "64 x 64 bounds-checked tiles"),
+    (300, 1100, 96, "128 x 128 bounds-checked tiles"),
+    (2048, 2048, 128, "streaming kernel, 256 x 128 tiles"),
+    (2048, 9216, 128, "streaming kernel, 256 x 256 tiles and a last round of 256 x 128"),
+    (1, 4096, 512, "M = 1: the fused call must not take the GEMV path"),
+)
+
+
+@pytest.mark.parametrize("m,n,k,what", FUSED_SHAPES)
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f8e4m3"))
+def test_fused_epilogue(gpu, ta, m, n, k, what):
+    """Bias and running maximum behind the alpha/beta step (include/skl-gfx950.h, fused section). int8:
+    C and *max equal the checker's GEMM followed by the two steps, bit for bit. Floating point: the fused call's C equals
+    the plain call's C plus the bias in one fp32 addition, bit for bit (same kernel, same summation), and
+    *max is the largest value written."""
+    rng = np.random.default_rng(m * 7 + n)
+    case = rowmajor_case(ta, m, n, k, alpha=1, beta=1 if m != 2048 else 0)
+    a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+    if case.is_int:
+        bias = rng.integers(-1 << 20, 1 << 20, n).astype(np.int32)
+        start = np.array([-(1 << 31)], np.int32)
+    else:
+        bias = rng.uniform(-4, 4, n).astype(np.float32)
+        start = np.array([-np.inf], np.float32)
+    checker_plain = run_oracle_gemm(case, a, b, c) if case.is_int else None
+    for mode in MODES:
+        if m == 1 and not case.is_int:
+            plain = None  # the plain M = 1 call sums with floating-point atomics: no bit-level anchor
+        else:
+            plain = run_gemm(gpu, "rc", case, a, b, c, mode)
+        for use_bias, use_max in ((True, True), (False, True), (True, False)):
+            got, top = run_fused_gemm(gpu, "rc", case, a, b, c, bias if use_bias else None,
+                                      start if use_max else None, mode)
+            if case.is_int:
+                want_c, want_top = fused_expectation(case, checker_plain, bias if use_bias else None,
+                                                     start if use_max else None)
+                assert np.array_equal(got, want_c), (what, mode, use_bias, use_max)
+                if use_max:
+                    assert top[0] == want_top[0], (what, mode)
+            elif plain is not None:
+                want_c, want_top = fused_expectation(case, plain, bias if use_bias else None,
+                                                     start if use_max else None)
+                assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8)), (what, mode, use_bias, use_max)
+                if use_max:
+                    assert top[0] == want_top[0], (what, mode)
+            else:
+                if not use_bias:
+                    support.assert_fp_gemm_close(case, a, b, c, got,
+                                                 extra_rel=support.FP8_MFMA_REL if ta.startswith("f8") else 0.0)
+                if use_max:
+                    assert top[0] == got.max(), (what, mode)
+    # a maximum already above every element stays
+    high = np.array([1 << 30], np.int32) if case.is_int else np.array([1e30], np.float32)
+    _, top = run_fused_gemm(gpu, "rc", case, a, b, c, None, high, "device")
+    assert top[0] == high[0]
+
+
+def test_fused_epilogue_blocked_form_and_null_descriptor(gpu):
+    """The rcprc form indexes the bias by the logical column (block * n0 + column in the block); a call
+    without descriptor operands is the plain GEMM. Odd blocks and strides: the any-stride kernel."""
+    rng = np.random.default_rng(5)
+    for ta in ("i8", "f16"):
+        case = support.GemmCase(ta, None, 2, 3, m0=3, n0=4, k0=5, m1=5, n1=3, k1=4, rsa0=5, csa0=1, rsa1=100, csa1=15,
+                                rsb0=4, csb0=1, rsb1=20, csb1=90, rsc0=1, csc0=3, rsc1=12, csc1=64)
+        a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+        n = case.n0 * case.n1
+        plain = run_gemm(gpu, "rcprc", case, a, b, c, "device")
+        bias = (rng.integers(-99, 99, n).astype(np.int32) if case.is_int else rng.uniform(-4, 4, n).astype(np.float32))
+        start = np.array([-(1 << 31)], np.int32) if case.is_int else np.array([-np.inf], np.float32)
+        for mode in MODES:
+            got, top = run_fused_gemm(gpu, "rcprc", case, a, b, c, bias, start, mode)
+            want_c, want_top = fused_expectation(case, plain, bias, start)
+            assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8)), (ta, mode)
+            assert top[0] == want_top[0]
+            got, _ = run_fused_gemm(gpu, "rcprc", case, a, b, c, None, None, mode)
+            assert np.array_equal(got.view(np.uint8), plain.view(np.uint8)), (ta, mode)
 
 
 def test_mixed_e4m3_e5m2(gpu):

@@ -234,3 +234,58 @@ def test_f32_to_f16_rounding_matches_numpy():
         want = x.astype(np.float16).view(np.uint16)
     got = np.fromiter((f(float(v)) for v in x), dtype=np.uint16, count=x.size)
     assert np.array_equal(got, want)
+
+
+FUSED_TYPES = ("i8", "bf16", "f16", "f8e4m3", "f8e5m2")
+
+
+def fused_expectation(case, plain, bias, max_in):
+    """C and *max after the fused steps, from the plain GEMM's result: the bias of the logical column
+    added in C's arithmetic (one fp32 addition / int32 wrap), the maximum over what was written."""
+    oc = support.blocked_offsets(case.m1, case.n1, case.m0, case.n0, case.rsc0, case.csc0, case.rsc1, case.csc1)
+    want = plain.copy()
+    if bias is not None:
+        with np.errstate(over="ignore"):
+            want[oc] = (plain[oc] + bias[None, :]).astype(plain.dtype)
+    top = None
+    if max_in is not None:
+        written = want[oc]
+        top = np.array([max(max_in[0], written.max())], dtype=plain.dtype)
+    return want, top
+
+
+@pytest.mark.parametrize("ta", FUSED_TYPES)
+def test_fused_steps_follow_the_plain_gemm(ta):
+    """Bias and maximum (src/gemm/fused-kernel-API.md:159-207) behind the alpha/beta step, checked
+    against the plain restatement plus numpy: strided and blocked forms, each step alone and both."""
+    rng = np.random.default_rng(31)
+    cases = (rowmajor_case(ta, 9, 14, 21, alpha=2, beta=3),
+             GemmCase(ta, None, 1, 0, m0=3, n0=4, k0=5, m1=5, n1=3, k1=4, rsa0=5, csa0=1, rsa1=100, csa1=15,
+                      rsb0=4, csb0=1, rsb1=20, csb1=90, rsc0=1, csc0=3, rsc1=12, csc1=64))
+    for case in cases:
+        a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+        n = case.n0 * case.n1
+        plain = run_oracle_gemm(case, a, b, c)
+        if case.is_int:
+            bias = rng.integers(-1 << 20, 1 << 20, n).astype(np.int32)
+            low = np.array([-(1 << 31)], np.int32)
+        else:
+            bias = rng.uniform(-4, 4, n).astype(np.float32)
+            low = np.array([-np.inf], np.float32)
+        blocked = not (case.m0 == case.n0 == case.k0 == 1)
+        name = "skl_gemm_fused_" + (case.stem() if blocked else case.stem().replace("rcprc", "rc"))[len("skl_gemm_"):] + "_oracle"
+        args = case.rcprc_args if blocked else (lambda a_, b_, c_: (case.m1, case.n1, case.k1, case.alpha, a_, case.rsa1,
+                                                                  case.csa1, b_, case.rsb1, case.csb1, case.beta,
+                                                                  c_, case.rsc1, case.csc1))
+        for use_bias, use_max in ((True, True), (True, False), (False, True), (False, False)):
+            for start in (low, None if not use_max else np.array([1 << 30 if case.is_int else 1e30], low.dtype)):
+                if start is None:
+                    continue
+                got, mx = c.copy(), start.copy()
+                getattr(oracle(), name)(*args(a, b, got), bias if use_bias else None, mx if use_max else None)
+                want, top = fused_expectation(case, plain, bias if use_bias else None, start if use_max else None)
+                assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (ta, blocked, use_bias, use_max)
+                if use_max:
+                    assert mx[0] == top[0], (ta, blocked, use_bias)
+                else:
+                    assert mx[0] == start[0]
