@@ -82,6 +82,20 @@ def wl_gemv(lib, rng):
                 name="int8 GEMV 1x4096x11008 (row-major W, beta=0)", kernel="gemv_kernel<int8 row-major>")
 
 
+def wl_gemv_large(lib, rng):
+    """The same kernel on a stream long enough that launch and tail no longer show: 235 MB of weights."""
+    k, n, nbuf = 8192, 28672, 2
+    w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(rand_i8(rng, k))
+    y = DeviceBuffer(4 * n)
+
+    def step(i):
+        lib.skl_gemm_i8_i8_i32_gfx950(1, n, k, 1, x, k, w[i % nbuf], n, 0, y, n)
+
+    return dict(fn=step, bytes=k * n + k + 4 * n, ops=2 * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
+                name="int8 GEMV 1x8192x28672 (row-major W, beta=0)", kernel="gemv_kernel<int8 row-major>")
+
+
 def wl_gemv_p4x1c(lib, rng):
     """Config 2 with W prepacked in the K-packed dot4 layout (B(4P+p, j) at P*rsb1 + 4j + p): same bytes."""
     k, n, nbuf = 4096, 11008, 8
@@ -232,6 +246,7 @@ WORKLOADS = {
     "gemv_i8": (wl_gemv, 2000, 100),
     "gemv_i8_p4x1c": (wl_gemv_p4x1c, 1000, 50),
     "gemv_bf16": (wl_gemv_bf16, 500, 50),
+    "gemv_i8_1x8192x28672": (wl_gemv_large, 300, 30),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2),
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2),
