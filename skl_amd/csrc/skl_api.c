@@ -163,6 +163,10 @@ static void gemm_on_device(const skl_gemm_desc *d) {
         skl_hip_launch_gemv(&g, 0);
         return;
       }
+      if (!fused && skl_hip_gemv_rows_supported(&g)) {
+        skl_hip_launch_gemv_rows(&g);
+        return;
+      }
       if (skl_hip_gemm_mfma_supported(&g)) {
         skl_hip_launch_gemm_mfma(&g);
         return;

@@ -288,6 +288,181 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// 2 <= M <= 8 rows of A against a row-major int8 B ("decode" with a small batch): still a stream over
+// B, so the M = 1 decomposition is kept - same strips, same loads, same 4x4 byte transposes - and every
+// transposed dword is multiplied with the packed x bytes of each of the MR rows (the transposes are shared:
+// (8 + 4 MR) / 16 VALU operations per byte of B). The rows are taken four at a time over the bytes held in
+// registers (64 sums per lane: two workgroups per compute unit). The eight row groups of a wave are laid
+// out inside each row of 16 lanes, so their sums are combined with three DPP rotations; the eight waves
+// meet in LDS, and the workgroups of a strip meet in one 64-bit slot per (row, column) like the M = 1 kernel.
+// ---------------------------------------------------------------------------
+constexpr int kMaxRows = 8;
+
+struct GemvRowsArgs {
+  const char *x;   // MR rows of K bytes, x_row bytes apart (4-byte aligned)
+  size_t x_row;
+  const char *b;
+  size_t b_sk, b_s1;
+  char *y;         // element (i, j) at i * y_row + j * y_s (elements)
+  size_t y_row, y_s;
+  size_t n, k;
+  skl_scalar alpha, beta;
+  void *acc;       // MR * n 64-bit slots, zero between calls
+  unsigned tiles, slabs;
+};
+
+// Sum over the eight lanes of a row of 16 that share a column group (same lane parity), in every lane:
+// three DPP rotations inside the row, no LDS crossbar.
+__device__ __forceinline__ int sum_over_row_groups(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x128 /* row_ror:8 */, 0xF, 0xF, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x124 /* row_ror:4 */, 0xF, 0xF, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x122 /* row_ror:2 */, 0xF, 0xF, false);
+  return v;
+}
+
+constexpr int kRowChunk = 4;  // rows of A multiplied per pass over the loaded bytes of B: 64 sums per lane
+
+template <int MR>
+__global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs p) {
+  using Md = Mode<kI8RowMajor>;
+  constexpr int kCols = Md::kCols, kWords = Md::kKPerLane / 4;
+  __shared__ int red[kWaves][MR][Md::kTileCols];
+
+  const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // Lane pairs read 32 adjacent bytes of a row; the eight row groups sit inside a row of 16 lanes, so that
+  // the lanes that share columns can be summed with DPP rotations: column lane = pair member + 2 * row of 16.
+  const int cl = (lane & 1) + 2 * (lane >> 4), rl = (lane >> 1) & 7;
+  const int part = wave * kRowLanes + rl;
+  const size_t k0 = (size_t)slab * Md::kKPerGroup + (size_t)part * Md::kKPerLane;
+  const size_t col = (size_t)tile * Md::kTileCols + (size_t)cl * kCols;
+  const bool live = col < p.n && k0 < p.k;
+
+  // B's bytes are loaded once and stay in registers for all passes.
+  uint4 rows[kLoadsPerLane];
+#pragma unroll
+  for (int r = 0; r < kLoadsPerLane; ++r) rows[r] = make_uint4(0, 0, 0, 0);
+  if (live) {
+    const char *wp = p.b + (col >> 6) * p.b_s1 + (col & 63) + k0 * p.b_sk;
+#pragma unroll
+    for (int r = 0; r < kLoadsPerLane; ++r)
+      if (k0 + (size_t)r < p.k) rows[r] = stream_load(wp + (size_t)r * p.b_sk);
+  }
+#pragma unroll
+  for (int i0 = 0; i0 < MR; i0 += kRowChunk) {
+    int acc[kRowChunk][kCols];
+#pragma unroll
+    for (int i = 0; i < kRowChunk; ++i)
+#pragma unroll
+      for (int j = 0; j < kCols; ++j) acc[i][j] = 0;
+    if (live) {
+      // x bytes of the lane's k range, four per dword, for the rows of this pass; k at or beyond K
+      // contributes zero
+      int xw[kRowChunk][kWords];
+#pragma unroll
+      for (int i = 0; i < kRowChunk; ++i) {
+        if (i0 + i >= MR) continue;
+        const int8_t *x = reinterpret_cast<const int8_t *>(p.x + (size_t)(i0 + i) * p.x_row);
+        if (k0 + Md::kKPerLane <= p.k) {
+          const int *xp = reinterpret_cast<const int *>(x + k0);  // k0 is a multiple of 8, rows are 4-byte aligned
+#pragma unroll
+          for (int q = 0; q < kWords; ++q) xw[i][q] = xp[q];
+        } else {
+#pragma unroll
+          for (int g = 0; g < kWords; ++g) {
+            unsigned w = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+              const size_t k = k0 + 4 * g + b;
+              w |= (k < p.k ? (unsigned)(uint8_t)x[k] : 0u) << (8 * b);
+            }
+            xw[i][g] = (int)w;
+          }
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < kLoadsPerLane / 4; ++g) {
+        const uint4 r0 = rows[4 * g], r1 = rows[4 * g + 1], r2 = rows[4 * g + 2], r3 = rows[4 * g + 3];
+        const unsigned a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
+        const unsigned a2[4] = {r2.x, r2.y, r2.z, r2.w}, a3[4] = {r3.x, r3.y, r3.z, r3.w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          unsigned t[4];
+          transpose4x4(a0[d], a1[d], a2[d], a3[d], t[0], t[1], t[2], t[3]);
+#pragma unroll
+          for (int i = 0; i < kRowChunk; ++i) {
+            if (i0 + i >= MR) continue;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+              acc[i][4 * d + c] = __builtin_amdgcn_sdot4((int)t[c], xw[i][g], acc[i][4 * d + c], false);
+          }
+        }
+      }
+    }
+    // The eight row groups of the wave hold sums of the same columns (every lane takes part);
+    // the first group hands the wave's sums to LDS.
+#pragma unroll
+    for (int i = 0; i < kRowChunk; ++i) {
+      if (i0 + i >= MR) continue;
+#pragma unroll
+      for (int j = 0; j < kCols; ++j) acc[i][j] = sum_over_row_groups(acc[i][j]);
+      if (rl == 0) {
+#pragma unroll
+        for (int j = 0; j < kCols; j += 4)
+          *reinterpret_cast<int4 *>(&red[wave][i0 + i][cl * kCols + j]) =
+              make_int4(acc[i][j], acc[i][j + 1], acc[i][j + 2], acc[i][j + 3]);
+      }
+    }
+  }
+  __syncthreads();
+  const size_t tile_col0 = (size_t)tile * Md::kTileCols;
+  // thread t: column t % 128, rows t / 128, t / 128 + 4, ... (512 threads: four rows at a time)
+  const int c = threadIdx.x % Md::kTileCols;
+  const size_t j = tile_col0 + c;
+  if (j >= p.n) return;
+  int *yv = reinterpret_cast<int *>(p.y);
+  int sum[(MR + 3) / 4];
+  unsigned long long now[(MR + 3) / 4];
+#pragma unroll
+  for (int q = 0; q < (MR + 3) / 4; ++q) {
+    const int i = threadIdx.x / Md::kTileCols + 4 * q;
+    sum[q] = 0;
+    if (i < MR) {
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) sum[q] += red[w][i][c];
+    }
+  }
+  if (p.slabs == 1) {
+#pragma unroll
+    for (int q = 0; q < (MR + 3) / 4; ++q) {
+      const int i = threadIdx.x / Md::kTileCols + 4 * q;
+      if (i < MR) skl_update(sum[q], yv + (size_t)i * p.y_row + j * p.y_s, p.alpha, p.beta);
+    }
+    return;
+  }
+  // all of the thread's atomics go out before the first result is looked at
+#pragma unroll
+  for (int q = 0; q < (MR + 3) / 4; ++q) {
+    const int i = threadIdx.x / Md::kTileCols + 4 * q;
+    if (i < MR) {
+      unsigned long long *slot = reinterpret_cast<unsigned long long *>(p.acc) + (size_t)i * p.n + j;
+      const unsigned long long mine = ((unsigned long long)(unsigned)sum[q] << 32) | 1ull;
+      now[q] = atomicAdd(slot, mine) + mine;
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < (MR + 3) / 4; ++q) {
+    const int i = threadIdx.x / Md::kTileCols + 4 * q;
+    if (i < MR && (unsigned)now[q] == p.slabs) {
+      unsigned long long *slot = reinterpret_cast<unsigned long long *>(p.acc) + (size_t)i * p.n + j;
+      __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
+      skl_update((int)(unsigned)(now[q] >> 32), yv + (size_t)i * p.y_row + j * p.y_s, p.alpha, p.beta);
+    }
+  }
+}
+
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 int mode_of(const skl_gemm_canon *g, int layout) {
@@ -330,6 +505,35 @@ int launch(const skl_gemm_canon *g, const Reduction &red) {
   return skl_check_launch("gemv");
 }
 
+
+template <int MR>
+int launch_rows(const skl_gemm_canon *g, const Reduction &red) {
+  using Md = Mode<kI8RowMajor>;
+  GemvRowsArgs p;
+  p.x = (const char *)g->a;
+  p.x_row = g->a_s0;
+  p.b = (const char *)g->b;
+  p.b_sk = g->b_sk;
+  p.b_s1 = g->b_s1;
+  p.y = (char *)g->c;
+  p.y_row = g->rsc0;
+  p.y_s = g->csc0;
+  p.n = g->n;
+  p.k = g->k;
+  p.alpha = g->alpha;
+  p.beta = g->beta;
+  p.acc = red.acc;
+  p.tiles = skl_div_up(g->n, Md::kTileCols);
+  p.slabs = skl_div_up(g->k, Md::kKPerGroup);
+  const size_t grid = (size_t)p.tiles * p.slabs;
+  if (grid > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemv: grid too large");
+    return -2;
+  }
+  gemv_rows_kernel<MR><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
+  return skl_check_launch("gemv_rows");
+}
+
 }  // namespace
 
 extern "C" int skl_hip_gemv_supported(const skl_gemm_canon *g, int layout) {
@@ -356,5 +560,34 @@ extern "C" int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout) {
     case kI8K4: return launch<kI8K4>(g, red);
     case kBF16: return launch<kBF16>(g, red);
     default: return launch<kF16>(g, red);
+  }
+}
+
+// 2 <= M <= 8, int8, row-major B: rows of A contiguous in K and 4-byte aligned, C rows inside one block of 64.
+extern "C" int skl_hip_gemv_rows_supported(const skl_gemm_canon *g) {
+  if (g->ta != SKL_DT_I8 || g->tb != SKL_DT_I8) return 0;
+  if (g->m < 2 || g->m > (size_t)kMaxRows || g->k == 0 || g->n == 0 || g->m * g->n > kMaxCols) return 0;
+  if (g->a_sk != 1 || ((uintptr_t)g->a & 3) != 0 || (g->a_s0 & 3) != 0) return 0;
+  if ((g->n % 16) != 0 || !aligned16(g->b) || (g->b_sk % 16) != 0) return 0;
+  if (g->b_s0 != 1 || (g->b_s1 % 16) != 0) return 0;
+  if (g->csc1 != 64 * g->csc0) return 0;
+  return 1;
+}
+
+extern "C" int skl_hip_launch_gemv_rows(const skl_gemm_canon *g) {
+  if (!skl_hip_gemv_rows_supported(g)) {
+    skl_hip_record_error(-2, "gemv_rows: unsupported problem");
+    return -2;
+  }
+  Reduction red;
+  if (!reduction_scratch(&red)) return -4;
+  switch (g->m) {
+    case 2: return launch_rows<2>(g, red);
+    case 3: return launch_rows<3>(g, red);
+    case 4: return launch_rows<4>(g, red);
+    case 5: return launch_rows<5>(g, red);
+    case 6: return launch_rows<6>(g, red);
+    case 7: return launch_rows<7>(g, red);
+    default: return launch_rows<8>(g, red);
   }
 }

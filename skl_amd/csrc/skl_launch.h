@@ -85,6 +85,9 @@ int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g);
  * int8 (`p4x1c`: B(p,j) at (p/4)*b_sk + j*4 + p%4). */
 int skl_hip_gemv_supported(const skl_gemm_canon *g, int layout);
 int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout);
+/* 2 <= M <= 8 rows against a row-major int8 B: the same stream over B with the transposes shared by the rows. */
+int skl_hip_gemv_rows_supported(const skl_gemm_canon *g);
+int skl_hip_launch_gemv_rows(const skl_gemm_canon *g);
 
 /* pack / unpack over elements of `esize` bytes (1, 2 or 4). */
 int skl_hip_launch_pack(int esize, size_t m, size_t n, const void *src, size_t rs, size_t cs,

@@ -104,3 +104,29 @@ def test_k_packed_int8_decode(gpu, n, k1):
     a, b, c = case.make_inputs(n * 3 + k1)
     for mode in ("device", "host"):
         assert np.array_equal(run_gemm(gpu, "dot4", case, a, b, c, mode), run_oracle_gemm(case, a, b, c))
+
+
+@pytest.mark.parametrize("m", (2, 3, 4, 5, 6, 7, 8))
+def test_small_batch_rows_bit_exact(gpu, m):
+    """2 to 8 rows of A against a row-major int8 B (the streaming kernel that shares the byte transposes
+    between the rows): the config-2 shape, ragged K, tiling edges, padded row strides of A, B and C,
+    alpha / beta with wrap-around, and back-to-back calls on the shared reduction scratch."""
+    rng = np.random.default_rng(40 + m)
+    shapes = ((11008, 4096, 0, 0, 0), (1040, 129, 0, 32, 16), (16, 4, 4, 0, 0), (2048, 1000, 24, 16, 48),
+              (33 * 16, 515, 0, 0, 0))
+    for (n, k, pad_a, pad_b, pad_c) in shapes:
+        for alpha, beta in ((1, 0), (0x01010101, -77)):
+            case = rowmajor_case("i8", m, n, k, alpha, beta, rsa=k + pad_a if (k + pad_a) % 4 == 0 else None,
+                                 rsb=n + pad_b, rsc=n + pad_c)
+            a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+            c[:] = rng.integers(-2 ** 31, 2 ** 31, size=c.size)
+            want = run_oracle_gemm(case, a, b, c)
+            for mode in ("device", "host"):
+                assert np.array_equal(run_gemm(gpu, "rowmajor", case, a, b, c, mode), want), (m, n, k, mode)
+
+
+def test_small_batch_unaligned_rows_fall_back(gpu):
+    """Rows of A that are not 4-byte aligned (odd row stride) are served by the tile kernels: same result."""
+    case = rowmajor_case("i8", 4, 1024, 131, 3, 2, rsa=133)
+    a, b, c = case.make_inputs(77)
+    assert np.array_equal(run_gemm(gpu, "rowmajor", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
