@@ -62,6 +62,11 @@ struct MfmaArgs {
   const char *bias;  // fused epilogue: per-column addend and running maximum of C's type, or null
   char *max;
   unsigned tiles_m, tiles_n;
+  // Split along K (bounds-checked kernel only): workgroup b works on tile b % (tiles_m * tiles_n) and on the
+  // slices [split * slices_per_split, ...) with split = b / (tiles_m * tiles_n); splits > 1 stores the raw
+  // sums to partial[split][m][n] (row-major, 4-byte elements) for gemm_split_reduce_kernel.
+  unsigned splits, slices_per_split;
+  char *partial;
 };
 
 // The fused steps behind the alpha/beta step, for one lane: bias of the lane's column, running maximum.
@@ -345,7 +350,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   unsigned tm, tn;
-  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const unsigned tiles = p.tiles_m * p.tiles_n, split = blockIdx.x / tiles;
+  tile_of_block(blockIdx.x % tiles, p.tiles_m, p.tiles_n, tm, tn);
   const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
@@ -363,10 +369,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-  const size_t slices = (p.k * ES + kSliceBytes - 1) / kSliceBytes;
+  const size_t all_slices = (p.k * ES + kSliceBytes - 1) / kSliceBytes;
+  const size_t s_begin = (size_t)split * p.slices_per_split;  // the host makes every split non-empty
+  const size_t slices = all_slices - s_begin < p.slices_per_split ? all_slices : s_begin + p.slices_per_split;
   v4i ra[TileA::kPerThread], rb[TileB::kPerThread];
-  la.template fetch<GUARDED>(ra, 0, p.k);
-  lb.template fetch<GUARDED>(rb, 0, p.k);
+  la.template fetch<GUARDED>(ra, s_begin, p.k);
+  lb.template fetch<GUARDED>(rb, s_begin, p.k);
   la.stash(smem, ra);
   lb.stash(smem + TileA::kBytes, rb);
   __syncthreads();
@@ -378,10 +386,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
 #pragma unroll
   for (int j = 0; j < NI; ++j) fb[0][j] = read_frag<ES, BN, B_KC, FRB>(smem + TileA::kBytes, wn + j * 32, 0);
 
-  for (size_t s = 0; s < slices; ++s) {
-    const char *ta = smem + (s & 1) * kStage;
+  for (size_t s = s_begin; s < slices; ++s) {
+    const char *ta = smem + ((s - s_begin) & 1) * kStage;
     const char *tb = ta + TileA::kBytes;
-    char *na = smem + ((s + 1) & 1) * kStage;
+    char *na = smem + ((s - s_begin + 1) & 1) * kStage;
     // Next slice: global -> registers while this one is multiplied. The last
     // iteration fetches its own slice again (in range, never consumed) so that
     // the loop body has no branch around the loads.
@@ -421,7 +429,24 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
     for (int j = 0; j < NI; ++j) fb[0][j] = read_frag<ES, BN, B_KC, FRB>(na + TileA::kBytes, wn + j * 32, 0);
   }
 
-  // Epilogue: lane l of a 32x32 block holds column l%32 and rows 8*(r/4) + 4*(l/32) + r%4. When C is
+  // Lane l of a 32x32 block holds column l%32 and rows 8*(r/4) + 4*(l/32) + r%4.
+  if (p.splits > 1) {  // a share of K: the raw sums go to this split's M x N plane
+    AccElem *plane = reinterpret_cast<AccElem *>(p.partial) + (size_t)split * p.m * p.n;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const size_t col = n0 + wn + j * 32 + (lane & 31);
+      if (col >= p.n) continue;
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const size_t row = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+          if (row < p.m) plane[row * p.n + col] = acc[i][j][r];
+        }
+    }
+    return;
+  }
+  // Epilogue. When C is
   // updated, the old values of kEpilogueBatch blocks are all requested before the first of them is used
   // (a load behind a store that may alias it would wait for that store: one exposed memory latency per
   // element). C is written once and not read again: non-temporal stores keep it out of the operands' caches.
@@ -964,6 +989,44 @@ int launch_ring(const MfmaArgs &args) {
   return skl_check_launch("gemm_mfma_ring");
 }
 
+// C = beta*C + alpha * (sum of the splits' planes, in split order), then the fused steps: the second
+// half of a GEMM whose K range was shared out between workgroups.
+template <typename T>
+__global__ void __launch_bounds__(256) gemm_split_reduce_kernel(MfmaArgs p) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.m * p.n) return;
+  const size_t row = idx / p.n, col = idx % p.n;
+  const T *plane = reinterpret_cast<const T *>(p.partial) + idx;
+  T sum = plane[0];
+  for (unsigned q = 1; q < p.splits; ++q) {
+    if constexpr (std::is_same<T, int>::value)
+      sum = (int)((unsigned)sum + (unsigned)plane[(size_t)q * p.m * p.n]);
+    else
+      sum = __fadd_rn(sum, plane[(size_t)q * p.m * p.n]);
+  }
+  T *c = reinterpret_cast<T *>(p.c) + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + (col >> 6) * p.csc1 + (col & 63) * p.csc0;
+  skl_update(sum, c, p.alpha, p.beta);
+  if (p.bias || p.max) {
+    T v = *c;
+    if (p.bias) {
+      v = skl_add_bias(v, reinterpret_cast<const T *>(p.bias)[col]);
+      *c = v;
+    }
+    if (p.max && v > skl_lowest<T>()) skl_atomic_max(reinterpret_cast<T *>(p.max), v);
+  }
+}
+
+// How many ways K is shared out when a problem has too few tiles for the chip: enough to put about two
+// workgroups on every compute unit, each share at least kMinSlicesPerSplit slices long, planes within 64 MiB.
+constexpr size_t kMinSlicesPerSplit = 8, kSplitFromSlices = 32, kSplitPlaneLimit = size_t(64) << 20;
+inline unsigned splits_for(size_t tiles, size_t slices, size_t m, size_t n) {
+  if (tiles >= 256 || slices < kSplitFromSlices) return 1;
+  size_t want = (512 + tiles - 1) / tiles;
+  if (want > slices / kMinSlicesPerSplit) want = slices / kMinSlicesPerSplit;
+  while (want > 1 && want * m * n * 4 > kSplitPlaneLimit) --want;
+  return (unsigned)(want < 1 ? 1 : want);
+}
+
 template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED>
 int launch_one(const MfmaArgs &args) {
   constexpr int ES = Kind<TA>::ES;
@@ -981,13 +1044,31 @@ int launch_one(const MfmaArgs &args) {
   MfmaArgs p = args;
   p.tiles_m = skl_div_up(p.m, BM);
   p.tiles_n = skl_div_up(p.n, BN);
-  const size_t grid = (size_t)p.tiles_m * p.tiles_n;
+  const size_t tiles = (size_t)p.tiles_m * p.tiles_n;
+  const size_t slices = (p.k * ES + kSliceBytes - 1) / kSliceBytes;
+  p.splits = splits_for(tiles, slices, p.m, p.n);
+  p.slices_per_split = (unsigned)((slices + p.splits - 1) / p.splits);
+  p.splits = (unsigned)((slices + p.slices_per_split - 1) / p.slices_per_split);  // no empty share
+  if (p.splits > 1) {
+    p.partial = (char *)skl_workspace((size_t)p.splits * p.m * p.n * 4);
+    if (!p.partial) return -4;
+  }
+  const size_t grid = tiles * p.splits;
   if (grid > 0x7FFFFFFFu) {
     skl_hip_record_error(-2, "gemm_mfma: grid too large");
     return -2;
   }
   kernel<<<(unsigned)grid, NT, lds, skl_current_stream()>>>(p);
-  return skl_check_launch("gemm_mfma");
+  int rc = skl_check_launch("gemm_mfma");
+  if (rc != 0 || p.splits == 1) return rc;
+  using AccElem = decltype(typename Kind<TA>::Acc{}.x);
+  const size_t blocks = (p.m * p.n + 255) / 256;
+  if (blocks > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemm_mfma: grid too large");
+    return -2;
+  }
+  gemm_split_reduce_kernel<AccElem><<<(unsigned)blocks, 256, 0, skl_current_stream()>>>(p);
+  return skl_check_launch("gemm_split_reduce");
 }
 
 template <int TA, int TB, bool A_KC, bool B_KC>
@@ -1079,6 +1160,7 @@ extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
   p.alpha = g->alpha, p.beta = g->beta;
   p.bias = (const char *)g->bias, p.max = (char *)g->max;
   p.tiles_m = p.tiles_n = 0;
+  p.splits = 1, p.slices_per_split = 0, p.partial = nullptr;
   switch (g->ta * 8 + g->tb) {
     case SKL_DT_I8 * 8 + SKL_DT_I8: return launch_layout<SKL_DT_I8, SKL_DT_I8>(p);
 #ifndef SKL_MFMA_INT8_ONLY  // kernel-development builds compile one operand kind only

@@ -255,6 +255,33 @@ def test_fused_epilogue_blocked_form_and_null_descriptor(gpu):
             assert np.array_equal(got.view(np.uint8), plain.view(np.uint8)), (ta, mode)
 
 
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f16", "f8e4m3"))
+@pytest.mark.parametrize("m,n,k", ((9, 1000, 4096), (16, 11008, 4096), (40, 300, 8192), (130, 520, 5000)))
+def test_few_tiles_long_k_shares_k_between_workgroups(gpu, ta, m, n, k):
+    """A problem with few output tiles and a long K is shared out along K: raw sums per share, then one
+    pass that adds the shares in order and applies alpha / beta (and the fused steps). int8 must stay
+    bit-exact, floating point inside the reference's bound; two runs give the same bits."""
+    if ta != "i8":
+        k -= k % 8  # 16-byte aligned rows for the 16-bit kinds
+    case = rowmajor_case(ta, m, n, k, alpha=2, beta=3)
+    a, b, c = case.make_inputs(m * 1000 + n)
+    for mode in MODES:
+        got = run_gemm(gpu, "rc", case, a, b, c, mode)
+        if case.is_int:
+            assert np.array_equal(got, run_oracle_gemm(case, a, b, c)), (m, n, k, mode)
+        else:
+            support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=support.FP8_MFMA_REL if ta.startswith("f8") else 0.0)
+            assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
+    # fused steps ride on the second pass
+    bias = (np.arange(n) % 7 - 3).astype(np.int32 if case.is_int else np.float32)
+    start = np.array([-(1 << 31)], np.int32) if case.is_int else np.array([-np.inf], np.float32)
+    plain = run_gemm(gpu, "rc", case, a, b, c, "device")
+    got, top = run_fused_gemm(gpu, "rc", case, a, b, c, bias, start, "device")
+    want_c, want_top = fused_expectation(case, plain, bias, start)
+    assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8))
+    assert top[0] == want_top[0]
+
+
 def test_mixed_e4m3_e5m2(gpu):
     for (m, n, k) in ((13, 21, 37), (128, 192, 256)):
         case = rowmajor_case("f8e4m3", m, n, k, 1.0, 0.0, tb="f8e5m2")
