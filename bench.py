@@ -96,6 +96,22 @@ def wl_gemv_large(lib, rng):
                 name="int8 GEMV 1x8192x28672 (row-major W, beta=0)", kernel="gemv_kernel<int8 row-major>")
 
 
+def _wl_small_batch(m):
+    def build(lib, rng):
+        k, n, nbuf = 4096, 11008, 8
+        w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+        x = DeviceBuffer.from_array(rand_i8(rng, m * k))
+        y = DeviceBuffer(4 * m * n)
+
+        def step(i):
+            lib.skl_gemm_i8_i8_i32_gfx950(m, n, k, 1, x, k, w[i % nbuf], n, 0, y, n)
+
+        kernel = "gemv_rows_kernel" if m <= 8 else "gemm_mfma_kernel (K shared between workgroups) + gemm_split_reduce_kernel"
+        return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
+                    name=f"int8 GEMM {m}x4096x11008 (decode with a batch of {m}: still a stream over W)", kernel=kernel)
+    return build
+
+
 def wl_gemv_p4x1c(lib, rng):
     """Config 2 with W prepacked in the K-packed dot4 layout (B(4P+p, j) at P*rsb1 + 4j + p): same bytes."""
     k, n, nbuf = 4096, 11008, 8
@@ -247,6 +263,8 @@ WORKLOADS = {
     "gemv_i8_p4x1c": (wl_gemv_p4x1c, 1000, 50),
     "gemv_bf16": (wl_gemv_bf16, 500, 50),
     "gemv_i8_1x8192x28672": (wl_gemv_large, 300, 30),
+    "gemm_i8_4x4096x11008": (_wl_small_batch(4), 500, 50),
+    "gemm_i8_16x4096x11008": (_wl_small_batch(16), 300, 30),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2),
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2),
