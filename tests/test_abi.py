@@ -50,3 +50,25 @@ def test_missing_library_fails_loudly(tmp_path):
         assert "no CPU fallback" in str(e)
     else:
         raise AssertionError("loading a missing library must raise")
+
+
+def test_headers_compile_as_c99_c11_and_cxx(tmp_path):
+    """The public headers are what an SKL caller includes: they must be valid C99 for a compiler without
+    `_Float16` (gcc 11: 16-bit patterns, no f16 -> f16 prototypes) and for one with it (ROCm's clang), and C++."""
+    src = tmp_path / "use.c"
+    src.write_text('#include "skl-gfx950.h"\n'
+                   'int probe(void) {\n'
+                   '  skl_gfx950_epilogue_t ep = {0, 0};\n'
+                   '  skl_gemm_i8_i8_i32_gfx950(0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0);\n'
+                   '  skl_gemm_fused_i8rc_i8rc_i32rc_gfx950(0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, &ep);\n'
+                   '  return (int)skl_hip_te();\n'
+                   '}\n')
+    inc = os.path.join(ROOT, "include")
+    clang = "/opt/rocm/lib/llvm/bin/clang"
+    cmds = [["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only", "-I", inc, str(src)],
+            ["g++", "-x", "c++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", inc, str(src)]]
+    if os.path.exists(clang):
+        cmds.append([clang, "-std=c11", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only", "-I", inc, str(src)])
+    for cmd in cmds:
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        assert proc.returncode == 0, (cmd[0], proc.stderr[-2000:])
