@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
 
 Prints ONE JSON line. The headline (`value`) is the int8 GEMV decode shape
-(1x4096 times 4096x11008, BASELINE config 2) in GB/s of algorithmic bytes with
+(1x4096 times 4096x11008, benchmark configuration 2) in GB/s of algorithmic bytes with
 all operands resident in HBM; a "step" is one GEMV call on the next of several
 weight matrices (their total size exceeds the 256 MiB last-level cache, so the
 stream comes from HBM). `extra` carries the dense workloads (TOPS / TFLOP/s and
@@ -199,7 +199,7 @@ def wl_gemm_bf16(lib, rng):
 
 
 def wl_f16_pipeline(lib, rng):
-    """BASELINE config 5: pack A, pack B, panel GEMM, unpack C - one step is the whole pipeline."""
+    """benchmark configuration 5: pack A, pack B, panel GEMM, unpack C - one step is the whole pipeline."""
     te, m, k, n = 64, 4096, 4096, 14336
     a = DeviceBuffer.from_array(rng.uniform(-1, 1, m * k).astype(np.float16).view(np.uint16))
     b = DeviceBuffer.from_array(rng.uniform(-1, 1, k * n).astype(np.float16).view(np.uint16))

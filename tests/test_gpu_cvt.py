@@ -119,7 +119,7 @@ def test_tails_and_misaligned_pointers(gpu, n, src_off, dst_off):
 
 
 def test_config4_operand_preparation(gpu):
-    """fp32 ~ N(0,1) -> E4M3 / E5M2 with saturation, scale 1 (BASELINE config 4's
+    """fp32 ~ N(0,1) -> E4M3 / E5M2 with saturation, scale 1 (benchmark configuration 4's
     input preparation), 4M elements, against the checker."""
     x = np.random.default_rng(0x5EED0040).normal(size=1 << 22).astype(np.float32)
     for fmt in FMTS:

@@ -1,4 +1,4 @@
-"""BASELINE's full-size configurations, checked through properties that do not
+"""The benchmark's full-size configurations, checked through properties that do not
 need the scalar checker to run at that size:
 
 * integer GEMM: Freivalds' identity  (A B) v = A (B v)  and  u^T (A B) = (u^T A) B  with

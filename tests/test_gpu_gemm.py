@@ -291,7 +291,7 @@ def test_mixed_e4m3_e5m2(gpu):
 
 
 def test_config1_int8_512_cubed_bit_exact(gpu):
-    """BASELINE config 1: 512^3, row-major, C = 0, alpha = 1, beta = 0."""
+    """benchmark configuration 1: 512^3, row-major, C = 0, alpha = 1, beta = 0."""
     case = rowmajor_case("i8", 512, 512, 512, 1, 0)
     a, b, c = case.make_inputs(0x5EED0010)
     c[:] = 0

@@ -1,5 +1,5 @@
 """GPU parity of the M == 1 streaming path with the CPU checker (bit-exact:
-integer sums are order-independent), at the BASELINE config-2 shape and around
+integer sums are order-independent), at the benchmark configuration 2 shape and around
 the kernel's tiling edges, including back-to-back calls that share the
 library's zero-initialised reduction scratch."""
 import numpy as np

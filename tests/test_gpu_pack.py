@@ -1,6 +1,6 @@
 """GPU parity of pack / unpack / transpose / panel pack with the CPU checker
 over the reference's test tables (whole destination buffers compared, so the
-stride gaps are a clobber check), plus the BASELINE config-5 shapes checked
+stride gaps are a clobber check), plus the benchmark configuration 5 shapes checked
 through the closed-form index map."""
 import numpy as np
 import pytest
@@ -92,7 +92,7 @@ def test_zero_extents_touch_nothing(gpu):
 
 
 def test_config5_pipeline_shapes(gpu):
-    """BASELINE config 5: pack A (4096x4096 f16 -> TE x 1 panels), pack B
+    """benchmark configuration 5: pack A (4096x4096 f16 -> TE x 1 panels), pack B
     (4096x14336 f16 -> 1 x TE panels), unpack C (TE x TE f32 blocks -> row-major
     4096x14336). Full size, device resident, checked against the closed-form
     index map (numpy) and by pack -> unpack round trip."""

@@ -79,7 +79,7 @@ def test_int8_against_exact_integer_matmul():
 
 
 def test_int8_config1_shape():
-    # BASELINE config 1: 512^3 row-major, alpha = 1, beta = 0, C = 0
+    # benchmark configuration 1: 512^3 row-major, alpha = 1, beta = 0, C = 0
     case = rowmajor_case("i8", 512, 512, 512, 1, 0)
     a, b, c = case.make_inputs(0x5EED0000)
     c[:] = 0
