@@ -140,6 +140,20 @@ def wl_gemv_bf16(lib, rng):
                 name="bf16 GEMV 1x4096x11008 (row-major W, beta=0)", kernel="gemv_kernel<bf16>")
 
 
+def wl_gemv_f8(lib, rng):
+    k, n, nbuf = 4096, 11008, 8
+    w = [DeviceBuffer.from_array(rng.integers(8, 127, size=k * n, dtype=np.uint8)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(rng.integers(8, 127, size=k, dtype=np.uint8))
+    y = DeviceBuffer(4 * n)
+    lib.skl_hip_memset(y, 0, 4 * n)
+
+    def step(i):
+        lib.skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950(1, n, k, 1.0, x, k, 1, w[i % nbuf], n, 1, 0.0, y, n, 1)
+
+    return dict(fn=step, bytes=k * n + k + 4 * n, ops=2 * k * n, bound="hbm", dtype="f8e4m3", keep=(w, x, y),
+                name="fp8 E4M3 GEMV 1x4096x11008 (row-major W, beta=0)", kernel="gemv_kernel<fp8 E4M3>")
+
+
 def _dense(lib, rng, name, fn_name, m, n, k, abytes, gen_a, gen_b, alpha, beta, ctype, dkey, col_major_a=False):
     a = DeviceBuffer.from_array(gen_a(m * k))
     b = DeviceBuffer.from_array(gen_b(k * n))
@@ -262,6 +276,7 @@ WORKLOADS = {
     "gemv_i8": (wl_gemv, 2000, 100),
     "gemv_i8_p4x1c": (wl_gemv_p4x1c, 1000, 50),
     "gemv_bf16": (wl_gemv_bf16, 500, 50),
+    "gemv_f8e4m3": (wl_gemv_f8, 1000, 50),
     "gemv_i8_1x8192x28672": (wl_gemv_large, 300, 30),
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 500, 50),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 300, 30),

@@ -30,7 +30,8 @@
 // for the workgroup's outstanding atomics before the ticket is taken is enough;
 // a device-scope fence would flush the whole L2 and costs ten times the kernel.)
 //
-// The same skeleton serves three more operand kinds: bf16 and f16 weights
+// The same skeleton serves more operand kinds: OCP fp8 weights and x (E4M3, E5M2 and E4M3 x with E5M2
+// weights; a lane owns 16 columns, the hardware conversions decode to fp32), bf16 and f16 weights
 // (a lane owns 8 columns, fp32 accumulation with v_fma, fp32 atomics between
 // workgroups - the summation order then varies from run to run, within the
 // reference's tolerance) and the K-packed int8 layout of the dot4 entry point
@@ -46,7 +47,7 @@
 namespace {
 
 // Kernel modes.
-enum { kI8RowMajor = 0, kI8K4 = 1, kBF16 = 2, kF16 = 3 };
+enum { kI8RowMajor = 0, kI8K4 = 1, kBF16 = 2, kF16 = 3, kF8E4M3 = 4, kF8E5M2 = 5, kF8Mixed = 6 /* E4M3 x, E5M2 B */ };
 
 constexpr int kColLanes = 8;                 // lanes side by side along a row: 8 x 16 B = one 128-byte line
 constexpr int kRowLanes = 64 / kColLanes;    // lane groups taking different rows
@@ -56,13 +57,14 @@ constexpr int kPartials = kWaves * kRowLanes;  // partial sums per column in a w
 
 template <int MODE>
 struct Mode {
-  static constexpr int kCols = MODE == kI8RowMajor ? 16 : MODE == kI8K4 ? 4 : 8;  // columns per lane
+  static constexpr bool kFp8 = MODE == kF8E4M3 || MODE == kF8E5M2 || MODE == kF8Mixed;
+  static constexpr int kCols = (MODE == kI8RowMajor || kFp8) ? 16 : MODE == kI8K4 ? 4 : 8;  // columns per lane
   static constexpr int kTileCols = kColLanes * kCols;                              // columns per workgroup
   static constexpr int kKPerLoad = MODE == kI8K4 ? 4 : 1;                          // k values per 128-bit load
   static constexpr int kKPerLane = kLoadsPerLane * kKPerLoad;
   static constexpr int kKPerGroup = kPartials * kKPerLane;                         // k per workgroup
   static constexpr int kES = (MODE == kBF16 || MODE == kF16) ? 2 : 1;
-  using Acc = typename std::conditional<(MODE == kBF16 || MODE == kF16), float, int>::type;
+  using Acc = typename std::conditional<(MODE == kBF16 || MODE == kF16 || kFp8), float, int>::type;
 };
 
 // Zero-initialised per-device scratch: one 64-bit slot per column (the floating-point modes use the
@@ -111,6 +113,7 @@ struct GemvArgs {
 
 // B is read once: a non-temporal 128-bit load.
 typedef unsigned u4v __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint4 stream_load(const char *p) {
   const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v *>(p));
   return make_uint4(v.x, v.y, v.z, v.w);
@@ -216,6 +219,34 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
           acc[1] = __builtin_amdgcn_sdot4((int)rows[r].y, xw[r], acc[1], false);
           acc[2] = __builtin_amdgcn_sdot4((int)rows[r].z, xw[r], acc[2], false);
           acc[3] = __builtin_amdgcn_sdot4((int)rows[r].w, xw[r], acc[3], false);
+        }
+      }
+    } else if constexpr (Md::kFp8) {
+      // OCP fp8 weights and x: the hardware conversions decode every code but the NaNs exactly as the
+      // reference's decode does (a NaN comes out with its sign set; it is a NaN either way), and the
+      // product of two fp8 values is exact in fp32, so a fused multiply-add rounds like multiply, then add.
+      constexpr bool x_e5m2 = MODE == kF8E5M2, b_e5m2 = MODE != kF8E4M3;
+      const uint8_t *x = reinterpret_cast<const uint8_t *>(p.x);
+#pragma unroll
+      for (int r = 0; r < kLoadsPerLane; ++r) {
+        const size_t k = k0 + r;
+        const int xb = k < p.k ? (int)x[k * p.x_sk] : 0;
+        const float xv = x_e5m2 ? __builtin_amdgcn_cvt_f32_bf8(xb, 0) : __builtin_amdgcn_cvt_f32_fp8(xb, 0);
+        const unsigned w[4] = {rows[r].x, rows[r].y, rows[r].z, rows[r].w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          v2f lo, hi;  // bytes 0, 1 and bytes 2, 3 of the dword: four consecutive columns
+          if constexpr (b_e5m2) {
+            lo = __builtin_amdgcn_cvt_pk_f32_bf8((int)w[d], false);
+            hi = __builtin_amdgcn_cvt_pk_f32_bf8((int)w[d], true);
+          } else {
+            lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[d], false);
+            hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[d], true);
+          }
+          acc[4 * d + 0] = __fmaf_rn(xv, lo.x, acc[4 * d + 0]);
+          acc[4 * d + 1] = __fmaf_rn(xv, lo.y, acc[4 * d + 1]);
+          acc[4 * d + 2] = __fmaf_rn(xv, hi.x, acc[4 * d + 2]);
+          acc[4 * d + 3] = __fmaf_rn(xv, hi.y, acc[4 * d + 3]);
         }
       }
     } else {
@@ -466,13 +497,16 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 int mode_of(const skl_gemm_canon *g, int layout) {
+  if (layout == 1) return (g->ta == SKL_DT_I8 && g->tb == SKL_DT_I8) ? kI8K4 : -1;
+  if (g->ta == SKL_DT_F8E4M3 && g->tb == SKL_DT_F8E5M2) return kF8Mixed;
   if (g->ta != g->tb) return -1;
-  if (layout == 1) return g->ta == SKL_DT_I8 ? kI8K4 : -1;
   switch (g->ta) {
     case SKL_DT_I8: return kI8RowMajor;
     case SKL_DT_BF16: return kBF16;
     case SKL_DT_F16: return kF16;
-    default: return -1;  // fp8 M = 1 goes to the matrix-core kernel
+    case SKL_DT_F8E4M3: return kF8E4M3;
+    case SKL_DT_F8E5M2: return kF8E5M2;
+    default: return -1;
   }
 }
 
@@ -541,7 +575,7 @@ extern "C" int skl_hip_gemv_supported(const skl_gemm_canon *g, int layout) {
   if (mode < 0) return 0;
   if (g->m != 1 || g->k == 0 || g->n == 0 || g->n > kMaxCols) return 0;
   const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1;
-  const size_t cols = mode == kI8RowMajor ? 16 : mode == kI8K4 ? 4 : 8;
+  const size_t cols = (mode == kI8RowMajor || mode >= kF8E4M3) ? 16 : mode == kI8K4 ? 4 : 8;
   if ((g->n % cols) != 0 || !aligned16(g->b) || ((g->b_sk * es) % 16) != 0) return 0;
   if (mode != kI8K4 && (g->b_s0 != 1 || ((g->b_s1 * es) % 16) != 0)) return 0;
   if (g->csc1 != 64 * g->csc0) return 0;  // y must be a flat strided vector
@@ -559,7 +593,10 @@ extern "C" int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout) {
     case kI8RowMajor: return launch<kI8RowMajor>(g, red);
     case kI8K4: return launch<kI8K4>(g, red);
     case kBF16: return launch<kBF16>(g, red);
-    default: return launch<kF16>(g, red);
+    case kF16: return launch<kF16>(g, red);
+    case kF8E4M3: return launch<kF8E4M3>(g, red);
+    case kF8E5M2: return launch<kF8E5M2>(g, red);
+    default: return launch<kF8Mixed>(g, red);
   }
 }
 

@@ -130,3 +130,38 @@ def test_small_batch_unaligned_rows_fall_back(gpu):
     case = rowmajor_case("i8", 4, 1024, 131, 3, 2, rsa=133)
     a, b, c = case.make_inputs(77)
     assert np.array_equal(run_gemm(gpu, "rowmajor", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
+
+
+FP8_PAIRS = (("f8e4m3", "f8e4m3"), ("f8e5m2", "f8e5m2"), ("f8e4m3", "f8e5m2"))
+
+
+@pytest.mark.parametrize("ta,tb", FP8_PAIRS)
+def test_fp8_rows_of_b_are_decoded_exactly(gpu, ta, tb):
+    """x = one-hot (1.0 at position p), alpha = 1, beta = 0: y is row p of B decoded to fp32. Every code
+    of the format (NaN codes aside) must come out as the format defines it, in the right column."""
+    n, k = 256, 24
+    one = 0x38 if ta == "f8e4m3" else 0x3C
+    table = support.decode_table(tb)
+    finite_codes = np.flatnonzero(np.isfinite(table)).astype(np.uint8)  # 0 * Inf would spoil whole columns
+    b = np.zeros(k * n, np.uint8)
+    for p in range(k):
+        b[p * n:(p + 1) * n] = finite_codes[(np.arange(n) * (2 * p + 1) + 5 * p) % finite_codes.size]
+    assert set(b.tolist()) == set(finite_codes.tolist())
+    for p in (0, 7, 8, 23):
+        x = np.zeros(k, np.uint8)
+        x[p] = one
+        case = rowmajor_case(ta, 1, n, k, 1.0, 0.0, tb=tb)
+        got = run_gemm(gpu, "rc", case, x, b, np.zeros(n, np.float32), "device")
+        assert np.array_equal(got.astype(np.float64), table[b[p * n:(p + 1) * n]]), (ta, tb, p)
+
+
+@pytest.mark.parametrize("ta,tb", FP8_PAIRS)
+@pytest.mark.parametrize("n,k", ((11008, 4096), (1040, 129), (16, 5), (2048, 1000)))
+def test_fp8_streaming_path_within_reference_bound(gpu, ta, tb, n, k):
+    """fp8 x and weights on the streaming kernel: fp32 accumulation (no matrix-core instruction), so the
+    reference's own elementwise bound holds without the fp8-MFMA allowance."""
+    case = rowmajor_case(ta, 1, n, k, 1.5, -0.5, tb=tb, rsb=n + 48)
+    a, b, c = case.make_inputs(n + 3 * k)
+    for mode in ("device", "host"):
+        got = run_gemm(gpu, "rc", case, a, b, c, mode)
+        support.assert_fp_gemm_close(case, a, b, c, got)
