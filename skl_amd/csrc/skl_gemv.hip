@@ -321,13 +321,15 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
 
 
 // ---------------------------------------------------------------------------
-// 2 <= M <= 8 rows of A against a row-major int8 B ("decode" with a small batch): still a stream over
+// 2 <= M <= 8 rows of A against a row-major B ("decode" with a small batch): still a stream over
 // B, so the M = 1 decomposition is kept - same strips, same loads, same 4x4 byte transposes - and every
 // transposed dword is multiplied with the packed x bytes of each of the MR rows (the transposes are shared:
 // (8 + 4 MR) / 16 VALU operations per byte of B). The rows are taken four at a time over the bytes held in
 // registers (64 sums per lane: two workgroups per compute unit). The eight row groups of a wave are laid
 // out inside each row of 16 lanes, so their sums are combined with three DPP rotations; the eight waves
 // meet in LDS, and the workgroups of a strip meet in one 64-bit slot per (row, column) like the M = 1 kernel.
+// The floating-point kinds (bf16, f16, fp8) run on the same skeleton: a loaded row of B is widened once and
+// multiplied with the x value of every row, fp32 sums, fp32 atomics and a ticket between workgroups.
 // ---------------------------------------------------------------------------
 constexpr int kMaxRows = 8;
 
@@ -340,7 +342,8 @@ struct GemvRowsArgs {
   size_t y_row, y_s;
   size_t n, k;
   skl_scalar alpha, beta;
-  void *acc;       // MR * n 64-bit slots, zero between calls
+  void *acc;       // MR * n 64-bit slots (floating point: fp32 values in the same region), zero between calls
+  unsigned *tickets;
   unsigned tiles, slabs;
 };
 
@@ -353,13 +356,23 @@ __device__ __forceinline__ int sum_over_row_groups(int v) {
   return v;
 }
 
+__device__ __forceinline__ float sum_over_row_groups(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xF, 0xF, false));
+  return v;
+}
+
 constexpr int kRowChunk = 4;  // rows of A multiplied per pass over the loaded bytes of B: 64 sums per lane
 
-template <int MR>
+template <int MR, int MODE>
 __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs p) {
-  using Md = Mode<kI8RowMajor>;
+  using Md = Mode<MODE>;
+  using Acc = typename Md::Acc;
   constexpr int kCols = Md::kCols, kWords = Md::kKPerLane / 4;
-  __shared__ int red[kWaves][MR][Md::kTileCols];
+  constexpr bool kInt = MODE == kI8RowMajor;
+  __shared__ Acc red[kWaves][MR][Md::kTileCols];
+  __shared__ unsigned ticket_s;
 
   const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -376,58 +389,99 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 #pragma unroll
   for (int r = 0; r < kLoadsPerLane; ++r) rows[r] = make_uint4(0, 0, 0, 0);
   if (live) {
-    const char *wp = p.b + (col >> 6) * p.b_s1 + (col & 63) + k0 * p.b_sk;
+    const char *wp = p.b + (col >> 6) * p.b_s1 + (col & 63) * Md::kES + k0 * p.b_sk;
 #pragma unroll
     for (int r = 0; r < kLoadsPerLane; ++r)
       if (k0 + (size_t)r < p.k) rows[r] = stream_load(wp + (size_t)r * p.b_sk);
   }
 #pragma unroll
   for (int i0 = 0; i0 < MR; i0 += kRowChunk) {
-    int acc[kRowChunk][kCols];
+    Acc acc[kRowChunk][kCols];
 #pragma unroll
     for (int i = 0; i < kRowChunk; ++i)
 #pragma unroll
       for (int j = 0; j < kCols; ++j) acc[i][j] = 0;
     if (live) {
-      // x bytes of the lane's k range, four per dword, for the rows of this pass; k at or beyond K
-      // contributes zero
-      int xw[kRowChunk][kWords];
+      if constexpr (kInt) {
+        // x bytes of the lane's k range, four per dword, for the rows of this pass; k at or beyond K
+        // contributes zero
+        int xw[kRowChunk][kWords];
 #pragma unroll
-      for (int i = 0; i < kRowChunk; ++i) {
-        if (i0 + i >= MR) continue;
-        const int8_t *x = reinterpret_cast<const int8_t *>(p.x + (size_t)(i0 + i) * p.x_row);
-        if (k0 + Md::kKPerLane <= p.k) {
-          const int *xp = reinterpret_cast<const int *>(x + k0);  // k0 is a multiple of 8, rows are 4-byte aligned
+        for (int i = 0; i < kRowChunk; ++i) {
+          if (i0 + i >= MR) continue;
+          const int8_t *x = reinterpret_cast<const int8_t *>(p.x + (size_t)(i0 + i) * p.x_row);
+          if (k0 + Md::kKPerLane <= p.k) {
+            const int *xp = reinterpret_cast<const int *>(x + k0);  // k0 is a multiple of 8, rows are 4-byte aligned
 #pragma unroll
-          for (int q = 0; q < kWords; ++q) xw[i][q] = xp[q];
-        } else {
+            for (int q = 0; q < kWords; ++q) xw[i][q] = xp[q];
+          } else {
 #pragma unroll
-          for (int g = 0; g < kWords; ++g) {
-            unsigned w = 0;
+            for (int g = 0; g < kWords; ++g) {
+              unsigned w = 0;
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-              const size_t k = k0 + 4 * g + b;
-              w |= (k < p.k ? (unsigned)(uint8_t)x[k] : 0u) << (8 * b);
+              for (int b = 0; b < 4; ++b) {
+                const size_t k = k0 + 4 * g + b;
+                w |= (k < p.k ? (unsigned)(uint8_t)x[k] : 0u) << (8 * b);
+              }
+              xw[i][g] = (int)w;
             }
-            xw[i][g] = (int)w;
           }
         }
-      }
 #pragma unroll
-      for (int g = 0; g < kLoadsPerLane / 4; ++g) {
-        const uint4 r0 = rows[4 * g], r1 = rows[4 * g + 1], r2 = rows[4 * g + 2], r3 = rows[4 * g + 3];
-        const unsigned a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
-        const unsigned a2[4] = {r2.x, r2.y, r2.z, r2.w}, a3[4] = {r3.x, r3.y, r3.z, r3.w};
+        for (int g = 0; g < kLoadsPerLane / 4; ++g) {
+          const uint4 r0 = rows[4 * g], r1 = rows[4 * g + 1], r2 = rows[4 * g + 2], r3 = rows[4 * g + 3];
+          const unsigned a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
+          const unsigned a2[4] = {r2.x, r2.y, r2.z, r2.w}, a3[4] = {r3.x, r3.y, r3.z, r3.w};
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          unsigned t[4];
-          transpose4x4(a0[d], a1[d], a2[d], a3[d], t[0], t[1], t[2], t[3]);
+          for (int d = 0; d < 4; ++d) {
+            unsigned t[4];
+            transpose4x4(a0[d], a1[d], a2[d], a3[d], t[0], t[1], t[2], t[3]);
+#pragma unroll
+            for (int i = 0; i < kRowChunk; ++i) {
+              if (i0 + i >= MR) continue;
+#pragma unroll
+              for (int c = 0; c < 4; ++c)
+                acc[i][4 * d + c] = __builtin_amdgcn_sdot4((int)t[c], xw[i][g], acc[i][4 * d + c], false);
+            }
+          }
+        }
+      } else {
+        // Floating-point kinds: a loaded row of B is widened once and multiplied with the x value of every row.
+#pragma unroll
+        for (int r = 0; r < kLoadsPerLane; ++r) {
+          const size_t k = k0 + r;
+          const unsigned w[4] = {rows[r].x, rows[r].y, rows[r].z, rows[r].w};
+          float wide[kCols];
+          if constexpr (Md::kFp8) {
+            constexpr bool b_e5m2 = MODE != kF8E4M3;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              const v2f lo = b_e5m2 ? __builtin_amdgcn_cvt_pk_f32_bf8((int)w[d], false) : __builtin_amdgcn_cvt_pk_f32_fp8((int)w[d], false);
+              const v2f hi = b_e5m2 ? __builtin_amdgcn_cvt_pk_f32_bf8((int)w[d], true) : __builtin_amdgcn_cvt_pk_f32_fp8((int)w[d], true);
+              wide[4 * d] = lo.x, wide[4 * d + 1] = lo.y, wide[4 * d + 2] = hi.x, wide[4 * d + 3] = hi.y;
+            }
+          } else {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              wide[2 * d] = widen16(w[d] & 0xFFFFu, MODE == kBF16);
+              wide[2 * d + 1] = widen16(w[d] >> 16, MODE == kBF16);
+            }
+          }
 #pragma unroll
           for (int i = 0; i < kRowChunk; ++i) {
             if (i0 + i >= MR) continue;
+            const char *xr = p.x + (size_t)(i0 + i) * p.x_row;
+            float xv = 0.0f;
+            if (k < p.k) {
+              if constexpr (Md::kFp8) {
+                const int xb = (int)reinterpret_cast<const uint8_t *>(xr)[k];
+                xv = MODE == kF8E5M2 ? __builtin_amdgcn_cvt_f32_bf8(xb, 0) : __builtin_amdgcn_cvt_f32_fp8(xb, 0);
+              } else {
+                xv = widen16(reinterpret_cast<const unsigned short *>(xr)[k], MODE == kBF16);
+              }
+            }
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
-              acc[i][4 * d + c] = __builtin_amdgcn_sdot4((int)t[c], xw[i][g], acc[i][4 * d + c], false);
+            for (int c = 0; c < kCols; ++c) acc[i][c] = __fmaf_rn(xv, wide[c], acc[i][c]);
           }
         }
       }
@@ -441,24 +495,22 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
       for (int j = 0; j < kCols; ++j) acc[i][j] = sum_over_row_groups(acc[i][j]);
       if (rl == 0) {
 #pragma unroll
-        for (int j = 0; j < kCols; j += 4)
-          *reinterpret_cast<int4 *>(&red[wave][i0 + i][cl * kCols + j]) =
-              make_int4(acc[i][j], acc[i][j + 1], acc[i][j + 2], acc[i][j + 3]);
+        for (int j = 0; j < kCols; ++j) red[wave][i0 + i][cl * kCols + j] = acc[i][j];
       }
     }
   }
   __syncthreads();
   const size_t tile_col0 = (size_t)tile * Md::kTileCols;
-  // thread t: column t % 128, rows t / 128, t / 128 + 4, ... (512 threads: four rows at a time)
-  const int c = threadIdx.x % Md::kTileCols;
+  // thread t: column t % kTileCols, rows t / kTileCols, + kRowStep, ...
+  constexpr int kRowStep = kWaves * 64 / Md::kTileCols, kPasses = (MR + kRowStep - 1) / kRowStep;
+  const int c = threadIdx.x % Md::kTileCols, row0 = threadIdx.x / Md::kTileCols;
   const size_t j = tile_col0 + c;
-  if (j >= p.n) return;
-  int *yv = reinterpret_cast<int *>(p.y);
-  int sum[(MR + 3) / 4];
-  unsigned long long now[(MR + 3) / 4];
+  const bool valid = j < p.n;
+  Acc *yv = reinterpret_cast<Acc *>(p.y);
+  Acc sum[kPasses];
 #pragma unroll
-  for (int q = 0; q < (MR + 3) / 4; ++q) {
-    const int i = threadIdx.x / Md::kTileCols + 4 * q;
+  for (int q = 0; q < kPasses; ++q) {
+    const int i = row0 + kRowStep * q;
     sum[q] = 0;
     if (i < MR) {
 #pragma unroll
@@ -467,30 +519,56 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
   }
   if (p.slabs == 1) {
 #pragma unroll
-    for (int q = 0; q < (MR + 3) / 4; ++q) {
-      const int i = threadIdx.x / Md::kTileCols + 4 * q;
-      if (i < MR) skl_update(sum[q], yv + (size_t)i * p.y_row + j * p.y_s, p.alpha, p.beta);
+    for (int q = 0; q < kPasses; ++q) {
+      const int i = row0 + kRowStep * q;
+      if (valid && i < MR) skl_update(sum[q], yv + (size_t)i * p.y_row + j * p.y_s, p.alpha, p.beta);
     }
     return;
   }
-  // all of the thread's atomics go out before the first result is looked at
+  if constexpr (kInt) {
+    // all of the thread's atomics go out before the first result is looked at
+    unsigned long long now[kPasses];
 #pragma unroll
-  for (int q = 0; q < (MR + 3) / 4; ++q) {
-    const int i = threadIdx.x / Md::kTileCols + 4 * q;
-    if (i < MR) {
-      unsigned long long *slot = reinterpret_cast<unsigned long long *>(p.acc) + (size_t)i * p.n + j;
-      const unsigned long long mine = ((unsigned long long)(unsigned)sum[q] << 32) | 1ull;
-      now[q] = atomicAdd(slot, mine) + mine;
+    for (int q = 0; q < kPasses; ++q) {
+      const int i = row0 + kRowStep * q;
+      if (valid && i < MR) {
+        unsigned long long *slot = reinterpret_cast<unsigned long long *>(p.acc) + (size_t)i * p.n + j;
+        const unsigned long long mine = ((unsigned long long)(unsigned)sum[q] << 32) | 1ull;
+        now[q] = atomicAdd(slot, mine) + mine;
+      }
     }
-  }
 #pragma unroll
-  for (int q = 0; q < (MR + 3) / 4; ++q) {
-    const int i = threadIdx.x / Md::kTileCols + 4 * q;
-    if (i < MR && (unsigned)now[q] == p.slabs) {
-      unsigned long long *slot = reinterpret_cast<unsigned long long *>(p.acc) + (size_t)i * p.n + j;
-      __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
-      skl_update((int)(unsigned)(now[q] >> 32), yv + (size_t)i * p.y_row + j * p.y_s, p.alpha, p.beta);
+    for (int q = 0; q < kPasses; ++q) {
+      const int i = row0 + kRowStep * q;
+      if (valid && i < MR && (unsigned)now[q] == p.slabs) {
+        unsigned long long *slot = reinterpret_cast<unsigned long long *>(p.acc) + (size_t)i * p.n + j;
+        __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
+        skl_update((int)(unsigned)(now[q] >> 32), yv + (size_t)i * p.y_row + j * p.y_s, p.alpha, p.beta);
+      }
     }
+  } else {
+    // fp32 sums between workgroups, then a ticket per strip, as in the M = 1 kernel
+    float *scratch = reinterpret_cast<float *>(p.acc);
+#pragma unroll
+    for (int q = 0; q < kPasses; ++q) {
+      const int i = row0 + kRowStep * q;
+      if (valid && i < MR) atomicAdd(&scratch[(size_t)i * p.n + j], sum[q]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) ticket_s = atomicAdd(&p.tickets[tile], 1u);
+    __syncthreads();
+    if (ticket_s != p.slabs - 1) return;
+#pragma unroll
+    for (int q = 0; q < kPasses; ++q) {
+      const int i = row0 + kRowStep * q;
+      if (valid && i < MR) {
+        const float total = atomicExch(&scratch[(size_t)i * p.n + j], 0.0f);  // read the total and leave zero behind
+        skl_update(total, yv + (size_t)i * p.y_row + j * p.y_s, p.alpha, p.beta);
+      }
+    }
+    if (threadIdx.x == 0) atomicExch(&p.tickets[tile], 0u);
   }
 }
 
@@ -540,15 +618,15 @@ int launch(const skl_gemm_canon *g, const Reduction &red) {
 }
 
 
-template <int MR>
+template <int MR, int MODE>
 int launch_rows(const skl_gemm_canon *g, const Reduction &red) {
-  using Md = Mode<kI8RowMajor>;
+  using Md = Mode<MODE>;
   GemvRowsArgs p;
   p.x = (const char *)g->a;
-  p.x_row = g->a_s0;
+  p.x_row = g->a_s0 * Md::kES;
   p.b = (const char *)g->b;
-  p.b_sk = g->b_sk;
-  p.b_s1 = g->b_s1;
+  p.b_sk = g->b_sk * Md::kES;
+  p.b_s1 = g->b_s1 * Md::kES;
   p.y = (char *)g->c;
   p.y_row = g->rsc0;
   p.y_s = g->csc0;
@@ -557,6 +635,7 @@ int launch_rows(const skl_gemm_canon *g, const Reduction &red) {
   p.alpha = g->alpha;
   p.beta = g->beta;
   p.acc = red.acc;
+  p.tickets = red.tickets;
   p.tiles = skl_div_up(g->n, Md::kTileCols);
   p.slabs = skl_div_up(g->k, Md::kKPerGroup);
   const size_t grid = (size_t)p.tiles * p.slabs;
@@ -564,8 +643,28 @@ int launch_rows(const skl_gemm_canon *g, const Reduction &red) {
     skl_hip_record_error(-2, "gemv: grid too large");
     return -2;
   }
-  gemv_rows_kernel<MR><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
+  gemv_rows_kernel<MR, MODE><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
   return skl_check_launch("gemv_rows");
+}
+
+// The floating-point kinds pay one multiply-add per element of B and row (there is no dot instruction over
+// k for them) and are bound by that from four rows on, where the tile kernels are faster: they stop at three.
+constexpr int kMaxRowsFloat = 3;
+
+template <int MODE>
+int launch_rows_of(const skl_gemm_canon *g, const Reduction &red) {
+  if constexpr (MODE != kI8RowMajor) {
+    return g->m == 2 ? launch_rows<2, MODE>(g, red) : launch_rows<3, MODE>(g, red);
+  } else
+  switch (g->m) {
+    case 2: return launch_rows<2, MODE>(g, red);
+    case 3: return launch_rows<3, MODE>(g, red);
+    case 4: return launch_rows<4, MODE>(g, red);
+    case 5: return launch_rows<5, MODE>(g, red);
+    case 6: return launch_rows<6, MODE>(g, red);
+    case 7: return launch_rows<7, MODE>(g, red);
+    default: return launch_rows<8, MODE>(g, red);
+  }
 }
 
 }  // namespace
@@ -600,13 +699,19 @@ extern "C" int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout) {
   }
 }
 
-// 2 <= M <= 8, int8, row-major B: rows of A contiguous in K and 4-byte aligned, C rows inside one block of 64.
+// 2 <= M <= 8 (int8) or 2 <= M <= 3 (bf16, f16, fp8), row-major B: rows of A contiguous in K (int8: 4-byte
+// aligned), C rows inside one block of 64.
 extern "C" int skl_hip_gemv_rows_supported(const skl_gemm_canon *g) {
-  if (g->ta != SKL_DT_I8 || g->tb != SKL_DT_I8) return 0;
-  if (g->m < 2 || g->m > (size_t)kMaxRows || g->k == 0 || g->n == 0 || g->m * g->n > kMaxCols) return 0;
-  if (g->a_sk != 1 || ((uintptr_t)g->a & 3) != 0 || (g->a_s0 & 3) != 0) return 0;
-  if ((g->n % 16) != 0 || !aligned16(g->b) || (g->b_sk % 16) != 0) return 0;
-  if (g->b_s0 != 1 || (g->b_s1 % 16) != 0) return 0;
+  const int mode = mode_of(g, 0);
+  if (mode < 0) return 0;
+  if (g->m < 2 || g->m > (size_t)(mode == kI8RowMajor ? kMaxRows : kMaxRowsFloat)) return 0;
+  if (g->k == 0 || g->n == 0 || g->m * g->n > kMaxCols) return 0;
+  const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1;
+  const size_t cols = es == 2 ? 8 : 16;
+  if (g->a_sk != 1) return 0;
+  if (mode == kI8RowMajor && ((((uintptr_t)g->a) & 3) != 0 || (g->a_s0 & 3) != 0)) return 0;
+  if ((g->n % cols) != 0 || !aligned16(g->b) || ((g->b_sk * es) % 16) != 0) return 0;
+  if (g->b_s0 != 1 || ((g->b_s1 * es) % 16) != 0) return 0;
   if (g->csc1 != 64 * g->csc0) return 0;
   return 1;
 }
@@ -618,13 +723,12 @@ extern "C" int skl_hip_launch_gemv_rows(const skl_gemm_canon *g) {
   }
   Reduction red;
   if (!reduction_scratch(&red)) return -4;
-  switch (g->m) {
-    case 2: return launch_rows<2>(g, red);
-    case 3: return launch_rows<3>(g, red);
-    case 4: return launch_rows<4>(g, red);
-    case 5: return launch_rows<5>(g, red);
-    case 6: return launch_rows<6>(g, red);
-    case 7: return launch_rows<7>(g, red);
-    default: return launch_rows<8>(g, red);
+  switch (mode_of(g, 0)) {
+    case kI8RowMajor: return launch_rows_of<kI8RowMajor>(g, red);
+    case kBF16: return launch_rows_of<kBF16>(g, red);
+    case kF16: return launch_rows_of<kF16>(g, red);
+    case kF8E4M3: return launch_rows_of<kF8E4M3>(g, red);
+    case kF8E5M2: return launch_rows_of<kF8E5M2>(g, red);
+    default: return launch_rows_of<kF8Mixed>(g, red);
   }
 }

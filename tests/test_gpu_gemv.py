@@ -165,3 +165,19 @@ def test_fp8_streaming_path_within_reference_bound(gpu, ta, tb, n, k):
     for mode in ("device", "host"):
         got = run_gemm(gpu, "rc", case, a, b, c, mode)
         support.assert_fp_gemm_close(case, a, b, c, got)
+
+
+@pytest.mark.parametrize("ta,tb", (("bf16", "bf16"), ("f16", "f16")) + FP8_PAIRS)
+@pytest.mark.parametrize("m", (2, 3))
+def test_small_batch_rows_floating_point(gpu, ta, tb, m):
+    """2 or 3 rows of A on the streaming kernel for bf16 / f16 / fp8: fp32 accumulation, the reference's
+    elementwise bound (no matrix-core allowance), strides with padding, both pointer modes, and a second
+    call right behind the first on the shared scratch."""
+    for (n, k) in ((11008, 4096), (1040, 136), (16, 8), (2048, 1000)):
+        case = rowmajor_case(ta, m, n, k, 1.5, -0.5, tb=tb, rsa=k + 8, rsb=n + 48, rsc=n + 3)
+        a, b, c = case.make_inputs(m * 100 + n + k)
+        for mode in ("device", "host"):
+            got = run_gemm(gpu, "rc", case, a, b, c, mode)
+            support.assert_fp_gemm_close(case, a, b, c, got)
+            again = run_gemm(gpu, "rc", case, a, b, c, mode)
+            support.assert_fp_gemm_close(case, a, b, c, again)
