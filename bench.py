@@ -96,6 +96,35 @@ def wl_gemv_large(lib, rng):
                 name="int8 GEMV 1x8192x28672 (row-major W, beta=0)", kernel="gemv_kernel<int8 row-major>")
 
 
+def wl_gemv_kc(lib, rng):
+    """The config-2 product with the weights stored column by column (B with K contiguous: a linear layer's
+    [out][in] weight): one dot product over contiguous memory per output, no sums between workgroups."""
+    k, n, nbuf = 4096, 11008, 8
+    w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(rand_i8(rng, k))
+    y = DeviceBuffer(4 * n)
+
+    def step(i):
+        lib.skl_gemm_i8rc_i8rc_i32rc_gfx950(1, n, k, 1, x, k, 1, w[i % nbuf], 1, k, 0, y, n, 1)
+
+    return dict(fn=step, bytes=k * n + k + 4 * n, ops=2 * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
+                name="int8 GEMV 1x4096x11008, W with K contiguous ([n][k]), beta=0", kernel="gemv_kc_kernel<int8>")
+
+
+def wl_gemv_kc_bf16(lib, rng):
+    k, n, nbuf = 4096, 11008, 4
+    w = [DeviceBuffer.from_array(bf16_bits(rng.normal(size=k * n) * 0.02)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(bf16_bits(rng.normal(size=k)))
+    y = DeviceBuffer(4 * n)
+    lib.skl_hip_memset(y, 0, 4 * n)
+
+    def step(i):
+        lib.skl_gemm_bf16rc_bf16rc_f32rc_gfx950(1, n, k, 1.0, x, k, 1, w[i % nbuf], 1, k, 0.0, y, n, 1)
+
+    return dict(fn=step, bytes=2 * k * n + 2 * k + 4 * n, ops=2 * k * n, bound="hbm", dtype="bf16", keep=(w, x, y),
+                name="bf16 GEMV 1x4096x11008, W with K contiguous ([n][k]), beta=0", kernel="gemv_kc_kernel<bf16>")
+
+
 def _wl_small_batch(m):
     def build(lib, rng):
         k, n, nbuf = 4096, 11008, 8
@@ -278,6 +307,8 @@ WORKLOADS = {
     "gemv_bf16": (wl_gemv_bf16, 500, 50),
     "gemv_f8e4m3": (wl_gemv_f8, 1000, 50),
     "gemv_i8_1x8192x28672": (wl_gemv_large, 300, 30),
+    "gemv_i8_kcontig": (wl_gemv_kc, 1000, 50),
+    "gemv_bf16_kcontig": (wl_gemv_kc_bf16, 500, 50),
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 500, 50),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 300, 30),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),

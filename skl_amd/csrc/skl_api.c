@@ -159,6 +159,10 @@ static void gemm_on_device(const skl_gemm_desc *d) {
       return;
     }
     if (canonicalize(d, &g)) {
+      if (!fused && skl_hip_gemv_kc_supported(&g)) {
+        skl_hip_launch_gemv_kc(&g);
+        return;
+      }
       if (!fused && g.m == 1 && skl_hip_gemv_supported(&g, 0)) {
         skl_hip_launch_gemv(&g, 0);
         return;

@@ -572,6 +572,143 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// B with K contiguous (column j is K consecutive elements, columns a fixed distance apart - how a linear
+// layer's weight [out][in] is stored): every output is a dot product over contiguous memory. A wave owns
+// two or four columns and walks K one KiB (64 lanes x 16 bytes) at a time, kKcUnroll KiB per column in
+// flight; the x values of a KiB are loaded once per row of A (1 to 4 rows) and reused by the columns.
+// The lanes' sums are combined inside the wave (DPP rotations, then two cross-lane exchanges), and
+// lane 0 writes the results: no sums between workgroups, no scratch, a fixed summation order.
+// ---------------------------------------------------------------------------
+constexpr int kKcUnroll = 4, kKcWaves = 4, kKcMaxRows = 4;
+// Columns per wave: two with one row of A (twice the waves in flight measured 8.4 us against 11.2 us with four
+// on the 45 MB case), four with more rows, where the x values a wave loads are shared by more columns.
+constexpr int kc_cols(int rows) { return rows == 1 ? 2 : 4; }
+
+struct GemvKcArgs {
+  const char *x;   // rows of A: K contiguous elements, x_row bytes apart
+  size_t x_row;
+  const char *b;   // column j at b + j * b_col (bytes)
+  size_t b_col;
+  char *y;         // element (i, j) at i * y_row + j * y_s (elements)
+  size_t y_row, y_s;
+  size_t n, kbytes;
+  skl_scalar alpha, beta;
+};
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+  // rows of 16 lanes: four DPP rotations leave the row's sum in every lane; the four rows are then combined
+  // through the cross-lane network (two exchanges per value, once per wave). The row-swap instructions
+  // (v_permlane16_swap / v_permlane32_swap) are not used: given the same value for both operands the
+  // compiler folds the sum of their two results into twice the first one.
+  unsigned u;
+#define SKL_ROTATE_ADD(ctrl)                                                              \
+  u = (unsigned)__builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, false); \
+  v += __builtin_bit_cast(T, u);
+  SKL_ROTATE_ADD(0x128)
+  SKL_ROTATE_ADD(0x124)
+  SKL_ROTATE_ADD(0x122)
+  SKL_ROTATE_ADD(0x121)
+#undef SKL_ROTATE_ADD
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// acc += sum over the 16 bytes of w and x (elements of kind MODE)
+template <int MODE>
+__device__ __forceinline__ void dot16(const uint4 &w, const uint4 &x, typename Mode<MODE>::Acc &acc) {
+  const unsigned ww[4] = {w.x, w.y, w.z, w.w}, xx[4] = {x.x, x.y, x.z, x.w};
+  if constexpr (MODE == kI8RowMajor) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) acc = __builtin_amdgcn_sdot4((int)ww[d], (int)xx[d], acc, false);
+  } else if constexpr (Mode<MODE>::kFp8) {
+    constexpr bool x_e5m2 = MODE == kF8E5M2, b_e5m2 = MODE != kF8E4M3;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const v2f w_lo = b_e5m2 ? __builtin_amdgcn_cvt_pk_f32_bf8((int)ww[d], false) : __builtin_amdgcn_cvt_pk_f32_fp8((int)ww[d], false);
+      const v2f w_hi = b_e5m2 ? __builtin_amdgcn_cvt_pk_f32_bf8((int)ww[d], true) : __builtin_amdgcn_cvt_pk_f32_fp8((int)ww[d], true);
+      const v2f x_lo = x_e5m2 ? __builtin_amdgcn_cvt_pk_f32_bf8((int)xx[d], false) : __builtin_amdgcn_cvt_pk_f32_fp8((int)xx[d], false);
+      const v2f x_hi = x_e5m2 ? __builtin_amdgcn_cvt_pk_f32_bf8((int)xx[d], true) : __builtin_amdgcn_cvt_pk_f32_fp8((int)xx[d], true);
+      acc = __fmaf_rn(x_lo.x, w_lo.x, acc);
+      acc = __fmaf_rn(x_lo.y, w_lo.y, acc);
+      acc = __fmaf_rn(x_hi.x, w_hi.x, acc);
+      acc = __fmaf_rn(x_hi.y, w_hi.y, acc);
+    }
+  } else {
+    constexpr bool bf = MODE == kBF16;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      acc = __fmaf_rn(widen16(xx[d] & 0xFFFFu, bf), widen16(ww[d] & 0xFFFFu, bf), acc);
+      acc = __fmaf_rn(widen16(xx[d] >> 16, bf), widen16(ww[d] >> 16, bf), acc);
+    }
+  }
+}
+
+template <int MODE, int MR>
+__global__ void __launch_bounds__(kKcWaves * 64) gemv_kc_kernel(GemvKcArgs p) {
+  using Acc = typename Mode<MODE>::Acc;
+  constexpr int kKcCols = kc_cols(MR);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const size_t col0 = ((size_t)blockIdx.x * kKcWaves + wave) * kKcCols;
+  if (col0 >= p.n) return;  // whole waves leave; no barrier follows
+  Acc acc[MR][kKcCols];
+#pragma unroll
+  for (int i = 0; i < MR; ++i)
+#pragma unroll
+    for (int c = 0; c < kKcCols; ++c) acc[i][c] = 0;
+  const char *col_ptr[kKcCols];
+#pragma unroll
+  for (int c = 0; c < kKcCols; ++c) {
+    const size_t col = col0 + c < p.n ? col0 + c : p.n - 1;  // a column past the end repeats the last one; not written
+    col_ptr[c] = p.b + col * p.b_col;
+  }
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  for (size_t base = 0; base < p.kbytes; base += (size_t)kKcUnroll * 1024) {
+    uint4 w[kKcUnroll][kKcCols], xs[kKcUnroll][MR];
+    if (base + (size_t)kKcUnroll * 1024 <= p.kbytes) {  // the whole block is inside K: no per-load checks
+#pragma unroll
+      for (int u = 0; u < kKcUnroll; ++u) {
+        const size_t off = base + (size_t)u * 1024 + (size_t)lane * 16;
+#pragma unroll
+        for (int c = 0; c < kKcCols; ++c) w[u][c] = stream_load(col_ptr[c] + off);
+#pragma unroll
+        for (int i = 0; i < MR; ++i) xs[u][i] = *reinterpret_cast<const uint4 *>(p.x + (size_t)i * p.x_row + off);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < kKcUnroll; ++u) {
+        const size_t off = base + (size_t)u * 1024 + (size_t)lane * 16;
+        const bool in = off < p.kbytes;  // K bytes are a multiple of 16: a 16-byte piece is inside or outside
+#pragma unroll
+        for (int c = 0; c < kKcCols; ++c) w[u][c] = in ? stream_load(col_ptr[c] + off) : zero;
+#pragma unroll
+        for (int i = 0; i < MR; ++i) xs[u][i] = in ? *reinterpret_cast<const uint4 *>(p.x + (size_t)i * p.x_row + off) : zero;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kKcUnroll; ++u)
+#pragma unroll
+      for (int i = 0; i < MR; ++i)
+#pragma unroll
+        for (int c = 0; c < kKcCols; ++c) dot16<MODE>(w[u][c], xs[u][i], acc[i][c]);
+  }
+#pragma unroll
+  for (int i = 0; i < MR; ++i)
+#pragma unroll
+    for (int c = 0; c < kKcCols; ++c) acc[i][c] = wave_sum(acc[i][c]);
+  if (lane == 0) {
+    Acc *yv = reinterpret_cast<Acc *>(p.y);
+#pragma unroll
+    for (int i = 0; i < MR; ++i)
+#pragma unroll
+      for (int c = 0; c < kKcCols; ++c)
+        if (col0 + c < p.n) skl_update(acc[i][c], yv + (size_t)i * p.y_row + (col0 + c) * p.y_s, p.alpha, p.beta);
+  }
+}
+
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 int mode_of(const skl_gemm_canon *g, int layout) {
@@ -667,6 +804,41 @@ int launch_rows_of(const skl_gemm_canon *g, const Reduction &red) {
   }
 }
 
+
+template <int MODE, int MR>
+int launch_kc(const skl_gemm_canon *g) {
+  constexpr size_t es = Mode<MODE>::kES;
+  GemvKcArgs p;
+  p.x = (const char *)g->a;
+  p.x_row = g->a_s0 * es;
+  p.b = (const char *)g->b;
+  p.b_col = g->b_s0 * es;
+  p.y = (char *)g->c;
+  p.y_row = g->rsc0;
+  p.y_s = g->csc0;
+  p.n = g->n;
+  p.kbytes = g->k * es;
+  p.alpha = g->alpha;
+  p.beta = g->beta;
+  const size_t grid = (g->n + kKcWaves * kc_cols(MR) - 1) / (kKcWaves * kc_cols(MR));
+  if (grid > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemv: grid too large");
+    return -2;
+  }
+  gemv_kc_kernel<MODE, MR><<<(unsigned)grid, kKcWaves * 64, 0, skl_current_stream()>>>(p);
+  return skl_check_launch("gemv_kc");
+}
+
+template <int MODE>
+int launch_kc_of(const skl_gemm_canon *g) {
+  switch (g->m) {
+    case 1: return launch_kc<MODE, 1>(g);
+    case 2: return launch_kc<MODE, 2>(g);
+    case 3: return launch_kc<MODE, 3>(g);
+    default: return launch_kc<MODE, 4>(g);
+  }
+}
+
 }  // namespace
 
 extern "C" int skl_hip_gemv_supported(const skl_gemm_canon *g, int layout) {
@@ -730,5 +902,34 @@ extern "C" int skl_hip_launch_gemv_rows(const skl_gemm_canon *g) {
     case kF8E4M3: return launch_rows_of<kF8E4M3>(g, red);
     case kF8E5M2: return launch_rows_of<kF8E5M2>(g, red);
     default: return launch_rows_of<kF8Mixed>(g, red);
+  }
+}
+
+// 1 <= M <= 4 against a B whose columns are contiguous in K (16-byte aligned columns and rows of A, K bytes a
+// multiple of 16, columns a fixed distance apart).
+extern "C" int skl_hip_gemv_kc_supported(const skl_gemm_canon *g) {
+  const int mode = mode_of(g, 0);
+  if (mode < 0) return 0;
+  if (g->m < 1 || g->m > (size_t)kKcMaxRows || g->k == 0 || g->n == 0) return 0;
+  const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1;
+  if (g->b_sk != 1 || g->a_sk != 1 || ((g->k * es) % 16) != 0) return 0;
+  if (!aligned16(g->b) || ((g->b_s0 * es) % 16) != 0 || (g->n > 64 && g->b_s1 != 64 * g->b_s0)) return 0;
+  if (!aligned16(g->a) || (g->m > 1 && ((g->a_s0 * es) % 16) != 0)) return 0;
+  if (g->n > 64 && g->csc1 != 64 * g->csc0) return 0;
+  return 1;
+}
+
+extern "C" int skl_hip_launch_gemv_kc(const skl_gemm_canon *g) {
+  if (!skl_hip_gemv_kc_supported(g)) {
+    skl_hip_record_error(-2, "gemv_kc: unsupported problem");
+    return -2;
+  }
+  switch (mode_of(g, 0)) {
+    case kI8RowMajor: return launch_kc_of<kI8RowMajor>(g);
+    case kBF16: return launch_kc_of<kBF16>(g);
+    case kF16: return launch_kc_of<kF16>(g);
+    case kF8E4M3: return launch_kc_of<kF8E4M3>(g);
+    case kF8E5M2: return launch_kc_of<kF8E5M2>(g);
+    default: return launch_kc_of<kF8Mixed>(g);
   }
 }

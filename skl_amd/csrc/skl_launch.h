@@ -88,6 +88,9 @@ int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout);
 /* 2 <= M <= 8 rows against a row-major int8 B: the same stream over B with the transposes shared by the rows. */
 int skl_hip_gemv_rows_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_rows(const skl_gemm_canon *g);
+/* 1 <= M <= 4 against a B with K contiguous (b_sk == 1): one dot product over contiguous memory per output. */
+int skl_hip_gemv_kc_supported(const skl_gemm_canon *g);
+int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
 
 /* pack / unpack over elements of `esize` bytes (1, 2 or 4). */
 int skl_hip_launch_pack(int esize, size_t m, size_t n, const void *src, size_t rs, size_t cs,

@@ -181,3 +181,37 @@ def test_small_batch_rows_floating_point(gpu, ta, tb, m):
             support.assert_fp_gemm_close(case, a, b, c, got)
             again = run_gemm(gpu, "rc", case, a, b, c, mode)
             support.assert_fp_gemm_close(case, a, b, c, again)
+
+
+def _kc_case(ta, tb, m, n, k, alpha, beta, pad=0):
+    """Row-major A (m x k), B with K contiguous (column j at j * (k + pad)), row-major C."""
+    return GemmCase(ta, tb, alpha, beta, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=k + pad, csa1=1,
+                    rsb0=0, csb0=0, rsb1=1, csb1=k + pad, rsc0=0, csc0=0, rsc1=n + 5, csc1=1)
+
+
+@pytest.mark.parametrize("m", (1, 2, 3, 4))
+def test_k_contiguous_b_int8_bit_exact(gpu, m):
+    """B stored column by column (a linear layer's [out][in] weight): one dot product over contiguous memory per
+    output, no sums between workgroups. Config-2 sizes, K tails of every residue of 16 bytes per KiB, few columns."""
+    rng = np.random.default_rng(60 + m)
+    for (n, k, pad) in ((11008, 4096, 0), (1037, 4096 + 16, 16), (5, 16, 0), (70, 1008, 32), (513, 5040, 0)):
+        for alpha, beta in ((1, 0), (-3, 2)):
+            case = _kc_case("i8", None, m, n, k, alpha, beta, pad)
+            a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+            want = run_oracle_gemm(case, a, b, c)
+            for mode in ("device", "host"):
+                assert np.array_equal(run_gemm(gpu, "rc", case, a, b, c, mode), want), (m, n, k, mode)
+
+
+@pytest.mark.parametrize("ta,tb", (("bf16", "bf16"), ("f16", "f16")) + FP8_PAIRS)
+@pytest.mark.parametrize("m", (1, 4))
+def test_k_contiguous_b_floating_point(gpu, ta, tb, m):
+    """Same layout for bf16 / f16 / fp8: fp32 accumulation in a fixed order - inside the reference's bound,
+    and the same bits on every run."""
+    for (n, k, pad) in ((11008, 4096, 0), (1037, 1040, 16), (5, 16, 0)):
+        case = _kc_case(ta, tb, m, n, k, 1.5, -0.5, pad)
+        a, b, c = case.make_inputs(m * 31 + n + k)
+        for mode in ("device", "host"):
+            got = run_gemm(gpu, "rc", case, a, b, c, mode)
+            support.assert_fp_gemm_close(case, a, b, c, got)
+            assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
