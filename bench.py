@@ -234,6 +234,27 @@ def wl_gemm_f8_8192(lib, rng, fmt_b="f8e4m3"):
                 name=name, kernel="gemm_mfma_ring_kernel")
 
 
+def wl_gemm_f8_layout(a_rows_contig, b_cols_contig):
+    """The same fp8 product through the full-stride (rc) entry point with other operand layouts: the A and B
+    buffers are random fp8 data either way, only the strides the call passes differ."""
+    def build(lib, rng):
+        m = n = k = 8192
+        a = _fp8_operand(lib, rng, m * k, "f8e4m3")
+        b = _fp8_operand(lib, rng, k * n, "f8e4m3")
+        c = DeviceBuffer.from_array(np.zeros(m * n, np.float32))
+        rsa, csa = (k, 1) if a_rows_contig else (1, m)
+        rsb, csb = (1, k) if b_cols_contig else (n, 1)
+
+        def step(i):
+            lib.skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950(m, n, k, 1.0, a, rsa, csa, b, rsb, csb, 0.0, c, n, 1)
+
+        name = (f"fp8 E4M3xE4M3 GEMM 8192^3 ({'row' if a_rows_contig else 'column'}-major A, "
+                f"{'column' if b_cols_contig else 'row'}-major B, alpha=1, beta=0)")
+        return dict(fn=step, bytes=m * k + k * n + 8 * m * n, ops=2 * m * n * k, bound="mfma", dtype="f8",
+                    keep=(a, b, c), name=name, kernel="gemm_mfma_ring_kernel")
+    return build
+
+
 def wl_gemm_bf16(lib, rng):
     m, n, k = 2048, 4096, 4096
     return _dense(lib, rng, "bf16 GEMM 2048x4096x4096 (row-major, alpha=1, beta=1)", "skl_gemm_bf16_bf16_f32_gfx950",
@@ -314,6 +335,8 @@ WORKLOADS = {
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2),
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2),
+    "gemm_f8e4m3_8192_rowmajor_a": (wl_gemm_f8_layout(True, False), 10, 2),
+    "gemm_f8e4m3_8192_kcontig": (wl_gemm_f8_layout(True, True), 10, 2),
     "gemm_bf16_2048x4096x4096": (wl_gemm_bf16, 20, 3),
     "pipeline_f16_4096x4096x14336": (wl_f16_pipeline, 5, 1),
     "gemm_i8_512": (wl_gemm_i8_512, 200, 20),
