@@ -150,6 +150,69 @@ static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g) {
   return 1;
 }
 
+/* The streaming kernels in the order they are tried; 1 if one of them took the problem. */
+static int gemv_on_device(const skl_gemm_canon *g) {
+  if (skl_hip_gemv_kc_supported(g)) return skl_hip_launch_gemv_kc(g), 1;
+  if (g->m == 1 && skl_hip_gemv_supported(g, 0)) return skl_hip_launch_gemv(g, 0), 1;
+  if (skl_hip_gemv_rows_supported(g)) return skl_hip_launch_gemv_rows(g), 1;
+  return 0;
+}
+
+/* C^T = B^T A^T: a problem with a few columns (matrix times vector, the reference's "small-N" regime,
+ * src/gemm/README.md:126) is a problem with a few rows once the roles of A and B are exchanged. Products
+ * commute exactly and the order of the sum over k is untouched, so the result is the same. */
+static void transposed_view(const skl_gemm_canon *g, skl_gemm_canon *t) {
+  *t = *g;
+  t->ta = g->tb;
+  t->tb = g->ta;
+  t->m = g->n;
+  t->n = g->m;
+  t->a = g->b;
+  t->a_s0 = g->b_s0;
+  t->a_s1 = g->b_s1;
+  t->a_sk = g->b_sk;
+  t->b = g->a;
+  t->b_s0 = g->a_s0;
+  t->b_s1 = g->a_s1;
+  t->b_sk = g->a_sk;
+  t->rsc0 = g->csc0;
+  t->rsc1 = g->csc1;
+  t->csc0 = g->rsc0;
+  t->csc1 = g->rsc1;
+}
+
+/* 1 if `g` (possibly with the roles exchanged) has a kernel other than the any-stride one. */
+static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
+  skl_gemm_canon t;
+  if (!fused && g->n <= 8 && g->n < g->m) {
+    transposed_view(g, &t);
+    if (launch ? gemv_on_device(&t)
+               : (skl_hip_gemv_kc_supported(&t) || (t.m == 1 && skl_hip_gemv_supported(&t, 0)) ||
+                  skl_hip_gemv_rows_supported(&t)))
+      return 1;
+  }
+  if (skl_hip_gemm_mfma_supported(g)) return launch ? (skl_hip_launch_gemm_mfma(g), 1) : 1;
+  return 0;
+}
+
+/* B has few columns (at most 64, fewer than C has rows) and a layout that none of the kernels reads - typically
+ * the row-major k x n matrix of a matrix-vector product, whose rows are shorter than 16 bytes. Such a B is small:
+ * it is copied into scratch memory as columns contiguous in K, 16-byte aligned, and the problem runs on that copy. */
+static int gemm_with_gathered_b(const skl_gemm_canon *g, int fused) {
+  skl_gemm_canon h = *g;
+  const size_t es = elem_size(g->tb);
+  const size_t kp = (g->k * es + 15) / 16 * 16 / es;
+  if (g->n > SKL_TE || g->n >= g->m || es > 2) return 0;
+  h.b = (const void *)(uintptr_t)256; /* stands for the aligned copy while asking who would take it */
+  h.b_sk = 1;
+  h.b_s0 = kp;
+  h.b_s1 = SKL_TE * kp;
+  if (!gemm_fast_path(&h, fused, 0)) return 0;
+  h.b = skl_hip_gather_columns((int)es, g->n, g->k, g->b, g->b_s0, g->b_s1, g->b_sk, kp);
+  if (!h.b) return 0;
+  return gemm_fast_path(&h, fused, 1);
+}
+
 static void gemm_on_device(const skl_gemm_desc *d) {
   skl_gemm_canon g;
   const int fused = d->bias != NULL || d->max != NULL; /* the M = 1 kernels have no fused steps */
@@ -159,21 +222,13 @@ static void gemm_on_device(const skl_gemm_desc *d) {
       return;
     }
     if (canonicalize(d, &g)) {
-      if (!fused && skl_hip_gemv_kc_supported(&g)) {
-        skl_hip_launch_gemv_kc(&g);
-        return;
-      }
-      if (!fused && g.m == 1 && skl_hip_gemv_supported(&g, 0)) {
-        skl_hip_launch_gemv(&g, 0);
-        return;
-      }
-      if (!fused && skl_hip_gemv_rows_supported(&g)) {
-        skl_hip_launch_gemv_rows(&g);
-        return;
-      }
-      if (skl_hip_gemm_mfma_supported(&g)) {
-        skl_hip_launch_gemm_mfma(&g);
-        return;
+      if (!fused && gemv_on_device(&g)) return;
+      if (gemm_fast_path(&g, fused, 1)) return;
+      if (gemm_with_gathered_b(&g, fused)) return;
+      if (!fused) { /* the same for an A of few rows: it is the B of the exchanged problem */
+        skl_gemm_canon t;
+        transposed_view(&g, &t);
+        if (gemm_with_gathered_b(&t, 0)) return;
       }
     }
   }

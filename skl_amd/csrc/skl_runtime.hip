@@ -17,6 +17,7 @@ constexpr int kMaxDevices = 16;
 struct DeviceState {
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
+  void *operand_scratch = nullptr;  // kOperandScratchBytes, allocated on first use, never moved
 };
 
 std::mutex g_mutex;
@@ -74,6 +75,20 @@ void *skl_workspace(size_t bytes) {
   return p;
 }
 
+void *skl_operand_scratch(size_t bytes) {
+  if (bytes > kOperandScratchBytes) return nullptr;
+  int dev = 0;
+  if (skl_check_hip(hipGetDevice(&dev), "hipGetDevice") != 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  DeviceState &st = g_devices[dev];
+  if (!st.operand_scratch && hipMalloc(&st.operand_scratch, kOperandScratchBytes) != hipSuccess) {
+    (void)hipGetLastError();
+    st.operand_scratch = nullptr;
+    skl_hip_record_error(SKL_HIP_ERR_WORKSPACE, "skl_operand_scratch");
+  }
+  return st.operand_scratch;
+}
+
 extern "C" {
 
 int skl_hip_init(int device) {
@@ -100,10 +115,11 @@ void skl_hip_shutdown(void) {
     return;
   }
   for (int d = 0; d < kMaxDevices; ++d) {
-    if (!g_devices[d].workspace) continue;
+    if (!g_devices[d].workspace && !g_devices[d].operand_scratch) continue;
     if (hipSetDevice(d) == hipSuccess) {
       (void)hipDeviceSynchronize();
-      (void)hipFree(g_devices[d].workspace);
+      if (g_devices[d].workspace) (void)hipFree(g_devices[d].workspace);
+      if (g_devices[d].operand_scratch) (void)hipFree(g_devices[d].operand_scratch);
     }
     g_devices[d] = DeviceState{};
   }

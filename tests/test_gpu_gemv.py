@@ -215,3 +215,60 @@ def test_k_contiguous_b_floating_point(gpu, ta, tb, m):
             got = run_gemm(gpu, "rc", case, a, b, c, mode)
             support.assert_fp_gemm_close(case, a, b, c, got)
             assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
+
+
+def _few_columns_case(ta, tb, m, n, k, alpha, beta, a_rows_contiguous, b_cols_contiguous, pad=0):
+    """A tall problem with 1..8 columns: A row-major (lda = k + pad) or column-major (lda = m + pad); B column by
+    column (a vector with unit stride when n == 1) or row-major; C row-major with a padded row."""
+    rsa, csa = (k + pad, 1) if a_rows_contiguous else (1, m + pad)
+    rsb, csb = (1, k + pad) if b_cols_contiguous else (n, 1)
+    return GemmCase(ta, tb, alpha, beta, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=rsa, csa1=csa,
+                    rsb0=0, csb0=0, rsb1=rsb, csb1=csb, rsc0=0, csc0=0, rsc1=n + 3, csc1=1)
+
+
+@pytest.mark.parametrize("n", (1, 2, 3, 4, 8))
+def test_few_columns_int8_bit_exact(gpu, n):
+    """Matrix times vector (and up to 8 vectors): served by the streaming kernels with the roles of A and B
+    exchanged. Every pairing of operand layouts, sizes on and off the kernels' alignment rules (those fall back
+    to the tile kernels) - all bit-exact."""
+    rng = np.random.default_rng(90 + n)
+    for (m, k, pad) in ((11008, 4096, 0), (1037, 1040, 16), (5, 16, 0), (513, 1000, 0), (4096, 4096, 64)):
+        for a_rows in (True, False):
+            for b_cols in (True, False):
+                for alpha, beta in ((1, 0), (-3, 2)):
+                    case = _few_columns_case("i8", None, m, n, k, alpha, beta, a_rows, b_cols, pad)
+                    a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+                    want = run_oracle_gemm(case, a, b, c)
+                    got = run_gemm(gpu, "rc", case, a, b, c, "device")
+                    assert np.array_equal(got, want), (m, n, k, a_rows, b_cols, alpha, beta)
+
+
+@pytest.mark.parametrize("ta,tb", (("bf16", "bf16"), ("f16", "f16")) + FP8_PAIRS)
+@pytest.mark.parametrize("n", (1, 3))
+def test_few_columns_floating_point(gpu, ta, tb, n):
+    """The E4M3 x E5M2 pair has no exchanged form on the streaming kernels (they decode the vector as E4M3) and
+    runs on the matrix-core kernels, whose fp8 summation term is allowed for."""
+    extra = support.FP8_MFMA_REL if ta != tb else 0.0
+    for (m, k, pad) in ((11008, 4096, 0), (1037, 1040, 16), (5, 16, 0)):
+        for a_rows in (True, False):
+            case = _few_columns_case(ta, tb, m, n, k, 1.5, -0.5, a_rows, True, pad)
+            a, b, c = case.make_inputs(n * 17 + m + k)
+            for mode in ("device", "host"):
+                got = run_gemm(gpu, "rc", case, a, b, c, mode)
+                support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=extra)
+
+
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f8e4m3"))
+def test_few_rows_of_a_in_a_layout_no_kernel_reads(gpu, ta):
+    """A with 2..40 rows stored column by column (rows 2..40 elements apart: below the kernels' 16-byte rule): A is
+    copied into scratch memory with K contiguous and the problem leaves the any-stride kernel. int8 bit-exact."""
+    for (m, n, k) in ((2, 11008, 4096), (3, 1040, 1000), (7, 4096, 512), (40, 2048, 777)):
+        case = GemmCase(ta, None, 2 if ta == "i8" else 1.5, 1 if ta == "i8" else -0.5, m0=1, n0=1, k0=1, m1=m, n1=n,
+                        k1=k, rsa0=0, csa0=0, rsa1=1, csa1=m, rsb0=0, csb0=0, rsb1=n, csb1=1, rsc0=0, csc0=0,
+                        rsc1=n, csc1=1)
+        a, b, c = case.make_inputs(m + n + k)
+        got = run_gemm(gpu, "rc", case, a, b, c, "device")
+        if ta == "i8":
+            assert np.array_equal(got, run_oracle_gemm(case, a, b, c)), (m, n, k)
+        else:
+            support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=support.FP8_MFMA_REL if ta.startswith("f8") else 0.0)
