@@ -158,6 +158,10 @@ static int gemv_on_device(const skl_gemm_canon *g) {
   return 0;
 }
 
+static int gemv_would_take(const skl_gemm_canon *g) {
+  return skl_hip_gemv_kc_supported(g) || (g->m == 1 && skl_hip_gemv_supported(g, 0)) || skl_hip_gemv_rows_supported(g);
+}
+
 /* C^T = B^T A^T: a problem with a few columns (matrix times vector, the reference's "small-N" regime,
  * src/gemm/README.md:126) is a problem with a few rows once the roles of A and B are exchanged. Products
  * commute exactly and the order of the sum over k is untouched, so the result is the same. */
@@ -181,36 +185,57 @@ static void transposed_view(const skl_gemm_canon *g, skl_gemm_canon *t) {
   t->csc1 = g->rsc1;
 }
 
-/* 1 if `g` (possibly with the roles exchanged) has a kernel other than the any-stride one. */
+/* Offers `g` to every kernel but the any-stride one; 1 if one of them takes it. With `launch` == 0 only asks. */
 static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
   skl_gemm_canon t;
-  if (!fused && g->n <= 8 && g->n < g->m) {
-    transposed_view(g, &t);
-    if (launch ? gemv_on_device(&t)
-               : (skl_hip_gemv_kc_supported(&t) || (t.m == 1 && skl_hip_gemv_supported(&t, 0)) ||
-                  skl_hip_gemv_rows_supported(&t)))
-      return 1;
+  if (!fused) {
+    if (launch ? gemv_on_device(g) : gemv_would_take(g)) return 1;
+    if (g->n <= 8 && g->n < g->m) {
+      transposed_view(g, &t);
+      if (launch ? gemv_on_device(&t) : gemv_would_take(&t)) return 1;
+    }
   }
   if (skl_hip_gemm_mfma_supported(g)) return launch ? (skl_hip_launch_gemm_mfma(g), 1) : 1;
   return 0;
 }
 
-/* B has few columns (at most 64, fewer than C has rows) and a layout that none of the kernels reads - typically
- * the row-major k x n matrix of a matrix-vector product, whose rows are shorter than 16 bytes. Such a B is small:
- * it is copied into scratch memory as columns contiguous in K, 16-byte aligned, and the problem runs on that copy. */
-static int gemm_with_gathered_b(const skl_gemm_canon *g, int fused) {
-  skl_gemm_canon h = *g;
-  const size_t es = elem_size(g->tb);
-  const size_t kp = (g->k * es + 15) / 16 * 16 / es;
-  if (g->n > SKL_TE || g->n >= g->m || es > 2) return 0;
-  h.b = (const void *)(uintptr_t)256; /* stands for the aligned copy while asking who would take it */
-  h.b_sk = 1;
-  h.b_s0 = kp;
-  h.b_s1 = SKL_TE * kp;
-  if (!gemm_fast_path(&h, fused, 0)) return 0;
-  h.b = skl_hip_gather_columns((int)es, g->n, g->k, g->b, g->b_s0, g->b_s1, g->b_sk, kp);
-  if (!h.b) return 0;
-  return gemm_fast_path(&h, fused, 1);
+/* An operand in a layout that none of the kernels reads - a leading dimension that is not a multiple of 16 bytes,
+ * the row-major k x n matrix of a matrix-vector product, no unit stride at all - is copied into scratch memory as
+ * rows contiguous in K, 16-byte aligned, and the problem runs on the copy: B alone, A alone, or both, whichever
+ * the kernels accept first. Worth a copy only when the product is not tiny. */
+static int gemm_with_realigned_operands(const skl_gemm_canon *g, int fused) {
+  const size_t esa = elem_size(g->ta), esb = elem_size(g->tb);
+  const size_t kpa = (g->k * esa + 15) / 16 * 16 / esa, kpb = (g->k * esb + 15) / 16 * 16 / esb;
+  const size_t bytes_a = (g->m * kpa * esa + 255) / 256 * 256, bytes_b = g->n * kpb * esb;
+  int which;
+  if (esa > 2 || esb > 2 || g->m * g->n * g->k < ((size_t)1 << 18)) return 0;
+  for (which = 1; which <= 3; ++which) { /* 1: B, 2: A, 3: both */
+    skl_gemm_canon h = *g;
+    const int copy_a = (which & 2) != 0, copy_b = (which & 1) != 0;
+    char *scratch;
+    if (copy_a) {
+      h.a = (const void *)(uintptr_t)256; /* stands for the aligned copy while asking who would take it */
+      h.a_sk = 1, h.a_s0 = kpa, h.a_s1 = SKL_TE * kpa;
+    }
+    if (copy_b) {
+      h.b = (const void *)(uintptr_t)256;
+      h.b_sk = 1, h.b_s0 = kpb, h.b_s1 = SKL_TE * kpb;
+    }
+    if (!gemm_fast_path(&h, fused, 0)) continue;
+    scratch = skl_hip_operand_scratch((copy_a ? bytes_a : 0) + (copy_b ? bytes_b : 0));
+    if (!scratch) return 0;
+    if (copy_a) {
+      if (skl_hip_launch_realign((int)esa, g->m, g->k, g->a, g->a_s0, g->a_s1, g->a_sk, scratch, kpa) != 0) return 0;
+      h.a = scratch;
+      scratch += bytes_a;
+    }
+    if (copy_b) {
+      if (skl_hip_launch_realign((int)esb, g->n, g->k, g->b, g->b_s0, g->b_s1, g->b_sk, scratch, kpb) != 0) return 0;
+      h.b = scratch;
+    }
+    return gemm_fast_path(&h, fused, 1);
+  }
+  return 0;
 }
 
 static void gemm_on_device(const skl_gemm_desc *d) {
@@ -222,14 +247,8 @@ static void gemm_on_device(const skl_gemm_desc *d) {
       return;
     }
     if (canonicalize(d, &g)) {
-      if (!fused && gemv_on_device(&g)) return;
       if (gemm_fast_path(&g, fused, 1)) return;
-      if (gemm_with_gathered_b(&g, fused)) return;
-      if (!fused) { /* the same for an A of few rows: it is the B of the exchanged problem */
-        skl_gemm_canon t;
-        transposed_view(&g, &t);
-        if (gemm_with_gathered_b(&t, 0)) return;
-      }
+      if (gemm_with_realigned_operands(&g, fused)) return;
     }
   }
   skl_hip_launch_gemm_generic(d);

@@ -14,11 +14,6 @@ hipStream_t skl_current_stream();
 // only meaningful inside one launch sequence on one stream.
 void *skl_workspace(size_t bytes);
 
-// A second, fixed block per device for a small operand copied into another layout ahead of a launch that may itself
-// use (and grow) the workspace. nullptr if `bytes` exceeds its size. Same ordering rule as the workspace.
-constexpr size_t kOperandScratchBytes = size_t(4) << 20;
-void *skl_operand_scratch(size_t bytes);
-
 // Records a HIP failure for skl_hip_last_error() and returns its code.
 int skl_check_hip(hipError_t e, const char *what);
 

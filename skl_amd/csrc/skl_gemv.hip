@@ -844,28 +844,6 @@ int launch_kc_of(const skl_gemm_canon *g) {
 
 }  // namespace
 
-// dst[j * kp + p] = B(p, j) for p < k, zero up to kp: a few columns of any layout as rows contiguous in K.
-template <typename T>
-__global__ void __launch_bounds__(256) gather_columns_kernel(const T *__restrict__ b, size_t s0, size_t s1, size_t sk,
-                                                             T *__restrict__ dst, size_t n, size_t k, size_t kp) {
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= n * kp) return;
-  const size_t j = idx / kp, p = idx % kp;
-  dst[idx] = p < k ? b[(j / 64) * s1 + (j % 64) * s0 + p * sk] : T(0);
-}
-
-extern "C" void *skl_hip_gather_columns(int esize, size_t n, size_t k, const void *b, size_t s0, size_t s1, size_t sk,
-                                        size_t kp) {
-  void *dst = skl_operand_scratch(n * kp * (size_t)esize);
-  if (!dst) return nullptr;
-  const unsigned grid = skl_div_up(n * kp, 256);
-  if (esize == 1)
-    gather_columns_kernel<uint8_t><<<grid, 256, 0, skl_current_stream()>>>((const uint8_t *)b, s0, s1, sk, (uint8_t *)dst, n, k, kp);
-  else
-    gather_columns_kernel<uint16_t><<<grid, 256, 0, skl_current_stream()>>>((const uint16_t *)b, s0, s1, sk, (uint16_t *)dst, n, k, kp);
-  return skl_check_launch("gather_columns") == 0 ? dst : nullptr;
-}
-
 extern "C" int skl_hip_gemv_supported(const skl_gemm_canon *g, int layout) {
   const int mode = mode_of(g, layout);
   if (mode < 0) return 0;

@@ -92,11 +92,13 @@ int skl_hip_launch_gemv_rows(const skl_gemm_canon *g);
 int skl_hip_gemv_kc_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
 
-/* Copies the n columns of a small B (element (p, j) at (j/64)*s1 + (j%64)*s0 + p*sk, `esize` 1 or 2 bytes) into a
- * per-device scratch block as n rows contiguous in K, kp >= k elements apart and zero-filled beyond k. Returns the
- * copy, or NULL when n*kp*esize exceeds the block (4 MiB) or the launch failed. Ordered on the current stream. */
-void *skl_hip_gather_columns(int esize, size_t n, size_t k, const void *b, size_t s0, size_t s1, size_t sk,
-                             size_t kp);
+/* A block of per-device scratch memory for operands copied into another layout ahead of a launch (grows on demand;
+ * ordered on the current stream like the workspace of the split reductions, which it does not share). */
+void *skl_hip_operand_scratch(size_t bytes);
+/* Copies a GEMM operand in the canonical description (element (x, p) at (x/64)*s1 + (x%64)*s0 + p*sk, `esize` 1 or
+ * 2 bytes) into rows contiguous in K: dst[x*kp + p], zero-filled for k <= p < kp. */
+int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_t s0, size_t s1, size_t sk,
+                           void *dst, size_t kp);
 
 /* pack / unpack over elements of `esize` bytes (1, 2 or 4). */
 int skl_hip_launch_pack(int esize, size_t m, size_t n, const void *src, size_t rs, size_t cs,

@@ -33,6 +33,25 @@ struct PackArgs {
   int blocked_along_c;  // lanes run along columns when touching the blocked matrix
 };
 
+template <typename T>
+__global__ void __launch_bounds__(kThreads) realign_kernel(const T *__restrict__ src, T *__restrict__ dst, size_t x, size_t k,
+                                                           size_t kp, size_t s0, size_t s1, size_t sk, unsigned tiles_p,
+                                                           int along_x) {
+  __shared__ T tile[kTile][kTile + 3];  // [p][x]
+  const size_t x0 = (size_t)(blockIdx.x / tiles_p) * kTile, p0 = (size_t)(blockIdx.x % tiles_p) * kTile;
+  const int fast = threadIdx.x % kTile, slow = threadIdx.x / kTile;
+  for (int it = slow; it < kTile; it += kThreads / kTile) {
+    const int xi = along_x ? fast : it, pi = along_x ? it : fast;
+    const size_t xx = x0 + xi, pp = p0 + pi;
+    tile[pi][xi] = (xx < x && pp < k) ? src[(xx / 64) * s1 + (xx % 64) * s0 + pp * sk] : T(0);
+  }
+  __syncthreads();
+  for (int it = slow; it < kTile; it += kThreads / kTile) {
+    const size_t xx = x0 + it, pp = p0 + fast;
+    if (xx < x && pp < kp) dst[xx * kp + pp] = tile[fast][it];
+  }
+}
+
 template <typename T, bool PACK>
 __global__ void __launch_bounds__(kThreads) pack_tile_kernel(const T *__restrict__ src, T *__restrict__ dst, PackArgs p) {
   __shared__ T tile[kTile][kTile + (sizeof(T) == 4 ? 1 : sizeof(T) == 2 ? 2 : 4)];
@@ -319,6 +338,28 @@ int skl_hip_launch_unpack(int esize, size_t m0, size_t n0, const void *src, size
   const size_t eff_rs0 = m0 > 1 ? rs0 : rs1, eff_cs0 = n0 > 1 ? cs0 : cs1;
   p.blocked_along_c = eff_cs0 <= eff_rs0;
   return dispatch(esize, false, src, dst, p);
+}
+
+// A GEMM operand in the canonical blocked description - element (x, p) at (x/64)*s1 + (x%64)*s0 + p*sk, x along M
+// or N, p along K - copied into rows contiguous in K: dst[x*kp + p], zero for k <= p < kp. 64 x 64 tiles through
+// LDS, read with lanes along x when the source is contiguous there and along p otherwise, written along p.
+int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_t s0, size_t s1, size_t sk,
+                           void *dst, size_t kp) {
+  if (x == 0 || kp == 0) return 0;
+  const size_t tiles_p = (kp + kTile - 1) / kTile, tiles = ((x + kTile - 1) / kTile) * tiles_p;
+  if (tiles > 0x7FFFFFFFu || (esize != 1 && esize != 2)) {
+    skl_hip_record_error(-2, "realign: problem too large");
+    return -2;
+  }
+  const int along_x = s0 == 1 && sk != 1;
+  hipStream_t st = skl_current_stream();
+  if (esize == 1)
+    realign_kernel<uint8_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint8_t *)src, (uint8_t *)dst, x, k, kp, s0, s1, sk,
+                                                                (unsigned)tiles_p, along_x);
+  else
+    realign_kernel<uint16_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint16_t *)src, (uint16_t *)dst, x, k, kp, s0, s1,
+                                                                 sk, (unsigned)tiles_p, along_x);
+  return skl_check_launch("realign");
 }
 
 }  // extern "C"

@@ -17,7 +17,8 @@ constexpr int kMaxDevices = 16;
 struct DeviceState {
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
-  void *operand_scratch = nullptr;  // kOperandScratchBytes, allocated on first use, never moved
+  void *operand_scratch = nullptr;  // copies of operands in another layout; apart from the workspace so that
+  size_t operand_bytes = 0;         // a launch that grows the workspace keeps the copies it was given
 };
 
 std::mutex g_mutex;
@@ -75,20 +76,6 @@ void *skl_workspace(size_t bytes) {
   return p;
 }
 
-void *skl_operand_scratch(size_t bytes) {
-  if (bytes > kOperandScratchBytes) return nullptr;
-  int dev = 0;
-  if (skl_check_hip(hipGetDevice(&dev), "hipGetDevice") != 0 || dev >= kMaxDevices) return nullptr;
-  std::lock_guard<std::mutex> lock(g_mutex);
-  DeviceState &st = g_devices[dev];
-  if (!st.operand_scratch && hipMalloc(&st.operand_scratch, kOperandScratchBytes) != hipSuccess) {
-    (void)hipGetLastError();
-    st.operand_scratch = nullptr;
-    skl_hip_record_error(SKL_HIP_ERR_WORKSPACE, "skl_operand_scratch");
-  }
-  return st.operand_scratch;
-}
-
 extern "C" {
 
 int skl_hip_init(int device) {
@@ -105,6 +92,29 @@ int skl_hip_init(int device) {
   int rc = skl_check_hip(hipSetDevice(device), "hipSetDevice");
   if (rc != 0) return rc;
   return skl_workspace(1) ? SKL_HIP_OK : SKL_HIP_ERR_WORKSPACE;
+}
+
+void *skl_hip_operand_scratch(size_t bytes) {
+  int dev = 0;
+  if (skl_check_hip(hipGetDevice(&dev), "hipGetDevice") != 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  DeviceState &st = g_devices[dev];
+  if (st.operand_bytes >= bytes && st.operand_scratch) return st.operand_scratch;
+  if (st.operand_scratch) {
+    // Earlier launches may still read the old block.
+    if (skl_check_hip(hipDeviceSynchronize(), "operand scratch grow: synchronize") != 0) return nullptr;
+    (void)hipFree(st.operand_scratch);
+    st.operand_scratch = nullptr;
+    st.operand_bytes = 0;
+  }
+  const size_t want = bytes < (size_t(4) << 20) ? (size_t(4) << 20) : bytes;
+  if (hipMalloc(&st.operand_scratch, want) != hipSuccess) {
+    (void)hipGetLastError();  // the caller falls back to a kernel that needs no copy
+    st.operand_scratch = nullptr;
+    return nullptr;
+  }
+  st.operand_bytes = want;
+  return st.operand_scratch;
 }
 
 void skl_hip_shutdown(void) {

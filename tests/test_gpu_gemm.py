@@ -366,3 +366,25 @@ def test_whole_tile_streaming_kernel(gpu, ta, a_kc, b_kc, m, n):
         bound = (gamma + extra) * abs(alpha) * (np.abs(A) @ np.abs(B)) + gamma * abs(beta) * np.abs(C)
         err = np.abs(got[oc] - exact)
         assert np.all(err <= bound + np.abs(exact) * 2.0 ** -22), float((err / (bound + 1e-30)).max())
+
+
+@pytest.mark.parametrize("ta,tb", (("i8", "i8"), ("bf16", "bf16"), ("f16", "f16"), ("f8e4m3", "f8e5m2")))
+def test_leading_dimensions_off_the_16_byte_rule(gpu, ta, tb):
+    """Operands whose leading dimension is not a multiple of 16 bytes, or that have no unit stride at all, are
+    copied into aligned scratch memory and multiplied by the matrix-core kernels instead of the any-stride one:
+    A alone, B alone, both; row- and column-major. Same bar as everywhere: int8 bit-exact over the whole C buffer,
+    floating point inside the reference's bound."""
+    from support import GemmCase
+    m, n, k = 300, 260, 777
+    layouts = {  # (rsa, csa), (rsb, csb)
+        "A odd lda": ((k + 1, 1), (n + 12, 1)),
+        "B odd ldb": ((k + 7, 1), (n + 1, 1)),
+        "both odd": ((k, 1), (n + 3, 1)),
+        "column-major, odd": ((1, m + 1), (1, k + 5)),
+        "no unit stride": ((2 * k, 2), (3 * n, 3)),
+    }
+    for name, ((rsa, csa), (rsb, csb)) in layouts.items():
+        alpha, beta = (2, -1) if ta == "i8" else (1.5, -0.5)
+        case = GemmCase(ta, tb, alpha, beta, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=rsa, csa1=csa,
+                        rsb0=0, csb0=0, rsb1=rsb, csb1=csb, rsc0=0, csc0=0, rsc1=n + 2, csc1=1)
+        check(gpu, "rc", case, 7000 + len(name), "device")
