@@ -207,7 +207,7 @@ static int gemm_with_realigned_operands(const skl_gemm_canon *g, int fused) {
   const size_t esa = elem_size(g->ta), esb = elem_size(g->tb);
   const size_t kpa = (g->k * esa + 15) / 16 * 16 / esa, kpb = (g->k * esb + 15) / 16 * 16 / esb;
   const size_t bytes_a = (g->m * kpa * esa + 255) / 256 * 256, bytes_b = g->n * kpb * esb;
-  int which;
+  int which, done;
   if (esa > 2 || esb > 2 || g->m * g->n * g->k < ((size_t)1 << 18)) return 0;
   for (which = 1; which <= 3; ++which) { /* 1: B, 2: A, 3: both */
     skl_gemm_canon h = *g;
@@ -222,18 +222,21 @@ static int gemm_with_realigned_operands(const skl_gemm_canon *g, int fused) {
       h.b_sk = 1, h.b_s0 = kpb, h.b_s1 = SKL_TE * kpb;
     }
     if (!gemm_fast_path(&h, fused, 0)) continue;
+    skl_hip_sequence_begin();
     scratch = skl_hip_operand_scratch((copy_a ? bytes_a : 0) + (copy_b ? bytes_b : 0));
-    if (!scratch) return 0;
-    if (copy_a) {
-      if (skl_hip_launch_realign((int)esa, g->m, g->k, g->a, g->a_s0, g->a_s1, g->a_sk, scratch, kpa) != 0) return 0;
+    done = scratch != NULL;
+    if (done && copy_a) {
+      done = skl_hip_launch_realign((int)esa, g->m, g->k, g->a, g->a_s0, g->a_s1, g->a_sk, scratch, kpa) == 0;
       h.a = scratch;
       scratch += bytes_a;
     }
-    if (copy_b) {
-      if (skl_hip_launch_realign((int)esb, g->n, g->k, g->b, g->b_s0, g->b_s1, g->b_sk, scratch, kpb) != 0) return 0;
+    if (done && copy_b) {
+      done = skl_hip_launch_realign((int)esb, g->n, g->k, g->b, g->b_s0, g->b_s1, g->b_sk, scratch, kpb) == 0;
       h.b = scratch;
     }
-    return gemm_fast_path(&h, fused, 1);
+    if (done) done = gemm_fast_path(&h, fused, 1);
+    skl_hip_sequence_end();
+    return done;
   }
   return 0;
 }

@@ -1018,6 +1018,12 @@ __global__ void __launch_bounds__(256) gemm_split_reduce_kernel(MfmaArgs p) {
 
 // How many ways K is shared out when a problem has too few tiles for the chip: enough to put about two
 // workgroups on every compute unit, each share at least kMinSlicesPerSplit slices long, planes within 64 MiB.
+struct SequenceGuard {
+  const bool held;
+  explicit SequenceGuard(bool hold) : held(hold) { if (held) skl_hip_sequence_begin(); }
+  ~SequenceGuard() { if (held) skl_hip_sequence_end(); }
+};
+
 constexpr size_t kMinSlicesPerSplit = 8, kSplitFromSlices = 32, kSplitPlaneLimit = size_t(64) << 20;
 inline unsigned splits_for(size_t tiles, size_t slices, size_t m, size_t n) {
   if (tiles >= 256 || slices < kSplitFromSlices) return 1;
@@ -1049,6 +1055,7 @@ int launch_one(const MfmaArgs &args) {
   p.splits = splits_for(tiles, slices, p.m, p.n);
   p.slices_per_split = (unsigned)((slices + p.splits - 1) / p.splits);
   p.splits = (unsigned)((slices + p.slices_per_split - 1) / p.slices_per_split);  // no empty share
+  SequenceGuard sequence(p.splits > 1);  // the partial sums travel from this kernel to the next through the workspace
   if (p.splits > 1) {
     p.partial = (char *)skl_workspace((size_t)p.splits * p.m * p.n * 4);
     if (!p.partial) return -4;

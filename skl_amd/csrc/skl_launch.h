@@ -92,9 +92,14 @@ int skl_hip_launch_gemv_rows(const skl_gemm_canon *g);
 int skl_hip_gemv_kc_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
 
-/* A block of per-device scratch memory for operands copied into another layout ahead of a launch (grows on demand;
- * ordered on the current stream like the workspace of the split reductions, which it does not share). */
+/* A block of per-device scratch memory for operands copied into another layout ahead of a launch (grows on demand,
+ * NULL when the device has no room; apart from the workspace of the split reductions). */
 void *skl_hip_operand_scratch(size_t bytes);
+/* Brackets a sequence of launches that hands data from one kernel to the next through per-device scratch memory
+ * (operand copies, partial sums), so that sequences of different host threads do not interleave on a stream.
+ * Recursive. */
+void skl_hip_sequence_begin(void);
+void skl_hip_sequence_end(void);
 /* Copies a GEMM operand in the canonical description (element (x, p) at (x/64)*s1 + (x%64)*s0 + p*sk, `esize` 1 or
  * 2 bytes) into rows contiguous in K: dst[x*kp + p], zero-filled for k <= p < kp. */
 int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_t s0, size_t s1, size_t sk,

@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <vector>
 
 #include "../../include/skl-hip.h"
 #include "skl_device.hpp"
@@ -14,12 +15,22 @@ namespace {
 
 constexpr int kMaxDevices = 16;
 
-struct DeviceState {
-  void *workspace = nullptr;
-  size_t workspace_bytes = 0;
-  void *operand_scratch = nullptr;  // copies of operands in another layout; apart from the workspace so that
-  size_t operand_bytes = 0;         // a launch that grows the workspace keeps the copies it was given
+// A block that only ever grows. The block it replaces is kept until shutdown: another thread may have been
+// handed its address and not launched yet, and kernels in flight may still use it.
+struct Scratch {
+  void *ptr = nullptr;
+  size_t bytes = 0;
 };
+
+struct DeviceState {
+  Scratch workspace;  // partial sums of the split reductions (never more than kWorkspaceBytes are asked for)
+  Scratch operands;   // copies of operands in another layout; apart from the workspace so that a launch which
+                      // uses the workspace keeps the copies it was given
+  std::vector<void *> retired;
+};
+
+constexpr size_t kWorkspaceBytes = size_t(64) << 20;
+constexpr size_t kOperandBytes = size_t(4) << 20;
 
 std::mutex g_mutex;
 DeviceState g_devices[kMaxDevices];
@@ -51,29 +62,42 @@ int skl_check_hip(hipError_t e, const char *what) {
 
 hipStream_t skl_current_stream() { return t_stream; }
 
-void *skl_workspace(size_t bytes) {
-  int dev = 0;
-  if (skl_check_hip(hipGetDevice(&dev), "hipGetDevice") != 0 || dev >= kMaxDevices) return nullptr;
-  std::lock_guard<std::mutex> lock(g_mutex);
-  DeviceState &st = g_devices[dev];
-  if (st.workspace_bytes >= bytes) return st.workspace;
-  if (st.workspace) {
-    // Earlier launches may still read the old block.
-    if (skl_check_hip(hipDeviceSynchronize(), "workspace grow: synchronize") != 0) return nullptr;
-    (void)hipFree(st.workspace);
-    st.workspace = nullptr;
-    st.workspace_bytes = 0;
-  }
-  size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes;
+namespace {
+
+std::recursive_mutex g_sequence;
+
+// Under g_mutex. At least `floor` bytes, and at least twice the block replaced, so that retired blocks add up to
+// less than the live one.
+void *grow(DeviceState &st, Scratch &sc, size_t bytes, size_t floor, const char *what, bool record) {
+  if (sc.ptr && sc.bytes >= bytes) return sc.ptr;
+  size_t want = bytes < floor ? floor : bytes;
+  if (want < 2 * sc.bytes) want = 2 * sc.bytes;
   void *p = nullptr;
-  if (hipMalloc(&p, want) != hipSuccess) {
+  if (hipMalloc(&p, want) != hipSuccess && (want == bytes || hipMalloc(&p, want = bytes) != hipSuccess)) {
     (void)hipGetLastError();
-    skl_hip_record_error(SKL_HIP_ERR_WORKSPACE, "skl_workspace");
+    if (record) skl_hip_record_error(SKL_HIP_ERR_WORKSPACE, what);
     return nullptr;
   }
-  st.workspace = p;
-  st.workspace_bytes = want;
+  (void)hipGetLastError();
+  if (sc.ptr) st.retired.push_back(sc.ptr);
+  sc.ptr = p;
+  sc.bytes = want;
   return p;
+}
+
+DeviceState *current_device_state() {
+  int dev = 0;
+  if (skl_check_hip(hipGetDevice(&dev), "hipGetDevice") != 0 || dev >= kMaxDevices) return nullptr;
+  return &g_devices[dev];
+}
+
+}  // namespace
+
+void *skl_workspace(size_t bytes) {
+  DeviceState *st = current_device_state();
+  if (!st) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  return grow(*st, st->workspace, bytes, kWorkspaceBytes, "skl_workspace", true);
 }
 
 extern "C" {
@@ -95,27 +119,15 @@ int skl_hip_init(int device) {
 }
 
 void *skl_hip_operand_scratch(size_t bytes) {
-  int dev = 0;
-  if (skl_check_hip(hipGetDevice(&dev), "hipGetDevice") != 0 || dev >= kMaxDevices) return nullptr;
+  DeviceState *st = current_device_state();
+  if (!st) return nullptr;
   std::lock_guard<std::mutex> lock(g_mutex);
-  DeviceState &st = g_devices[dev];
-  if (st.operand_bytes >= bytes && st.operand_scratch) return st.operand_scratch;
-  if (st.operand_scratch) {
-    // Earlier launches may still read the old block.
-    if (skl_check_hip(hipDeviceSynchronize(), "operand scratch grow: synchronize") != 0) return nullptr;
-    (void)hipFree(st.operand_scratch);
-    st.operand_scratch = nullptr;
-    st.operand_bytes = 0;
-  }
-  const size_t want = bytes < (size_t(4) << 20) ? (size_t(4) << 20) : bytes;
-  if (hipMalloc(&st.operand_scratch, want) != hipSuccess) {
-    (void)hipGetLastError();  // the caller falls back to a kernel that needs no copy
-    st.operand_scratch = nullptr;
-    return nullptr;
-  }
-  st.operand_bytes = want;
-  return st.operand_scratch;
+  // not recorded as an error: the caller falls back to a kernel that needs no copy
+  return grow(*st, st->operands, bytes, kOperandBytes, "skl_hip_operand_scratch", false);
 }
+
+void skl_hip_sequence_begin(void) { g_sequence.lock(); }
+void skl_hip_sequence_end(void) { g_sequence.unlock(); }
 
 void skl_hip_shutdown(void) {
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -125,13 +137,15 @@ void skl_hip_shutdown(void) {
     return;
   }
   for (int d = 0; d < kMaxDevices; ++d) {
-    if (!g_devices[d].workspace && !g_devices[d].operand_scratch) continue;
+    DeviceState &st = g_devices[d];
+    if (!st.workspace.ptr && !st.operands.ptr && st.retired.empty()) continue;
     if (hipSetDevice(d) == hipSuccess) {
       (void)hipDeviceSynchronize();
-      if (g_devices[d].workspace) (void)hipFree(g_devices[d].workspace);
-      if (g_devices[d].operand_scratch) (void)hipFree(g_devices[d].operand_scratch);
+      if (st.workspace.ptr) (void)hipFree(st.workspace.ptr);
+      if (st.operands.ptr) (void)hipFree(st.operands.ptr);
+      for (void *p : st.retired) (void)hipFree(p);
     }
-    g_devices[d] = DeviceState{};
+    st = DeviceState{};
   }
   (void)hipSetDevice(prev);
 }

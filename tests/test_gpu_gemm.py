@@ -388,3 +388,43 @@ def test_leading_dimensions_off_the_16_byte_rule(gpu, ta, tb):
         case = GemmCase(ta, tb, alpha, beta, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=rsa, csa1=csa,
                         rsb0=0, csb0=0, rsb1=rsb, csb1=csb, rsc0=0, csc0=0, rsc1=n + 2, csc1=1)
         check(gpu, "rc", case, 7000 + len(name), "device")
+
+
+def test_host_threads_share_one_device(gpu):
+    """The entry points are re-entrant like the reference's: host threads may call them at the same time on one
+    device (here all on the default stream). Problems whose kernels hand data to each other through the library's
+    per-device scratch memory - K shared between workgroups, operands copied into aligned memory, few columns - must
+    not pick up each other's data. int8, so every result is compared bit for bit."""
+    import threading
+    from support import GemmCase
+
+    def rc(m, n, k, rsa, csa, rsb, csb):
+        return GemmCase("i8", None, 3, -2, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=rsa, csa1=csa,
+                        rsb0=0, csb0=0, rsb1=rsb, csb1=csb, rsc0=0, csc0=0, rsc1=n, csc1=1)
+
+    cases = [rc(16, 2048, 4096, 4096, 1, 2048, 1),      # few tiles, long K: partial sums in the workspace
+             rc(300, 260, 777, 778, 1, 261, 1),         # odd leading dimensions: both operands copied
+             rc(1037, 2, 1040, 1040, 1, 2, 1),          # matrix times two vectors, row-major B: B copied
+             rc(24, 1024, 8192, 8192, 1, 1024, 1)]
+    jobs = []
+    for i, case in enumerate(cases):
+        a, b, c = case.make_inputs(9100 + i)
+        jobs.append((case, a, b, c, run_oracle_gemm(case, a, b, c)))
+    failures = []
+
+    def worker(t):
+        try:
+            for it in range(6):
+                case, a, b, c, want = jobs[(t + it) % len(jobs)]
+                got = run_gemm(gpu, "rc", case, a, b, c, "device")
+                if not np.array_equal(got, want):
+                    failures.append((t, it, (t + it) % len(jobs)))
+        except Exception as e:  # noqa: BLE001 - reported by the assertion below
+            failures.append((t, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not failures, failures
