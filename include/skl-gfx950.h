@@ -19,6 +19,7 @@
 #ifndef SKL_GFX950_H
 #define SKL_GFX950_H
 
+#include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -233,6 +234,15 @@ void skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(size_t m, size_t n, size_t k1, int32_t
                                           size_t rsa1, size_t csa1, const int8_t *b, size_t rsb1,
                                           int32_t beta, int32_t *c, size_t rsc);
 
+/* 4 x 8 by 8 x 4 block products ("fat dot product" layout): A in row-major 4 x 8 blocks, block (I, P) at
+ * I*rsa1 + P*32; B in row-major 8 x 4 blocks, block (P, J) at P*rsb1 + J*32; C in row-major 4 x 4 blocks, block
+ * (I, J) at I*rsc1 + J*16. C = A*B, or C += A*B with `accum`. The reference documents this entry point and its
+ * layouts (src/gemm/packed-gemm.md:270-298) and ships no implementation of it; the arithmetic is that of
+ * ref/gemm/gemm_i8rcprc_i8rcprc_i32rcprc.c:10-37 with m0 = n0 = 4, k0 = 8, alpha = 1 and beta = accum. */
+void skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4_gfx950(size_t m1, size_t n1, size_t k1, const int8_t *a, size_t rsa1,
+                                                 const int8_t *b, size_t rsb1, int32_t *c, size_t rsc1,
+                                                 bool accum);
+
 /* ======================================================================== */
 /* pack / unpack / transpose                                                 */
 /* ======================================================================== */
@@ -257,6 +267,19 @@ void skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(size_t m, size_t n, size_t k1, int32_t
 SKL_GFX950_DECLARE_PACK(8, uint8_t)
 SKL_GFX950_DECLARE_PACK(16, uint16_t)
 SKL_GFX950_DECLARE_PACK(32, uint32_t)
+
+/* Packers of the 4 x 8 / 8 x 4 / 4 x 4 block layouts above, from and to a row-major matrix with row stride
+ * `rs`; blocks of one block row are contiguous, block rows `rs1` apart; partial blocks are filled with `pad`.
+ * src/pack/README.md:172-178 names these four kernels as required for that GEMM and gives no prototypes; the
+ * argument list follows skl_pack_e16_e16rcptex1c (src/pack/pack_e16_xsfmmbase.h:49), the element rule is that of
+ * ref/pack/pack_e8rc_e8rcprc.c:10-35 / ref/pack/unpack_e8rcprc_e8rc.c:10-37. */
+void skl_pack_e8_e8p4x8_gfx950(size_t m, size_t n, const uint8_t *src, size_t rs, uint8_t *dst, size_t rs1,
+                               uint8_t pad);
+void skl_pack_e8_e8p8x4_gfx950(size_t m, size_t n, const uint8_t *src, size_t rs, uint8_t *dst, size_t rs1,
+                               uint8_t pad);
+void skl_pack_e32_e32p4x4_gfx950(size_t m, size_t n, const uint32_t *src, size_t rs, uint32_t *dst, size_t rs1,
+                                 uint32_t pad);
+void skl_unpack_e32p4x4_e32_gfx950(size_t m, size_t n, const uint32_t *src, size_t rs1, uint32_t *dst, size_t rs);
 
 /* ======================================================================== */
 /* OFP8 / OFP4 conversions: (dst, src, scale, n)                             */

@@ -226,12 +226,12 @@ static int gemm_with_realigned_operands(const skl_gemm_canon *g, int fused) {
     scratch = skl_hip_operand_scratch((copy_a ? bytes_a : 0) + (copy_b ? bytes_b : 0));
     done = scratch != NULL;
     if (done && copy_a) {
-      done = skl_hip_launch_realign((int)esa, g->m, g->k, g->a, g->a_s0, g->a_s1, g->a_sk, scratch, kpa) == 0;
+      done = skl_hip_launch_realign((int)esa, g->m, g->k, g->a, SKL_TE, g->a_s0, g->a_s1, 1, 0, g->a_sk, scratch, kpa) == 0;
       h.a = scratch;
       scratch += bytes_a;
     }
     if (done && copy_b) {
-      done = skl_hip_launch_realign((int)esb, g->n, g->k, g->b, g->b_s0, g->b_s1, g->b_sk, scratch, kpb) == 0;
+      done = skl_hip_launch_realign((int)esb, g->n, g->k, g->b, SKL_TE, g->b_s0, g->b_s1, 1, 0, g->b_sk, scratch, kpb) == 0;
       h.b = scratch;
     }
     if (done) done = gemm_fast_path(&h, fused, 1);
@@ -239,6 +239,47 @@ static int gemm_with_realigned_operands(const skl_gemm_canon *g, int fused) {
     return done;
   }
   return 0;
+}
+
+/* Any other blocking (the 4x8 / 8x4 / 4x4 blocks of src/gemm/packed-gemm.md:270-298, blocks of 32, ...): A and B
+ * are copied into rows contiguous in K, C is unpacked into a row-major scratch matrix - always, since even a call
+ * with beta == 0 reads C where the product is an exact zero - multiplied there, and packed back. M and N are
+ * whole numbers of blocks, so packing writes exactly the elements the reference writes. */
+static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
+  const size_t M = d->m0 * d->m1, N = d->n0 * d->n1, K = d->k0 * d->k1;
+  const size_t esa = elem_size(d->ta), esb = elem_size(d->tb);
+  const size_t kpa = (K * esa + 15) / 16 * 16 / esa, kpb = (K * esb + 15) / 16 * 16 / esb;
+  const size_t bytes_a = (M * kpa * esa + 255) / 256 * 256, bytes_b = (N * kpb * esb + 255) / 256 * 256;
+  skl_gemm_canon h;
+  char *scratch;
+  int done;
+  if (esa > 2 || esb > 2 || M * N * K < ((size_t)1 << 18)) return 0;
+  memset(&h, 0, sizeof h);
+  h.ta = d->ta, h.tb = d->tb;
+  h.m = M, h.n = N, h.k = K;
+  h.a = h.b = (const void *)(uintptr_t)256;
+  h.c = (void *)(uintptr_t)256;
+  h.a_sk = 1, h.a_s0 = kpa, h.a_s1 = SKL_TE * kpa;
+  h.b_sk = 1, h.b_s0 = kpb, h.b_s1 = SKL_TE * kpb;
+  h.rsc0 = N, h.rsc1 = SKL_TE * N, h.csc0 = 1, h.csc1 = SKL_TE;
+  h.alpha = d->alpha, h.beta = d->beta;
+  h.bias = d->bias, h.max = d->max;
+  if (!gemm_fast_path(&h, fused, 0)) return 0;
+  skl_hip_sequence_begin();
+  scratch = skl_hip_operand_scratch(bytes_a + bytes_b + M * N * 4);
+  done = scratch != NULL;
+  if (done) {
+    h.a = scratch, h.b = scratch + bytes_a, h.c = scratch + bytes_a + bytes_b;
+    done = skl_hip_launch_realign((int)esa, M, K, d->a, d->m0, d->rsa0, d->rsa1, d->k0, d->csa0, d->csa1, scratch, kpa) == 0 &&
+           skl_hip_launch_realign((int)esb, N, K, d->b, d->n0, d->csb0, d->csb1, d->k0, d->rsb0, d->rsb1,
+                                  scratch + bytes_a, kpb) == 0 &&
+           skl_hip_launch_unpack(4, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, M, N, h.c, N, 1) == 0;
+  }
+  if (done) done = gemm_fast_path(&h, fused, 1);
+  if (done)
+    done = skl_hip_launch_pack(4, M, N, h.c, N, 1, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, 0) == 0;
+  skl_hip_sequence_end();
+  return done;
 }
 
 static void gemm_on_device(const skl_gemm_desc *d) {
@@ -252,6 +293,8 @@ static void gemm_on_device(const skl_gemm_desc *d) {
     if (canonicalize(d, &g)) {
       if (gemm_fast_path(&g, fused, 1)) return;
       if (gemm_with_realigned_operands(&g, fused)) return;
+    } else if (gemm_through_copies(d, fused)) {
+      return;
     }
   }
   skl_hip_launch_gemm_generic(d);
@@ -440,6 +483,15 @@ void skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(size_t m, size_t n, size_t k1, int32_t
                                            beta, c, 0, 0, rsc, 1);
 }
 
+/* src/gemm/packed-gemm.md:270-298 */
+void skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4_gfx950(size_t m1, size_t n1, size_t k1, const int8_t *a, size_t rsa1,
+                                                 const int8_t *b, size_t rsb1, int32_t *c, size_t rsc1,
+                                                 bool accum) {
+  skl_gemm_desc d = {SKL_DT_I8, SKL_DT_I8, 4, 4, 8, m1, n1, k1, a, 8, 1, rsa1, 32, b, 4, 1, rsb1, 32,
+                     c, 4, 1, rsc1, 16, {.i = 1}, {.i = accum ? 1 : 0}, NULL, NULL};
+  gemm_run(&d, __func__);
+}
+
 /* ------------------------------------------------------------------------ */
 /* pack / unpack / transpose                                                 */
 /* ------------------------------------------------------------------------ */
@@ -527,6 +579,23 @@ static void unpack_run(int esize, size_t m0, size_t n0, const void *src, size_t 
 DEFINE_PACK_FAMILY(8, uint8_t, 1)
 DEFINE_PACK_FAMILY(16, uint16_t, 2)
 DEFINE_PACK_FAMILY(32, uint32_t, 4)
+
+/* Block layouts of the 4x8x4 block GEMM (src/gemm/packed-gemm.md:270-298, src/pack/README.md:172-178). */
+void skl_pack_e8_e8p4x8_gfx950(size_t m, size_t n, const uint8_t *src, size_t rs, uint8_t *dst, size_t rs1,
+                               uint8_t pad) {
+  pack_run(1, m, n, src, rs, 1, 4, 8, dst, 8, 1, rs1, 32, pad, __func__);
+}
+void skl_pack_e8_e8p8x4_gfx950(size_t m, size_t n, const uint8_t *src, size_t rs, uint8_t *dst, size_t rs1,
+                               uint8_t pad) {
+  pack_run(1, m, n, src, rs, 1, 8, 4, dst, 4, 1, rs1, 32, pad, __func__);
+}
+void skl_pack_e32_e32p4x4_gfx950(size_t m, size_t n, const uint32_t *src, size_t rs, uint32_t *dst, size_t rs1,
+                                 uint32_t pad) {
+  pack_run(4, m, n, src, rs, 1, 4, 4, dst, 4, 1, rs1, 16, pad, __func__);
+}
+void skl_unpack_e32p4x4_e32_gfx950(size_t m, size_t n, const uint32_t *src, size_t rs1, uint32_t *dst, size_t rs) {
+  unpack_run(4, 4, 4, src, 4, 1, rs1, 16, m, n, dst, rs, 1, __func__);
+}
 
 /* ------------------------------------------------------------------------ */
 /* cvt                                                                       */

@@ -100,10 +100,11 @@ void *skl_hip_operand_scratch(size_t bytes);
  * Recursive. */
 void skl_hip_sequence_begin(void);
 void skl_hip_sequence_end(void);
-/* Copies a GEMM operand in the canonical description (element (x, p) at (x/64)*s1 + (x%64)*s0 + p*sk, `esize` 1 or
- * 2 bytes) into rows contiguous in K: dst[x*kp + p], zero-filled for k <= p < kp. */
-int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_t s0, size_t s1, size_t sk,
-                           void *dst, size_t kp);
+/* Copies a GEMM operand in the reference's blocked description (element (x, p), x along M or N and p along K, at
+ * (x/x0)*s1 + (x%x0)*s0 + (p/k0)*sk1 + (p%k0)*sk0; `esize` 1 or 2 bytes) into rows contiguous in K:
+ * dst[x*kp + p], zero-filled for k <= p < kp. */
+int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_t x0, size_t s0, size_t s1, size_t k0,
+                           size_t sk0, size_t sk1, void *dst, size_t kp);
 
 /* pack / unpack over elements of `esize` bytes (1, 2 or 4). */
 int skl_hip_launch_pack(int esize, size_t m, size_t n, const void *src, size_t rs, size_t cs,

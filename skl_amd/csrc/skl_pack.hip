@@ -33,21 +33,27 @@ struct PackArgs {
   int blocked_along_c;  // lanes run along columns when touching the blocked matrix
 };
 
+// Blocked source of a realigning copy: element (x, p) at (x/x0)*s1 + (x%x0)*s0 + (p/k0)*sk1 + (p%k0)*sk0.
+struct RealignSource {
+  size_t x0, s0, s1, k0, sk0, sk1;
+};
+
 template <typename T>
 __global__ void __launch_bounds__(kThreads) realign_kernel(const T *__restrict__ src, T *__restrict__ dst, size_t x, size_t k,
-                                                           size_t kp, size_t s0, size_t s1, size_t sk, unsigned tiles_p,
-                                                           int along_x) {
+                                                           size_t kp, RealignSource f, unsigned tiles_p, int along_x) {
   __shared__ T tile[kTile][kTile + 3];  // [p][x]
-  const size_t x0 = (size_t)(blockIdx.x / tiles_p) * kTile, p0 = (size_t)(blockIdx.x % tiles_p) * kTile;
+  const size_t x_base = (size_t)(blockIdx.x / tiles_p) * kTile, p_base = (size_t)(blockIdx.x % tiles_p) * kTile;
   const int fast = threadIdx.x % kTile, slow = threadIdx.x / kTile;
   for (int it = slow; it < kTile; it += kThreads / kTile) {
     const int xi = along_x ? fast : it, pi = along_x ? it : fast;
-    const size_t xx = x0 + xi, pp = p0 + pi;
-    tile[pi][xi] = (xx < x && pp < k) ? src[(xx / 64) * s1 + (xx % 64) * s0 + pp * sk] : T(0);
+    const size_t xx = x_base + xi, pp = p_base + pi;
+    tile[pi][xi] = (xx < x && pp < k)
+                       ? src[(xx / f.x0) * f.s1 + (xx % f.x0) * f.s0 + (pp / f.k0) * f.sk1 + (pp % f.k0) * f.sk0]
+                       : T(0);
   }
   __syncthreads();
   for (int it = slow; it < kTile; it += kThreads / kTile) {
-    const size_t xx = x0 + it, pp = p0 + fast;
+    const size_t xx = x_base + it, pp = p_base + fast;
     if (xx < x && pp < kp) dst[xx * kp + pp] = tile[fast][it];
   }
 }
@@ -340,25 +346,28 @@ int skl_hip_launch_unpack(int esize, size_t m0, size_t n0, const void *src, size
   return dispatch(esize, false, src, dst, p);
 }
 
-// A GEMM operand in the canonical blocked description - element (x, p) at (x/64)*s1 + (x%64)*s0 + p*sk, x along M
-// or N, p along K - copied into rows contiguous in K: dst[x*kp + p], zero for k <= p < kp. 64 x 64 tiles through
-// LDS, read with lanes along x when the source is contiguous there and along p otherwise, written along p.
-int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_t s0, size_t s1, size_t sk,
-                           void *dst, size_t kp) {
+// A GEMM operand in the reference's blocked description - element (x, p), x along M or N and p along K, at
+// (x/x0)*s1 + (x%x0)*s0 + (p/k0)*sk1 + (p%k0)*sk0 - copied into rows contiguous in K: dst[x*kp + p], zero for
+// k <= p < kp. 64 x 64 tiles through LDS, read with lanes along x when the source is contiguous there and along p
+// otherwise, written along p.
+int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_t x0, size_t s0, size_t s1, size_t k0,
+                           size_t sk0, size_t sk1, void *dst, size_t kp) {
   if (x == 0 || kp == 0) return 0;
   const size_t tiles_p = (kp + kTile - 1) / kTile, tiles = ((x + kTile - 1) / kTile) * tiles_p;
-  if (tiles > 0x7FFFFFFFu || (esize != 1 && esize != 2)) {
-    skl_hip_record_error(-2, "realign: problem too large");
+  if (tiles > 0x7FFFFFFFu || (esize != 1 && esize != 2) || x0 == 0 || k0 == 0) {
+    skl_hip_record_error(-2, "realign: bad problem");
     return -2;
   }
-  const int along_x = s0 == 1 && sk != 1;
+  const RealignSource f = {x0, s0, s1, k0, sk0, sk1};
+  const size_t step_x = x0 > 1 ? s0 : s1, step_p = k0 > 1 ? sk0 : sk1;
+  const int along_x = step_x == 1 && step_p != 1;
   hipStream_t st = skl_current_stream();
   if (esize == 1)
-    realign_kernel<uint8_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint8_t *)src, (uint8_t *)dst, x, k, kp, s0, s1, sk,
+    realign_kernel<uint8_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint8_t *)src, (uint8_t *)dst, x, k, kp, f,
                                                                 (unsigned)tiles_p, along_x);
   else
-    realign_kernel<uint16_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint16_t *)src, (uint16_t *)dst, x, k, kp, s0, s1,
-                                                                 sk, (unsigned)tiles_p, along_x);
+    realign_kernel<uint16_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint16_t *)src, (uint16_t *)dst, x, k, kp, f,
+                                                                 (unsigned)tiles_p, along_x);
   return skl_check_launch("realign");
 }
 

@@ -2,6 +2,7 @@
 
 Each character is one C parameter: ``z`` size_t, ``p`` pointer, ``i`` int32_t,
 ``f`` float, ``d`` double, ``b`` uint8_t, ``h`` uint16_t, ``w`` uint32_t,
+``B`` bool,
 ``H`` a ``_Float16`` passed by value, ``E`` a pointer to a ``skl_gfx950_epilogue_t``.
 Names are given without the implementation suffix (``_gfx950`` for the GPU
 library); the parameter order is the reference's (include/skl-gfx950.h cites
@@ -34,6 +35,7 @@ CTYPES = {
     "b": ctypes.c_uint8,
     "h": ctypes.c_uint16,
     "w": ctypes.c_uint32,
+    "B": ctypes.c_bool,
     "H": HalfByValue,
     "E": ctypes.c_void_p,
 }
@@ -159,6 +161,11 @@ def gfx950_only():
     for name, s in GEMM_PANEL.items():
         sigs[name] = _panel(s)
     sigs["skl_gemm_i8rcp1x4_i8p4x1c_i32"] = "zzzipzzpzipz"
+    sigs["skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4"] = "zzzpzpzpzB"   # m1 n1 k1 a rsa1 b rsb1 c rsc1 accum
+    sigs["skl_pack_e8_e8p4x8"] = "zzpzpzb"                        # m n src rs dst rs1 pad
+    sigs["skl_pack_e8_e8p8x4"] = "zzpzpzb"
+    sigs["skl_pack_e32_e32p4x4"] = "zzpzpzw"
+    sigs["skl_unpack_e32p4x4_e32"] = "zzpzpz"                     # m n src rs1 dst rs
     for name, sig in GEMM_FUSED.items():
         sigs[name] = sig + "E"
     for w, pad in _PAD.items():

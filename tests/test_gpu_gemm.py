@@ -428,3 +428,50 @@ def test_host_threads_share_one_device(gpu):
     for th in threads:
         th.join()
     assert not failures, failures
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_block4x8x4_entry_point(gpu, mode):
+    """`skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4` (documented by the reference without an implementation): small
+    problems on the any-stride kernel, larger ones through aligned copies on the matrix cores; block rows with
+    gaps between them; C = A*B and C += A*B; empty dimensions. Whole C buffer compared bit for bit."""
+    from test_oracle_gemm import block4x8x4_case
+    shapes = [(1, 1, 1, 0), (3, 2, 5, 7), (0, 2, 2, 0), (2, 0, 2, 0), (2, 2, 0, 0), (64, 96, 40, 0), (33, 50, 129, 48),
+              (256, 8, 64, 16)]
+    for i, (m1, n1, k1, gap) in enumerate(shapes):
+        for accum in (False, True):
+            case = block4x8x4_case(m1, n1, k1, 32 * k1 + gap, 32 * n1 + gap, 16 * n1 + gap, accum)
+            a, b, c = case.make_inputs(8100 + i)
+            want = run_oracle_gemm(case, a, b, c)
+            if mode == "host":
+                got = c.copy()
+                gpu.skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4_gfx950(m1, n1, k1, a, case.rsa1, b, case.rsb1, got, case.rsc1, accum)
+                skl_amd.check_error()
+            else:
+                bufs = [skl_amd.DeviceBuffer.from_array(x) for x in (a, b, c)]
+                gpu.skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4_gfx950(m1, n1, k1, bufs[0], case.rsa1, bufs[1], case.rsb1, bufs[2],
+                                                                case.rsc1, accum)
+                assert gpu.skl_hip_synchronize() == 0
+                skl_amd.check_error()
+                got = bufs[2].download(c.dtype, c.size)
+                for d in bufs:
+                    d.free()
+            assert np.array_equal(got, want), (m1, n1, k1, gap, accum)
+
+
+@pytest.mark.parametrize("ta,tb", (("i8", "i8"), ("bf16", "bf16"), ("f16", "f16"), ("f8e4m3", "f8e4m3"), ("f8e5m2", "f8e5m2")))
+def test_blockings_no_kernel_reads_in_place(gpu, ta, tb):
+    """Blocks of other sizes than 1, 64 or the whole matrix (3 x 5 x 7, 32 x 32 x 16 column-major blocks with
+    gaps, the 4 x 8 x 4 format): operands copied, C unpacked, multiplied and packed back. beta != 0 and beta == 0;
+    gaps in C must come back untouched."""
+    from support import GemmCase
+    blockings = [
+        dict(m0=3, n0=5, k0=7, m1=40, n1=30, k1=20, rsa0=7, csa0=1, rsa1=7 * 3 * 20 + 4, csa1=21, rsb0=5, csb0=1,
+             rsb1=5 * 7 * 30 + 1, csb1=35, rsc0=5, csc0=1, rsc1=15 * 30 + 3, csc1=15),
+        dict(m0=32, n0=32, k0=16, m1=5, n1=6, k1=9, rsa0=1, csa0=32, rsa1=512, csa1=5 * 512, rsb0=1, csb0=16,
+             rsb1=512, csb1=9 * 512 + 16, rsc0=1, csc0=33, rsc1=33 * 32, csc1=5 * 33 * 32),
+    ]
+    for i, blk in enumerate(blockings):
+        for alpha, beta in (((2, -1) if ta == "i8" else (1.5, -0.5)), ((1, 0) if ta == "i8" else (1.0, 0.0))):
+            case = GemmCase(ta, tb, alpha, beta, **blk)
+            check(gpu, "rcprc", case, 8200 + i, "device")

@@ -186,3 +186,32 @@ def test_vector_paths_pack_and_unpack(gpu, w):
                           lambda s, d: (*tail, s, *bs, row["m"], row["n"], d, row["rs"], row["cs"]),
                           packed, plain, "device")
         assert np.array_equal(got_u, want_u), ("unpack", row)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_block4x8x4_packers(gpu, mode):
+    """The four packers of the 4 x 8 / 8 x 4 / 4 x 4 block layouts (src/pack/README.md:172-178) against the checker's
+    general pack / unpack with those block sizes and strides, and against numpy's reshape of the packed buffer;
+    partial blocks padded, gaps between block rows untouched; pack -> unpack returns the matrix."""
+    rng = np.random.default_rng(4848)
+    for (m, n, gap) in ((4, 8, 0), (8, 8, 0), (7, 13, 5), (64, 96, 0), (129, 130, 32), (1, 1, 3)):
+        for name, w, (m0, n0) in (("skl_pack_e8_e8p4x8", 8, (4, 8)), ("skl_pack_e8_e8p8x4", 8, (8, 4)),
+                                  ("skl_pack_e32_e32p4x4", 32, (4, 4))):
+            m1, n1 = -(-m // m0), -(-n // n0)
+            rs, rs1 = n + 3, n1 * m0 * n0 + gap
+            src = rng.integers(0, 1 << w, size=m * rs, dtype=np.uint64).astype(DT[w])
+            dst = rng.integers(0, 1 << w, size=m1 * rs1, dtype=np.uint64).astype(DT[w])
+            want = dst.copy()
+            getattr(oracle(), f"skl_pack_e{w}rc_e{w}rcprc_oracle")(m, n, src, rs, 1, m0, n0, want, n0, 1, rs1, m0 * n0, PAD[w])
+            got = run_inout(gpu, name + "_gfx950", lambda s, d: (m, n, s, rs, d, rs1, PAD[w]), src, dst, mode)
+            assert np.array_equal(got, want), (name, m, n, gap)
+            blocks = np.stack([got[i * rs1:i * rs1 + n1 * m0 * n0] for i in range(m1)]).reshape(m1, n1, m0, n0)
+            dense = np.full((m1 * m0, n1 * n0), PAD[w], DT[w])
+            dense[:m, :n] = src.reshape(m, rs)[:, :n]
+            assert np.array_equal(blocks.transpose(0, 2, 1, 3).reshape(m1 * m0, n1 * n0), dense)
+            if name == "skl_pack_e32_e32p4x4":
+                back = rng.integers(0, 1 << 32, size=m * rs, dtype=np.uint64).astype(np.uint32)
+                want_back = back.copy()
+                want_back.reshape(m, rs)[:, :n] = src.reshape(m, rs)[:, :n]
+                got_back = run_inout(gpu, "skl_unpack_e32p4x4_e32_gfx950", lambda s, d: (m, n, s, rs1, d, rs), got, back, mode)
+                assert np.array_equal(got_back, want_back), (m, n, gap)

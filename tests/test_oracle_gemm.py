@@ -289,3 +289,27 @@ def test_fused_steps_follow_the_plain_gemm(ta):
                     assert mx[0] == top[0], (ta, blocked, use_bias)
                 else:
                     assert mx[0] == start[0]
+
+
+def block4x8x4_case(m1, n1, k1, rsa1=None, rsb1=None, rsc1=None, accum=False):
+    """The 4 x 8 by 8 x 4 block product of src/gemm/packed-gemm.md:270-298 as a blocked GEMM: "block dimensions
+    m0 = 4, n0 = 4, k0 = 8; intra-block row strides rsa0 = 8, rsb0 = 4, rsc0 = 4; all intra-block column strides
+    equal to 1", block-row-major with csa1 = 32, csb1 = 32, csc1 = 16."""
+    return support.GemmCase("i8", None, 1, 1 if accum else 0, m0=4, n0=4, k0=8, m1=m1, n1=n1, k1=k1,
+                            rsa0=8, csa0=1, rsa1=rsa1 if rsa1 is not None else 32 * k1, csa1=32,
+                            rsb0=4, csb0=1, rsb1=rsb1 if rsb1 is not None else 32 * n1, csb1=32,
+                            rsc0=4, csc0=1, rsc1=rsc1 if rsc1 is not None else 16 * n1, csc1=16)
+
+
+def test_block4x8x4_layout_against_numpy_blocks():
+    """Pins the checker on that layout without its own index arithmetic: the buffers reshaped into
+    [block row][block column][row][column] arrays, the product formed block by block with numpy in 64 bits."""
+    m1, n1, k1 = 5, 3, 4
+    for accum in (False, True):
+        case = block4x8x4_case(m1, n1, k1, accum=accum)
+        a, b, c = case.make_inputs(77 + accum)
+        got = support.run_oracle_gemm(case, a, b, c)
+        A = a.astype(np.int64).reshape(m1, k1, 4, 8)
+        B = b.astype(np.int64).reshape(k1, n1, 8, 4)
+        want = np.einsum("ipak,pjkb->ijab", A, B) + (c.astype(np.int64).reshape(m1, n1, 4, 4) if accum else 0)
+        assert np.array_equal(got.reshape(m1, n1, 4, 4), want.astype(np.int32))
