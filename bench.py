@@ -27,7 +27,7 @@ import skl_amd  # noqa: E402
 from skl_amd import DeviceBuffer  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
-MFMA_PEAK_TOPS = {"i8": 5000.0, "f8": 5000.0, "bf16": 2500.0, "f16": 2500.0}
+MFMA_PEAK_TOPS = {"i8": 5000.0, "f8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "f32": 157.3, "f64": 78.6}
 METRIC = "GEMM TOPS (int8/fp8/bf16) + GEMV HBM GB/s on 1 MI355X, % of roofline"
 
 
@@ -262,6 +262,26 @@ def wl_gemm_bf16(lib, rng):
                   1.0, 1.0, np.float32, "bf16")
 
 
+def wl_gemm_f32(lib, rng):
+    """f32 and f64 results are defined operation by operation (a rounded multiply, then a rounded add, k ascending),
+    so they run on the vector ALUs, not the matrix cores; the published fp32 / fp64 peaks are the denominators."""
+    m = n = k = 4096
+    d = _dense(lib, rng, "f32 GEMM 4096^3 (row-major, alpha=1, beta=0; bit-identical to the reference)",
+               "skl_gemm_f32_f32_f32_gfx950", m, n, k, 4, lambda c: rng.normal(size=c).astype(np.float32),
+               lambda c: rng.normal(size=c).astype(np.float32), 1.0, 0.0, np.float32, "f32")
+    d["kernel"] = "gemm_tiled_kernel"
+    return d
+
+
+def wl_gemm_f64(lib, rng):
+    m = n = k = 4096
+    d = _dense(lib, rng, "f64 GEMM 4096^3 (row-major, alpha=1, beta=0; bit-identical to the reference)",
+               "skl_gemm_f64_f64_f64_gfx950", m, n, k, 8, lambda c: rng.normal(size=c), lambda c: rng.normal(size=c),
+               1.0, 0.0, np.float64, "f64")
+    d["kernel"] = "gemm_tiled_kernel"
+    return d
+
+
 def wl_f16_pipeline(lib, rng):
     """benchmark configuration 5: pack A, pack B, panel GEMM, unpack C - one step is the whole pipeline."""
     te, m, k, n = 64, 4096, 4096, 14336
@@ -338,6 +358,8 @@ WORKLOADS = {
     "gemm_f8e4m3_8192_rowmajor_a": (wl_gemm_f8_layout(True, False), 10, 2),
     "gemm_f8e4m3_8192_kcontig": (wl_gemm_f8_layout(True, True), 10, 2),
     "gemm_bf16_2048x4096x4096": (wl_gemm_bf16, 20, 3),
+    "gemm_f32_4096": (wl_gemm_f32, 5, 1),
+    "gemm_f64_4096": (wl_gemm_f64, 5, 1),
     "pipeline_f16_4096x4096x14336": (wl_f16_pipeline, 5, 1),
     "gemm_i8_512": (wl_gemm_i8_512, 200, 20),
     "cvt_f32_f8e4m3_8192sq": (wl_cvt, 20, 3),

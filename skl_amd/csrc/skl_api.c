@@ -297,6 +297,11 @@ static void gemm_on_device(const skl_gemm_desc *d) {
       return;
     }
   }
+  if (d->k0 * d->k1 != 0 && !fused && canonicalize(d, &g) && skl_hip_gemm_tiled_supported(&g) &&
+      g.m * g.n * g.k >= ((size_t)1 << 15)) {
+    skl_hip_launch_gemm_tiled(&g);
+    return;
+  }
   skl_hip_launch_gemm_generic(d);
 }
 

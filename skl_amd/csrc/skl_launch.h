@@ -75,6 +75,10 @@ typedef struct {
 } skl_gemm_canon;
 
 int skl_hip_launch_gemm_generic(const skl_gemm_desc *d);
+/* Register-tiled kernel for f32, f64 and f16 -> f16 (bit-identical to the any-stride kernel); any strides of the
+ * canonical form, no fused steps. */
+int skl_hip_gemm_tiled_supported(const skl_gemm_canon *g);
+int skl_hip_launch_gemm_tiled(const skl_gemm_canon *g);
 /* Returns 1 if the canonical problem meets the matrix-core kernels' alignment
  * rules (16-byte aligned bases and strides along the non-unit dimensions). */
 int skl_hip_gemm_mfma_supported(const skl_gemm_canon *g);

@@ -122,9 +122,9 @@ def test_ragged_mid_size_bounds_checked_tiles(gpu, ta):
 
 
 def test_f32_f64_bit_identical_to_the_checker(gpu):
-    """The f32 and f64 contractions run on the any-stride kernel, which evaluates the reference's loop
-    with a separately rounded multiply and add: for finite data the result equals the checker's
-    (and the compiled reference's) bit for bit, stride gaps included."""
+    """The f32 and f64 contractions evaluate the reference's loop with a separately rounded multiply and add: for
+    finite data the result equals the checker's (and the compiled reference's) bit for bit, stride gaps
+    included. (A row-major case on the register-tiled kernel, a blocking only the any-stride kernel takes.)"""
     rng = np.random.default_rng(91)
     for ta in ("f32", "f64"):
         for case in (rowmajor_case(ta, 33, 47, 129, alpha=1.5, beta=-0.25, rsa=131, rsb=50, rsc=49),
@@ -475,3 +475,35 @@ def test_blockings_no_kernel_reads_in_place(gpu, ta, tb):
         for alpha, beta in (((2, -1) if ta == "i8" else (1.5, -0.5)), ((1, 0) if ta == "i8" else (1.0, 0.0))):
             case = GemmCase(ta, tb, alpha, beta, **blk)
             check(gpu, "rcprc", case, 8200 + i, "device")
+
+
+@pytest.mark.parametrize("ta", ("f32", "f64", "f16h"))
+def test_register_tiled_kernel_bit_identical(gpu, ta):
+    """f32, f64 and f16 -> f16 on the register-tiled kernel: the same bits as the checker over the whole C buffer.
+    Both tile sizes (64 x 64; 128 x 128 from 512 tiles on), every pairing of row- and column-major operands, 64-row
+    panels, ragged edges in M, N and K, K shorter than one slab, beta == 0 and != 0."""
+    from support import GemmCase
+    te = support.TE
+
+    def rc(m, n, k, a_rows, b_rows, alpha, beta):
+        rsa, csa = (k + 3, 1) if a_rows else (1, m + 1)
+        rsb, csb = (n + 2, 1) if b_rows else (1, k + 5)
+        return GemmCase(ta, None, alpha, beta, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=rsa, csa1=csa,
+                        rsb0=0, csb0=0, rsb1=rsb, csb1=csb, rsc0=0, csc0=0, rsc1=n + 1, csc1=1)
+
+    cases = []
+    for a_rows in (True, False):
+        for b_rows in (True, False):
+            cases.append(rc(130, 203, 77, a_rows, b_rows, 1.5, -0.5))
+            cases.append(rc(64, 64, 5, a_rows, b_rows, 1.0, 0.0))
+    cases.append(rc(2890, 2950, 24, True, True, 0.5, 2.0))     # 128 x 128 tiles, ragged
+    cases.append(rc(2944, 2944, 9, False, True, 1.0, 0.0))
+    # 64-row panels of A and B, 64 x 64 blocks of C (the panel entry points' layout)
+    m1, n1, k = 3, 5, 50
+    cases.append(GemmCase(ta, None, 2.0, 1.0, m0=te, n0=te, k0=1, m1=m1, n1=n1, k1=k, rsa0=1, csa0=0, rsa1=k * te, csa1=te,
+                          rsb0=0, csb0=1, rsb1=te, csb1=k * te, rsc0=te, csc0=1, rsc1=n1 * te * te, csc1=te * te))
+    for i, case in enumerate(cases):
+        a, b, c = case.make_inputs(9300 + i)
+        want = run_oracle_gemm(case, a, b, c)
+        got = run_gemm(gpu, "rcprc", case, a, b, c, "device")
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (ta, i, vars(case))
