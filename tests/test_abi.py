@@ -56,12 +56,12 @@ def test_headers_compile_as_c99_c11_and_cxx(tmp_path):
     """The public headers are what an SKL caller includes: they must be valid C99 for a compiler without
     `_Float16` (gcc 11: 16-bit patterns, no f16 -> f16 prototypes) and for one with it (ROCm's clang), and C++."""
     src = tmp_path / "use.c"
-    src.write_text('#include "skl-gfx950.h"\n'
+    src.write_text('#include "skl-gfx950-compat.h"\n'
                    'int probe(void) {\n'
                    '  skl_gfx950_epilogue_t ep = {0, 0};\n'
-                   '  skl_gemm_i8_i8_i32_gfx950(0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0);\n'
+                   '  skl_gemm_i8_i8_i32_zve32x_x390(0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0);\n'
                    '  skl_gemm_fused_i8rc_i8rc_i32rc_gfx950(0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, &ep);\n'
-                   '  return (int)skl_hip_te();\n'
+                   '  return (int)skl_get_ete_xsfmmbase();\n'
                    '}\n')
     inc = os.path.join(ROOT, "include")
     clang = "/opt/rocm/lib/llvm/bin/clang"
@@ -72,3 +72,47 @@ def test_headers_compile_as_c99_c11_and_cxx(tmp_path):
     for cmd in cmds:
         proc = subprocess.run(cmd, capture_output=True, text=True)
         assert proc.returncode == 0, (cmd[0], proc.stderr[-2000:])
+
+
+def _compat_defines():
+    text = open(os.path.join(ROOT, "include", "skl-gfx950-compat.h")).read()
+    return re.findall(r"^#define\s+(skl_\w+)\s+(skl_\w+_gfx950)\s+/\*\s*([\w/.\-]+):(\d+)\s*\*/", text, re.M)
+
+
+def test_compat_header_targets_are_declared():
+    """Every name of the reference that include/skl-gfx950-compat.h maps has a declared, exported target."""
+    defines = _compat_defines()
+    assert len(defines) >= 80
+    declared = declared_functions("skl-gfx950.h")
+    cdll = ctypes.CDLL(skl_amd.library_path())
+    for name, target, _, _ in defines:
+        assert target in declared and hasattr(cdll, target), (name, target)
+
+
+def test_compat_header_agrees_with_the_reference_prototypes(tmp_path):
+    """Type-level check of the drop-in boundary: behind the compat header, each of the reference's own headers
+    re-declares this library's functions (its names are macros for ours), and a C compiler rejects a
+    re-declaration whose parameter list differs. The reference's headers refuse to be read without their RISC-V
+    feature macros, which are defined here for the syntax check only; nothing of the reference is compiled."""
+    import pytest
+    ref = "/root/reference"
+    clang = "/opt/rocm/lib/llvm/bin/clang"
+    if not (os.path.isdir(ref) and os.path.exists(clang)):
+        pytest.skip("needs the reference checkout and a compiler with __bf16 / _Float16")
+    features = ("zve32x zve32f zve64d zvfh zvfbfwma zvfbfmin zvfofp8min zvfofp4min xsfmmbase xsfmm32a8i xsfmm32a8f "
+                "xsfmm32a16f xsfmm32a32f xsfvqdotq").split()
+    flags = [f"-D__riscv_{f}=1000000" for f in features]
+    headers = sorted({h for _, _, h, _ in _compat_defines()})
+    assert len(headers) >= 40
+    for h in headers:
+        src = tmp_path / "t.c"
+        src.write_text(f'#include "skl-gfx950-compat.h"\n#include "{h}"\n')
+        proc = subprocess.run([clang, "-std=gnu2x", "-fsyntax-only", *flags, "-I", os.path.join(ROOT, "include"),
+                               "-I", os.path.join(ref, "include"), "-I", ref, str(src)], capture_output=True, text=True)
+        assert proc.returncode == 0, (h, proc.stderr[-1500:])
+    # the check bites: an argument of another type is rejected
+    src.write_text('#include "skl-gfx950-compat.h"\n'
+                   'void skl_transpose_e8_zve32x(size_t m, size_t n, const uint8_t *a, size_t rsa, uint8_t *at, int rsat);\n')
+    proc = subprocess.run([clang, "-std=gnu2x", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), str(src)],
+                          capture_output=True, text=True)
+    assert proc.returncode != 0 and "conflicting types" in proc.stderr
