@@ -1,5 +1,5 @@
-/* A C caller of the library with ordinary malloc'ed buffers - the literal drop-in use: the same calls an
- * SKL program makes, with the suffix _gfx950. Checks int8 GEMM (strided, alpha / beta), the fused bias +
+/* A C caller of the library with ordinary malloc'ed buffers - the literal drop-in use: the calls an SKL
+ * program makes, under SKL's own function names (skl-gfx950-compat.h maps them), plus this library's fused form. Checks int8 GEMM (strided, alpha / beta), the fused bias +
  * maximum epilogue, a 16-bit panel pack / unpack round trip and the saturating fp32 -> E4M3 conversion
  * against plain loops written from the definitions. Prints "dropin ok" and returns 0 on success. */
 #include <stdint.h>
@@ -7,7 +7,7 @@
 #include <stdlib.h>
 #include <string.h>
 
-#include "skl-gfx950.h"
+#include "skl-gfx950-compat.h"
 
 static uint64_t rng_state = 0x9E3779B97F4A7C15ull;
 static uint32_t next_u32(void) {
@@ -56,12 +56,26 @@ int main(void) {
     bad = 1;
   }
 
+  /* the same product through SKL's row-major entry point: C = A*B */
+  skl_gemm_i8_i8_i32_zve32x_x390(M, N, K, 1, a, LDA, b, LDB, 0, c, LDC);
+  bad |= check_error("int8 GEMM");
+  for (int i = 0; i < M && !bad; ++i)
+    for (int j = 0; j < N; ++j) {
+      int32_t acc = 0;
+      for (int p = 0; p < K; ++p) acc += (int32_t)a[i * LDA + p] * (int32_t)b[p * LDB + j];
+      if (c[i * LDC + j] != acc) {
+        fprintf(stderr, "int8 GEMM differs at (%d, %d)\n", i, j);
+        bad = 1;
+        break;
+      }
+    }
+
   /* 16-bit panels: pack 70 x 96 into TE x 1 column panels and unpack again */
   {
-    const size_t te = skl_hip_te(), m1 = (M + te - 1) / te;
+    const size_t te = skl_get_ete_xsfmmbase(), m1 = (M + te - 1) / te;
     uint16_t *src = malloc(2 * M * N), *panels = malloc(2 * m1 * N * te), *back = calloc(M * N, 2);
     for (int i = 0; i < M * N; ++i) src[i] = (uint16_t)next_u32();
-    skl_pack_e16_e16rcptex1c_gfx950(M, N, src, N, panels, N * te, te, 0);
+    skl_pack_e16_e16rcptex1c_xsfmmbase(M, N, src, N, panels, N * te, te, 0);
     for (int i = 0; i < M && !bad; ++i)
       for (int j = 0; j < N; ++j)
         if (panels[(i / te) * N * te + j * te + i % te] != src[i * N + j]) {
@@ -83,7 +97,7 @@ int main(void) {
     const float x[4] = {1.0f, 448.0f, 1e6f, -0.0f};
     const uint8_t expect[4] = {0x38, 0x7E, 0x7E, 0x80};
     uint8_t q[4] = {0, 0, 0, 0};
-    skl_cvt_sat_f32_f8e4m3_gfx950(q, x, 1.0f, 4);
+    skl_cvt_sat_f32_f8e4m3_zvfofp8min(q, x, 1.0f, 4);
     bad |= check_error("cvt");
     if (memcmp(q, expect, 4) != 0) {
       fprintf(stderr, "cvt differs: %02x %02x %02x %02x\n", q[0], q[1], q[2], q[3]);
