@@ -186,15 +186,18 @@ static void transposed_view(const skl_gemm_canon *g, skl_gemm_canon *t) {
 }
 
 /* Offers `g` to every kernel but the any-stride one; 1 if one of them takes it. With `launch` == 0 only asks. */
-static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
+static int gemv_paths(const skl_gemm_canon *g, int launch) {
   skl_gemm_canon t;
-  if (!fused) {
-    if (launch ? gemv_on_device(g) : gemv_would_take(g)) return 1;
-    if (g->n <= 8 && g->n < g->m) {
-      transposed_view(g, &t);
-      if (launch ? gemv_on_device(&t) : gemv_would_take(&t)) return 1;
-    }
+  if (launch ? gemv_on_device(g) : gemv_would_take(g)) return 1;
+  if (g->n <= 8 && g->n < g->m) {
+    transposed_view(g, &t);
+    if (launch ? gemv_on_device(&t) : gemv_would_take(&t)) return 1;
   }
+  return 0;
+}
+
+static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
+  if (!fused && gemv_paths(g, launch)) return 1;
   if (skl_hip_gemm_mfma_supported(g)) return launch ? (skl_hip_launch_gemm_mfma(g), 1) : 1;
   return 0;
 }
@@ -239,6 +242,33 @@ static int gemm_with_realigned_operands(const skl_gemm_canon *g, int fused) {
     return done;
   }
   return 0;
+}
+
+/* Ragged or misaligned problems large enough for the streaming kernel: A and B copied into scratch memory padded
+ * to whole tiles (the rows beyond M and N are never written and what they hold only reaches elements of C that do
+ * not exist; K is zero-filled), C updated in place. */
+static int gemm_padded_to_tiles(const skl_gemm_canon *g) {
+  size_t mp, np, kp;
+  const int tile_cols = skl_hip_gemm_mfma_padded_plan(g, &mp, &np, &kp);
+  const size_t esa = elem_size(g->ta), esb = elem_size(g->tb);
+  skl_gemm_canon h = *g;
+  char *scratch;
+  int done;
+  if (!tile_cols) return 0;
+  skl_hip_sequence_begin();
+  scratch = skl_hip_operand_scratch(mp * kp * esa + np * kp * esb);
+  done = scratch != NULL &&
+         skl_hip_launch_realign((int)esa, g->m, g->k, g->a, SKL_TE, g->a_s0, g->a_s1, 1, 0, g->a_sk, scratch, kp) == 0 &&
+         skl_hip_launch_realign((int)esb, g->n, g->k, g->b, SKL_TE, g->b_s0, g->b_s1, 1, 0, g->b_sk,
+                                scratch + mp * kp * esa, kp) == 0;
+  if (done) {
+    h.a = scratch, h.a_sk = 1, h.a_s0 = kp, h.a_s1 = SKL_TE * kp;
+    h.b = scratch + mp * kp * esa, h.b_sk = 1, h.b_s0 = kp, h.b_s1 = SKL_TE * kp;
+    h.k = kp;
+    done = skl_hip_launch_gemm_mfma_padded(&h, tile_cols) == 0;
+  }
+  skl_hip_sequence_end();
+  return done;
 }
 
 /* Any other blocking (the 4x8 / 8x4 / 4x4 blocks of src/gemm/packed-gemm.md:270-298, blocks of 32, ...): A and B
@@ -291,6 +321,8 @@ static void gemm_on_device(const skl_gemm_desc *d) {
       return;
     }
     if (canonicalize(d, &g)) {
+      if (!fused && gemv_paths(&g, 1)) return;
+      if (gemm_padded_to_tiles(&g)) return;
       if (gemm_fast_path(&g, fused, 1)) return;
       if (gemm_with_realigned_operands(&g, fused)) return;
     } else if (gemm_through_copies(d, fused)) {

@@ -691,7 +691,9 @@ __device__ __forceinline__ Frag join_pieces(const Piece (&pc)[N]) {
 
 constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BN>
+// EDGE: the operands are copies padded to whole tiles, C is not - its last tile rows / columns end at p.m / p.n and
+// the epilogue touches nothing beyond them.
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false>
 __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   using KA = Kind<TA>;
   using M = Mma<TA, TB>;
@@ -928,47 +930,53 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
+    if (EDGE && col >= p.n) continue;
     fused.column(col);
     const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
 #pragma unroll
     for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
       AccElem *out[kEpilogueBatch][4];
+      size_t first_row[kEpilogueBatch][4];
 #pragma unroll
       for (int i = 0; i < kEpilogueBatch; ++i)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block of 64
+          first_row[i][g] = row;
           out[i][g] = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
         }
+      auto inside = [&](int i, int r) { return !EDGE || first_row[i][r >> 2] + (r & 3) < p.m; };
       if (init) {
 #pragma unroll
         for (int i = 0; i < kEpilogueBatch; ++i)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             AccElem *dst = out[i][r >> 2] + (r & 3) * p.rsc0;
-            __builtin_nontemporal_store(fused.apply(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta)), dst);
+            if (inside(i, r))
+              __builtin_nontemporal_store(fused.apply(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta)), dst);
           }
       } else {
         AccElem old[kEpilogueBatch][16];
 #pragma unroll
         for (int i = 0; i < kEpilogueBatch; ++i)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) old[i][r] = out[i][r >> 2][(r & 3) * p.rsc0];
+          for (int r = 0; r < 16; ++r) old[i][r] = inside(i, r) ? out[i][r >> 2][(r & 3) * p.rsc0] : AccElem(0);
 #pragma unroll
         for (int i = 0; i < kEpilogueBatch; ++i)
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            __builtin_nontemporal_store(fused.apply(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta)), out[i][r >> 2] + (r & 3) * p.rsc0);
+            if (inside(i, r))
+              __builtin_nontemporal_store(fused.apply(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta)), out[i][r >> 2] + (r & 3) * p.rsc0);
       }
     }
   }
   fused.finish();
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BN>
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false>
 int launch_ring(const MfmaArgs &args) {
   constexpr int lds = kRingStages * (256 + BN) * kRingSlice;
-  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN>;
+  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE>;
   static bool configured = false;
   if (!configured) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -978,8 +986,8 @@ int launch_ring(const MfmaArgs &args) {
     configured = true;
   }
   MfmaArgs p = args;
-  p.tiles_m = (unsigned)(p.m / 256);
-  p.tiles_n = (unsigned)(p.n / BN);
+  p.tiles_m = (unsigned)((p.m + (EDGE ? 255 : 0)) / 256);
+  p.tiles_n = (unsigned)((p.n + (EDGE ? BN - 1 : 0)) / BN);
   const size_t grid = (size_t)p.tiles_m * p.tiles_n;
   if (grid > 0x7FFFFFFFu) {
     skl_hip_record_error(-2, "gemm_mfma: grid too large");
@@ -1149,6 +1157,84 @@ extern "C" int skl_hip_gemm_mfma_supported(const skl_gemm_canon *g) {
   if (!operand_ok(g->b, es, g->b_s1, g->b_s0, g->b_sk, g->n, g->k)) return 0;
   if (((uintptr_t)g->c & 3) != 0) return 0;
   return 1;
+}
+
+namespace {
+
+// Would the problem, as it lies in memory, run on the streaming kernel? (The rule of launch_tile.)
+bool streams_in_place(const skl_gemm_canon *g, size_t es) {
+  if (!skl_hip_gemm_mfma_supported(g) || g->m % 256 != 0 || (g->k * es) % 128 != 0) return false;
+  const size_t tiles_m = g->m / 256;
+  return (g->n % 256 == 0 && tiles_m * (g->n / 256) >= 200) || (g->n % 128 == 0 && tiles_m * (g->n / 128) >= 96);
+}
+
+template <int TA, int TB>
+int launch_padded(const MfmaArgs &p, size_t tile_cols) {
+  return tile_cols == 256 ? launch_ring<TA, TB, true, true, 256, true>(p) : launch_ring<TA, TB, true, true, 128, true>(p);
+}
+
+}  // namespace
+
+// A problem the streaming kernel does not take as it lies in memory - ragged M, N or K, operands off the 16-byte
+// rule - can still run on it from copies of A and B padded to whole tiles (rows contiguous in K, `*kp` elements
+// apart, `*mp` / `*np` of them, K zero-filled to whole slice pairs) while C stays where it is. Returns the tile
+// width (256 or 128) when that is worth it: enough tiles to fill the chip, at most 30 % of padding, and not a
+// problem that streams in place anyway; else 0.
+extern "C" int skl_hip_gemm_mfma_padded_plan(const skl_gemm_canon *g, size_t *mp, size_t *np, size_t *kp) {
+  if (g->m == 0 || g->n == 0 || g->k == 0 || g->ta > SKL_DT_F8E5M2 || g->tb > SKL_DT_F8E5M2) return 0;
+  const bool fp8a = g->ta >= SKL_DT_F8E4M3, fp8b = g->tb >= SKL_DT_F8E4M3;
+  if (!(g->ta == g->tb || (fp8a && fp8b)) || ((uintptr_t)g->c & 3) != 0) return 0;
+  const size_t es = (g->ta == SKL_DT_BF16 || g->ta == SKL_DT_F16) ? 2 : 1;
+  if (streams_in_place(g, es)) return 0;
+  const size_t tiles_m = (g->m + 255) / 256;
+  int tile_cols = 0;
+  if (tiles_m * ((g->n + 255) / 256) >= 200) tile_cols = 256;
+  else if (tiles_m * ((g->n + 127) / 128) >= 96) tile_cols = 128;
+  if (!tile_cols) return 0;
+  *mp = tiles_m * 256;
+  *np = (g->n + tile_cols - 1) / tile_cols * tile_cols;
+  *kp = (g->k * es + 127) / 128 * 128 / es;
+  const double padded = (double)*mp * (double)*np * (double)*kp, exact = (double)g->m * (double)g->n * (double)g->k;
+  if (padded > 1.3 * exact || *kp * es * 256 >= (size_t(1) << 31)) return 0;  // offsets inside a tile stay in 32 bits
+  return tile_cols;
+}
+
+// `g` describes the padded copies (a_sk == b_sk == 1, rows kp apart in flat blocks of 64, k == kp) and the true
+// m, n and C; `tile_cols` is what the plan returned.
+extern "C" int skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile_cols) {
+  const size_t es = (g->ta == SKL_DT_BF16 || g->ta == SKL_DT_F16) ? 2 : 1;
+  if ((tile_cols != 256 && tile_cols != 128) || g->a_sk != 1 || g->b_sk != 1 || (g->k * es) % 128 != 0 ||
+      g->a_s1 != 64 * g->a_s0 || g->b_s1 != 64 * g->b_s0 || ((g->a_s0 * es) & 15) != 0 || ((g->b_s0 * es) & 15) != 0 ||
+      ((uintptr_t)g->a & 15) != 0 || ((uintptr_t)g->b & 15) != 0 || ((uintptr_t)g->c & 3) != 0) {
+    skl_hip_record_error(-2, "gemm_mfma_padded: not a padded problem");
+    return -2;
+  }
+  MfmaArgs p;
+  p.a = (const char *)g->a;
+  p.b = (const char *)g->b;
+  p.c = (char *)g->c;
+  p.m = g->m, p.n = g->n, p.k = g->k;
+  p.a_s1 = g->a_s1, p.a_s0 = g->a_s0, p.a_sk = g->a_sk;
+  p.b_s1 = g->b_s1, p.b_s0 = g->b_s0, p.b_sk = g->b_sk;
+  p.rsc0 = g->rsc0, p.csc0 = g->csc0, p.rsc1 = g->rsc1, p.csc1 = g->csc1;
+  p.alpha = g->alpha, p.beta = g->beta;
+  p.bias = (const char *)g->bias, p.max = (char *)g->max;
+  p.tiles_m = p.tiles_n = 0;
+  p.splits = 1, p.slices_per_split = 0, p.partial = nullptr;
+  switch (g->ta * 8 + g->tb) {
+    case SKL_DT_I8 * 8 + SKL_DT_I8: return launch_padded<SKL_DT_I8, SKL_DT_I8>(p, tile_cols);
+#ifndef SKL_MFMA_INT8_ONLY
+    case SKL_DT_BF16 * 8 + SKL_DT_BF16: return launch_padded<SKL_DT_BF16, SKL_DT_BF16>(p, tile_cols);
+    case SKL_DT_F16 * 8 + SKL_DT_F16: return launch_padded<SKL_DT_F16, SKL_DT_F16>(p, tile_cols);
+    case SKL_DT_F8E4M3 * 8 + SKL_DT_F8E4M3: return launch_padded<SKL_DT_F8E4M3, SKL_DT_F8E4M3>(p, tile_cols);
+    case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E5M2: return launch_padded<SKL_DT_F8E5M2, SKL_DT_F8E5M2>(p, tile_cols);
+    case SKL_DT_F8E4M3 * 8 + SKL_DT_F8E5M2: return launch_padded<SKL_DT_F8E4M3, SKL_DT_F8E5M2>(p, tile_cols);
+    case SKL_DT_F8E5M2 * 8 + SKL_DT_F8E4M3: return launch_padded<SKL_DT_F8E5M2, SKL_DT_F8E4M3>(p, tile_cols);
+#endif
+    default:
+      skl_hip_record_error(-2, "gemm_mfma_padded: operand type pair");
+      return -2;
+  }
 }
 
 extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {

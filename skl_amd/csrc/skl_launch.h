@@ -84,6 +84,12 @@ int skl_hip_launch_gemm_tiled(const skl_gemm_canon *g);
 int skl_hip_gemm_mfma_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g);
 
+/* The streaming kernel on copies of A and B padded to whole tiles (see skl_gemm_mfma.hip): the plan returns the tile
+ * width (256 / 128) and the padded extents when that pays, else 0; the launch takes the canonical description of the
+ * copies (K contiguous, rows *kp apart, k == *kp) with the true m, n and C. */
+int skl_hip_gemm_mfma_padded_plan(const skl_gemm_canon *g, size_t *mp, size_t *np, size_t *kp);
+int skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile_cols);
+
 /* M == 1 streaming kernels: y[j*csc] = beta*y + alpha * sum_p x[p*x_sk] * B(p,j).
  * `layout`: 0 = B row-major (b_s0 == 1 within 64-blocks), 1 = K4-interleaved
  * int8 (`p4x1c`: B(p,j) at (p/4)*b_sk + j*4 + p%4). */

@@ -58,6 +58,74 @@ __global__ void __launch_bounds__(kThreads) realign_kernel(const T *__restrict__
   }
 }
 
+// The two common sources of a realigning copy, with 16-byte stores on the aligned side. Flat K (k0 == 1).
+//
+// Source rows contiguous in K: one thread per 16-byte piece of a destination row, fetched with the widest loads
+// the source's alignment allows (VEC bytes: 16, 4, or one element).
+template <int ES, int VEC>
+__global__ void __launch_bounds__(kThreads) realign_rows_kernel(const char *__restrict__ src, char *__restrict__ dst, size_t x,
+                                                                size_t kbytes, size_t pitch, RealignSource f) {
+  const size_t pieces_per_row = pitch / 16;
+  const size_t idx = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (idx >= x * pieces_per_row) return;
+  const size_t xx = idx / pieces_per_row, off = (idx % pieces_per_row) * 16;
+  const char *row = src + ((xx / f.x0) * f.s1 + (xx % f.x0) * f.s0) * ES;
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (off + 16 <= kbytes) {
+    if constexpr (VEC == 16) {
+      v = *reinterpret_cast<const uint4 *>(row + off);
+    } else if constexpr (VEC == 4) {
+      const unsigned *w = reinterpret_cast<const unsigned *>(row + off);
+      v = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+      unsigned char b[16];
+#pragma unroll
+      for (int i = 0; i < 16; i += ES) {
+        if constexpr (ES == 1) b[i] = (unsigned char)row[off + i];
+        else *reinterpret_cast<uint16_t *>(b + i) = *reinterpret_cast<const uint16_t *>(row + off + i);
+      }
+      v = *reinterpret_cast<const uint4 *>(b);
+    }
+  } else if (off < kbytes) {  // the piece that holds the end of K: element by element, zero beyond
+    unsigned char b[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    for (size_t i = 0; off + i < kbytes; ++i) b[i] = (unsigned char)row[off + i];
+    v = *reinterpret_cast<const uint4 *>(b);
+  }
+  *reinterpret_cast<uint4 *>(dst + xx * pitch + off) = v;
+}
+
+// Source contiguous along x (runs of x0 elements, blocks s1 apart), K strided: a 64 x 64 tile is read with lanes
+// along x, kept in LDS with K contiguous (row pitch 64 elements + 4 bytes: lanes along x hit distinct banks), and
+// written as 16-byte pieces of the destination rows.
+template <typename T>
+__global__ void __launch_bounds__(kThreads) realign_transpose_kernel(const T *__restrict__ src, char *__restrict__ dst, size_t x,
+                                                                     size_t k, size_t pitch, RealignSource f, unsigned tiles_p) {
+  constexpr int kRowBytes = kTile * (int)sizeof(T), kLdsPitch = kRowBytes + 4;
+  __shared__ __attribute__((aligned(16))) char tile[kTile * kLdsPitch];
+  const size_t x_base = (size_t)(blockIdx.x / tiles_p) * kTile, p_base = (size_t)(blockIdx.x % tiles_p) * kTile;
+  {
+    const int xi = threadIdx.x % kTile, pr = threadIdx.x / kTile;
+    const size_t xx = x_base + xi;
+    const T *col = src + (xx / f.x0) * f.s1 + (xx % f.x0) * f.s0;
+#pragma unroll 4
+    for (int pi = pr; pi < kTile; pi += kThreads / kTile) {
+      const size_t pp = p_base + pi;
+      const T v = (xx < x && pp < k) ? col[pp * f.sk1] : T(0);
+      *reinterpret_cast<T *>(tile + xi * kLdsPitch + pi * (int)sizeof(T)) = v;
+    }
+  }
+  __syncthreads();
+  constexpr int kPiecesPerRow = kRowBytes / 16, kPieces = kTile * kPiecesPerRow;
+#pragma unroll
+  for (int piece = threadIdx.x; piece < kPieces; piece += kThreads) {
+    const int xi = piece / kPiecesPerRow, off = (piece % kPiecesPerRow) * 16;
+    const size_t xx = x_base + xi, byte = p_base * sizeof(T) + off;
+    if (xx >= x || byte >= pitch) continue;  // the pitch is a whole number of 16-byte pieces
+    const unsigned *w = reinterpret_cast<const unsigned *>(tile + xi * kLdsPitch + off);
+    *reinterpret_cast<uint4 *>(dst + xx * pitch + byte) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
 template <typename T, bool PACK>
 __global__ void __launch_bounds__(kThreads) pack_tile_kernel(const T *__restrict__ src, T *__restrict__ dst, PackArgs p) {
   __shared__ T tile[kTile][kTile + (sizeof(T) == 4 ? 1 : sizeof(T) == 2 ? 2 : 4)];
@@ -362,6 +430,36 @@ int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_
   const size_t step_x = x0 > 1 ? s0 : s1, step_p = k0 > 1 ? sk0 : sk1;
   const int along_x = step_x == 1 && step_p != 1;
   hipStream_t st = skl_current_stream();
+  const size_t es = (size_t)esize, pitch = kp * es;
+  if (k0 == 1 && pitch % 16 == 0 && ((uintptr_t)dst & 15) == 0) {
+    if (sk1 == 1) {  // rows contiguous in K
+      const size_t blocks = (x * (pitch / 16) + kThreads - 1) / kThreads;
+      if (blocks <= 0x7FFFFFFFu) {
+        const uintptr_t align = (uintptr_t)src | (x0 > 1 ? s0 * es : 0) | (s1 * es);
+        const char *s8 = (const char *)src;
+        char *d8 = (char *)dst;
+        const unsigned grid = (unsigned)blocks;
+        if (esize == 1) {
+          if (align % 16 == 0) realign_rows_kernel<1, 16><<<grid, kThreads, 0, st>>>(s8, d8, x, k * es, pitch, f);
+          else if (align % 4 == 0) realign_rows_kernel<1, 4><<<grid, kThreads, 0, st>>>(s8, d8, x, k * es, pitch, f);
+          else realign_rows_kernel<1, 1><<<grid, kThreads, 0, st>>>(s8, d8, x, k * es, pitch, f);
+        } else {
+          if (align % 16 == 0) realign_rows_kernel<2, 16><<<grid, kThreads, 0, st>>>(s8, d8, x, k * es, pitch, f);
+          else if (align % 4 == 0) realign_rows_kernel<2, 4><<<grid, kThreads, 0, st>>>(s8, d8, x, k * es, pitch, f);
+          else realign_rows_kernel<2, 2><<<grid, kThreads, 0, st>>>(s8, d8, x, k * es, pitch, f);
+        }
+        return skl_check_launch("realign_rows");
+      }
+    } else if (along_x) {
+      if (esize == 1)
+        realign_transpose_kernel<uint8_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint8_t *)src, (char *)dst, x, k, pitch, f,
+                                                                              (unsigned)tiles_p);
+      else
+        realign_transpose_kernel<uint16_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint16_t *)src, (char *)dst, x, k, pitch,
+                                                                               f, (unsigned)tiles_p);
+      return skl_check_launch("realign_transpose");
+    }
+  }
   if (esize == 1)
     realign_kernel<uint8_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint8_t *)src, (uint8_t *)dst, x, k, kp, f,
                                                                 (unsigned)tiles_p, along_x);

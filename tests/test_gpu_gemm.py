@@ -507,3 +507,37 @@ def test_register_tiled_kernel_bit_identical(gpu, ta):
         want = run_oracle_gemm(case, a, b, c)
         got = run_gemm(gpu, "rcprc", case, a, b, c, "device")
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (ta, i, vars(case))
+
+
+@pytest.mark.parametrize("ta,tb", (("i8", "i8"), ("bf16", "bf16"), ("f16", "f16"), ("f8e4m3", "f8e4m3"), ("f8e4m3", "f8e5m2")))
+def test_ragged_problems_on_padded_copies(gpu, ta, tb):
+    """Ragged M, N and K (and odd leading dimensions) on a problem large enough to fill the chip: A and B are copied
+    into tile-padded scratch memory and the streaming kernel runs with an epilogue that stops at C's true edges.
+    256 x 128 and 256 x 256 tiles, row- and column-major operands, beta == 0 and != 0, C with padded rows (the
+    clobber check), fused bias and maximum. int8 bit-exact, floating point inside the reference's bound."""
+    from support import GemmCase
+    fp8 = ta.startswith("f8")
+    shapes = [(1500, 2100, 500 if ta == "i8" or fp8 else 250, True, True),      # 6 x 17 tiles of 256 x 128
+              (3300, 4000, 250 if ta == "i8" or fp8 else 125, False, False),    # 13 x 16 tiles of 256 x 256
+              (1537, 2049, 1000, True, False)]
+    for i, (m, n, k, a_rows, b_rows) in enumerate(shapes):
+        rsa, csa = (k + 1, 1) if a_rows else (1, m + 3)
+        rsb, csb = (n + 5, 1) if b_rows else (1, k + 7)
+        alpha, beta = ((2, -1) if ta == "i8" else (1.5, -0.5)) if i != 1 else ((1, 0) if ta == "i8" else (1.0, 0.0))
+        case = GemmCase(ta, tb, alpha, beta, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=rsa, csa1=csa,
+                        rsb0=0, csb0=0, rsb1=rsb, csb1=csb, rsc0=0, csc0=0, rsc1=n + 3, csc1=1)
+        a, b, c = case.make_inputs(9500 + i)
+        got = run_gemm(gpu, "rc", case, a, b, c, "device")
+        if case.is_int:
+            want = run_oracle_gemm(case, a, b, c)
+            assert np.array_equal(got, want), (m, n, k)
+        else:
+            support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=support.FP8_MFMA_REL if fp8 else 0.0)
+        if i == 0 and ta == tb:
+            rng = np.random.default_rng(i)
+            bias = (rng.integers(-99, 99, n).astype(np.int32) if case.is_int else rng.uniform(-4, 4, n).astype(np.float32))
+            start = np.array([-(1 << 31)], np.int32) if case.is_int else np.array([-np.inf], np.float32)
+            fused, top = run_fused_gemm(gpu, "rc", case, a, b, c, bias, start, "device")
+            want_c, want_top = fused_expectation(case, got, bias, start)
+            assert np.array_equal(fused.view(np.uint8), want_c.view(np.uint8)), (ta, m, n, k)
+            assert top[0] == want_top[0]
