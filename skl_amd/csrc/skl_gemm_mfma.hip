@@ -754,16 +754,19 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   char *region_a = smem, *region_b = smem + TileA::kRegion;
   const unsigned addr_a = (unsigned)(size_t)LDS_PTR(char, smem), addr_b = addr_a + TileA::kRegion;
 
+  // K may be shared between `splits` workgroups per tile: p.k is then one share (whole slice pairs), split s
+  // starts s shares into K and leaves its raw sums in plane s of the workspace.
   unsigned tm, tn;
-  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const unsigned tiles = p.tiles_m * p.tiles_n, split = blockIdx.x / tiles;
+  tile_of_block(blockIdx.x % tiles, p.tiles_m, p.tiles_n, tm, tn);
   const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
 
   LA la;
   LB lb;
-  la.init(p.a, m0, p.a_s1, p.a_s0, p.a_sk);
-  lb.init(p.b, n0, p.b_s1, p.b_s0, p.b_sk);
+  la.init(p.a + (size_t)split * p.k * p.a_sk * ES, m0, p.a_s1, p.a_s0, p.a_sk);
+  lb.init(p.b + (size_t)split * p.k * p.b_sk * ES, n0, p.b_s1, p.b_s0, p.b_sk);
   RA ra;
   RB rb;
   ra.init(wm);
@@ -923,6 +926,22 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
+  if (p.splits > 1) {  // a share of K: the raw sums go to this split's M x N plane
+    AccElem *plane = reinterpret_cast<AccElem *>(p.partial) + (size_t)split * p.m * p.n;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const size_t col = n0 + wn + j * 32 + (lane & 31);
+      if (EDGE && col >= p.n) continue;
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const size_t row = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+          if (!EDGE || row < p.m) plane[row * p.n + col] = acc[i][j][r];
+        }
+    }
+    return;
+  }
   // Epilogue, as in the kernel above: old values requested kEpilogueBatch blocks at a time, non-temporal stores.
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
   const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
@@ -973,30 +992,6 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   fused.finish();
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false>
-int launch_ring(const MfmaArgs &args) {
-  constexpr int lds = kRingStages * (256 + BN) * kRingSlice;
-  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE>;
-  static bool configured = false;
-  if (!configured) {
-    int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                           "gemm_mfma_ring: LDS size");
-    if (rc != 0) return rc;
-    configured = true;
-  }
-  MfmaArgs p = args;
-  p.tiles_m = (unsigned)((p.m + (EDGE ? 255 : 0)) / 256);
-  p.tiles_n = (unsigned)((p.n + (EDGE ? BN - 1 : 0)) / BN);
-  const size_t grid = (size_t)p.tiles_m * p.tiles_n;
-  if (grid > 0x7FFFFFFFu) {
-    skl_hip_record_error(-2, "gemm_mfma: grid too large");
-    return -2;
-  }
-  kernel<<<(unsigned)grid, 512, lds, skl_current_stream()>>>(p);
-  return skl_check_launch("gemm_mfma_ring");
-}
-
 // C = beta*C + alpha * (sum of the splits' planes, in split order), then the fused steps: the second
 // half of a GEMM whose K range was shared out between workgroups.
 template <typename T>
@@ -1024,14 +1019,61 @@ __global__ void __launch_bounds__(256) gemm_split_reduce_kernel(MfmaArgs p) {
   }
 }
 
-// How many ways K is shared out when a problem has too few tiles for the chip: enough to put about two
-// workgroups on every compute unit, each share at least kMinSlicesPerSplit slices long, planes within 64 MiB.
 struct SequenceGuard {
   const bool held;
   explicit SequenceGuard(bool hold) : held(hold) { if (held) skl_hip_sequence_begin(); }
   ~SequenceGuard() { if (held) skl_hip_sequence_end(); }
 };
 
+constexpr size_t kRingMinSlicesPerSplit = 64;  // below 8 KiB of K per row the pass over the planes costs what the split saves
+
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false>
+int launch_ring(const MfmaArgs &args) {
+  constexpr int lds = kRingStages * (256 + BN) * kRingSlice;
+  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE>;
+  static bool configured = false;
+  if (!configured) {
+    int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "gemm_mfma_ring: LDS size");
+    if (rc != 0) return rc;
+    configured = true;
+  }
+  MfmaArgs p = args;
+  p.tiles_m = (unsigned)((p.m + (EDGE ? 255 : 0)) / 256);
+  p.tiles_n = (unsigned)((p.n + (EDGE ? BN - 1 : 0)) / BN);
+  const size_t tiles = (size_t)p.tiles_m * p.tiles_n;
+  // Tiles for at most half of the 256 compute units: K is shared between two workgroups per tile (each at least
+  // kRingMinSlicesPerSplit slices long) and a second pass adds the two planes and applies alpha / beta.
+  constexpr int ES = Kind<TA>::ES;
+  const size_t slices = p.k * ES / kRingSlice;
+  p.splits = (tiles <= 128 && slices % 4 == 0 && slices / 2 >= kRingMinSlicesPerSplit) ? 2 : 1;
+  SequenceGuard sequence(p.splits > 1);
+  if (p.splits > 1) {
+    p.partial = (char *)skl_workspace((size_t)p.splits * p.m * p.n * 4);
+    if (!p.partial) return -4;
+    p.k /= p.splits;  // one share; whole slice pairs
+  }
+  const size_t grid = tiles * p.splits;
+  if (grid > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemm_mfma: grid too large");
+    return -2;
+  }
+  kernel<<<(unsigned)grid, 512, lds, skl_current_stream()>>>(p);
+  int rc = skl_check_launch("gemm_mfma_ring");
+  if (rc != 0 || p.splits == 1) return rc;
+  using AccElem = decltype(typename Kind<TA>::Acc{}.x);
+  const size_t blocks = (p.m * p.n + 255) / 256;
+  if (blocks > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemm_mfma: grid too large");
+    return -2;
+  }
+  gemm_split_reduce_kernel<AccElem><<<(unsigned)blocks, 256, 0, skl_current_stream()>>>(p);
+  return skl_check_launch("gemm_split_reduce");
+}
+
+// How many ways K is shared out when a problem has too few tiles for the chip: enough to put about two
+// workgroups on every compute unit, each share at least kMinSlicesPerSplit slices long, planes within 64 MiB.
 constexpr size_t kMinSlicesPerSplit = 8, kSplitFromSlices = 32, kSplitPlaneLimit = size_t(64) << 20;
 inline unsigned splits_for(size_t tiles, size_t slices, size_t m, size_t n) {
   if (tiles >= 256 || slices < kSplitFromSlices) return 1;
@@ -1089,6 +1131,7 @@ int launch_one(const MfmaArgs &args) {
 template <int TA, int TB, bool A_KC, bool B_KC>
 int launch_tile(const MfmaArgs &p) {
   constexpr int ES = Kind<TA>::ES;
+  constexpr size_t kRing128FromTiles = 96;
   // The streaming kernel takes problems that its tiles divide evenly: 256 x 256 tiles when those
   // can fill the 256 compute units, 256 x 128 tiles for the sizes below that; everything else runs
   // on the small, bounds-checked kernel.
@@ -1111,7 +1154,7 @@ int launch_tile(const MfmaArgs &p) {
       }
       return launch_ring<TA, TB, A_KC, B_KC, 256>(p);
     }
-    if (p.n % 128 == 0 && tiles_m * (p.n / 128) >= 96) return launch_ring<TA, TB, A_KC, B_KC, 128>(p);
+    if (p.n % 128 == 0 && tiles_m * (p.n / 128) >= kRing128FromTiles) return launch_ring<TA, TB, A_KC, B_KC, 128>(p);
   }
   // Small problems: 64 x 64 tiles put four times as many workgroups on the chip.
   if (skl_div_up(p.m, 128) * (size_t)skl_div_up(p.n, 128) < 64) return launch_one<TA, TB, A_KC, B_KC, 64, 64, 2, 2, true>(p);

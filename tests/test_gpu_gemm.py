@@ -541,3 +541,35 @@ def test_ragged_problems_on_padded_copies(gpu, ta, tb):
             want_c, want_top = fused_expectation(case, got, bias, start)
             assert np.array_equal(fused.view(np.uint8), want_c.view(np.uint8)), (ta, m, n, k)
             assert top[0] == want_top[0]
+
+
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f8e4m3"))
+def test_streaming_kernel_shares_k_when_tiles_fill_half_the_chip(gpu, ta):
+    """96 to 128 tiles of 256 x 128: two workgroups per tile take half of K each, a second pass adds the planes and
+    applies alpha / beta and the fused steps. Whole tiles in place and a ragged problem on padded copies. int8
+    bit-exact; floating point inside the bound and the same bits on two runs."""
+    from support import GemmCase
+    k = 8192 if ta != "bf16" else 4096  # 8 KiB of K per row: the shortest K that is shared
+    for i, (m, n, kk, ld_extra) in enumerate(((1536, 2048, k, 0), (1500, 2040, k - 40, 1))):
+        case = GemmCase(ta, None, 2 if ta == "i8" else 1.5, -1 if ta == "i8" else -0.5, m0=1, n0=1, k0=1, m1=m, n1=n, k1=kk,
+                        rsa0=0, csa0=0, rsa1=kk + ld_extra, csa1=1, rsb0=0, csb0=0, rsb1=n + ld_extra, csb1=1,
+                        rsc0=0, csc0=0, rsc1=n + 2, csc1=1)
+        a, b, c = case.make_inputs(9700 + i)
+        got = run_gemm(gpu, "rc", case, a, b, c, "device")
+        if case.is_int:
+            # 25 G multiply-adds are minutes of the scalar checker; every partial sum here is below 2^53, so the
+            # fp64 matrix product of the widened operands is the exact integer result
+            A, B, C, oc = case.dense(a, b, c)
+            want = c.copy()
+            want[oc] = (case.alpha * (A @ B) + case.beta * C).astype(np.int64).astype(np.int32)
+            assert np.array_equal(got, want), (m, n, kk)
+        else:
+            support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=support.FP8_MFMA_REL if ta.startswith("f8") else 0.0)
+            assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, "device").view(np.uint8))
+        rng = np.random.default_rng(i)
+        bias = (rng.integers(-99, 99, n).astype(np.int32) if case.is_int else rng.uniform(-4, 4, n).astype(np.float32))
+        start = np.array([-(1 << 31)], np.int32) if case.is_int else np.array([-np.inf], np.float32)
+        fused, top = run_fused_gemm(gpu, "rc", case, a, b, c, bias, start, "device")
+        want_c, want_top = fused_expectation(case, got, bias, start)
+        assert np.array_equal(fused.view(np.uint8), want_c.view(np.uint8)), (ta, m, n, kk)
+        assert top[0] == want_top[0]
