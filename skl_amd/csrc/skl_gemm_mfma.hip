@@ -1154,7 +1154,10 @@ int launch_tile(const MfmaArgs &p) {
       }
       return launch_ring<TA, TB, A_KC, B_KC, 256>(p);
     }
-    if (p.n % 128 == 0 && tiles_m * (p.n / 128) >= kRing128FromTiles) return launch_ring<TA, TB, A_KC, B_KC, 128>(p);
+    // ... from 96 tiles on, or from 64 when K is long enough to be shared between two workgroups per tile
+    const size_t tiles128 = p.n % 128 == 0 ? tiles_m * (p.n / 128) : 0, slices = p.k * ES / kRingSlice;
+    if (tiles128 >= kRing128FromTiles || (tiles128 >= 64 && slices % 4 == 0 && slices / 2 >= kRingMinSlicesPerSplit))
+      return launch_ring<TA, TB, A_KC, B_KC, 128>(p);
   }
   // Small problems: 64 x 64 tiles put four times as many workgroups on the chip.
   // ... and for the 16-bit kinds up to 64 rows of A: a 128-row tile would fetch and multiply rows that do not exist

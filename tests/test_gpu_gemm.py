@@ -550,7 +550,7 @@ def test_streaming_kernel_shares_k_when_tiles_fill_half_the_chip(gpu, ta):
     bit-exact; floating point inside the bound and the same bits on two runs."""
     from support import GemmCase
     k = 8192 if ta != "bf16" else 4096  # 8 KiB of K per row: the shortest K that is shared
-    for i, (m, n, kk, ld_extra) in enumerate(((1536, 2048, k, 0), (1500, 2040, k - 40, 1))):
+    for i, (m, n, kk, ld_extra) in enumerate(((1536, 2048, k, 0), (1500, 2040, k - 40, 1), (256, 11008, k, 0))):  # 96, 96, 86 tiles
         case = GemmCase(ta, None, 2 if ta == "i8" else 1.5, -1 if ta == "i8" else -0.5, m0=1, n0=1, k0=1, m1=m, n1=n, k1=kk,
                         rsa0=0, csa0=0, rsa1=kk + ld_extra, csa1=1, rsb0=0, csb0=0, rsb1=n + ld_extra, csb1=1,
                         rsc0=0, csc0=0, rsc1=n + 2, csc1=1)
