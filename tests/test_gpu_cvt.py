@@ -133,3 +133,40 @@ def test_mixed_pointers_are_refused(gpu):
     gpu.skl_cvt_f32_f8e4m3_gfx950(d, x, 1.0, 16)
     assert gpu.skl_hip_last_error() == -1
     assert b"mixed" in gpu.skl_hip_last_error_string()
+
+
+@pytest.mark.parametrize("sat", (False, True))
+@pytest.mark.parametrize("fmt", FMTS)
+def test_f32_every_bit_pattern(gpu, fmt, sat):
+    """All 2^32 fp32 bit patterns through the GPU kernel against the CPU checker (which is itself compared with the
+    compiled reference over the same 2^32 inputs by test_oracle_cvt's exhaustive sweep). The checker runs on a pool of
+    threads while the GPU converts the next chunk: about four seconds per variant on the GPU host."""
+    from concurrent.futures import ThreadPoolExecutor
+    stem = f"skl_cvt_{'sat_' if sat else ''}f32_{fmt}"
+    chunk = 1 << 24
+    src, dst = skl_amd.DeviceBuffer(4 * chunk), skl_amd.DeviceBuffer(chunk)
+
+    def chunk_input(c):
+        return (np.arange(chunk, dtype=np.uint32) | np.uint32(c << 24)).view(np.float32)
+
+    def checker(c):
+        want = np.empty(chunk, np.uint8)
+        getattr(oracle(), stem + "_oracle")(want, chunk_input(c), 1.0, chunk)
+        return want
+
+    with ThreadPoolExecutor(max_workers=12) as pool:
+        window = 24
+        pending = {c: pool.submit(checker, c) for c in range(window)}
+        for c in range(256):
+            src.upload(chunk_input(c))
+            getattr(gpu, stem + "_gfx950")(dst, src, 1.0, chunk)
+            assert gpu.skl_hip_synchronize() == 0
+            got = dst.download(np.uint8)
+            want = pending.pop(c).result()
+            if c + window < 256:
+                pending[c + window] = pool.submit(checker, c + window)
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, (c, [(hex(int(chunk_input(c).view(np.uint32)[i])), hex(got[i]), hex(want[i])) for i in bad[:5]])
+            if c % 32 == 31:
+                print(f"{stem}: {c + 1} / 256 chunks equal", flush=True)
+    src.free(), dst.free()
