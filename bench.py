@@ -202,6 +202,15 @@ def wl_gemm_i8_8192(lib, rng):
                   8192, 1, lambda n: rand_i8(rng, n), lambda n: rand_i8(rng, n), 1, 0, np.int32, "i8")
 
 
+def wl_gemm_i8_4000(lib, rng):
+    """Ragged M, N, K: A and B are copied into tile-padded scratch memory, the streaming kernel runs on the copies."""
+    d = _dense(lib, rng, "int8 GEMM 4000^3 (row-major, alpha=1, beta=0; ragged: runs on tile-padded copies)",
+               "skl_gemm_i8_i8_i32_gfx950", 4000, 4000, 4000, 1, lambda n: rand_i8(rng, n), lambda n: rand_i8(rng, n), 1, 0,
+               np.int32, "i8")
+    d["kernel"] = "realign_rows_kernel + realign_transpose_kernel + gemm_mfma_ring_kernel<EDGE>"
+    return d
+
+
 def wl_gemm_i8_512(lib, rng):
     return _dense(lib, rng, "int8 GEMM 512^3 (row-major, alpha=1, beta=0)", "skl_gemm_i8_i8_i32_gfx950", 512, 512, 512,
                   1, lambda n: rand_i8(rng, n), lambda n: rand_i8(rng, n), 1, 0, np.int32, "i8")
@@ -357,6 +366,7 @@ WORKLOADS = {
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2),
     "gemm_f8e4m3_8192_rowmajor_a": (wl_gemm_f8_layout(True, False), 10, 2),
     "gemm_f8e4m3_8192_kcontig": (wl_gemm_f8_layout(True, True), 10, 2),
+    "gemm_i8_4000": (wl_gemm_i8_4000, 20, 3),
     "gemm_bf16_2048x4096x4096": (wl_gemm_bf16, 20, 3),
     "gemm_f32_4096": (wl_gemm_f32, 5, 1),
     "gemm_f64_4096": (wl_gemm_f64, 5, 1),
