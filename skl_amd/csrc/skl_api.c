@@ -106,6 +106,31 @@ static int flat_k(size_t k0, size_t k1, size_t s0, size_t s1, size_t *sk) {
   return 1;
 }
 
+static unsigned log2_of_power_of_two(size_t v) { /* 0 if v is not a power of two (or is 1) */
+  unsigned s = 0;
+  if (v < 2 || (v & (v - 1)) != 0) return 0;
+  while (((size_t)1 << s) < v) ++s;
+  return s;
+}
+
+/* C's part of the canonical form. With `small_blocks`, power-of-two blocks other than 64 (at least 4 rows) are
+ * accepted as they are - the matrix-core epilogues index them directly. */
+static int canonicalize_c(const skl_gemm_desc *d, skl_gemm_canon *g, int small_blocks) {
+  g->c = d->c;
+  g->c_row_shift = g->c_col_shift = 6;
+  if (!block64(d->m0, d->m1, d->rsc0, d->rsc1, &g->rsc0, &g->rsc1)) {
+    const unsigned s = log2_of_power_of_two(d->m0);
+    if (!small_blocks || s < 2) return 0;
+    g->c_row_shift = s, g->rsc0 = d->rsc0, g->rsc1 = d->rsc1;
+  }
+  if (!block64(d->n0, d->n1, d->csc0, d->csc1, &g->csc0, &g->csc1)) {
+    const unsigned s = log2_of_power_of_two(d->n0);
+    if (!small_blocks || s < 1) return 0;
+    g->c_col_shift = s, g->csc0 = d->csc0, g->csc1 = d->csc1;
+  }
+  return 1;
+}
+
 static int canonicalize(const skl_gemm_desc *d, skl_gemm_canon *g) {
   g->ta = d->ta;
   g->tb = d->tb;
@@ -123,9 +148,7 @@ static int canonicalize(const skl_gemm_desc *d, skl_gemm_canon *g) {
   if (!flat_k(d->k0, d->k1, d->rsb0, d->rsb1, &g->b_sk)) return 0;
   if (!block64(d->m0, d->m1, d->rsa0, d->rsa1, &g->a_s0, &g->a_s1)) return 0;
   if (!block64(d->n0, d->n1, d->csb0, d->csb1, &g->b_s0, &g->b_s1)) return 0;
-  if (!block64(d->m0, d->m1, d->rsc0, d->rsc1, &g->rsc0, &g->rsc1)) return 0;
-  if (!block64(d->n0, d->n1, d->csc0, d->csc1, &g->csc0, &g->csc1)) return 0;
-  return 1;
+  return canonicalize_c(d, g, 0);
 }
 
 /* The K4-interleaved int8 layout of the dot4 entry point, M == 1 only. */
@@ -145,6 +168,7 @@ static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g) {
   g->c = d->c;
   g->csc0 = d->csc1;
   g->csc1 = SKL_TE * d->csc1;
+  g->c_row_shift = g->c_col_shift = 6;
   g->alpha = d->alpha;
   g->beta = d->beta;
   return 1;
@@ -183,6 +207,8 @@ static void transposed_view(const skl_gemm_canon *g, skl_gemm_canon *t) {
   t->rsc1 = g->csc1;
   t->csc0 = g->rsc0;
   t->csc1 = g->rsc1;
+  t->c_row_shift = g->c_col_shift;
+  t->c_col_shift = g->c_row_shift;
 }
 
 /* Offers `g` to every kernel but the any-stride one; 1 if one of them takes it. With `launch` == 0 only asks. */
@@ -272,17 +298,20 @@ static int gemm_padded_to_tiles(const skl_gemm_canon *g) {
 }
 
 /* Any other blocking (the 4x8 / 8x4 / 4x4 blocks of src/gemm/packed-gemm.md:270-298, blocks of 32, ...): A and B
- * are copied into rows contiguous in K, C is unpacked into a row-major scratch matrix - always, since even a call
- * with beta == 0 reads C where the product is an exact zero - multiplied there, and packed back. M and N are
+ * are copied into rows contiguous in K, C is unpacked into a row-major scratch matrix - also for beta == 0 when C is
+ * floating point, since such a call still reads C where the product is an exact zero - multiplied there, and packed
+ * back. M and N are
  * whole numbers of blocks, so packing writes exactly the elements the reference writes. */
 static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   const size_t M = d->m0 * d->m1, N = d->n0 * d->n1, K = d->k0 * d->k1;
   const size_t esa = elem_size(d->ta), esb = elem_size(d->tb);
   const size_t kpa = (K * esa + 15) / 16 * 16 / esa, kpb = (K * esb + 15) / 16 * 16 / esb;
   const size_t bytes_a = (M * kpa * esa + 255) / 256 * 256, bytes_b = (N * kpb * esb + 255) / 256 * 256;
+  /* an integer C with beta == 0 is not read at all; a floating-point one is, where the product is an exact zero */
+  const int c_is_read = !(d->ta == SKL_DT_I8 && d->beta.i == 0);
   skl_gemm_canon h;
   char *scratch;
-  int done;
+  int done, c_in_place;
   if (esa > 2 || esb > 2 || M * N * K < ((size_t)1 << 18)) return 0;
   memset(&h, 0, sizeof h);
   h.ta = d->ta, h.tb = d->tb;
@@ -292,21 +321,34 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   h.a_sk = 1, h.a_s0 = kpa, h.a_s1 = SKL_TE * kpa;
   h.b_sk = 1, h.b_s0 = kpb, h.b_s1 = SKL_TE * kpb;
   h.rsc0 = N, h.rsc1 = SKL_TE * N, h.csc0 = 1, h.csc1 = SKL_TE;
+  h.c_row_shift = h.c_col_shift = 6;
   h.alpha = d->alpha, h.beta = d->beta;
   h.bias = d->bias, h.max = d->max;
+  /* C in power-of-two blocks (the 4 x 4 blocks of that format) can be updated where it is by the matrix-core
+   * kernels. Small blocks make their stores short (16 bytes per 4 x 4 block row), so that pays when C would
+   * otherwise travel three times (unpack, update, pack: 8192^3 in 4 x 4 blocks 890 against 1048 us), not when an
+   * integer C with beta == 0 is only packed (998 against 913 us). */
+  c_in_place = c_is_read && canonicalize_c(d, &h, 1);
+  if (!c_in_place) {
+    h.c = (void *)(uintptr_t)256;
+    h.rsc0 = N, h.rsc1 = SKL_TE * N, h.csc0 = 1, h.csc1 = SKL_TE;
+    h.c_row_shift = h.c_col_shift = 6;
+  }
   if (!gemm_fast_path(&h, fused, 0)) return 0;
   skl_hip_sequence_begin();
-  scratch = skl_hip_operand_scratch(bytes_a + bytes_b + M * N * 4);
+  scratch = skl_hip_operand_scratch(bytes_a + bytes_b + (c_in_place ? 0 : M * N * 4));
   done = scratch != NULL;
   if (done) {
-    h.a = scratch, h.b = scratch + bytes_a, h.c = scratch + bytes_a + bytes_b;
+    h.a = scratch, h.b = scratch + bytes_a;
+    if (!c_in_place) h.c = scratch + bytes_a + bytes_b;
     done = skl_hip_launch_realign((int)esa, M, K, d->a, d->m0, d->rsa0, d->rsa1, d->k0, d->csa0, d->csa1, scratch, kpa) == 0 &&
            skl_hip_launch_realign((int)esb, N, K, d->b, d->n0, d->csb0, d->csb1, d->k0, d->rsb0, d->rsb1,
                                   scratch + bytes_a, kpb) == 0 &&
-           skl_hip_launch_unpack(4, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, M, N, h.c, N, 1) == 0;
+           (c_in_place || !c_is_read ||
+            skl_hip_launch_unpack(4, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, M, N, h.c, N, 1) == 0);
   }
   if (done) done = gemm_fast_path(&h, fused, 1);
-  if (done)
+  if (done && !c_in_place)
     done = skl_hip_launch_pack(4, M, N, h.c, N, 1, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, 0) == 0;
   skl_hip_sequence_end();
   return done;

@@ -58,6 +58,7 @@ struct MfmaArgs {
   size_t a_s1, a_s0, a_sk;  // elements
   size_t b_s1, b_s0, b_sk;
   size_t rsc0, csc0, rsc1, csc1;
+  unsigned crs, ccs;  // log2 of C's block rows / columns (6 unless C comes in smaller power-of-two blocks; crs >= 2)
   skl_scalar alpha, beta;
   const char *bias;  // fused epilogue: per-column addend and running maximum of C's type, or null
   char *max;
@@ -458,7 +459,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
     const size_t col = n0 + wn + j * 32 + (lane & 31);
     if (GUARDED && col >= p.n) continue;
     fused.column(col);
-    const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
+    const size_t col_off = (col >> p.ccs) * p.csc1 + (col & ((size_t(1) << p.ccs) - 1)) * p.csc0;
 #pragma unroll
     for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
       AccElem *out[kEpilogueBatch][4];
@@ -466,8 +467,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
       for (int i = 0; i < kEpilogueBatch; ++i)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block of 64
-          out[i][g] = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
+          const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block (blocks have a multiple of 4 rows)
+          out[i][g] = c + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 + col_off;
         }
       auto in_range = [&](int i, int r) {
         return !GUARDED || m0 + wm + (i0 + i) * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3) < p.m;
@@ -951,7 +952,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
     if (EDGE && col >= p.n) continue;
     fused.column(col);
-    const size_t col_off = (col >> 6) * p.csc1 + (col & 63) * p.csc0;
+    const size_t col_off = (col >> p.ccs) * p.csc1 + (col & ((size_t(1) << p.ccs) - 1)) * p.csc0;
 #pragma unroll
     for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
       AccElem *out[kEpilogueBatch][4];
@@ -960,9 +961,9 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
       for (int i = 0; i < kEpilogueBatch; ++i)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block of 64
+          const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block (blocks have a multiple of 4 rows)
           first_row[i][g] = row;
-          out[i][g] = c + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + col_off;
+          out[i][g] = c + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 + col_off;
         }
       auto inside = [&](int i, int r) { return !EDGE || first_row[i][r >> 2] + (r & 3) < p.m; };
       if (init) {
@@ -1007,7 +1008,8 @@ __global__ void __launch_bounds__(256) gemm_split_reduce_kernel(MfmaArgs p) {
     else
       sum = __fadd_rn(sum, plane[(size_t)q * p.m * p.n]);
   }
-  T *c = reinterpret_cast<T *>(p.c) + (row >> 6) * p.rsc1 + (row & 63) * p.rsc0 + (col >> 6) * p.csc1 + (col & 63) * p.csc0;
+  T *c = reinterpret_cast<T *>(p.c) + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 +
+         (col >> p.ccs) * p.csc1 + (col & ((size_t(1) << p.ccs) - 1)) * p.csc0;
   skl_update(sum, c, p.alpha, p.beta);
   if (p.bias || p.max) {
     T v = *c;
@@ -1147,7 +1149,7 @@ int launch_tile(const MfmaArgs &p) {
         head.n = head_cols;
         tail.n = tail_cols;
         tail.b = p.b + (head_cols / 64) * p.b_s1 * ES;
-        tail.c = p.c + (head_cols / 64) * p.csc1 * sizeof(float);  // C elements are 4 bytes for every kind
+        tail.c = p.c + (head_cols >> p.ccs) * p.csc1 * sizeof(float);  // whole blocks; C elements are 4 bytes for every kind
         if (p.bias) tail.bias = p.bias + head_cols * sizeof(float);
         const int rc = launch_ring<TA, TB, A_KC, B_KC, 256>(head);
         return rc != 0 ? rc : launch_ring<TA, TB, A_KC, B_KC, 128>(tail);
@@ -1205,6 +1207,7 @@ extern "C" int skl_hip_gemm_mfma_supported(const skl_gemm_canon *g) {
   if (!operand_ok(g->a, es, g->a_s1, g->a_s0, g->a_sk, g->m, g->k)) return 0;
   if (!operand_ok(g->b, es, g->b_s1, g->b_s0, g->b_sk, g->n, g->k)) return 0;
   if (((uintptr_t)g->c & 3) != 0) return 0;
+  if (g->c_row_shift < 2 || g->c_row_shift > 6 || g->c_col_shift < 1 || g->c_col_shift > 6) return 0;
   return 1;
 }
 
@@ -1266,6 +1269,7 @@ extern "C" int skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile
   p.a_s1 = g->a_s1, p.a_s0 = g->a_s0, p.a_sk = g->a_sk;
   p.b_s1 = g->b_s1, p.b_s0 = g->b_s0, p.b_sk = g->b_sk;
   p.rsc0 = g->rsc0, p.csc0 = g->csc0, p.rsc1 = g->rsc1, p.csc1 = g->csc1;
+  p.crs = g->c_row_shift, p.ccs = g->c_col_shift;
   p.alpha = g->alpha, p.beta = g->beta;
   p.bias = (const char *)g->bias, p.max = (char *)g->max;
   p.tiles_m = p.tiles_n = 0;
@@ -1299,6 +1303,7 @@ extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
   p.a_s1 = g->a_s1, p.a_s0 = g->a_s0, p.a_sk = g->a_sk;
   p.b_s1 = g->b_s1, p.b_s0 = g->b_s0, p.b_sk = g->b_sk;
   p.rsc0 = g->rsc0, p.csc0 = g->csc0, p.rsc1 = g->rsc1, p.csc1 = g->csc1;
+  p.crs = g->c_row_shift, p.ccs = g->c_col_shift;
   p.alpha = g->alpha, p.beta = g->beta;
   p.bias = (const char *)g->bias, p.max = (char *)g->max;
   p.tiles_m = p.tiles_n = 0;

@@ -847,6 +847,7 @@ int launch_kc_of(const skl_gemm_canon *g) {
 extern "C" int skl_hip_gemv_supported(const skl_gemm_canon *g, int layout) {
   const int mode = mode_of(g, layout);
   if (mode < 0) return 0;
+  if (g->c_row_shift != 6 || g->c_col_shift != 6) return 0;  // C in blocks of 64 (or flat) only
   if (g->m != 1 || g->k == 0 || g->n == 0 || g->n > kMaxCols) return 0;
   const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1;
   const size_t cols = (mode == kI8RowMajor || mode >= kF8E4M3) ? 16 : mode == kI8K4 ? 4 : 8;
@@ -879,6 +880,7 @@ extern "C" int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout) {
 extern "C" int skl_hip_gemv_rows_supported(const skl_gemm_canon *g) {
   const int mode = mode_of(g, 0);
   if (mode < 0) return 0;
+  if (g->c_row_shift != 6 || g->c_col_shift != 6) return 0;  // C in blocks of 64 (or flat) only
   if (g->m < 2 || g->m > (size_t)(mode == kI8RowMajor ? kMaxRows : kMaxRowsFloat)) return 0;
   if (g->k == 0 || g->n == 0 || g->m * g->n > kMaxCols) return 0;
   const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1;
@@ -913,6 +915,7 @@ extern "C" int skl_hip_launch_gemv_rows(const skl_gemm_canon *g) {
 extern "C" int skl_hip_gemv_kc_supported(const skl_gemm_canon *g) {
   const int mode = mode_of(g, 0);
   if (mode < 0) return 0;
+  if (g->c_row_shift != 6 || g->c_col_shift != 6) return 0;  // C in blocks of 64 (or flat) only
   if (g->m < 1 || g->m > (size_t)kKcMaxRows || g->k == 0 || g->n == 0) return 0;
   const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1;
   if (g->b_sk != 1 || g->a_sk != 1 || ((g->k * es) % 16) != 0) return 0;

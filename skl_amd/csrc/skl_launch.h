@@ -59,7 +59,10 @@ typedef struct {
 /* Canonical form served by the matrix-core kernels: flat in K, blocked by 64
  * in M and N. A(i,p) = a[(i/64)*a_s1 + (i%64)*a_s0 + p*a_sk] with exactly one of
  * a_s0 / a_sk equal to 1; B(p,j) = b[(j/64)*b_s1 + (j%64)*b_s0 + p*b_sk]
- * likewise; C(i,j) = c[(i/64)*rsc1 + (i%64)*rsc0 + (j/64)*csc1 + (j%64)*csc0]. */
+ * likewise; C(i,j) = c[(i/R)*rsc1 + (i%R)*rsc0 + (j/S)*csc1 + (j%S)*csc0] with
+ * R = 1 << c_row_shift, S = 1 << c_col_shift: 64 x 64 blocks (shift 6) unless C
+ * comes in smaller power-of-two blocks (rows: at least 4), which only the
+ * matrix-core kernels address. */
 typedef struct {
   int ta, tb;
   size_t m, n, k;
@@ -69,6 +72,7 @@ typedef struct {
   size_t b_s1, b_s0, b_sk;
   void *c;
   size_t rsc0, csc0, rsc1, csc1;
+  unsigned c_row_shift, c_col_shift;
   skl_scalar alpha, beta;
   const void *bias; /* as in skl_gemm_desc */
   void *max;

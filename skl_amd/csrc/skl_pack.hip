@@ -94,23 +94,25 @@ __global__ void __launch_bounds__(kThreads) realign_rows_kernel(const char *__re
   *reinterpret_cast<uint4 *>(dst + xx * pitch + off) = v;
 }
 
-// Source contiguous along x (runs of x0 elements, blocks s1 apart), K strided: a 64 x 64 tile is read with lanes
-// along x, kept in LDS with K contiguous (row pitch 64 elements + 4 bytes: lanes along x hit distinct banks), and
-// written as 16-byte pieces of the destination rows.
+// Any other source (contiguous along x, blocked in K, no unit stride at all): a 64 x 64 tile is read with lanes
+// along the source's denser direction, kept in LDS with K contiguous (row pitch 64 elements + 4 bytes: lanes along
+// x hit distinct banks), and written as 16-byte pieces of the destination rows.
 template <typename T>
-__global__ void __launch_bounds__(kThreads) realign_transpose_kernel(const T *__restrict__ src, char *__restrict__ dst, size_t x,
-                                                                     size_t k, size_t pitch, RealignSource f, unsigned tiles_p) {
+__global__ void __launch_bounds__(kThreads) realign_tile_kernel(const T *__restrict__ src, char *__restrict__ dst, size_t x,
+                                                                size_t k, size_t pitch, RealignSource f, unsigned tiles_p,
+                                                                int along_x) {
   constexpr int kRowBytes = kTile * (int)sizeof(T), kLdsPitch = kRowBytes + 4;
   __shared__ __attribute__((aligned(16))) char tile[kTile * kLdsPitch];
   const size_t x_base = (size_t)(blockIdx.x / tiles_p) * kTile, p_base = (size_t)(blockIdx.x % tiles_p) * kTile;
   {
-    const int xi = threadIdx.x % kTile, pr = threadIdx.x / kTile;
-    const size_t xx = x_base + xi;
-    const T *col = src + (xx / f.x0) * f.s1 + (xx % f.x0) * f.s0;
+    const int fast = threadIdx.x % kTile, slow = threadIdx.x / kTile;
 #pragma unroll 4
-    for (int pi = pr; pi < kTile; pi += kThreads / kTile) {
-      const size_t pp = p_base + pi;
-      const T v = (xx < x && pp < k) ? col[pp * f.sk1] : T(0);
+    for (int it = slow; it < kTile; it += kThreads / kTile) {
+      const int xi = along_x ? fast : it, pi = along_x ? it : fast;
+      const size_t xx = x_base + xi, pp = p_base + pi;
+      const T v = (xx < x && pp < k)
+                      ? src[(xx / f.x0) * f.s1 + (xx % f.x0) * f.s0 + (pp / f.k0) * f.sk1 + (pp % f.k0) * f.sk0]
+                      : T(0);
       *reinterpret_cast<T *>(tile + xi * kLdsPitch + pi * (int)sizeof(T)) = v;
     }
   }
@@ -450,15 +452,18 @@ int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_
         }
         return skl_check_launch("realign_rows");
       }
-    } else if (along_x) {
-      if (esize == 1)
-        realign_transpose_kernel<uint8_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint8_t *)src, (char *)dst, x, k, pitch, f,
-                                                                              (unsigned)tiles_p);
-      else
-        realign_transpose_kernel<uint16_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint16_t *)src, (char *)dst, x, k, pitch,
-                                                                               f, (unsigned)tiles_p);
-      return skl_check_launch("realign_transpose");
     }
+  }
+  if (pitch % 16 == 0 && ((uintptr_t)dst & 15) == 0) {
+    // lanes along K when that is the source's denser direction (a unit or the smaller step), else along x
+    const int lanes_along_x = step_x < step_p;
+    if (esize == 1)
+      realign_tile_kernel<uint8_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint8_t *)src, (char *)dst, x, k, pitch, f,
+                                                                       (unsigned)tiles_p, lanes_along_x);
+    else
+      realign_tile_kernel<uint16_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint16_t *)src, (char *)dst, x, k, pitch, f,
+                                                                        (unsigned)tiles_p, lanes_along_x);
+    return skl_check_launch("realign_tile");
   }
   if (esize == 1)
     realign_kernel<uint8_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint8_t *)src, (uint8_t *)dst, x, k, kp, f,
