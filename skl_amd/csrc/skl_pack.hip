@@ -97,22 +97,42 @@ __global__ void __launch_bounds__(kThreads) realign_rows_kernel(const char *__re
 // Any other source (contiguous along x, blocked in K, no unit stride at all): a 64 x 64 tile is read with lanes
 // along the source's denser direction, kept in LDS with K contiguous (row pitch 64 elements + 4 bytes: lanes along
 // x hit distinct banks), and written as 16-byte pieces of the destination rows.
-template <typename T>
+// VECX > 1: the source is contiguous along x in runs that 4-byte loads can take (lanes along x, VECX elements each).
+template <typename T, int VECX>
 __global__ void __launch_bounds__(kThreads) realign_tile_kernel(const T *__restrict__ src, char *__restrict__ dst, size_t x,
                                                                 size_t k, size_t pitch, RealignSource f, unsigned tiles_p,
                                                                 int along_x) {
   constexpr int kRowBytes = kTile * (int)sizeof(T), kLdsPitch = kRowBytes + 4;
   __shared__ __attribute__((aligned(16))) char tile[kTile * kLdsPitch];
   const size_t x_base = (size_t)(blockIdx.x / tiles_p) * kTile, p_base = (size_t)(blockIdx.x % tiles_p) * kTile;
-  {
+  auto at = [&](size_t xx, size_t pp) {
+    return (xx / f.x0) * f.s1 + (xx % f.x0) * f.s0 + (pp / f.k0) * f.sk1 + (pp % f.k0) * f.sk0;
+  };
+  if constexpr (VECX > 1) {
+    constexpr int kLanesX = kTile / VECX, kRowsPerPass = kThreads / kLanesX;
+    const int xi = (threadIdx.x % kLanesX) * VECX, pr = threadIdx.x / kLanesX;
+#pragma unroll
+    for (int pi = pr; pi < kTile; pi += kRowsPerPass) {
+      const size_t xx = x_base + xi, pp = p_base + pi;
+      T v[VECX];
+      if (xx + VECX <= x && pp < k) {
+        const unsigned w = *reinterpret_cast<const unsigned *>(src + at(xx, pp));
+#pragma unroll
+        for (int e = 0; e < VECX; ++e) v[e] = (T)(w >> (8 * sizeof(T) * e));
+      } else {
+#pragma unroll
+        for (int e = 0; e < VECX; ++e) v[e] = (xx + e < x && pp < k) ? src[at(xx + e, pp)] : T(0);
+      }
+#pragma unroll
+      for (int e = 0; e < VECX; ++e) *reinterpret_cast<T *>(tile + (xi + e) * kLdsPitch + pi * (int)sizeof(T)) = v[e];
+    }
+  } else {
     const int fast = threadIdx.x % kTile, slow = threadIdx.x / kTile;
 #pragma unroll 4
     for (int it = slow; it < kTile; it += kThreads / kTile) {
       const int xi = along_x ? fast : it, pi = along_x ? it : fast;
       const size_t xx = x_base + xi, pp = p_base + pi;
-      const T v = (xx < x && pp < k)
-                      ? src[(xx / f.x0) * f.s1 + (xx % f.x0) * f.s0 + (pp / f.k0) * f.sk1 + (pp % f.k0) * f.sk0]
-                      : T(0);
+      const T v = (xx < x && pp < k) ? src[at(xx, pp)] : T(0);
       *reinterpret_cast<T *>(tile + xi * kLdsPitch + pi * (int)sizeof(T)) = v;
     }
   }
@@ -457,12 +477,18 @@ int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_
   if (pitch % 16 == 0 && ((uintptr_t)dst & 15) == 0) {
     // lanes along K when that is the source's denser direction (a unit or the smaller step), else along x
     const int lanes_along_x = step_x < step_p;
-    if (esize == 1)
-      realign_tile_kernel<uint8_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint8_t *)src, (char *)dst, x, k, pitch, f,
-                                                                       (unsigned)tiles_p, lanes_along_x);
-    else
-      realign_tile_kernel<uint16_t><<<(unsigned)tiles, kThreads, 0, st>>>((const uint16_t *)src, (char *)dst, x, k, pitch, f,
-                                                                        (unsigned)tiles_p, lanes_along_x);
+    // 4-byte loads along x: unit stride there in runs of a multiple of 4 bytes, everything else 4-byte aligned
+    const size_t run = x0 > 1 ? x0 : (size_t)1 << 20;  // x0 == 1 with s1 == 1 is one long run
+    const size_t other = ((uintptr_t)src) | (x0 > 1 ? s1 * es : 0) | (k0 > 1 ? sk0 * es : 0) | (sk1 * es);
+    const bool wide = lanes_along_x && step_x == 1 && (run * es) % 4 == 0 && other % 4 == 0;
+    const unsigned grid = (unsigned)tiles, tp = (unsigned)tiles_p;
+    if (esize == 1) {
+      if (wide) realign_tile_kernel<uint8_t, 4><<<grid, kThreads, 0, st>>>((const uint8_t *)src, (char *)dst, x, k, pitch, f, tp, 1);
+      else realign_tile_kernel<uint8_t, 1><<<grid, kThreads, 0, st>>>((const uint8_t *)src, (char *)dst, x, k, pitch, f, tp, lanes_along_x);
+    } else {
+      if (wide) realign_tile_kernel<uint16_t, 2><<<grid, kThreads, 0, st>>>((const uint16_t *)src, (char *)dst, x, k, pitch, f, tp, 1);
+      else realign_tile_kernel<uint16_t, 1><<<grid, kThreads, 0, st>>>((const uint16_t *)src, (char *)dst, x, k, pitch, f, tp, lanes_along_x);
+    }
     return skl_check_launch("realign_tile");
   }
   if (esize == 1)
