@@ -41,10 +41,11 @@ extern "C" {
 #define SKL_HIP_POINTERS_AUTO 0   /* ask the HIP runtime about every pointer (default) */
 #define SKL_HIP_POINTERS_DEVICE 1 /* caller promises device-accessible pointers: no queries */
 
-/* Selects `device` for the calling thread and creates the library's
- * per-device state (workspace for split reductions). Returns 0 or an error. */
+/* Selects `device` for the calling thread and creates the workspace for split
+ * reductions of its current stream (scratch memory is kept per stream and
+ * device, created at a stream's first call that needs it). Returns 0 or an error. */
 int skl_hip_init(int device);
-/* Releases every per-device workspace. Outstanding work is waited for. */
+/* Releases every scratch block of every device and stream. Outstanding work is waited for. */
 void skl_hip_shutdown(void);
 
 void *skl_hip_malloc(size_t bytes);

@@ -10,9 +10,14 @@
 // Stream the calling thread launches on (set through skl_hip_set_stream).
 hipStream_t skl_current_stream();
 
-// Per-device scratch used by split reductions. Grows on demand; contents are
-// only meaningful inside one launch sequence on one stream.
+// Scratch of the current stream (on the current device) used by split reductions. Grows on
+// demand; contents are only meaningful inside one launch sequence.
 void *skl_workspace(size_t bytes);
+
+// A block of the current stream (on the current device) that is zero when a kernel starts and
+// that every kernel leaves zero again: sums and counters shared by the workgroups of a launch.
+// Allocated and cleared at the first call; every caller asks for the same size.
+void *skl_zeroed_scratch(size_t bytes);
 
 // Records a HIP failure for skl_hip_last_error() and returns its code.
 int skl_check_hip(hipError_t e, const char *what);

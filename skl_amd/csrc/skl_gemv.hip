@@ -42,7 +42,6 @@
 // k, which v_dot4_i32_i8 consumes without any byte shuffling).
 #include <hip/hip_runtime.h>
 
-#include <mutex>
 #include <type_traits>
 
 #include "skl_device.hpp"
@@ -70,7 +69,7 @@ struct Mode {
   using Acc = typename std::conditional<(MODE == kBF16 || MODE == kF16 || kFp8), float, int>::type;
 };
 
-// Zero-initialised per-device scratch: one 64-bit slot per column (the floating-point modes use the
+// Zero-initialised scratch of the launching stream: one 64-bit slot per column (the floating-point modes use the
 // first 32 bits of the region as an fp32 array) + tickets.
 constexpr size_t kMaxCols = size_t(1) << 22;  // 4 Mi columns
 constexpr size_t kMaxTiles = kMaxCols / 32;
@@ -78,23 +77,13 @@ struct Reduction {
   void *acc = nullptr;          // kMaxCols 64-bit slots
   unsigned *tickets = nullptr;  // kMaxTiles counters
 };
-std::mutex g_mutex;
-Reduction g_reduction[16];
 
+// One block per stream and device: launches on different streams may run at the same time.
 bool reduction_scratch(Reduction *out) {
-  int dev = 0;
-  if (skl_check_hip(hipGetDevice(&dev), "hipGetDevice") != 0 || dev >= 16) return false;
-  std::lock_guard<std::mutex> lock(g_mutex);
-  Reduction &r = g_reduction[dev];
-  if (!r.acc) {
-    const size_t bytes = kMaxCols * 8 + kMaxTiles * sizeof(unsigned);
-    void *p = nullptr;
-    if (skl_check_hip(hipMalloc(&p, bytes), "gemv scratch") != 0) return false;
-    if (skl_check_hip(hipMemset(p, 0, bytes), "gemv scratch clear") != 0) return false;
-    r.acc = p;
-    r.tickets = (unsigned *)((char *)p + kMaxCols * 8);
-  }
-  *out = r;
+  void *p = skl_zeroed_scratch(kMaxCols * 8 + kMaxTiles * sizeof(unsigned));
+  if (!p) return false;
+  out->acc = p;
+  out->tickets = (unsigned *)((char *)p + kMaxCols * 8);
   return true;
 }
 

@@ -106,10 +106,10 @@ int skl_hip_launch_gemv_rows(const skl_gemm_canon *g);
 int skl_hip_gemv_kc_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
 
-/* A block of per-device scratch memory for operands copied into another layout ahead of a launch (grows on demand,
- * NULL when the device has no room; apart from the workspace of the split reductions). */
+/* A block of scratch memory of the current stream and device for operands copied into another layout ahead of a
+ * launch (grows on demand, NULL when the device has no room; apart from the workspace of the split reductions). */
 void *skl_hip_operand_scratch(size_t bytes);
-/* Brackets a sequence of launches that hands data from one kernel to the next through per-device scratch memory
+/* Brackets a sequence of launches that hands data from one kernel to the next through the stream's scratch memory
  * (operand copies, partial sums), so that sequences of different host threads do not interleave on a stream.
  * Recursive. */
 void skl_hip_sequence_begin(void);

@@ -22,10 +22,23 @@ struct Scratch {
   size_t bytes = 0;
 };
 
+// Scratch memory belongs to one stream of one device: kernels of different streams may run at the same time, and
+// each scratch block carries data from one kernel to the next (or between the workgroups of one kernel).
+struct StreamState {
+  hipStream_t stream = nullptr;
+  Scratch workspace;       // partial sums of the split reductions (never more than kWorkspaceBytes are asked for)
+  Scratch operands;        // copies of operands in another layout; apart from the workspace so that a launch which
+                           // uses the workspace keeps the copies it was given
+  void *zeroed = nullptr;  // block that is zero between launches (sums and counters shared by workgroups)
+  size_t zeroed_bytes = 0;
+};
+
+// Streams with scratch of their own per device; every further stream shares the last entry (calls on those
+// streams must then not overlap on the device).
+constexpr size_t kMaxStreamStates = 32;
+
 struct DeviceState {
-  Scratch workspace;  // partial sums of the split reductions (never more than kWorkspaceBytes are asked for)
-  Scratch operands;   // copies of operands in another layout; apart from the workspace so that a launch which
-                      // uses the workspace keeps the copies it was given
+  std::vector<StreamState> streams;
   std::vector<void *> retired;
 };
 
@@ -91,13 +104,47 @@ DeviceState *current_device_state() {
   return &g_devices[dev];
 }
 
+// Under g_mutex: the scratch of the calling thread's stream on this device.
+StreamState &current_stream_state(DeviceState &st) {
+  for (StreamState &s : st.streams)
+    if (s.stream == t_stream) return s;
+  if (st.streams.size() < kMaxStreamStates) {
+    st.streams.emplace_back();
+    st.streams.back().stream = t_stream;
+  }
+  return st.streams.back();
+}
+
 }  // namespace
 
 void *skl_workspace(size_t bytes) {
   DeviceState *st = current_device_state();
   if (!st) return nullptr;
   std::lock_guard<std::mutex> lock(g_mutex);
-  return grow(*st, st->workspace, bytes, kWorkspaceBytes, "skl_workspace", true);
+  return grow(*st, current_stream_state(*st).workspace, bytes, kWorkspaceBytes, "skl_workspace", true);
+}
+
+void *skl_zeroed_scratch(size_t bytes) {
+  DeviceState *st = current_device_state();
+  if (!st) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  StreamState &ss = current_stream_state(*st);
+  if (ss.zeroed) {
+    if (bytes <= ss.zeroed_bytes) return ss.zeroed;
+    skl_hip_record_error(SKL_HIP_ERR_BAD_ARGUMENT, "skl_zeroed_scratch: size differs from the first request");
+    return nullptr;
+  }
+  void *p = nullptr;
+  if (skl_check_hip(hipMalloc(&p, bytes), "zeroed scratch") != 0) return nullptr;
+  // Cleared on the stream that will use it, and finished before any other stream can be handed the block.
+  if (skl_check_hip(hipMemsetAsync(p, 0, bytes, t_stream), "zeroed scratch clear") != 0 ||
+      skl_check_hip(hipStreamSynchronize(t_stream), "zeroed scratch clear") != 0) {
+    (void)hipFree(p);
+    return nullptr;
+  }
+  ss.zeroed = p;
+  ss.zeroed_bytes = bytes;
+  return p;
 }
 
 extern "C" {
@@ -123,7 +170,7 @@ void *skl_hip_operand_scratch(size_t bytes) {
   if (!st) return nullptr;
   std::lock_guard<std::mutex> lock(g_mutex);
   // not recorded as an error: the caller falls back to a kernel that needs no copy
-  return grow(*st, st->operands, bytes, kOperandBytes, "skl_hip_operand_scratch", false);
+  return grow(*st, current_stream_state(*st).operands, bytes, kOperandBytes, "skl_hip_operand_scratch", false);
 }
 
 void skl_hip_sequence_begin(void) { g_sequence.lock(); }
@@ -138,11 +185,14 @@ void skl_hip_shutdown(void) {
   }
   for (int d = 0; d < kMaxDevices; ++d) {
     DeviceState &st = g_devices[d];
-    if (!st.workspace.ptr && !st.operands.ptr && st.retired.empty()) continue;
+    if (st.streams.empty() && st.retired.empty()) continue;
     if (hipSetDevice(d) == hipSuccess) {
       (void)hipDeviceSynchronize();
-      if (st.workspace.ptr) (void)hipFree(st.workspace.ptr);
-      if (st.operands.ptr) (void)hipFree(st.operands.ptr);
+      for (StreamState &s : st.streams) {
+        if (s.workspace.ptr) (void)hipFree(s.workspace.ptr);
+        if (s.operands.ptr) (void)hipFree(s.operands.ptr);
+        if (s.zeroed) (void)hipFree(s.zeroed);
+      }
       for (void *p : st.retired) (void)hipFree(p);
     }
     st = DeviceState{};

@@ -430,6 +430,76 @@ def test_host_threads_share_one_device(gpu):
     assert not failures, failures
 
 
+def test_host_threads_on_streams_of_their_own(gpu):
+    """Scratch memory (sums shared by the workgroups of a GEMV, partial sums of a shared K, operand copies) belongs
+    to the launching stream, so host threads with a stream each may have their kernels run at the same time. Every
+    thread enqueues its whole list of problems back to back, so that launches of different streams overlap on the
+    device, and compares bit for bit (int8)."""
+    import ctypes as ct
+    import threading
+    from skl_amd import DeviceBuffer
+    from support import GemmCase
+
+    hip = ct.CDLL("libamdhip64.so.7")
+    hip.hipStreamCreate.restype = hip.hipStreamDestroy.restype = ct.c_int
+
+    def rc(m, n, k, rsa, csa, rsb, csb):
+        return GemmCase("i8", None, 1, 0, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=rsa, csa1=csa,
+                        rsb0=0, csb0=0, rsb1=rsb, csb1=csb, rsc0=0, csc0=0, rsc1=n, csc1=1)
+
+    cases = [rc(1, 4096, 8192, 8192, 1, 4096, 1),       # GEMV: workgroups meet in the zeroed scratch
+             rc(4, 2048, 4096, 4096, 1, 2048, 1),       # a batch of four rows on the same scratch
+             rc(16, 2048, 4096, 4096, 1, 2048, 1),      # few tiles, long K: partial sums in the workspace
+             rc(300, 260, 777, 778, 1, 261, 1),         # odd leading dimensions: both operands copied
+             rc(1037, 2, 1040, 1040, 1, 2, 1)]          # matrix times two vectors, row-major B: B copied
+    jobs = []
+    for i, case in enumerate(cases):
+        a, b, c = case.make_inputs(9200 + i)
+        jobs.append((case, a, b, c, run_oracle_gemm(case, a, b, c)))
+    failures = []
+
+    def worker(t):
+        stream = ct.c_void_p()
+        bufs = []
+        try:
+            assert hip.hipStreamCreate(ct.byref(stream)) == 0
+            gpu.skl_hip_set_stream(stream.value)
+            gpu.skl_hip_set_pointer_mode(1)
+            for case, a, b, c, _ in jobs:
+                bufs.append((DeviceBuffer.from_array(a), DeviceBuffer.from_array(b), DeviceBuffer.from_array(c)))
+            for it in range(8):
+                for rep in range(3):
+                    for j in range(len(jobs)):
+                        idx = (j + t) % len(jobs)
+                        case = jobs[idx][0]
+                        da, db, dc = bufs[idx]
+                        gpu.skl_gemm_i8rc_i8rc_i32rc_gfx950(case.m1, case.n1, case.k1, 1, da, case.rsa1, case.csa1, db,
+                                                           case.rsb1, case.csb1, 0, dc, case.rsc1, case.csc1)
+                assert gpu.skl_hip_synchronize() == 0
+                skl_amd.check_error()
+                for idx, (case, a, b, c, want) in enumerate(jobs):
+                    if not np.array_equal(bufs[idx][2].download(c.dtype, c.size), want):
+                        failures.append((t, it, idx))
+        except Exception as e:  # noqa: BLE001 - reported by the assertion below
+            failures.append((t, repr(e)))
+        finally:
+            gpu.skl_hip_synchronize()
+            gpu.skl_hip_set_stream(None)
+            gpu.skl_hip_set_pointer_mode(0)
+            for trio in bufs:
+                for d in trio:
+                    d.free()
+            if stream:
+                hip.hipStreamDestroy(stream)
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not failures, failures
+
+
 @pytest.mark.parametrize("mode", MODES)
 def test_block4x8x4_entry_point(gpu, mode):
     """`skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4` (documented by the reference without an implementation): small
