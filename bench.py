@@ -135,7 +135,7 @@ def _wl_small_batch(m):
         def step(i):
             lib.skl_gemm_i8_i8_i32_gfx950(m, n, k, 1, x, k, w[i % nbuf], n, 0, y, n)
 
-        kernel = "gemv_rows_kernel" if m <= 8 else "gemm_mfma_kernel (K shared between workgroups) + gemm_split_reduce_kernel"
+        kernel = "gemv_rows_kernel" if m <= 3 else "gemv_mfma_scale_c_kernel + gemv_mfma_rows_kernel"
         return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
                     name=f"int8 GEMM {m}x4096x11008 (decode with a batch of {m}: still a stream over W)", kernel=kernel)
     return build
@@ -360,6 +360,7 @@ WORKLOADS = {
     "gemv_i8_kcontig": (wl_gemv_kc, 1000, 50),
     "gemv_bf16_kcontig": (wl_gemv_kc_bf16, 500, 50),
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 500, 50),
+    "gemm_i8_8x4096x11008": (_wl_small_batch(8), 300, 30),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 300, 30),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2),

@@ -178,12 +178,14 @@ static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g) {
 static int gemv_on_device(const skl_gemm_canon *g) {
   if (skl_hip_gemv_kc_supported(g)) return skl_hip_launch_gemv_kc(g), 1;
   if (g->m == 1 && skl_hip_gemv_supported(g, 0)) return skl_hip_launch_gemv(g, 0), 1;
+  if (skl_hip_gemv_mfma_rows_supported(g)) return skl_hip_launch_gemv_mfma_rows(g), 1;
   if (skl_hip_gemv_rows_supported(g)) return skl_hip_launch_gemv_rows(g), 1;
   return 0;
 }
 
 static int gemv_would_take(const skl_gemm_canon *g) {
-  return skl_hip_gemv_kc_supported(g) || (g->m == 1 && skl_hip_gemv_supported(g, 0)) || skl_hip_gemv_rows_supported(g);
+  return skl_hip_gemv_kc_supported(g) || (g->m == 1 && skl_hip_gemv_supported(g, 0)) ||
+         skl_hip_gemv_mfma_rows_supported(g) || skl_hip_gemv_rows_supported(g);
 }
 
 /* C^T = B^T A^T: a problem with a few columns (matrix times vector, the reference's "small-N" regime,

@@ -566,6 +566,122 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 
 
 // ---------------------------------------------------------------------------
+// 4 <= M <= 16 rows of int8 A against a row-major int8 B: still one pass over B at the speed it arrives, with
+// the multiply-adds on the matrix cores so that their number does not grow with the rows of A
+// (v_mfma_i32_16x16x64_i8: a 16 x 64 block of A times a 64 x 16 block of B). B never goes through LDS: a lane
+// loads 16 consecutive rows of 16 consecutive columns (128-bit non-temporal loads, 16 lanes side by side cover
+// 256 columns, the four lane groups of a wave take four ranges of 16 rows), transposes the 16 x 16 bytes in
+// registers (v_perm_b32) and then holds, for each of its 16 columns, the 16 consecutive k the instruction wants
+// from one lane. Instruction c of a block multiplies column c of every lane, i.e. the 16 columns 16 j + c of the
+// 256: which 16 columns share an instruction is free, and so is the order of k inside it as long as A's lanes
+// hold the same k in the same bytes - A's rows are contiguous in K, so one 128-bit load per block gives exactly
+// that. A wave takes kMfmaIters blocks of 64 rows with all loads in flight before the first use, the four waves
+// of a workgroup take consecutive k ranges of the same 256 columns and meet in LDS.
+// Workgroups that share columns meet in C itself: a first kernel scales C by beta (beta == 0: writes zeros, C is
+// not read), and every workgroup adds alpha times its partial sums with atomics that return nothing. int32
+// arithmetic wraps, so beta*c + alpha*s1 + alpha*s2 + ... equals beta*c + alpha*(s1 + s2 + ...) bit for bit.
+// (Partial sums in planes and a second kernel that adds them: 19 us for 16 x 4096 x 11008; 64-bit atomics that
+// carry an arrival count like the M = 1 kernel's: 19 us; this: 15 us, and 13 us for 5 rows.)
+// ---------------------------------------------------------------------------
+constexpr int kMfmaMinRows = 4, kMfmaMaxRows = 16, kMfmaWaves = 4, kMfmaIters = 2, kMfmaTileCols = 256;
+constexpr int kMfmaKPerGroup = kMfmaWaves * kMfmaIters * 64;
+constexpr int kMfmaPitch = kMfmaTileCols + 4;  // ints per row of the LDS block
+constexpr size_t kMfmaLds = (size_t)kMfmaWaves * 16 * kMfmaPitch * sizeof(int);
+
+struct GemvMfmaArgs {
+  const char *a;   // rows of A: K contiguous bytes, a_row bytes apart, 16-byte aligned
+  size_t a_row;
+  const char *b;   // B(k, j) at (j / 64) * b_s1 + j % 64 + k * b_sk
+  size_t b_sk, b_s1;
+  int *c;          // element (i, j) at i * c_row + j * c_s
+  size_t c_row, c_s;
+  size_t m, n, k;
+  skl_scalar alpha, beta;
+  unsigned tiles, slabs;
+};
+
+__global__ void __launch_bounds__(256) gemv_mfma_scale_c_kernel(GemvMfmaArgs p) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.m * p.n) return;
+  int *c = p.c + (idx / p.n) * p.c_row + (idx % p.n) * p.c_s;
+  *c = p.beta.i == 0 ? 0 : (int)((unsigned)p.beta.i * (unsigned)*c);
+}
+
+__global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfmaArgs p) {
+  extern __shared__ __attribute__((aligned(16))) int mfma_red_raw[];
+  int(*red)[16][kMfmaPitch] = reinterpret_cast<int(*)[16][kMfmaPitch]>(mfma_red_raw);
+  typedef int v4i __attribute__((ext_vector_type(4)));
+  const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int jl = lane & 15, g = lane >> 4;
+  const size_t col = (size_t)tile * kMfmaTileCols + (size_t)jl * 16;  // the lane's 16 columns: inside one block of 64
+  const size_t kwave = ((size_t)slab * kMfmaWaves + wave) * (64 * kMfmaIters);
+  const bool col_ok = col < p.n;  // n is a multiple of 16
+  const char *bp = p.b + (col >> 6) * p.b_s1 + (col & 63);
+
+  uint4 rows[kMfmaIters][16];
+  v4i xa[kMfmaIters];
+#pragma unroll
+  for (int it = 0; it < kMfmaIters; ++it) {
+    const size_t k0 = kwave + (size_t)it * 64 + (size_t)g * 16;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if (col_ok && k0 + r < p.k)
+        rows[it][r] = stream_load(bp + (k0 + r) * p.b_sk);
+      else
+        rows[it][r] = make_uint4(0, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < kMfmaIters; ++it) {
+    const size_t k0 = kwave + (size_t)it * 64 + (size_t)g * 16;  // k is a multiple of 16: a chunk is inside or outside
+    if ((size_t)jl < p.m && k0 < p.k)
+      xa[it] = *reinterpret_cast<const v4i *>(p.a + (size_t)jl * p.a_row + k0);
+    else
+      xa[it] = v4i{0, 0, 0, 0};
+  }
+  v4i acc[16];
+#pragma unroll
+  for (int c = 0; c < 16; ++c) acc[c] = v4i{0, 0, 0, 0};
+#pragma unroll
+  for (int it = 0; it < kMfmaIters; ++it) {
+    unsigned t[4][16];  // [group of four rows][column]: four k of one column per dword
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint4 r0 = rows[it][4 * q], r1 = rows[it][4 * q + 1], r2 = rows[it][4 * q + 2], r3 = rows[it][4 * q + 3];
+      const unsigned a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
+      const unsigned a2[4] = {r2.x, r2.y, r2.z, r2.w}, a3[4] = {r3.x, r3.y, r3.z, r3.w};
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        transpose4x4(a0[d], a1[d], a2[d], a3[d], t[q][4 * d], t[q][4 * d + 1], t[q][4 * d + 2], t[q][4 * d + 3]);
+    }
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const v4i bw = {(int)t[0][c], (int)t[1][c], (int)t[2][c], (int)t[3][c]};
+      acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[it], bw, acc[c], 0, 0, 0);
+    }
+  }
+  // acc[c][r] is row 4 g + r of C, column 16 jl + c of the tile.
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4)
+      *reinterpret_cast<int4 *>(&red[wave][4 * g + r][16 * jl + 4 * c4]) =
+          make_int4(acc[4 * c4][r], acc[4 * c4 + 1][r], acc[4 * c4 + 2][r], acc[4 * c4 + 3][r]);
+  __syncthreads();
+  const size_t j = (size_t)tile * kMfmaTileCols + threadIdx.x;  // 256 threads, 256 columns
+  if (j >= p.n) return;
+  for (size_t i = 0; i < p.m; ++i) {
+    unsigned sum = 0;
+#pragma unroll
+    for (int w = 0; w < kMfmaWaves; ++w) sum += (unsigned)red[w][i][threadIdx.x];
+    (void)__hip_atomic_fetch_add(p.c + i * p.c_row + j * p.c_s, (int)((unsigned)p.alpha.i * sum), __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+
+// ---------------------------------------------------------------------------
 // B with K contiguous (column j is K consecutive elements, columns a fixed distance apart - how a linear
 // layer's weight [out][in] is stored): every output is a dot product over contiguous memory. A wave owns
 // two or four columns and walks K one KiB (64 lanes x 16 bytes) at a time, kKcUnroll KiB per column in
@@ -897,6 +1013,63 @@ extern "C" int skl_hip_launch_gemv_rows(const skl_gemm_canon *g) {
     case kF8E5M2: return launch_rows_of<kF8E5M2>(g, red);
     default: return launch_rows_of<kF8Mixed>(g, red);
   }
+}
+
+// 4 <= M <= 16, int8, row-major B (flat or in panels of 64 columns), rows of A contiguous in K and 16-byte aligned,
+// K a multiple of 16, C rows inside one block of 64 and its columns a fixed distance apart. Problems with less than
+// 1 MiB of B are left to the kernels that need one launch.
+extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g) {
+  if (mode_of(g, 0) != kI8RowMajor) return 0;
+  if (g->c_row_shift != 6 || g->c_col_shift != 6) return 0;
+  if (g->m < (size_t)kMfmaMinRows || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;
+  if ((g->k % 16) != 0 || (g->n % 16) != 0 || g->k * g->n < (size_t(1) << 20)) return 0;
+  if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % 16) != 0) return 0;
+  if (g->b_s0 != 1 || !aligned16(g->b) || (g->b_sk % 16) != 0 || (g->b_s1 % 16) != 0) return 0;
+  if (g->csc1 != 64 * g->csc0) return 0;
+  return 1;
+}
+
+extern "C" int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g) {
+  if (!skl_hip_gemv_mfma_rows_supported(g)) {
+    skl_hip_record_error(-2, "gemv_mfma_rows: unsupported problem");
+    return -2;
+  }
+  static bool configured = false;  // racing threads would set the same value
+  if (!configured) {
+    int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_mfma_rows_kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLds),
+                           "gemv_mfma_rows: LDS size");
+    if (rc != 0) return rc;
+    configured = true;
+  }
+  GemvMfmaArgs p;
+  p.a = (const char *)g->a;
+  p.a_row = g->a_s0;
+  p.b = (const char *)g->b;
+  p.b_sk = g->b_sk;
+  p.b_s1 = g->b_s1;
+  p.c = (int *)g->c;
+  p.c_row = g->rsc0;
+  p.c_s = g->csc0;
+  p.m = g->m;
+  p.n = g->n;
+  p.k = g->k;
+  p.alpha = g->alpha;
+  p.beta = g->beta;
+  p.tiles = skl_div_up(g->n, kMfmaTileCols);
+  p.slabs = skl_div_up(g->k, kMfmaKPerGroup);
+  const size_t grid = (size_t)p.tiles * p.slabs, cells = (g->m * g->n + 255) / 256;
+  if (grid > 0x7FFFFFFFu || cells > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemv_mfma_rows: grid too large");
+    return -2;
+  }
+  if (g->beta.i != 1) {  // beta == 1: C is the starting value as it is
+    gemv_mfma_scale_c_kernel<<<(unsigned)cells, 256, 0, skl_current_stream()>>>(p);
+    int rc = skl_check_launch("gemv_mfma_scale_c");
+    if (rc != 0) return rc;
+  }
+  gemv_mfma_rows_kernel<<<(unsigned)grid, kMfmaWaves * 64, kMfmaLds, skl_current_stream()>>>(p);
+  return skl_check_launch("gemv_mfma_rows");
 }
 
 // 1 <= M <= 4 against a B whose columns are contiguous in K (16-byte aligned columns and rows of A, K bytes a

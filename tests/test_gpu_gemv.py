@@ -125,6 +125,43 @@ def test_small_batch_rows_bit_exact(gpu, m):
                 assert np.array_equal(run_gemm(gpu, "rowmajor", case, a, b, c, mode), want), (m, n, k, mode)
 
 
+@pytest.mark.parametrize("m", (4, 5, 8, 9, 13, 16))
+def test_decode_batch_on_the_matrix_cores_bit_exact(gpu, m):
+    """4 to 16 rows of A against a row-major int8 B of at least 1 MiB (the stream over B whose multiply-adds run
+    on the matrix cores and whose workgroups add into C with atomics): the config-2 weights, K and N off the
+    kernel's 512 x 256 blocks, a K of a single block, padded row strides of A, B and C (whole-buffer compare:
+    the padding must survive), beta 0 / 1 / other with wrap-around, a C full of extreme values, both pointer modes."""
+    rng = np.random.default_rng(400 + m)
+    shapes = ((11008, 4096, 0, 0, 0), (4112, 528, 16, 32, 16), (16 * 4099, 16, 0, 0, 3), (2064, 1008, 48, 16, 48),
+              (256, 4096, 0, 0, 0))
+    for (n, k, pad_a, pad_b, pad_c) in shapes:
+        for alpha, beta in ((1, 0), (0x01010101, -77), (-3, 1)):
+            case = rowmajor_case("i8", m, n, k, alpha, beta, rsa=k + pad_a, rsb=n + pad_b, rsc=n + pad_c)
+            a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+            c[:] = rng.integers(-2 ** 31, 2 ** 31, size=c.size)
+            want = run_oracle_gemm(case, a, b, c)
+            for mode in ("device", "host"):
+                assert np.array_equal(run_gemm(gpu, "rowmajor", case, a, b, c, mode), want), (m, n, k, alpha, beta, mode)
+
+
+def test_decode_batch_on_the_matrix_cores_panels_and_strided_c(gpu):
+    """The same kernel with a column-major C through the full-stride entry point, and with B in panels of 64
+    columns (the 1 x TE panel format) through the blocked one."""
+    rng = np.random.default_rng(77)
+    m, n, k = 12, 2560, 1024
+    case = GemmCase("i8", None, 3, -5, m0=1, n0=1, k0=1, m1=m, n1=n, k1=k, rsa0=0, csa0=0, rsa1=k, csa1=1,
+                    rsb0=0, csb0=0, rsb1=n, csb1=1, rsc0=0, csc0=0, rsc1=1, csc1=m + 3)
+    a, b, c = case.make_inputs(6)
+    c[:] = rng.integers(-2 ** 31, 2 ** 31, size=c.size)
+    assert np.array_equal(run_gemm(gpu, "rc", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
+    # B in panels of 64 columns with 16 rows of A: blocked description, m0 = 16 rows in one block
+    n1 = 40
+    case = GemmCase("i8", None, 1, 0, m0=16, n0=64, k0=1, m1=1, n1=n1, k1=k, rsa0=k, csa0=0, rsa1=16 * k, csa1=1,
+                    rsb0=0, csb0=1, rsb1=64, csb1=k * 64, rsc0=64 * n1, csc0=1, rsc1=16 * 64 * n1, csc1=64)
+    a, b, c = case.make_inputs(7)
+    assert np.array_equal(run_gemm(gpu, "rcprc", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
+
+
 def test_small_batch_unaligned_rows_fall_back(gpu):
     """Rows of A that are not 4-byte aligned (odd row stride) are served by the tile kernels: same result."""
     case = rowmajor_case("i8", 4, 1024, 131, 3, 2, rsa=133)
