@@ -141,6 +141,21 @@ def _wl_small_batch(m):
     return build
 
 
+def wl_small_batch_f8(lib, rng):
+    """Decode with a batch of 16 against fp8 weights: the stream over W with the matrix cores multiplying."""
+    m, k, n, nbuf = 16, 4096, 11008, 8
+    w = [DeviceBuffer.from_array(rng.integers(8, 127, size=k * n, dtype=np.uint8)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(rng.integers(8, 127, size=m * k, dtype=np.uint8))
+    y = DeviceBuffer(4 * m * n)
+
+    def step(i):
+        lib.skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950(m, n, k, 1.0, x, k, 1, w[i % nbuf], n, 1, 0.0, y, n, 1)
+
+    return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="f8e4m3", keep=(w, x, y),
+                name="fp8 E4M3 GEMM 16x4096x11008 (decode with a batch of 16)",
+                kernel="gemv_mfma_rows_kernel<fp8 E4M3> + gemv_mfma_add_planes_kernel")
+
+
 def wl_gemv_p4x1c(lib, rng):
     """Config 2 with W prepacked in the K-packed dot4 layout (B(4P+p, j) at P*rsb1 + 4j + p): same bytes."""
     k, n, nbuf = 4096, 11008, 8
@@ -362,6 +377,7 @@ WORKLOADS = {
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 500, 50),
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 300, 30),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 300, 30),
+    "gemm_f8e4m3_16x4096x11008": (wl_small_batch_f8, 300, 30),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2),
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2),

@@ -582,6 +582,11 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 // arithmetic wraps, so beta*c + alpha*s1 + alpha*s2 + ... equals beta*c + alpha*(s1 + s2 + ...) bit for bit.
 // (Partial sums in planes and a second kernel that adds them: 19 us for 16 x 4096 x 11008; 64-bit atomics that
 // carry an arrival count like the M = 1 kernel's: 19 us; this: 15 us, and 13 us for 5 rows.)
+// OCP fp8 (E4M3, E5M2, E4M3 A with E5M2 B) runs on the same skeleton with v_mfma_f32_16x16x32_{fp8,bf8}_{fp8,bf8}
+// (8 bytes of K per lane: two instructions per column and block). Floating-point sums depend on their order and
+// the reference's epilogue rounds beta*c + alpha*acc in one place, so here each workgroup stores its raw sums to
+// its own plane of the stream's workspace and a second kernel adds the planes in order, applies alpha / beta and
+// the fused steps: deterministic, at the accuracy of the fp8 matrix-core instructions like the tile kernels.
 // ---------------------------------------------------------------------------
 constexpr int kMfmaMinRows = 4, kMfmaMaxRows = 16, kMfmaWaves = 4, kMfmaIters = 2, kMfmaTileCols = 256;
 constexpr int kMfmaKPerGroup = kMfmaWaves * kMfmaIters * 64;
@@ -598,6 +603,9 @@ struct GemvMfmaArgs {
   size_t m, n, k;
   skl_scalar alpha, beta;
   unsigned tiles, slabs;
+  float *planes;        // fp8: slabs planes of m x n raw sums
+  const float *bias;    // fp8: fused steps of the second pass, or null
+  float *max;
 };
 
 __global__ void __launch_bounds__(256) gemv_mfma_scale_c_kernel(GemvMfmaArgs p) {
@@ -607,9 +615,33 @@ __global__ void __launch_bounds__(256) gemv_mfma_scale_c_kernel(GemvMfmaArgs p) 
   *c = p.beta.i == 0 ? 0 : (int)((unsigned)p.beta.i * (unsigned)*c);
 }
 
+// C = beta*C + alpha * (sum of the planes, in order), then bias and maximum: the second pass of the fp8 kinds.
+__global__ void __launch_bounds__(256) gemv_mfma_add_planes_kernel(GemvMfmaArgs p) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.m * p.n) return;
+  const float *plane = p.planes + idx;
+  float sum = plane[0];
+  for (unsigned q = 1; q < p.slabs; ++q) sum = __fadd_rn(sum, plane[(size_t)q * p.m * p.n]);
+  const size_t col = idx % p.n;
+  float *c = reinterpret_cast<float *>(p.c) + (idx / p.n) * p.c_row + col * p.c_s;
+  skl_update(sum, c, p.alpha, p.beta);
+  if (p.bias || p.max) {
+    float v = *c;
+    if (p.bias) {
+      v = skl_add_bias(v, p.bias[col]);
+      *c = v;
+    }
+    if (p.max && v > skl_lowest<float>()) skl_atomic_max(p.max, v);
+  }
+}
+
+template <int MODE>
 __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfmaArgs p) {
+  constexpr bool kInt = MODE == kI8RowMajor;
+  using Acc = typename Mode<MODE>::Acc;  // int or float: 4 bytes either way
+  typedef Acc v4acc __attribute__((ext_vector_type(4)));
   extern __shared__ __attribute__((aligned(16))) int mfma_red_raw[];
-  int(*red)[16][kMfmaPitch] = reinterpret_cast<int(*)[16][kMfmaPitch]>(mfma_red_raw);
+  Acc(*red)[16][kMfmaPitch] = reinterpret_cast<Acc(*)[16][kMfmaPitch]>(mfma_red_raw);
   typedef int v4i __attribute__((ext_vector_type(4)));
   const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -640,9 +672,9 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
     else
       xa[it] = v4i{0, 0, 0, 0};
   }
-  v4i acc[16];
+  v4acc acc[16];
 #pragma unroll
-  for (int c = 0; c < 16; ++c) acc[c] = v4i{0, 0, 0, 0};
+  for (int c = 0; c < 16; ++c) acc[c] = v4acc{0, 0, 0, 0};
 #pragma unroll
   for (int it = 0; it < kMfmaIters; ++it) {
     unsigned t[4][16];  // [group of four rows][column]: four k of one column per dword
@@ -657,8 +689,26 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
     }
 #pragma unroll
     for (int c = 0; c < 16; ++c) {
-      const v4i bw = {(int)t[0][c], (int)t[1][c], (int)t[2][c], (int)t[3][c]};
-      acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[it], bw, acc[c], 0, 0, 0);
+      if constexpr (kInt) {
+        const v4i bw = {(int)t[0][c], (int)t[1][c], (int)t[2][c], (int)t[3][c]};
+        acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[it], bw, acc[c], 0, 0, 0);
+      } else {
+        // 8 bytes of K per lane and instruction: the lane's 16 k in two halves, A's bytes split the same way
+        const long a_lo = (long)(((unsigned long long)(unsigned)xa[it].y << 32) | (unsigned)xa[it].x);
+        const long a_hi = (long)(((unsigned long long)(unsigned)xa[it].w << 32) | (unsigned)xa[it].z);
+        const long b_lo = (long)(((unsigned long long)t[1][c] << 32) | t[0][c]);
+        const long b_hi = (long)(((unsigned long long)t[3][c] << 32) | t[2][c]);
+        if constexpr (MODE == kF8E4M3) {
+          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a_lo, b_lo, acc[c], 0, 0, 0);
+          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a_hi, b_hi, acc[c], 0, 0, 0);
+        } else if constexpr (MODE == kF8E5M2) {
+          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(a_lo, b_lo, acc[c], 0, 0, 0);
+          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(a_hi, b_hi, acc[c], 0, 0, 0);
+        } else {  // E4M3 A, E5M2 B
+          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(a_lo, b_lo, acc[c], 0, 0, 0);
+          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(a_hi, b_hi, acc[c], 0, 0, 0);
+        }
+      }
     }
   }
   // acc[c][r] is row 4 g + r of C, column 16 jl + c of the tile.
@@ -666,17 +716,27 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
   for (int r = 0; r < 4; ++r)
 #pragma unroll
     for (int c4 = 0; c4 < 4; ++c4)
-      *reinterpret_cast<int4 *>(&red[wave][4 * g + r][16 * jl + 4 * c4]) =
-          make_int4(acc[4 * c4][r], acc[4 * c4 + 1][r], acc[4 * c4 + 2][r], acc[4 * c4 + 3][r]);
+      *reinterpret_cast<v4acc *>(&red[wave][4 * g + r][16 * jl + 4 * c4]) =
+          v4acc{acc[4 * c4][r], acc[4 * c4 + 1][r], acc[4 * c4 + 2][r], acc[4 * c4 + 3][r]};
   __syncthreads();
   const size_t j = (size_t)tile * kMfmaTileCols + threadIdx.x;  // 256 threads, 256 columns
   if (j >= p.n) return;
-  for (size_t i = 0; i < p.m; ++i) {
-    unsigned sum = 0;
+  if constexpr (kInt) {
+    for (size_t i = 0; i < p.m; ++i) {
+      unsigned sum = 0;
 #pragma unroll
-    for (int w = 0; w < kMfmaWaves; ++w) sum += (unsigned)red[w][i][threadIdx.x];
-    (void)__hip_atomic_fetch_add(p.c + i * p.c_row + j * p.c_s, (int)((unsigned)p.alpha.i * sum), __ATOMIC_RELAXED,
-                                 __HIP_MEMORY_SCOPE_AGENT);
+      for (int w = 0; w < kMfmaWaves; ++w) sum += (unsigned)red[w][i][threadIdx.x];
+      (void)__hip_atomic_fetch_add(p.c + i * p.c_row + j * p.c_s, (int)((unsigned)p.alpha.i * sum), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+    }
+  } else {
+    float *plane = p.planes + (size_t)slab * p.m * p.n;
+    for (size_t i = 0; i < p.m; ++i) {
+      float sum = red[0][i][threadIdx.x];
+#pragma unroll
+      for (int w = 1; w < kMfmaWaves; ++w) sum = __fadd_rn(sum, red[w][i][threadIdx.x]);
+      plane[i * p.n + j] = sum;
+    }
   }
 }
 
@@ -1015,32 +1075,77 @@ extern "C" int skl_hip_launch_gemv_rows(const skl_gemm_canon *g) {
   }
 }
 
-// 4 <= M <= 16, int8, row-major B (flat or in panels of 64 columns), rows of A contiguous in K and 16-byte aligned,
-// K a multiple of 16, C rows inside one block of 64 and its columns a fixed distance apart. Problems with less than
-// 1 MiB of B are left to the kernels that need one launch.
+// 4 <= M <= 16, int8 or fp8, row-major B (flat or in panels of 64 columns), rows of A contiguous in K and 16-byte
+// aligned, K a multiple of 16, C rows inside one block of 64 and its columns a fixed distance apart. Problems with
+// less than 1 MiB of B are left to the kernels that need one launch.
 extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g) {
-  if (mode_of(g, 0) != kI8RowMajor) return 0;
+  const int mode = mode_of(g, 0);
+  if (mode != kI8RowMajor && mode != kF8E4M3 && mode != kF8E5M2 && mode != kF8Mixed) return 0;
   if (g->c_row_shift != 6 || g->c_col_shift != 6) return 0;
   if (g->m < (size_t)kMfmaMinRows || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;
   if ((g->k % 16) != 0 || (g->n % 16) != 0 || g->k * g->n < (size_t(1) << 20)) return 0;
   if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % 16) != 0) return 0;
   if (g->b_s0 != 1 || !aligned16(g->b) || (g->b_sk % 16) != 0 || (g->b_s1 % 16) != 0) return 0;
   if (g->csc1 != 64 * g->csc0) return 0;
+  if (mode == kI8RowMajor && (g->bias || g->max)) return 0;  // the fused steps ride on the second pass of the fp8 kinds
+  // fp8: one plane of raw sums per 512 k, inside the workspace's usual 64 MiB
+  const size_t slabs = (g->k + kMfmaKPerGroup - 1) / kMfmaKPerGroup;
+  if (mode != kI8RowMajor && slabs * g->m * g->n * sizeof(float) > (size_t(64) << 20)) return 0;
   return 1;
 }
+
+namespace {
+
+template <int MODE>
+int launch_mfma_rows(const GemvMfmaArgs &args) {
+  auto kernel = gemv_mfma_rows_kernel<MODE>;
+  static bool configured = false;  // per instantiation; racing threads would set the same value
+  if (!configured) {
+    int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLds),
+                           "gemv_mfma_rows: LDS size");
+    if (rc != 0) return rc;
+    configured = true;
+  }
+  GemvMfmaArgs p = args;
+  const size_t grid = (size_t)p.tiles * p.slabs, cells = (p.m * p.n + 255) / 256;
+  if (grid > 0x7FFFFFFFu || cells > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemv_mfma_rows: grid too large");
+    return -2;
+  }
+  if constexpr (MODE == kI8RowMajor) {
+    if (p.beta.i != 1) {  // beta == 1: C is the starting value as it is
+      gemv_mfma_scale_c_kernel<<<(unsigned)cells, 256, 0, skl_current_stream()>>>(p);
+      int rc = skl_check_launch("gemv_mfma_scale_c");
+      if (rc != 0) return rc;
+    }
+    kernel<<<(unsigned)grid, kMfmaWaves * 64, kMfmaLds, skl_current_stream()>>>(p);
+    return skl_check_launch("gemv_mfma_rows");
+  } else {
+    // The planes travel from the first kernel to the second through the stream's workspace: other host threads
+    // on this stream must not get in between.
+    skl_hip_sequence_begin();
+    int rc = -4;
+    p.planes = (float *)skl_workspace((size_t)p.slabs * p.m * p.n * sizeof(float));
+    if (p.planes) {
+      kernel<<<(unsigned)grid, kMfmaWaves * 64, kMfmaLds, skl_current_stream()>>>(p);
+      rc = skl_check_launch("gemv_mfma_rows");
+      if (rc == 0) {
+        gemv_mfma_add_planes_kernel<<<(unsigned)cells, 256, 0, skl_current_stream()>>>(p);
+        rc = skl_check_launch("gemv_mfma_add_planes");
+      }
+    }
+    skl_hip_sequence_end();
+    return rc;
+  }
+}
+
+}  // namespace
 
 extern "C" int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g) {
   if (!skl_hip_gemv_mfma_rows_supported(g)) {
     skl_hip_record_error(-2, "gemv_mfma_rows: unsupported problem");
     return -2;
-  }
-  static bool configured = false;  // racing threads would set the same value
-  if (!configured) {
-    int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_mfma_rows_kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLds),
-                           "gemv_mfma_rows: LDS size");
-    if (rc != 0) return rc;
-    configured = true;
   }
   GemvMfmaArgs p;
   p.a = (const char *)g->a;
@@ -1058,18 +1163,15 @@ extern "C" int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g) {
   p.beta = g->beta;
   p.tiles = skl_div_up(g->n, kMfmaTileCols);
   p.slabs = skl_div_up(g->k, kMfmaKPerGroup);
-  const size_t grid = (size_t)p.tiles * p.slabs, cells = (g->m * g->n + 255) / 256;
-  if (grid > 0x7FFFFFFFu || cells > 0x7FFFFFFFu) {
-    skl_hip_record_error(-2, "gemv_mfma_rows: grid too large");
-    return -2;
+  p.planes = nullptr;
+  p.bias = (const float *)g->bias;
+  p.max = (float *)g->max;
+  switch (mode_of(g, 0)) {
+    case kI8RowMajor: return launch_mfma_rows<kI8RowMajor>(p);
+    case kF8E4M3: return launch_mfma_rows<kF8E4M3>(p);
+    case kF8E5M2: return launch_mfma_rows<kF8E5M2>(p);
+    default: return launch_mfma_rows<kF8Mixed>(p);
   }
-  if (g->beta.i != 1) {  // beta == 1: C is the starting value as it is
-    gemv_mfma_scale_c_kernel<<<(unsigned)cells, 256, 0, skl_current_stream()>>>(p);
-    int rc = skl_check_launch("gemv_mfma_scale_c");
-    if (rc != 0) return rc;
-  }
-  gemv_mfma_rows_kernel<<<(unsigned)grid, kMfmaWaves * 64, kMfmaLds, skl_current_stream()>>>(p);
-  return skl_check_launch("gemv_mfma_rows");
 }
 
 // 1 <= M <= 4 against a B whose columns are contiguous in K (16-byte aligned columns and rows of A, K bytes a

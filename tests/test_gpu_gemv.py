@@ -162,6 +162,53 @@ def test_decode_batch_on_the_matrix_cores_panels_and_strided_c(gpu):
     assert np.array_equal(run_gemm(gpu, "rcprc", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
 
 
+@pytest.mark.parametrize("ta,tb", (("f8e4m3", "f8e4m3"), ("f8e5m2", "f8e5m2"), ("f8e4m3", "f8e5m2")))
+@pytest.mark.parametrize("m", (4, 7, 16))
+def test_decode_batch_on_the_matrix_cores_fp8(gpu, ta, tb, m):
+    """The fp8 kinds of the same kernel (raw sums in planes, a second pass adds them in order): the reference's
+    bound widened by the accuracy of the fp8 matrix-core instructions, shapes off the kernel's blocks, padded
+    strides, the same bits on a second run, and the fused steps (bias, maximum) applied to the same sums."""
+    from gpu_support import run_fused_gemm
+    from test_oracle_gemm import fused_expectation
+    for (n, k, pad) in ((11008, 4096, 0), (4112, 528, 16), (2064, 1008, 48)):
+        case = rowmajor_case(ta, m, n, k, 1.5, -0.5, tb=tb, rsa=k + pad, rsb=n + pad, rsc=n + pad)
+        a, b, c = case.make_inputs(m * 100 + n + k)
+        for mode in ("device", "host"):
+            got = run_gemm(gpu, "rc", case, a, b, c, mode)
+            support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=support.FP8_MFMA_REL)
+            assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
+        if ta != tb:
+            continue  # the mixed pair has no fused entry point
+        bias = (np.arange(n) % 7 - 3).astype(np.float32)
+        start = np.array([-np.inf], np.float32)
+        plain = run_gemm(gpu, "rc", case, a, b, c, "device")
+        got, top = run_fused_gemm(gpu, "rc", case, a, b, c, bias, start, "device")
+        want_c, want_top = fused_expectation(case, plain, bias, start)
+        assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8))
+        assert top[0] == want_top[0]
+
+
+def test_decode_batch_on_the_matrix_cores_decodes_fp8_exactly(gpu):
+    """A = rows of one-hot vectors (1.0 at position p of row i), alpha = 1, beta = 0: row i of C is row p_i of B
+    decoded to fp32 - every finite code of both formats must come out as the format defines it, in its column,
+    whichever lane group and half of the instruction its k falls into."""
+    m, n, k = 16, 4096, 256
+    for ta, tb in (("f8e4m3", "f8e4m3"), ("f8e5m2", "f8e5m2"), ("f8e4m3", "f8e5m2")):
+        one = 0x38 if ta == "f8e4m3" else 0x3C
+        table = support.decode_table(tb)
+        finite_codes = np.flatnonzero(np.isfinite(table)).astype(np.uint8)  # 0 * Inf would spoil whole columns
+        b = finite_codes[(np.arange(k * n) * 7 + np.arange(k * n) // n) % finite_codes.size].astype(np.uint8)
+        for base in (0, 5, 64 + 8, 128 + 48 - 15):
+            a = np.zeros(m * k, np.uint8)
+            for i in range(m):
+                a[i * k + base + i] = one
+            case = rowmajor_case(ta, m, n, k, 1.0, 0.0, tb=tb)
+            got = run_gemm(gpu, "rc", case, a, b, np.zeros(m * n, np.float32), "device").reshape(m, n)
+            for i in range(m):
+                p = base + i
+                assert np.array_equal(got[i].astype(np.float64), table[b[p * n:(p + 1) * n]]), (ta, tb, base, i)
+
+
 def test_small_batch_unaligned_rows_fall_back(gpu):
     """Rows of A that are not 4-byte aligned (odd row stride) are served by the tile kernels: same result."""
     case = rowmajor_case("i8", 4, 1024, 131, 3, 2, rsa=133)
