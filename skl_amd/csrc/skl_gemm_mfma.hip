@@ -1000,13 +1000,23 @@ __global__ void __launch_bounds__(256) gemm_split_reduce_kernel(MfmaArgs p) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= p.m * p.n) return;
   const size_t row = idx / p.n, col = idx % p.n;
+  // Eight planes are requested before the first is used (one memory round trip per eight, not per plane); the
+  // sum still runs over the planes in order, starting from plane 0 itself.
   const T *plane = reinterpret_cast<const T *>(p.partial) + idx;
+  const size_t mn = p.m * p.n;
   T sum = plane[0];
-  for (unsigned q = 1; q < p.splits; ++q) {
-    if constexpr (std::is_same<T, int>::value)
-      sum = (int)((unsigned)sum + (unsigned)plane[(size_t)q * p.m * p.n]);
-    else
-      sum = __fadd_rn(sum, plane[(size_t)q * p.m * p.n]);
+  for (unsigned q0 = 1; q0 < p.splits; q0 += 8) {
+    T v[8];
+#pragma unroll
+    for (unsigned u = 0; u < 8; ++u) v[u] = q0 + u < p.splits ? plane[(size_t)(q0 + u) * mn] : T(0);
+#pragma unroll
+    for (unsigned u = 0; u < 8; ++u) {
+      if (q0 + u >= p.splits) continue;
+      if constexpr (std::is_same<T, int>::value)
+        sum = (int)((unsigned)sum + (unsigned)v[u]);
+      else
+        sum = __fadd_rn(sum, v[u]);
+    }
   }
   T *c = reinterpret_cast<T *>(p.c) + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 +
          (col >> p.ccs) * p.csc1 + (col & ((size_t(1) << p.ccs) - 1)) * p.csc0;

@@ -619,9 +619,19 @@ __global__ void __launch_bounds__(256) gemv_mfma_scale_c_kernel(GemvMfmaArgs p) 
 __global__ void __launch_bounds__(256) gemv_mfma_add_planes_kernel(GemvMfmaArgs p) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= p.m * p.n) return;
+  // Eight planes are requested before the first is used (one memory round trip per eight, not per plane); the
+  // sum still runs over the planes in order, starting from plane 0 itself.
   const float *plane = p.planes + idx;
+  const size_t mn = p.m * p.n;
   float sum = plane[0];
-  for (unsigned q = 1; q < p.slabs; ++q) sum = __fadd_rn(sum, plane[(size_t)q * p.m * p.n]);
+  for (unsigned q0 = 1; q0 < p.slabs; q0 += 8) {
+    float v[8];
+#pragma unroll
+    for (unsigned u = 0; u < 8; ++u) v[u] = q0 + u < p.slabs ? plane[(size_t)(q0 + u) * mn] : 0.0f;
+#pragma unroll
+    for (unsigned u = 0; u < 8; ++u)
+      if (q0 + u < p.slabs) sum = __fadd_rn(sum, v[u]);
+  }
   const size_t col = idx % p.n;
   float *c = reinterpret_cast<float *>(p.c) + (idx / p.n) * p.c_row + col * p.c_s;
   skl_update(sum, c, p.alpha, p.beta);
