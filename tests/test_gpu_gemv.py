@@ -106,6 +106,36 @@ def test_k_packed_int8_decode(gpu, n, k1):
         assert np.array_equal(run_gemm(gpu, "dot4", case, a, b, c, mode), run_oracle_gemm(case, a, b, c))
 
 
+def _exact_int8_gemv(x, w, k, n):
+    """x (k) times row-major w (k x n) in exact integer arithmetic, through fp64 BLAS in slices of K."""
+    acc = np.zeros(n, np.float64)
+    for k0 in range(0, k, 2048):
+        k1 = min(k, k0 + 2048)
+        acc += x[k0:k1].astype(np.float64) @ w[k0 * n:k1 * n].reshape(k1 - k0, n).astype(np.float64)
+    return acc.astype(np.int64).astype(np.int32)
+
+
+def test_long_streams_take_sixteen_loads_per_lane(gpu):
+    """A stream of more than two rounds of workgroups (here 138 MB of int8 / fp8 weights, 143 MB of bf16, 134 MB in
+    the K-packed layout) runs with sixteen loads per lane and groups of 1024 rows: ragged K against those groups,
+    int8 bit for bit, floating point inside the reference's bound."""
+    rng = np.random.default_rng(88)
+    n, k = 8192, 16900
+    x, w = rng.integers(-128, 128, k, dtype=np.int8), rng.integers(-128, 128, k * n, dtype=np.int8)
+    case = rowmajor_case("i8", 1, n, k, -3, 5)
+    c = rng.integers(-2 ** 31, 2 ** 31, size=n).astype(np.int32)
+    want = (5 * c.astype(np.int64) - 3 * _exact_int8_gemv(x, w, k, n).astype(np.int64)).astype(np.int32)
+    assert np.array_equal(run_gemm(gpu, "rowmajor", case, x, w, c, "device"), want)
+    k1 = 4100  # K-packed: B(4P + p, j) at P * 4n + 4j + p
+    case = support.dot4_case(1, n, k1, alpha=1, beta=0)
+    a, b, c = case.make_inputs(3)
+    assert np.array_equal(run_gemm(gpu, "dot4", case, a, b, c, "device"), run_oracle_gemm(case, a, b, c))
+    for ta, kk in (("bf16", 8712), ("f8e4m3", 16900)):
+        case = rowmajor_case(ta, 1, n, kk, 1.5, -0.5)
+        a, b, c = case.make_inputs(kk)
+        support.assert_fp_gemm_close(case, a, b, c, run_gemm(gpu, "rc", case, a, b, c, "device"))
+
+
 @pytest.mark.parametrize("m", (2, 3, 4, 5, 6, 7, 8))
 def test_small_batch_rows_bit_exact(gpu, m):
     """2 to 8 rows of A against a row-major int8 B (the streaming kernel that shares the byte transposes
