@@ -141,6 +141,21 @@ def _wl_small_batch(m):
     return build
 
 
+def wl_small_batch_bf16(lib, rng):
+    """Decode with a batch of 8 against bf16 weights (90 MB): the stream over W with the matrix cores multiplying."""
+    m, k, n, nbuf = 8, 4096, 11008, 4
+    w = [DeviceBuffer.from_array(bf16_bits(rng.normal(size=k * n) * 0.02)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(bf16_bits(rng.normal(size=m * k)))
+    y = DeviceBuffer(4 * m * n)
+
+    def step(i):
+        lib.skl_gemm_bf16_bf16_f32_gfx950(m, n, k, 1.0, x, k, w[i % nbuf], n, 0.0, y, n)
+
+    return dict(fn=step, bytes=2 * k * n + 2 * m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="bf16",
+                keep=(w, x, y), name="bf16 GEMM 8x4096x11008 (decode with a batch of 8)",
+                kernel="gemv_mfma_rows_kernel<bf16> + gemv_mfma_add_planes_kernel")
+
+
 def wl_small_batch_f8(lib, rng):
     """Decode with a batch of 16 against fp8 weights: the stream over W with the matrix cores multiplying."""
     m, k, n, nbuf = 16, 4096, 11008, 8
@@ -378,6 +393,7 @@ WORKLOADS = {
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 300, 30),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 300, 30),
     "gemm_f8e4m3_16x4096x11008": (wl_small_batch_f8, 300, 30),
+    "gemm_bf16_8x4096x11008": (wl_small_batch_bf16, 300, 30),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2),
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2),

@@ -568,7 +568,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 
 
 // ---------------------------------------------------------------------------
-// 4 <= M <= 16 rows of int8 A against a row-major int8 B: still one pass over B at the speed it arrives, with
+// 4 <= M <= 16 rows of int8 A (other kinds, below: from two rows) against a row-major B: still one pass over B at the speed it arrives, with
 // the multiply-adds on the matrix cores so that their number does not grow with the rows of A
 // (v_mfma_i32_16x16x64_i8: a 16 x 64 block of A times a 64 x 16 block of B). B never goes through LDS: a lane
 // loads 16 consecutive rows of 16 consecutive columns (128-bit non-temporal loads, 16 lanes side by side cover
@@ -577,7 +577,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 // from one lane. Instruction c of a block multiplies column c of every lane, i.e. the 16 columns 16 j + c of the
 // 256: which 16 columns share an instruction is free, and so is the order of k inside it as long as A's lanes
 // hold the same k in the same bytes - A's rows are contiguous in K, so one 128-bit load per block gives exactly
-// that. A wave takes kMfmaIters blocks of 64 rows with all loads in flight before the first use, the four waves
+// that. A wave takes two blocks of 64 rows with all 32 loads in flight before the first use, the four waves
 // of a workgroup take consecutive k ranges of the same 256 columns and meet in LDS.
 // Workgroups that share columns meet in C itself: a first kernel scales C by beta (beta == 0: writes zeros, C is
 // not read), and every workgroup adds alpha times its partial sums with atomics that return nothing. int32
@@ -590,15 +590,26 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 // its own plane of the stream's workspace and a second kernel adds the planes in order, applies alpha / beta and
 // the fused steps: deterministic, at the accuracy of the fp8 matrix-core instructions like the tile kernels.
 // ---------------------------------------------------------------------------
-constexpr int kMfmaMinRows = 4, kMfmaMaxRows = 16, kMfmaWaves = 4, kMfmaIters = 2, kMfmaTileCols = 256;
-constexpr int kMfmaKPerGroup = kMfmaWaves * kMfmaIters * 64;
-constexpr int kMfmaPitch = kMfmaTileCols + 4;  // ints per row of the LDS block
-constexpr size_t kMfmaLds = (size_t)kMfmaWaves * 16 * kMfmaPitch * sizeof(int);
+// bf16 / f16: a 128-bit load holds 8 columns and v_mfma_f32_16x16x32_{bf16,f16} wants 8 consecutive k per lane, so a
+// lane loads 8 rows of 8 columns and transposes 8 x 8 halfwords (one v_perm_b32 per dword of the result); 16 lanes
+// cover 128 columns, the four lane groups 32 rows, a wave takes four such blocks. Raw sums in planes like fp8.
+constexpr int kMfmaMinRowsInt8 = 4, kMfmaMaxRows = 16, kMfmaWaves = 4;
+template <int ES>
+struct MfmaShape {
+  static constexpr int kLaneCols = 16 / ES;           // columns in a 128-bit load = instructions per block
+  static constexpr int kLaneRows = 16 / ES;           // rows a lane loads per block = k per lane and instruction(s)
+  static constexpr int kBlockK = 4 * kLaneRows;       // 64 or 32
+  static constexpr int kIters = 32 / kLaneRows;       // blocks per wave: 32 loads in flight per lane
+  static constexpr int kTileCols = 16 * kLaneCols;    // 256 or 128
+  static constexpr int kKPerGroup = kMfmaWaves * kIters * kBlockK;  // 512
+  static constexpr int kPitch = kTileCols + 4;        // 4-byte words per row of the LDS block
+  static constexpr size_t kLds = (size_t)kMfmaWaves * 16 * kPitch * 4;
+};
 
 struct GemvMfmaArgs {
-  const char *a;   // rows of A: K contiguous bytes, a_row bytes apart, 16-byte aligned
+  const char *a;   // rows of A: K contiguous elements, a_row bytes apart, 16-byte aligned
   size_t a_row;
-  const char *b;   // B(k, j) at (j / 64) * b_s1 + j % 64 + k * b_sk
+  const char *b;   // B(k, j) at (j / 64) * b_s1 + (j % 64) * elemsize + k * b_sk (bytes)
   size_t b_sk, b_s1;
   int *c;          // element (i, j) at i * c_row + j * c_s
   size_t c_row, c_s;
@@ -649,27 +660,30 @@ __global__ void __launch_bounds__(256) gemv_mfma_add_planes_kernel(GemvMfmaArgs 
 
 template <int MODE>
 __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfmaArgs p) {
-  constexpr bool kInt = MODE == kI8RowMajor;
+  constexpr bool kInt = MODE == kI8RowMajor, k16 = MODE == kBF16 || MODE == kF16;
+  constexpr int ES = k16 ? 2 : 1;
+  using Sh = MfmaShape<ES>;
+  constexpr int LC = Sh::kLaneCols, LR = Sh::kLaneRows, ITERS = Sh::kIters;
   using Acc = typename Mode<MODE>::Acc;  // int or float: 4 bytes either way
   typedef Acc v4acc __attribute__((ext_vector_type(4)));
-  extern __shared__ __attribute__((aligned(16))) int mfma_red_raw[];
-  Acc(*red)[16][kMfmaPitch] = reinterpret_cast<Acc(*)[16][kMfmaPitch]>(mfma_red_raw);
   typedef int v4i __attribute__((ext_vector_type(4)));
+  extern __shared__ __attribute__((aligned(16))) int mfma_red_raw[];
+  Acc(*red)[16][Sh::kPitch] = reinterpret_cast<Acc(*)[16][Sh::kPitch]>(mfma_red_raw);
   const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int jl = lane & 15, g = lane >> 4;
-  const size_t col = (size_t)tile * kMfmaTileCols + (size_t)jl * 16;  // the lane's 16 columns: inside one block of 64
-  const size_t kwave = ((size_t)slab * kMfmaWaves + wave) * (64 * kMfmaIters);
-  const bool col_ok = col < p.n;  // n is a multiple of 16
-  const char *bp = p.b + (col >> 6) * p.b_s1 + (col & 63);
+  const size_t col = (size_t)tile * Sh::kTileCols + (size_t)jl * LC;  // the lane's columns: inside one block of 64
+  const size_t kwave = ((size_t)slab * kMfmaWaves + wave) * (Sh::kBlockK * ITERS);
+  const bool col_ok = col < p.n;  // n is a multiple of the columns per lane
+  const char *bp = p.b + (col >> 6) * p.b_s1 + (col & 63) * ES;
 
-  uint4 rows[kMfmaIters][16];
-  v4i xa[kMfmaIters];
+  uint4 rows[ITERS][LR];
+  v4i xa[ITERS];
 #pragma unroll
-  for (int it = 0; it < kMfmaIters; ++it) {
-    const size_t k0 = kwave + (size_t)it * 64 + (size_t)g * 16;
+  for (int it = 0; it < ITERS; ++it) {
+    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * LR;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
+    for (int r = 0; r < LR; ++r) {
       if (col_ok && k0 + r < p.k)
         rows[it][r] = stream_load(bp + (k0 + r) * p.b_sk);
       else
@@ -677,33 +691,55 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
     }
   }
 #pragma unroll
-  for (int it = 0; it < kMfmaIters; ++it) {
-    const size_t k0 = kwave + (size_t)it * 64 + (size_t)g * 16;  // k is a multiple of 16: a chunk is inside or outside
+  for (int it = 0; it < ITERS; ++it) {
+    // k is a multiple of the rows per lane: a 16-byte piece of a row of A is inside or outside
+    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * LR;
     if ((size_t)jl < p.m && k0 < p.k)
-      xa[it] = *reinterpret_cast<const v4i *>(p.a + (size_t)jl * p.a_row + k0);
+      xa[it] = *reinterpret_cast<const v4i *>(p.a + (size_t)jl * p.a_row + k0 * ES);
     else
       xa[it] = v4i{0, 0, 0, 0};
   }
-  v4acc acc[16];
+  v4acc acc[LC];
 #pragma unroll
-  for (int c = 0; c < 16; ++c) acc[c] = v4acc{0, 0, 0, 0};
+  for (int c = 0; c < LC; ++c) acc[c] = v4acc{0, 0, 0, 0};
 #pragma unroll
-  for (int it = 0; it < kMfmaIters; ++it) {
-    unsigned t[4][16];  // [group of four rows][column]: four k of one column per dword
+  for (int it = 0; it < ITERS; ++it) {
+    unsigned t[4][LC];  // [dword of the operand][column]: the lane's k of one column, ascending
+    if constexpr (k16) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint4 r0 = rows[it][4 * q], r1 = rows[it][4 * q + 1], r2 = rows[it][4 * q + 2], r3 = rows[it][4 * q + 3];
-      const unsigned a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
-      const unsigned a2[4] = {r2.x, r2.y, r2.z, r2.w}, a3[4] = {r3.x, r3.y, r3.z, r3.w};
+      for (int q = 0; q < 4; ++q) {  // rows 2q and 2q + 1 of the block
+        const uint4 lo = rows[it][2 * q], hi = rows[it][2 * q + 1];
+        const unsigned l4[4] = {lo.x, lo.y, lo.z, lo.w}, h4[4] = {hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
-      for (int d = 0; d < 4; ++d)
-        transpose4x4(a0[d], a1[d], a2[d], a3[d], t[q][4 * d], t[q][4 * d + 1], t[q][4 * d + 2], t[q][4 * d + 3]);
+        for (int d = 0; d < 4; ++d) {  // dword d holds columns 2d and 2d + 1
+          t[q][2 * d] = __builtin_amdgcn_perm(h4[d], l4[d], 0x05040100u);      // low halves: row 2q, row 2q + 1
+          t[q][2 * d + 1] = __builtin_amdgcn_perm(h4[d], l4[d], 0x07060302u);  // high halves
+        }
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint4 r0 = rows[it][4 * q], r1 = rows[it][4 * q + 1], r2 = rows[it][4 * q + 2], r3 = rows[it][4 * q + 3];
+        const unsigned a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
+        const unsigned a2[4] = {r2.x, r2.y, r2.z, r2.w}, a3[4] = {r3.x, r3.y, r3.z, r3.w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          transpose4x4(a0[d], a1[d], a2[d], a3[d], t[q][4 * d], t[q][4 * d + 1], t[q][4 * d + 2], t[q][4 * d + 3]);
+      }
     }
 #pragma unroll
-    for (int c = 0; c < 16; ++c) {
+    for (int c = 0; c < LC; ++c) {
+      const v4i bw = {(int)t[0][c], (int)t[1][c], (int)t[2][c], (int)t[3][c]};
       if constexpr (kInt) {
-        const v4i bw = {(int)t[0][c], (int)t[1][c], (int)t[2][c], (int)t[3][c]};
         acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[it], bw, acc[c], 0, 0, 0);
+      } else if constexpr (MODE == kBF16) {
+        typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+        acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, xa[it]), __builtin_bit_cast(v8bf, bw),
+                                                         acc[c], 0, 0, 0);
+      } else if constexpr (MODE == kF16) {
+        typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+        acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, xa[it]), __builtin_bit_cast(v8h, bw),
+                                                        acc[c], 0, 0, 0);
       } else {
         // 8 bytes of K per lane and instruction: the lane's 16 k in two halves, A's bytes split the same way
         const long a_lo = (long)(((unsigned long long)(unsigned)xa[it].y << 32) | (unsigned)xa[it].x);
@@ -723,30 +759,33 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
       }
     }
   }
-  // acc[c][r] is row 4 g + r of C, column 16 jl + c of the tile.
+  // acc[c][r] is row 4 g + r of C, column LC jl + c of the tile.
 #pragma unroll
   for (int r = 0; r < 4; ++r)
 #pragma unroll
-    for (int c4 = 0; c4 < 4; ++c4)
-      *reinterpret_cast<v4acc *>(&red[wave][4 * g + r][16 * jl + 4 * c4]) =
+    for (int c4 = 0; c4 < LC / 4; ++c4)
+      *reinterpret_cast<v4acc *>(&red[wave][4 * g + r][LC * jl + 4 * c4]) =
           v4acc{acc[4 * c4][r], acc[4 * c4 + 1][r], acc[4 * c4 + 2][r], acc[4 * c4 + 3][r]};
   __syncthreads();
-  const size_t j = (size_t)tile * kMfmaTileCols + threadIdx.x;  // 256 threads, 256 columns
+  // 256 threads: one column each (two rows of C at a time for the 128-column tiles)
+  constexpr int kRowStep = kMfmaWaves * 64 / Sh::kTileCols;
+  const int tc = threadIdx.x % Sh::kTileCols;
+  const size_t j = (size_t)tile * Sh::kTileCols + tc;
   if (j >= p.n) return;
   if constexpr (kInt) {
-    for (size_t i = 0; i < p.m; ++i) {
+    for (size_t i = threadIdx.x / Sh::kTileCols; i < p.m; i += kRowStep) {
       unsigned sum = 0;
 #pragma unroll
-      for (int w = 0; w < kMfmaWaves; ++w) sum += (unsigned)red[w][i][threadIdx.x];
+      for (int w = 0; w < kMfmaWaves; ++w) sum += (unsigned)red[w][i][tc];
       (void)__hip_atomic_fetch_add(p.c + i * p.c_row + j * p.c_s, (int)((unsigned)p.alpha.i * sum), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
     }
   } else {
     float *plane = p.planes + (size_t)slab * p.m * p.n;
-    for (size_t i = 0; i < p.m; ++i) {
-      float sum = red[0][i][threadIdx.x];
+    for (size_t i = threadIdx.x / Sh::kTileCols; i < p.m; i += kRowStep) {
+      float sum = red[0][i][tc];
 #pragma unroll
-      for (int w = 1; w < kMfmaWaves; ++w) sum = __fadd_rn(sum, red[w][i][threadIdx.x]);
+      for (int w = 1; w < kMfmaWaves; ++w) sum = __fadd_rn(sum, red[w][i][tc]);
       plane[i * p.n + j] = sum;
     }
   }
@@ -1095,21 +1134,29 @@ extern "C" int skl_hip_launch_gemv_rows(const skl_gemm_canon *g) {
   }
 }
 
-// 4 <= M <= 16, int8 or fp8, row-major B (flat or in panels of 64 columns), rows of A contiguous in K and 16-byte
-// aligned, K a multiple of 16, C rows inside one block of 64 and its columns a fixed distance apart. Problems with
+// 4 <= M <= 16 (int8) or 2 <= M <= 16 (fp8, bf16, f16), row-major B (flat or in panels of 64 columns), rows of A contiguous in K and
+// 16-byte aligned, K and N multiples of 16 bytes of elements, C rows inside one block of 64 and its columns a fixed
+// distance apart. Problems with
 // less than 1 MiB of B are left to the kernels that need one launch.
 extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g) {
   const int mode = mode_of(g, 0);
-  if (mode != kI8RowMajor && mode != kF8E4M3 && mode != kF8E5M2 && mode != kF8Mixed) return 0;
+  if (mode < 0 || mode == kI8K4) return 0;
+  const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1, piece = 16 / es;  // elements in 16 bytes
   if (g->c_row_shift != 6 || g->c_col_shift != 6) return 0;
-  if (g->m < (size_t)kMfmaMinRows || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;
-  if ((g->k % 16) != 0 || (g->n % 16) != 0 || g->k * g->n < (size_t(1) << 20)) return 0;
-  if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % 16) != 0) return 0;
-  if (g->b_s0 != 1 || !aligned16(g->b) || (g->b_sk % 16) != 0 || (g->b_s1 % 16) != 0) return 0;
+  // Fewest rows from which this kernel is the faster one for 1 x 4096 x 11008 weights: int8 13.1 us whatever the
+  // rows against 11.2 / 12.9 / 14.6 us for 2 / 3 / 4 rows on the kernel that shares the byte transposes; fp8 13.7 us
+  // against 17.9 us for 2 rows; bf16 20.5 us against 27.1 us. (One row: int8 12.8 against 10.3 us, fp8 13.5 against
+  // 11.5 us, bf16 20.4 against 21.6 us - left to the M = 1 kernel, which uses no matrix cores.)
+  const size_t min_rows = mode == kI8RowMajor ? kMfmaMinRowsInt8 : 2;
+  if (g->m < min_rows || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;
+  if ((g->k % piece) != 0 || (g->n % piece) != 0 || g->k * g->n * es < (size_t(1) << 20)) return 0;
+  if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % piece) != 0) return 0;
+  if (g->b_s0 != 1 || !aligned16(g->b) || (g->b_sk % piece) != 0 || (g->b_s1 % piece) != 0) return 0;
   if (g->csc1 != 64 * g->csc0) return 0;
   if (mode == kI8RowMajor && (g->bias || g->max)) return 0;  // the fused steps ride on the second pass of the fp8 kinds
-  // fp8: one plane of raw sums per 512 k, inside the workspace's usual 64 MiB
-  const size_t slabs = (g->k + kMfmaKPerGroup - 1) / kMfmaKPerGroup;
+  // floating point: one plane of raw sums per 512 k, inside the workspace's usual 64 MiB
+  const size_t slabs = (g->k + MfmaShape<1>::kKPerGroup - 1) / MfmaShape<1>::kKPerGroup;
+  static_assert(MfmaShape<1>::kKPerGroup == MfmaShape<2>::kKPerGroup, "one group length for every kind");
   if (mode != kI8RowMajor && slabs * g->m * g->n * sizeof(float) > (size_t(64) << 20)) return 0;
   return 1;
 }
@@ -1118,6 +1165,8 @@ namespace {
 
 template <int MODE>
 int launch_mfma_rows(const GemvMfmaArgs &args) {
+  using Sh = MfmaShape<(MODE == kBF16 || MODE == kF16) ? 2 : 1>;
+  constexpr size_t kMfmaLds = Sh::kLds;
   auto kernel = gemv_mfma_rows_kernel<MODE>;
   static bool configured = false;  // per instantiation; racing threads would set the same value
   if (!configured) {
@@ -1128,6 +1177,8 @@ int launch_mfma_rows(const GemvMfmaArgs &args) {
     configured = true;
   }
   GemvMfmaArgs p = args;
+  p.tiles = skl_div_up(p.n, Sh::kTileCols);
+  p.slabs = skl_div_up(p.k, Sh::kKPerGroup);
   const size_t grid = (size_t)p.tiles * p.slabs, cells = (p.m * p.n + 255) / 256;
   if (grid > 0x7FFFFFFFu || cells > 0x7FFFFFFFu) {
     skl_hip_record_error(-2, "gemv_mfma_rows: grid too large");
@@ -1169,10 +1220,12 @@ extern "C" int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g) {
   }
   GemvMfmaArgs p;
   p.a = (const char *)g->a;
-  p.a_row = g->a_s0;
+  const int mode = mode_of(g, 0);
+  const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1;
+  p.a_row = g->a_s0 * es;
   p.b = (const char *)g->b;
-  p.b_sk = g->b_sk;
-  p.b_s1 = g->b_s1;
+  p.b_sk = g->b_sk * es;
+  p.b_s1 = g->b_s1 * es;
   p.c = (int *)g->c;
   p.c_row = g->rsc0;
   p.c_s = g->csc0;
@@ -1181,13 +1234,14 @@ extern "C" int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g) {
   p.k = g->k;
   p.alpha = g->alpha;
   p.beta = g->beta;
-  p.tiles = skl_div_up(g->n, kMfmaTileCols);
-  p.slabs = skl_div_up(g->k, kMfmaKPerGroup);
+  p.tiles = p.slabs = 0;  // set per kind
   p.planes = nullptr;
   p.bias = (const float *)g->bias;
   p.max = (float *)g->max;
-  switch (mode_of(g, 0)) {
+  switch (mode) {
     case kI8RowMajor: return launch_mfma_rows<kI8RowMajor>(p);
+    case kBF16: return launch_mfma_rows<kBF16>(p);
+    case kF16: return launch_mfma_rows<kF16>(p);
     case kF8E4M3: return launch_mfma_rows<kF8E4M3>(p);
     case kF8E5M2: return launch_mfma_rows<kF8E5M2>(p);
     default: return launch_mfma_rows<kF8Mixed>(p);

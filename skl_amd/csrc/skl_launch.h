@@ -102,8 +102,8 @@ int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout);
 /* 2 <= M <= 8 rows against a row-major int8 B: the same stream over B with the transposes shared by the rows. */
 int skl_hip_gemv_rows_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_rows(const skl_gemm_canon *g);
-/* 4 <= M <= 16 rows against a row-major int8 or fp8 B: the same stream with the multiply-adds on the matrix cores
- * (fp8: with the fused steps, if any). */
+/* 4 <= M <= 16 rows against a row-major int8 B, 2 <= M <= 16 against an fp8 / bf16 / f16 one: the same stream with
+ * the multiply-adds on the matrix cores (floating point: with the fused steps, if any). */
 int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g);
 /* 1 <= M <= 4 against a B with K contiguous (b_sk == 1): one dot product over contiguous memory per output. */

@@ -193,7 +193,7 @@ def test_decode_batch_on_the_matrix_cores_panels_and_strided_c(gpu):
 
 
 @pytest.mark.parametrize("ta,tb", (("f8e4m3", "f8e4m3"), ("f8e5m2", "f8e5m2"), ("f8e4m3", "f8e5m2")))
-@pytest.mark.parametrize("m", (4, 7, 16))
+@pytest.mark.parametrize("m", (2, 7, 16))
 def test_decode_batch_on_the_matrix_cores_fp8(gpu, ta, tb, m):
     """The fp8 kinds of the same kernel (raw sums in planes, a second pass adds them in order): the reference's
     bound widened by the accuracy of the fp8 matrix-core instructions, shapes off the kernel's blocks, padded
@@ -216,6 +216,49 @@ def test_decode_batch_on_the_matrix_cores_fp8(gpu, ta, tb, m):
         want_c, want_top = fused_expectation(case, plain, bias, start)
         assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8))
         assert top[0] == want_top[0]
+
+
+@pytest.mark.parametrize("ta", ("bf16", "f16"))
+@pytest.mark.parametrize("m", (2, 7, 16))
+def test_decode_batch_on_the_matrix_cores_16bit(gpu, ta, m):
+    """bf16 / f16 on the same kernel (8 x 8 halfword transposes, v_mfma_f32_16x16x32): products are exact in fp32
+    and the sums are fp32, so the reference's own bound holds; shapes off the kernel's 512 x 128 blocks, padded
+    strides, the same bits on a second run and with the fused steps."""
+    from gpu_support import run_fused_gemm
+    from test_oracle_gemm import fused_expectation
+    for (n, k, pad) in ((11008, 4096, 0), (4104, 520, 8), (2056, 1000, 24)):
+        case = rowmajor_case(ta, m, n, k, 1.5, -0.5, rsa=k + pad, rsb=n + pad, rsc=n + pad)
+        a, b, c = case.make_inputs(m * 100 + n + k)
+        for mode in ("device", "host"):
+            got = run_gemm(gpu, "rc", case, a, b, c, mode)
+            support.assert_fp_gemm_close(case, a, b, c, got)
+            assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
+        bias = (np.arange(n) % 7 - 3).astype(np.float32)
+        start = np.array([-np.inf], np.float32)
+        plain = run_gemm(gpu, "rc", case, a, b, c, "device")
+        got, top = run_fused_gemm(gpu, "rc", case, a, b, c, bias, start, "device")
+        want_c, want_top = fused_expectation(case, plain, bias, start)
+        assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8))
+        assert top[0] == want_top[0]
+
+
+def test_decode_batch_on_the_matrix_cores_16bit_one_hot(gpu):
+    """Rows of A with a single 1.0 each: row i of C is row p_i of B widened to fp32, exactly and in the right
+    columns, for positions in every lane group and every halfword of a lane's eight."""
+    m, n, k = 16, 4096, 256
+    rng = np.random.default_rng(5)
+    for ta in ("bf16", "f16"):
+        b = support.ETYPES[ta].gen(rng, k * n)
+        wide = support.ETYPES[ta].widen(b).reshape(k, n)
+        one = 0x3F80 if ta == "bf16" else 0x3C00
+        for base in (0, 3, 32 + 8, 128 + 48 - 15):
+            a = np.zeros(m * k, np.uint16)
+            for i in range(m):
+                a[i * k + base + i] = one
+            case = rowmajor_case(ta, m, n, k, 1.0, 0.0)
+            got = run_gemm(gpu, "rc", case, a, b, np.zeros(m * n, np.float32), "device").reshape(m, n)
+            for i in range(m):
+                assert np.array_equal(got[i].astype(np.float64), wide[base + i]), (ta, base, i)
 
 
 def test_decode_batch_on_the_matrix_cores_decodes_fp8_exactly(gpu):
@@ -284,17 +327,20 @@ def test_fp8_streaming_path_within_reference_bound(gpu, ta, tb, n, k):
 @pytest.mark.parametrize("ta,tb", (("bf16", "bf16"), ("f16", "f16")) + FP8_PAIRS)
 @pytest.mark.parametrize("m", (2, 3))
 def test_small_batch_rows_floating_point(gpu, ta, tb, m):
-    """2 or 3 rows of A on the streaming kernel for bf16 / f16 / fp8: fp32 accumulation, the reference's
-    elementwise bound (no matrix-core allowance), strides with padding, both pointer modes, and a second
-    call right behind the first on the shared scratch."""
+    """2 or 3 rows of A for bf16 / f16 / fp8: with less than 1 MiB of B (or K off the 16-byte rule) on the
+    streaming kernel with fp32 multiply-adds - the reference's elementwise bound, no matrix-core allowance -,
+    larger ones on the kernel that multiplies on the matrix cores (fp8: with the allowance of those instructions).
+    Strides with padding, both pointer modes, and a second call right behind the first on the shared scratch."""
     for (n, k) in ((11008, 4096), (1040, 136), (16, 8), (2048, 1000)):
         case = rowmajor_case(ta, m, n, k, 1.5, -0.5, tb=tb, rsa=k + 8, rsb=n + 48, rsc=n + 3)
         a, b, c = case.make_inputs(m * 100 + n + k)
+        on_matrix_cores = ta.startswith("f8") and n * k >= (1 << 20) and k % 16 == 0
+        extra = support.FP8_MFMA_REL if on_matrix_cores else 0.0
         for mode in ("device", "host"):
             got = run_gemm(gpu, "rc", case, a, b, c, mode)
-            support.assert_fp_gemm_close(case, a, b, c, got)
+            support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=extra)
             again = run_gemm(gpu, "rc", case, a, b, c, mode)
-            support.assert_fp_gemm_close(case, a, b, c, again)
+            support.assert_fp_gemm_close(case, a, b, c, again, extra_rel=extra)
 
 
 def _kc_case(ta, tb, m, n, k, alpha, beta, pad=0):
