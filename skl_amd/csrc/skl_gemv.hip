@@ -1,9 +1,11 @@
 // skl_gemv.hip - the M == 1 ("decode") path: y = beta*y + alpha * x*B, a pure
-// HBM stream over B. No matrix cores: the kernel is bound by how fast B's bytes
-// arrive, so the design is about memory-level parallelism and coalescing.
-// Three kernels: gemv_kernel (M = 1, row-major or K-packed B; described below),
-// gemv_rows_kernel (a few rows of A against a row-major B) and gemv_kc_kernel
-// (1 to 4 rows of A against a B with K contiguous), each introduced where it is defined.
+// HBM stream over B. The one-row kernels use no matrix cores: they are bound by how
+// fast B's bytes arrive, so the design is about memory-level parallelism and coalescing.
+// Four kernels: gemv_kernel (M = 1, row-major or K-packed B; described below),
+// gemv_rows_kernel (a few rows of A against a row-major B), gemv_mfma_rows_kernel (up to
+// 16 rows of A against a row-major B: the same stream, B transposed in registers and
+// multiplied on the matrix cores) and gemv_kc_kernel (1 to 4 rows of A against a B with K
+// contiguous), each introduced where it is defined.
 //
 // The reference has no separate GEMV API: M == 1 is a branch inside its GEMM
 // dispatchers (src/gemm/gemm_bf16_bf16_f32_zvfbfwma_x390.c:1220-1224,
