@@ -1138,8 +1138,20 @@ extern "C" int skl_hip_launch_gemv_rows(const skl_gemm_canon *g) {
 
 // 4 <= M <= 16 (int8) or 2 <= M <= 16 (fp8, bf16, f16), row-major B (flat or in panels of 64 columns), rows of A contiguous in K and
 // 16-byte aligned, K and N multiples of 16 bytes of elements, C rows inside one block of 64 and its columns a fixed
-// distance apart. Problems with
-// less than 1 MiB of B are left to the kernels that need one launch.
+// distance apart. Small problems are left to the kernels that need one launch.
+// Bytes of B from which the two launches of this path beat the one launch of gemv_rows_kernel (measured on
+// 2048^2, 4096^2, 8192 x 1024, 4096 x 8192 and 4096 x 11008: e.g. int8 with 4 rows 8.0 against 8.9 us at 16 MiB,
+// 13.9 against 13.3 us at 43 MiB; bf16 with 2 rows 6.9 against 8.5 us at 8 MiB, 9.7 against 9.3 us at 16 MiB). Row
+// counts the other kernel does not take (int8 above 8, floating point above 3) come here from 1 MiB on.
+namespace {
+size_t mfma_rows_min_bytes(int mode, size_t m) {
+  constexpr size_t MiB = size_t(1) << 20;
+  if (mode == kI8RowMajor) return m == 4 ? 40 * MiB : m == 5 ? 12 * MiB : m <= 7 ? 4 * MiB : MiB;
+  if (mode == kBF16 || mode == kF16) return m <= 3 ? 12 * MiB : MiB;
+  return m == 2 ? 12 * MiB : MiB;  // fp8
+}
+}  // namespace
+
 extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g) {
   const int mode = mode_of(g, 0);
   if (mode < 0 || mode == kI8K4) return 0;
@@ -1151,7 +1163,7 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g) {
   // 11.5 us, bf16 20.4 against 21.6 us - left to the M = 1 kernel, which uses no matrix cores.)
   const size_t min_rows = mode == kI8RowMajor ? kMfmaMinRowsInt8 : 2;
   if (g->m < min_rows || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;
-  if ((g->k % piece) != 0 || (g->n % piece) != 0 || g->k * g->n * es < (size_t(1) << 20)) return 0;
+  if ((g->k % piece) != 0 || (g->n % piece) != 0 || g->k * g->n * es < mfma_rows_min_bytes(mode, g->m)) return 0;
   if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % piece) != 0) return 0;
   if (g->b_s0 != 1 || !aligned16(g->b) || (g->b_sk % piece) != 0 || (g->b_s1 % piece) != 0) return 0;
   if (g->csc1 != 64 * g->csc0) return 0;

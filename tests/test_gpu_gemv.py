@@ -203,11 +203,15 @@ def test_decode_batch_on_the_matrix_cores_fp8(gpu, ta, tb, m):
     for (n, k, pad) in ((11008, 4096, 0), (4112, 528, 16), (2064, 1008, 48)):
         case = rowmajor_case(ta, m, n, k, 1.5, -0.5, tb=tb, rsa=k + pad, rsb=n + pad, rsc=n + pad)
         a, b, c = case.make_inputs(m * 100 + n + k)
+        # two or three rows against less than 12 MiB of B run on the kernel with fp32 multiply-adds (sums between
+        # workgroups through atomics: no fixed order, and not the sums of the fused call)
+        here = m >= 4 or n * k >= (12 << 20)
         for mode in ("device", "host"):
             got = run_gemm(gpu, "rc", case, a, b, c, mode)
             support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=support.FP8_MFMA_REL)
-            assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
-        if ta != tb:
+            if here:
+                assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
+        if ta != tb or not here:
             continue  # the mixed pair has no fused entry point
         bias = (np.arange(n) % 7 - 3).astype(np.float32)
         start = np.array([-np.inf], np.float32)
@@ -229,10 +233,16 @@ def test_decode_batch_on_the_matrix_cores_16bit(gpu, ta, m):
     for (n, k, pad) in ((11008, 4096, 0), (4104, 520, 8), (2056, 1000, 24)):
         case = rowmajor_case(ta, m, n, k, 1.5, -0.5, rsa=k + pad, rsb=n + pad, rsc=n + pad)
         a, b, c = case.make_inputs(m * 100 + n + k)
+        # two or three rows against less than 12 MiB of B run on the kernel with fp32 multiply-adds (sums between
+        # workgroups through atomics: no fixed order, and not the sums of the fused call)
+        here = m >= 4 or 2 * n * k >= (12 << 20)
         for mode in ("device", "host"):
             got = run_gemm(gpu, "rc", case, a, b, c, mode)
             support.assert_fp_gemm_close(case, a, b, c, got)
-            assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
+            if here:
+                assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
+        if not here:
+            continue
         bias = (np.arange(n) % 7 - 3).astype(np.float32)
         start = np.array([-np.inf], np.float32)
         plain = run_gemm(gpu, "rc", case, a, b, c, "device")
