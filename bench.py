@@ -419,6 +419,9 @@ MEASURED_TRAFFIC_BYTES = {
     "cvt_f32_f8e4m3_8192sq": int((131135 * 1.998 + 65536) * 1024),
     "gemm_i8_8192": int((393396 * 1.998 + 262144) * 1024),
     "copy_u32_4096sq": int((32800.3 * 1.998 + 65536) * 1024),
+    # both kernels of the call
+    "gemm_i8_16x4096x11008": int(((22336.6 + 17.1) * 1.998 + 5504 + 688) * 1024),
+    "gemm_bf16_8x4096x11008": int(((44343.8 + 1397.5) * 1.998 + 2752 + 344) * 1024),
 }
 
 
