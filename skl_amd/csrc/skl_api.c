@@ -226,8 +226,8 @@ static int gemv_paths(const skl_gemm_canon *g, int launch) {
 
 static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
   if (!fused && gemv_paths(g, launch)) return 1;
-  /* the decode-batch kernel of the fp8 kinds applies the fused steps itself, so that a call gives the same bits
-   * with and without them */
+  /* the decode-batch kernel of the floating-point kinds applies the fused steps itself, so that a call gives the
+   * same bits with and without them */
   if (fused && skl_hip_gemv_mfma_rows_supported(g)) return launch ? (skl_hip_launch_gemv_mfma_rows(g), 1) : 1;
   if (skl_hip_gemm_mfma_supported(g)) return launch ? (skl_hip_launch_gemm_mfma(g), 1) : 1;
   return 0;

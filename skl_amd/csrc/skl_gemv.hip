@@ -570,8 +570,8 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 
 
 // ---------------------------------------------------------------------------
-// 4 <= M <= 16 rows of int8 A (other kinds, below: from two rows) against a row-major B: still one pass over B at the speed it arrives, with
-// the multiply-adds on the matrix cores so that their number does not grow with the rows of A
+// 4 <= M <= 16 rows of int8 A (other kinds, below: from two rows) against a row-major B: still one pass over B
+// at the speed it arrives, with the multiply-adds on the matrix cores so that their number does not grow with the rows of A
 // (v_mfma_i32_16x16x64_i8: a 16 x 64 block of A times a 64 x 16 block of B). B never goes through LDS: a lane
 // loads 16 consecutive rows of 16 consecutive columns (128-bit non-temporal loads, 16 lanes side by side cover
 // 256 columns, the four lane groups of a wave take four ranges of 16 rows), transposes the 16 x 16 bytes in
@@ -591,10 +591,10 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 // the reference's epilogue rounds beta*c + alpha*acc in one place, so here each workgroup stores its raw sums to
 // its own plane of the stream's workspace and a second kernel adds the planes in order, applies alpha / beta and
 // the fused steps: deterministic, at the accuracy of the fp8 matrix-core instructions like the tile kernels.
-// ---------------------------------------------------------------------------
 // bf16 / f16: a 128-bit load holds 8 columns and v_mfma_f32_16x16x32_{bf16,f16} wants 8 consecutive k per lane, so a
 // lane loads 8 rows of 8 columns and transposes 8 x 8 halfwords (one v_perm_b32 per dword of the result); 16 lanes
 // cover 128 columns, the four lane groups 32 rows, a wave takes four such blocks. Raw sums in planes like fp8.
+// ---------------------------------------------------------------------------
 constexpr int kMfmaMinRowsInt8 = 4, kMfmaMaxRows = 16, kMfmaWaves = 4;
 template <int ES>
 struct MfmaShape {
@@ -618,8 +618,8 @@ struct GemvMfmaArgs {
   size_t m, n, k;
   skl_scalar alpha, beta;
   unsigned tiles, slabs;
-  float *planes;        // fp8: slabs planes of m x n raw sums
-  const float *bias;    // fp8: fused steps of the second pass, or null
+  float *planes;        // floating point: slabs planes of m x n raw sums
+  const float *bias;    // floating point: fused steps of the second pass, or null
   float *max;
 };
 
@@ -630,7 +630,7 @@ __global__ void __launch_bounds__(256) gemv_mfma_scale_c_kernel(GemvMfmaArgs p) 
   *c = p.beta.i == 0 ? 0 : (int)((unsigned)p.beta.i * (unsigned)*c);
 }
 
-// C = beta*C + alpha * (sum of the planes, in order), then bias and maximum: the second pass of the fp8 kinds.
+// C = beta*C + alpha * (sum of the planes, in order), then bias and maximum: the second pass of the floating-point kinds.
 __global__ void __launch_bounds__(256) gemv_mfma_add_planes_kernel(GemvMfmaArgs p) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= p.m * p.n) return;
@@ -1167,7 +1167,7 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g) {
   if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % piece) != 0) return 0;
   if (g->b_s0 != 1 || !aligned16(g->b) || (g->b_sk % piece) != 0 || (g->b_s1 % piece) != 0) return 0;
   if (g->csc1 != 64 * g->csc0) return 0;
-  if (mode == kI8RowMajor && (g->bias || g->max)) return 0;  // the fused steps ride on the second pass of the fp8 kinds
+  if (mode == kI8RowMajor && (g->bias || g->max)) return 0;  // the fused steps ride on the second pass (floating point)
   // floating point: one plane of raw sums per 512 k, inside the workspace's usual 64 MiB
   const size_t slabs = (g->k + MfmaShape<1>::kKPerGroup - 1) / MfmaShape<1>::kKPerGroup;
   static_assert(MfmaShape<1>::kKPerGroup == MfmaShape<2>::kKPerGroup, "one group length for every kind");
