@@ -151,14 +151,20 @@ static int canonicalize(const skl_gemm_desc *d, skl_gemm_canon *g) {
   return canonicalize_c(d, g, 0);
 }
 
-/* The K4-interleaved int8 layout of the dot4 entry point, M == 1 only. */
-static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g) {
-  if (d->ta != SKL_DT_I8 || d->m0 * d->m1 != 1 || d->k0 != 4 || d->n0 != 1) return 0;
+/* The K4-interleaved int8 layout of the dot4 entry point: one row of A (`rows` == 0), or up to 16 rows that are
+ * contiguous in K and lie in one block of C's rows. */
+static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g, int rows) {
+  if (d->ta != SKL_DT_I8 || d->k0 != 4 || d->n0 != 1) return 0;
+  if (rows ? (d->m0 != 1 || d->m1 < 2 || d->m1 > 16) : d->m0 * d->m1 != 1) return 0;
   if (d->rsb0 != 1 || d->csb1 != 4 || d->csa0 != 1) return 0;
   if (!(d->k1 == 1 || d->csa1 == 4)) return 0;
   memset(g, 0, sizeof *g);
   g->ta = g->tb = SKL_DT_I8;
-  g->m = 1;
+  g->m = d->m1;
+  g->a_s0 = d->rsa1;
+  g->a_s1 = SKL_TE * d->rsa1;
+  g->rsc0 = d->rsc1;
+  g->rsc1 = SKL_TE * d->rsc1;
   g->n = d->n1;
   g->k = 4 * d->k1;
   g->a = d->a;
@@ -178,14 +184,14 @@ static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g) {
 static int gemv_on_device(const skl_gemm_canon *g) {
   if (skl_hip_gemv_kc_supported(g)) return skl_hip_launch_gemv_kc(g), 1;
   if (g->m == 1 && skl_hip_gemv_supported(g, 0)) return skl_hip_launch_gemv(g, 0), 1;
-  if (skl_hip_gemv_mfma_rows_supported(g)) return skl_hip_launch_gemv_mfma_rows(g), 1;
+  if (skl_hip_gemv_mfma_rows_supported(g, 0)) return skl_hip_launch_gemv_mfma_rows(g, 0), 1;
   if (skl_hip_gemv_rows_supported(g)) return skl_hip_launch_gemv_rows(g), 1;
   return 0;
 }
 
 static int gemv_would_take(const skl_gemm_canon *g) {
   return skl_hip_gemv_kc_supported(g) || (g->m == 1 && skl_hip_gemv_supported(g, 0)) ||
-         skl_hip_gemv_mfma_rows_supported(g) || skl_hip_gemv_rows_supported(g);
+         skl_hip_gemv_mfma_rows_supported(g, 0) || skl_hip_gemv_rows_supported(g);
 }
 
 /* C^T = B^T A^T: a problem with a few columns (matrix times vector, the reference's "small-N" regime,
@@ -228,7 +234,7 @@ static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
   if (!fused && gemv_paths(g, launch)) return 1;
   /* the decode-batch kernel of the floating-point kinds applies the fused steps itself, so that a call gives the
    * same bits with and without them */
-  if (fused && skl_hip_gemv_mfma_rows_supported(g)) return launch ? (skl_hip_launch_gemv_mfma_rows(g), 1) : 1;
+  if (fused && skl_hip_gemv_mfma_rows_supported(g, 0)) return launch ? (skl_hip_launch_gemv_mfma_rows(g, 0), 1) : 1;
   if (skl_hip_gemm_mfma_supported(g)) return launch ? (skl_hip_launch_gemm_mfma(g), 1) : 1;
   return 0;
 }
@@ -363,8 +369,12 @@ static void gemm_on_device(const skl_gemm_desc *d) {
   skl_gemm_canon g;
   const int fused = d->bias != NULL || d->max != NULL; /* the M = 1 kernels have no fused steps */
   if (d->k0 * d->k1 != 0 && d->ta <= SKL_DT_F8E5M2) {
-    if (!fused && canonicalize_k4(d, &g) && skl_hip_gemv_supported(&g, 1)) {
+    if (!fused && canonicalize_k4(d, &g, 0) && skl_hip_gemv_supported(&g, 1)) {
       skl_hip_launch_gemv(&g, 1);
+      return;
+    }
+    if (!fused && canonicalize_k4(d, &g, 1) && skl_hip_gemv_mfma_rows_supported(&g, 1)) {
+      skl_hip_launch_gemv_mfma_rows(&g, 1);
       return;
     }
     if (canonicalize(d, &g)) {

@@ -596,14 +596,20 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 // cover 128 columns, the four lane groups 32 rows, a wave takes four such blocks. Raw sums in planes like fp8.
 // ---------------------------------------------------------------------------
 constexpr int kMfmaMinRowsInt8 = 4, kMfmaMaxRows = 16, kMfmaWaves = 4;
-template <int ES>
+// The K-packed int8 layout of the dot4 entry point (B(4P + p, j) at P * b_sk + 4 j + p) needs no transposes at all:
+// a 128-bit load holds four columns times four k, so four loads at consecutive P give a lane the 16 consecutive k
+// of four columns, dword c of the four loads being the operand of column c. 16 lanes cover 64 columns (256 bytes
+// of a row of groups), a block is 64 k by 64 columns and four instructions, a wave takes four blocks.
+template <int ES, bool K4 = false>
 struct MfmaShape {
-  static constexpr int kLaneCols = 16 / ES;           // columns in a 128-bit load = instructions per block
-  static constexpr int kLaneRows = 16 / ES;           // rows a lane loads per block = k per lane and instruction(s)
-  static constexpr int kBlockK = 4 * kLaneRows;       // 64 or 32
-  static constexpr int kIters = 32 / kLaneRows;       // blocks per wave: 32 loads in flight per lane
-  static constexpr int kTileCols = 16 * kLaneCols;    // 256 or 128
-  static constexpr int kKPerGroup = kMfmaWaves * kIters * kBlockK;  // 512
+  static constexpr int kLaneCols = K4 ? 4 : 16 / ES;  // columns in a 128-bit load = instructions per block
+  static constexpr int kLaneRows = K4 ? 4 : 16 / ES;  // loads of a lane per block
+  static constexpr int kKPerLoad = K4 ? 4 : 1;        // k a load covers: kLaneRows * kKPerLoad = k per lane and block
+  static constexpr int kBlockK = 4 * kLaneRows * kKPerLoad;  // 64 or 32
+  static constexpr int kIters = K4 ? 4 : 32 / kLaneRows;  // blocks per wave: 32 loads in flight per lane (K-packed: 16 -
+                                                          // with 32 the kernel needs 378 registers, one wave per SIMD)
+  static constexpr int kTileCols = 16 * kLaneCols;    // 256, 128 or 64
+  static constexpr int kKPerGroup = kMfmaWaves * kIters * kBlockK;  // 512 (K-packed: 1024)
   static constexpr int kPitch = kTileCols + 4;        // 4-byte words per row of the LDS block
   static constexpr size_t kLds = (size_t)kMfmaWaves * 16 * kPitch * 4;
 };
@@ -662,9 +668,10 @@ __global__ void __launch_bounds__(256) gemv_mfma_add_planes_kernel(GemvMfmaArgs 
 
 template <int MODE>
 __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfmaArgs p) {
-  constexpr bool kInt = MODE == kI8RowMajor, k16 = MODE == kBF16 || MODE == kF16;
+  constexpr bool kInt = MODE == kI8RowMajor || MODE == kI8K4, k16 = MODE == kBF16 || MODE == kF16;
+  constexpr bool kPacked = MODE == kI8K4;
   constexpr int ES = k16 ? 2 : 1;
-  using Sh = MfmaShape<ES>;
+  using Sh = MfmaShape<ES, kPacked>;
   constexpr int LC = Sh::kLaneCols, LR = Sh::kLaneRows, ITERS = Sh::kIters;
   using Acc = typename Mode<MODE>::Acc;  // int or float: 4 bytes either way
   typedef Acc v4acc __attribute__((ext_vector_type(4)));
@@ -677,25 +684,26 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
   const size_t col = (size_t)tile * Sh::kTileCols + (size_t)jl * LC;  // the lane's columns: inside one block of 64
   const size_t kwave = ((size_t)slab * kMfmaWaves + wave) * (Sh::kBlockK * ITERS);
   const bool col_ok = col < p.n;  // n is a multiple of the columns per lane
-  const char *bp = p.b + (col >> 6) * p.b_s1 + (col & 63) * ES;
+  const char *bp = kPacked ? p.b + col * 4 : p.b + (col >> 6) * p.b_s1 + (col & 63) * ES;
+  constexpr int kLaneK = LR * Sh::kKPerLoad;  // k of a lane per block: 16 bytes of A
 
   uint4 rows[ITERS][LR];
   v4i xa[ITERS];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * LR;
+    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * kLaneK;
 #pragma unroll
     for (int r = 0; r < LR; ++r) {
-      if (col_ok && k0 + r < p.k)
-        rows[it][r] = stream_load(bp + (k0 + r) * p.b_sk);
+      if (col_ok && k0 + (size_t)r * Sh::kKPerLoad < p.k)
+        rows[it][r] = stream_load(bp + (k0 / Sh::kKPerLoad + r) * p.b_sk);
       else
         rows[it][r] = make_uint4(0, 0, 0, 0);
     }
   }
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    // k is a multiple of the rows per lane: a 16-byte piece of a row of A is inside or outside
-    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * LR;
+    // k is a multiple of a lane's k per block: a 16-byte piece of a row of A is inside or outside
+    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * kLaneK;
     if ((size_t)jl < p.m && k0 < p.k)
       xa[it] = *reinterpret_cast<const v4i *>(p.a + (size_t)jl * p.a_row + k0 * ES);
     else
@@ -707,7 +715,12 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     unsigned t[4][LC];  // [dword of the operand][column]: the lane's k of one column, ascending
-    if constexpr (k16) {
+    if constexpr (kPacked) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        t[q][0] = rows[it][q].x, t[q][1] = rows[it][q].y, t[q][2] = rows[it][q].z, t[q][3] = rows[it][q].w;
+      }
+    } else if constexpr (k16) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {  // rows 2q and 2q + 1 of the block
         const uint4 lo = rows[it][2 * q], hi = rows[it][2 * q + 1];
@@ -1152,9 +1165,18 @@ size_t mfma_rows_min_bytes(int mode, size_t m) {
 }
 }  // namespace
 
-extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g) {
-  const int mode = mode_of(g, 0);
-  if (mode < 0 || mode == kI8K4) return 0;
+extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int layout) {
+  const int mode = mode_of(g, layout);
+  if (mode < 0) return 0;
+  if (mode == kI8K4) {
+    // B(4P + p, j) at P * b_sk + 4 j + p; 2 to 16 rows (no other kernel reads this layout with more than one row)
+    if (g->c_row_shift != 6 || g->c_col_shift != 6 || g->bias || g->max) return 0;
+    if (g->m < 2 || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;
+    if ((g->k % 16) != 0 || (g->n % 4) != 0 || g->k * g->n < (size_t(1) << 20)) return 0;
+    if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % 16) != 0) return 0;
+    if (!aligned16(g->b) || (g->b_sk % 16) != 0) return 0;
+    return g->csc1 == 64 * g->csc0;
+  }
   const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1, piece = 16 / es;  // elements in 16 bytes
   if (g->c_row_shift != 6 || g->c_col_shift != 6) return 0;
   // Fewest rows from which this kernel is the faster one for 1 x 4096 x 11008 weights: int8 13.1 us whatever the
@@ -1170,7 +1192,7 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g) {
   if (mode == kI8RowMajor && (g->bias || g->max)) return 0;  // the fused steps ride on the second pass (floating point)
   // floating point: one plane of raw sums per 512 k, inside the workspace's usual 64 MiB
   const size_t slabs = (g->k + MfmaShape<1>::kKPerGroup - 1) / MfmaShape<1>::kKPerGroup;
-  static_assert(MfmaShape<1>::kKPerGroup == MfmaShape<2>::kKPerGroup, "one group length for every kind");
+  static_assert(MfmaShape<1>::kKPerGroup == MfmaShape<2>::kKPerGroup, "one group length for every floating-point kind");
   if (mode != kI8RowMajor && slabs * g->m * g->n * sizeof(float) > (size_t(64) << 20)) return 0;
   return 1;
 }
@@ -1179,7 +1201,7 @@ namespace {
 
 template <int MODE>
 int launch_mfma_rows(const GemvMfmaArgs &args) {
-  using Sh = MfmaShape<(MODE == kBF16 || MODE == kF16) ? 2 : 1>;
+  using Sh = MfmaShape<(MODE == kBF16 || MODE == kF16) ? 2 : 1, MODE == kI8K4>;
   constexpr size_t kMfmaLds = Sh::kLds;
   auto kernel = gemv_mfma_rows_kernel<MODE>;
   static bool configured = false;  // per instantiation; racing threads would set the same value
@@ -1198,7 +1220,7 @@ int launch_mfma_rows(const GemvMfmaArgs &args) {
     skl_hip_record_error(-2, "gemv_mfma_rows: grid too large");
     return -2;
   }
-  if constexpr (MODE == kI8RowMajor) {
+  if constexpr (MODE == kI8RowMajor || MODE == kI8K4) {
     if (p.beta.i != 1) {  // beta == 1: C is the starting value as it is
       gemv_mfma_scale_c_kernel<<<(unsigned)cells, 256, 0, skl_current_stream()>>>(p);
       int rc = skl_check_launch("gemv_mfma_scale_c");
@@ -1227,14 +1249,14 @@ int launch_mfma_rows(const GemvMfmaArgs &args) {
 
 }  // namespace
 
-extern "C" int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g) {
-  if (!skl_hip_gemv_mfma_rows_supported(g)) {
+extern "C" int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g, int layout) {
+  if (!skl_hip_gemv_mfma_rows_supported(g, layout)) {
     skl_hip_record_error(-2, "gemv_mfma_rows: unsupported problem");
     return -2;
   }
   GemvMfmaArgs p;
   p.a = (const char *)g->a;
-  const int mode = mode_of(g, 0);
+  const int mode = mode_of(g, layout);
   const size_t es = (mode == kBF16 || mode == kF16) ? 2 : 1;
   p.a_row = g->a_s0 * es;
   p.b = (const char *)g->b;
@@ -1254,6 +1276,7 @@ extern "C" int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g) {
   p.max = (float *)g->max;
   switch (mode) {
     case kI8RowMajor: return launch_mfma_rows<kI8RowMajor>(p);
+    case kI8K4: return launch_mfma_rows<kI8K4>(p);
     case kBF16: return launch_mfma_rows<kBF16>(p);
     case kF16: return launch_mfma_rows<kF16>(p);
     case kF8E4M3: return launch_mfma_rows<kF8E4M3>(p);

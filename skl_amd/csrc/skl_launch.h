@@ -103,9 +103,10 @@ int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout);
 int skl_hip_gemv_rows_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_rows(const skl_gemm_canon *g);
 /* 4 <= M <= 16 rows against a row-major int8 B, 2 <= M <= 16 against an fp8 / bf16 / f16 one: the same stream with
- * the multiply-adds on the matrix cores (floating point: with the fused steps, if any). */
-int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g);
-int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g);
+ * the multiply-adds on the matrix cores (floating point: with the fused steps, if any). `layout` as for the M == 1
+ * kernels: 1 = K4-interleaved int8 B, 2 <= M <= 16. */
+int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int layout);
+int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g, int layout);
 /* 1 <= M <= 4 against a B with K contiguous (b_sk == 1): one dot product over contiguous memory per output. */
 int skl_hip_gemv_kc_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);

@@ -106,6 +106,24 @@ def test_k_packed_int8_decode(gpu, n, k1):
         assert np.array_equal(run_gemm(gpu, "dot4", case, a, b, c, mode), run_oracle_gemm(case, a, b, c))
 
 
+@pytest.mark.parametrize("m", (2, 3, 7, 16))
+def test_k_packed_int8_decode_batches(gpu, m):
+    """The dot4 layout with 2 to 16 rows of A (src/gemm/gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.c:645-660 has its own
+    kernels for these): the K-packed B is read in place by the decode-batch kernel - four loads give a lane 16 k of
+    four columns, no transposes. The config-2 weights prepacked, N and K off the kernel's 2048 x 64 blocks, padded
+    strides of A, B and C, alpha / beta with wrap-around, both pointer modes; whole-buffer compare."""
+    rng = np.random.default_rng(600 + m)
+    for (n, k1, pad_a, pad_b, pad_c) in ((11008, 1024, 0, 0, 0), (4100, 132, 16, 32, 5), (2052, 516, 48, 16, 0)):
+        for alpha, beta in ((1, 0), (0x01010101, -77), (-3, 1)):
+            case = support.dot4_case(m, n, k1, alpha=alpha, beta=beta, rsa1=4 * k1 + pad_a, rsb1=4 * n + pad_b,
+                                     rsc1=n + pad_c)
+            a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+            c[:] = rng.integers(-2 ** 31, 2 ** 31, size=c.size)
+            want = run_oracle_gemm(case, a, b, c)
+            for mode in ("device", "host"):
+                assert np.array_equal(run_gemm(gpu, "dot4", case, a, b, c, mode), want), (m, n, k1, alpha, beta, mode)
+
+
 def _exact_int8_gemv(x, w, k, n):
     """x (k) times row-major w (k x n) in exact integer arithmetic, through fp64 BLAS in slices of K."""
     acc = np.zeros(n, np.float64)
