@@ -365,6 +365,32 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   return done;
 }
 
+/* K-packed B with more rows of A than one call of the decode-batch kernel takes: chunks of 16 rows, one pass over
+ * B each. Up to 112 rows that is cheaper than copying B into a layout the tile kernels read (17 x 4096 x 11008:
+ * 126 us on copies). Every chunk is checked before the first is launched. */
+static int k4_in_row_chunks(const skl_gemm_desc *d) {
+  skl_gemm_canon g;
+  int launch;
+  if (d->ta != SKL_DT_I8 || d->k0 != 4 || d->m0 != 1 || d->m1 <= 16 || d->m1 > 112) return 0;
+  for (launch = 0; launch < 2; ++launch) {
+    size_t i;
+    for (i = 0; i < d->m1; i += 16) {
+      skl_gemm_desc part = *d;
+      part.m1 = d->m1 - i < 16 ? d->m1 - i : 16;
+      part.a = (const char *)d->a + i * d->rsa1;
+      part.c = (char *)d->c + 4 * i * d->rsc1;
+      if (part.m1 == 1) {
+        if (!canonicalize_k4(&part, &g, 0) || !skl_hip_gemv_supported(&g, 1)) return 0;
+        if (launch) skl_hip_launch_gemv(&g, 1);
+      } else {
+        if (!canonicalize_k4(&part, &g, 1) || !skl_hip_gemv_mfma_rows_supported(&g, 1)) return 0;
+        if (launch) skl_hip_launch_gemv_mfma_rows(&g, 1);
+      }
+    }
+  }
+  return 1;
+}
+
 static void gemm_on_device(const skl_gemm_desc *d) {
   skl_gemm_canon g;
   const int fused = d->bias != NULL || d->max != NULL; /* the M = 1 kernels have no fused steps */
@@ -377,6 +403,7 @@ static void gemm_on_device(const skl_gemm_desc *d) {
       skl_hip_launch_gemv_mfma_rows(&g, 1);
       return;
     }
+    if (!fused && k4_in_row_chunks(d)) return;
     if (canonicalize(d, &g)) {
       if (!fused && gemv_paths(&g, 1)) return;
       if (gemm_padded_to_tiles(&g)) return;
