@@ -185,6 +185,21 @@ def wl_gemv_p4x1c(lib, rng):
                 name="int8 GEMV 1x4096x11008 (W in the p4x1c K-packed layout, beta=0)", kernel="gemv_kernel<int8 K-packed>")
 
 
+def wl_small_batch_p4x1c(lib, rng):
+    """Decode with a batch of 16 against the same prepacked weights: the K-packed B read in place, no transposes."""
+    m, k, n, nbuf = 16, 4096, 11008, 8
+    w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(rand_i8(rng, m * k))
+    y = DeviceBuffer(4 * m * n)
+
+    def step(i):
+        lib.skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(m, n, k // 4, 1, x, k, 4, w[i % nbuf], 4 * n, 0, y, n)
+
+    return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
+                name="int8 GEMM 16x4096x11008 (W in the p4x1c K-packed layout, decode with a batch of 16)",
+                kernel="gemv_mfma_scale_c_kernel + gemv_mfma_rows_kernel<int8 K-packed>")
+
+
 def wl_gemv_bf16(lib, rng):
     k, n, nbuf = 4096, 11008, 4
     w = [DeviceBuffer.from_array(bf16_bits(rng.normal(size=k * n) * 0.02)) for _ in range(nbuf)]
@@ -392,6 +407,7 @@ WORKLOADS = {
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 500, 50),
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 300, 30),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 300, 30),
+    "gemm_i8_p4x1c_16x4096x11008": (wl_small_batch_p4x1c, 300, 30),
     "gemm_f8e4m3_16x4096x11008": (wl_small_batch_f8, 300, 30),
     "gemm_bf16_8x4096x11008": (wl_small_batch_bf16, 300, 30),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
