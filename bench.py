@@ -5,12 +5,16 @@
 
 Prints ONE JSON line. The headline (`value`) is the int8 GEMV decode shape
 (1x4096 times 4096x11008, benchmark configuration 2) in GB/s of algorithmic bytes with
-all operands resident in HBM; a "step" is one GEMV call on the next of several
-weight matrices (their total size exceeds the 256 MiB last-level cache, so the
-stream comes from HBM). `extra` carries the dense workloads (TOPS / TFLOP/s and
-fraction of the MFMA roofline) and the pack / cvt streams, each timed the same
-way. `cpu_baseline` is the reference's scalar routine (or, where that library
-was not built, the CPU checker) timed on this host for the same shape.
+all operands resident in HBM. A "step" is `config.calls_per_step` GEMV calls back to back,
+each on the next of eight weight matrices (their total size exceeds the 256 MiB last-level
+cache, so the stream comes from HBM): one 10 us call per step would time the synchronisation
+around the step, not the kernel. `value` comes from the wall clock around the K steps,
+`roofline.achieved` from HIP events on the library's stream around the same calls.
+`roofline.configs` is the table of the other benchmark configurations (TOPS / TFLOP/s or GB/s and
+fraction of the roofline, each timed the same way), `roofline.measured_peak` what a plain read of
+the same buffers reaches on this device (and, per table row, what the matrix cores reach on register
+operands), `extra` the full records. `cpu_baseline` is the reference's scalar routine (or, where that
+library was not built, the CPU checker) timed on this host for the same shape.
 """
 import argparse
 import json
@@ -29,31 +33,32 @@ from skl_amd import DeviceBuffer  # noqa: E402
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TOPS = {"i8": 5000.0, "f8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "f32": 157.3, "f64": 78.6}
 METRIC = "GEMM TOPS (int8/fp8/bf16) + GEMV HBM GB/s on 1 MI355X, % of roofline"
+LLC_BYTES = 256 << 20  # buffers of HBM-bound workloads are rotated so that a step streams more than this
 
 
 class Timer:
-    """Times `steps` calls of fn(i) after `warmup` untimed ones: wall clock around a
+    """Times `steps` steps of `calls` calls of fn(i) each after `warmup` untimed steps: wall clock around a
     synchronised region, and HIP events on the library's stream inside it."""
 
     def __init__(self, lib):
         self.lib = lib
         self.e0, self.e1 = lib.skl_hip_event_create(), lib.skl_hip_event_create()
 
-    def run(self, fn, steps, warmup):
+    def run(self, fn, steps, warmup, calls=1):
         lib = self.lib
-        for i in range(warmup):
+        for i in range(warmup * calls):
             fn(i)
         lib.skl_hip_synchronize()
         t0 = time.perf_counter()
         lib.skl_hip_event_record(self.e0)
-        for i in range(steps):
-            fn(warmup + i)
+        for i in range(steps * calls):
+            fn(i)
         lib.skl_hip_event_record(self.e1)
         ev_ms = lib.skl_hip_event_elapsed_ms(self.e0, self.e1)
         lib.skl_hip_synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3
         skl_amd.check_error()
-        return wall_ms / steps, ev_ms / steps
+        return wall_ms / steps, ev_ms / (steps * calls)
 
 
 def rand_i8(rng, n):
@@ -371,61 +376,149 @@ def wl_cvt(lib, rng):
 
 
 def wl_pack_a(lib, rng):
-    te, m, k = 64, 4096, 4096
-    a = DeviceBuffer.from_array(rng.integers(0, 1 << 16, m * k, dtype=np.uint16))
-    ap = DeviceBuffer(2 * m * k)
+    te, m, k, nbuf = 64, 4096, 4096, 5   # 5 x (32 + 32 MiB): more than the last-level cache between two uses
+    a = [DeviceBuffer.from_array(rng.integers(0, 1 << 16, m * k, dtype=np.uint16)) for _ in range(nbuf)]
+    ap = [DeviceBuffer(2 * m * k) for _ in range(nbuf)]
 
     def step(i):
-        lib.skl_pack_e16_e16rcptex1c_gfx950(m, k, a, k, ap, k * te, te, 0)
+        lib.skl_pack_e16_e16rcptex1c_gfx950(m, k, a[i % nbuf], k, ap[i % nbuf], k * te, te, 0)
 
     return dict(fn=step, bytes=4 * m * k, ops=m * k, bound="hbm", dtype="u16", keep=(a, ap),
-                name="pack e16 4096x4096 -> TEx1 column panels", kernel="pack_vec_kernel (transposing)")
+                name="pack e16 4096x4096 -> TEx1 column panels (5 buffer pairs rotated)",
+                kernel="pack_vec_kernel (transposing)")
+
+
+def wl_pack_b(lib, rng):
+    """Configuration 5's B: row-major 4096 x 14336 f16 into 1 x TE row panels (a copy-like pack, 112 + 112 MiB)."""
+    te, k, n, nbuf = 64, 4096, 14336, 2
+    b = [DeviceBuffer.from_array(rng.integers(0, 1 << 16, k * n, dtype=np.uint16)) for _ in range(nbuf)]
+    bp = [DeviceBuffer(2 * k * n) for _ in range(nbuf)]
+
+    def step(i):
+        lib.skl_pack_e16rc_e16rcprc_gfx950(k, n, b[i % nbuf], n, 1, 1, te, bp[i % nbuf], te, 1, te, k * te, 0)
+
+    return dict(fn=step, bytes=4 * k * n, ops=k * n, bound="hbm", dtype="u16", keep=(b, bp),
+                name="pack e16 4096x14336 -> 1xTE row panels (2 buffer pairs rotated)", kernel="pack_vec_kernel (copy-like)")
+
+
+def wl_unpack_c(lib, rng):
+    """Configuration 5's C: TE x TE blocks of f32 back to row-major 4096 x 14336 (224 + 224 MiB)."""
+    te, m, n = 64, 4096, 14336
+    n1 = n // te
+    cp = DeviceBuffer.from_array(rng.integers(0, 1 << 32, m * n, dtype=np.uint32))
+    c = DeviceBuffer(4 * m * n)
+
+    def step(i):
+        lib.skl_unpack_e32rcprc_e32rc_gfx950(te, te, cp, te, 1, n1 * te * te, te * te, m, n, c, n, 1)
+
+    return dict(fn=step, bytes=8 * m * n, ops=m * n, bound="hbm", dtype="u32", keep=(cp, c),
+                name="unpack e32 TExTE blocks -> row-major 4096x14336", kernel="pack_vec_kernel (copy-like)")
 
 
 def wl_copy(lib, rng):
     """Plain copy through the pack kernel (one block = the whole matrix): the
     known-size stream the HBM traffic counters are calibrated against."""
     m = n = 4096
-    src = DeviceBuffer.from_array(rng.integers(0, 1 << 32, m * n, dtype=np.uint32))
-    dst = DeviceBuffer(4 * m * n)
+    nbuf = 3   # 3 x (64 + 64 MiB)
+    src = [DeviceBuffer.from_array(rng.integers(0, 1 << 32, m * n, dtype=np.uint32)) for _ in range(nbuf)]
+    dst = [DeviceBuffer(4 * m * n) for _ in range(nbuf)]
 
     def step(i):
-        lib.skl_pack_e32rc_e32rcprc_gfx950(m, n, src, n, 1, m, n, dst, n, 1, 0, 0, 0)
+        lib.skl_pack_e32rc_e32rcprc_gfx950(m, n, src[i % nbuf], n, 1, m, n, dst[i % nbuf], n, 1, 0, 0, 0)
 
     return dict(fn=step, bytes=8 * m * n, ops=m * n, bound="hbm", dtype="u32", keep=(src, dst),
-                name="copy 4096x4096 u32 (64 MiB read + 64 MiB write)", kernel="pack_vec_kernel (copy)")
+                name="copy 4096x4096 u32 (64 MiB read + 64 MiB write, 3 buffer pairs rotated)", kernel="pack_vec_kernel (copy)")
 
 
+def wl_peak_hbm_read(lib, rng):
+    """The ceiling of the headline: a plain read (128-bit non-temporal loads, nothing else) of the same eight
+    45 MB buffers the GEMV streams, one launch per buffer."""
+    k, n, nbuf = 4096, 11008, 8
+    w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+
+    def step(i):
+        lib.skl_hip_probe_hbm_read(w[i % nbuf], k * n)
+
+    return dict(fn=step, bytes=k * n, ops=0, bound="hbm", dtype="u8", keep=(w,),
+                name="plain read of 45 MB (8 buffers rotated): what a streaming kernel can reach on that many bytes",
+                kernel="probe_read_kernel")
+
+
+def _wl_peak_mfma(kind, dkey, random_operands):
+    def build(lib, rng):
+        iters = 20000
+        ops = lib.skl_hip_probe_mfma(kind, random_operands, 16)  # also loads the kernel
+        lib.skl_hip_synchronize()
+        ops = ops / 16 * iters
+
+        def step(i):
+            lib.skl_hip_probe_mfma(kind, random_operands, iters)
+
+        what = "pseudo-random" if random_operands else "all-equal"
+        return dict(fn=step, bytes=0, ops=ops, bound="mfma", dtype=dkey, keep=(),
+                    name=f"matrix cores alone, {dkey} 32x32 instructions on register operands ({what} values)",
+                    kernel="probe_mfma_kernel")
+    return build
+
+
+# key: (builder, default steps, default warm-up steps, calls per step)
 WORKLOADS = {
-    "gemv_i8": (wl_gemv, 2000, 100),
-    "gemv_i8_p4x1c": (wl_gemv_p4x1c, 1000, 50),
-    "gemv_bf16": (wl_gemv_bf16, 500, 50),
-    "gemv_f8e4m3": (wl_gemv_f8, 1000, 50),
-    "gemv_i8_1x8192x28672": (wl_gemv_large, 300, 30),
-    "gemv_i8_kcontig": (wl_gemv_kc, 1000, 50),
-    "gemv_bf16_kcontig": (wl_gemv_kc_bf16, 500, 50),
-    "gemm_i8_4x4096x11008": (_wl_small_batch(4), 500, 50),
-    "gemm_i8_8x4096x11008": (_wl_small_batch(8), 300, 30),
-    "gemm_i8_16x4096x11008": (_wl_small_batch(16), 300, 30),
-    "gemm_i8_p4x1c_16x4096x11008": (wl_small_batch_p4x1c, 300, 30),
-    "gemm_f8e4m3_16x4096x11008": (wl_small_batch_f8, 300, 30),
-    "gemm_bf16_8x4096x11008": (wl_small_batch_bf16, 300, 30),
-    "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2),
-    "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2),
-    "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2),
-    "gemm_f8e4m3_8192_rowmajor_a": (wl_gemm_f8_layout(True, False), 10, 2),
-    "gemm_f8e4m3_8192_kcontig": (wl_gemm_f8_layout(True, True), 10, 2),
-    "gemm_i8_4000": (wl_gemm_i8_4000, 20, 3),
-    "gemm_bf16_2048x4096x4096": (wl_gemm_bf16, 20, 3),
-    "gemm_f32_4096": (wl_gemm_f32, 5, 1),
-    "gemm_f64_4096": (wl_gemm_f64, 5, 1),
-    "pipeline_f16_4096x4096x14336": (wl_f16_pipeline, 5, 1),
-    "gemm_i8_512": (wl_gemm_i8_512, 200, 20),
-    "cvt_f32_f8e4m3_8192sq": (wl_cvt, 20, 3),
-    "pack_e16_4096sq": (wl_pack_a, 20, 3),
-    "copy_u32_4096sq": (wl_copy, 20, 3),
+    "gemv_i8": (wl_gemv, 20, 5, 128),
+    "peak_hbm_read": (wl_peak_hbm_read, 20, 5, 128),
+    "gemv_i8_p4x1c": (wl_gemv_p4x1c, 10, 2, 128),
+    "gemv_bf16": (wl_gemv_bf16, 10, 2, 64),
+    "gemv_f8e4m3": (wl_gemv_f8, 10, 2, 128),
+    "gemv_i8_1x8192x28672": (wl_gemv_large, 10, 2, 32),
+    "gemv_i8_kcontig": (wl_gemv_kc, 10, 2, 128),
+    "gemv_bf16_kcontig": (wl_gemv_kc_bf16, 10, 2, 64),
+    "gemm_i8_4x4096x11008": (_wl_small_batch(4), 10, 2, 64),
+    "gemm_i8_8x4096x11008": (_wl_small_batch(8), 10, 2, 64),
+    "gemm_i8_16x4096x11008": (_wl_small_batch(16), 10, 2, 64),
+    "gemm_i8_p4x1c_16x4096x11008": (wl_small_batch_p4x1c, 10, 2, 64),
+    "gemm_f8e4m3_16x4096x11008": (wl_small_batch_f8, 10, 2, 64),
+    "gemm_bf16_8x4096x11008": (wl_small_batch_bf16, 10, 2, 32),
+    "peak_mfma_i8_random": (_wl_peak_mfma(0, "i8", 1), 3, 1, 1),
+    "peak_mfma_i8_constant": (_wl_peak_mfma(0, "i8", 0), 3, 1, 1),
+    "peak_mfma_f8_random": (_wl_peak_mfma(2, "f8", 1), 3, 1, 1),
+    "peak_mfma_f8_constant": (_wl_peak_mfma(2, "f8", 0), 3, 1, 1),
+    "peak_mfma_bf16_random": (_wl_peak_mfma(1, "bf16", 1), 3, 1, 1),
+    "peak_mfma_bf16_constant": (_wl_peak_mfma(1, "bf16", 0), 3, 1, 1),
+    "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2, 1),
+    "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2, 1),
+    "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2, 1),
+    "gemm_f8e4m3_8192_rowmajor_a": (wl_gemm_f8_layout(True, False), 10, 2, 1),
+    "gemm_f8e4m3_8192_kcontig": (wl_gemm_f8_layout(True, True), 10, 2, 1),
+    "gemm_i8_4000": (wl_gemm_i8_4000, 10, 2, 2),
+    "gemm_bf16_2048x4096x4096": (wl_gemm_bf16, 10, 2, 4),
+    "gemm_f32_4096": (wl_gemm_f32, 5, 1, 1),
+    "gemm_f64_4096": (wl_gemm_f64, 5, 1, 1),
+    "pipeline_f16_4096x4096x14336": (wl_f16_pipeline, 5, 1, 1),
+    "gemm_i8_512": (wl_gemm_i8_512, 10, 2, 64),
+    "cvt_f32_f8e4m3_8192sq": (wl_cvt, 10, 2, 2),
+    "pack_e16_4096sq": (wl_pack_a, 10, 2, 10),
+    "pack_e16_4096x14336_row_panels": (wl_pack_b, 10, 2, 2),
+    "unpack_e32_4096x14336": (wl_unpack_c, 10, 2, 2),
+    "copy_u32_4096sq": (wl_copy, 10, 2, 6),
 }
 HEADLINE = "gemv_i8"
+
+# The benchmark configurations as rows of `roofline.configs`: label -> workload key.
+CONFIG_TABLE = {
+    "C1 int8 512^3": "gemm_i8_512",
+    "C2 int8 GEMV 1x4096x11008": "gemv_i8",
+    "C3 bf16 2048x4096x4096 beta=1": "gemm_bf16_2048x4096x4096",
+    "C4 fp8 E4M3xE4M3 8192^3": "gemm_f8e4m3_8192",
+    "C4 fp8 E4M3xE5M2 8192^3": "gemm_f8e4m3_f8e5m2_8192",
+    "C5 f16 pack+GEMM+unpack 4096x4096x14336": "pipeline_f16_4096x4096x14336",
+    "C5 pack A": "pack_e16_4096sq",
+    "C5 pack B": "pack_e16_4096x14336_row_panels",
+    "C5 unpack C": "unpack_e32_4096x14336",
+    "C4 cvt f32->E4M3": "cvt_f32_f8e4m3_8192sq",
+    "target int8 8192^3": "gemm_i8_8192",
+}
+# Which probe is the measured ceiling of a workload's kind.
+MEASURED_PEAK_OF = {"hbm": "peak_hbm_read", "i8": "peak_mfma_i8_random", "f8": "peak_mfma_f8_random",
+                    "bf16": "peak_mfma_bf16_random", "f16": "peak_mfma_bf16_random"}
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
 # dispatch), FETCH_SIZE scaled by 1.998 (what it under-reads on a 64 MiB copy), WRITE_SIZE by 1.000;
@@ -442,28 +535,29 @@ MEASURED_TRAFFIC_BYTES = {
 
 
 def measure(lib, key, steps=None, warmup=None, seed=0x5EED0000):
-    builder, dsteps, dwarm = WORKLOADS[key]
+    builder, dsteps, dwarm, calls = WORKLOADS[key]
     steps = steps or dsteps
     warmup = dwarm if warmup is None else warmup
     rng = np.random.default_rng(seed)
     wl = builder(lib, rng)
-    wall_ms, ev_ms = Timer(lib).run(wl["fn"], steps, warmup)
-    out = dict(workload=key, name=wl["name"], steps=steps, warmup=warmup, ms_per_step=wall_ms, event_ms_per_step=ev_ms,
-               dtype=wl["dtype"])
-    sec = ev_ms * 1e-3
+    wall_ms, ev_ms = Timer(lib).run(wl["fn"], steps, warmup, calls)
+    out = dict(workload=key, name=wl["name"], steps=steps, warmup=warmup, calls_per_step=calls, ms_per_step=wall_ms,
+               event_ms_per_call=ev_ms, dtype=wl["dtype"])
+    sec, wall_sec = ev_ms * 1e-3, wall_ms * 1e-3 / calls
     if wl["bound"] == "hbm":
         gbs = wl["bytes"] / sec / 1e9
-        out.update(value=wl["bytes"] / (wall_ms * 1e-3) / 1e9, unit="GB/s",
+        out.update(value=wl["bytes"] / wall_sec / 1e9, unit="GB/s",
                    roofline=dict(bound="hbm", achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=gbs / HBM_PEAK_GBS,
                                  traffic=None, kernel=wl["kernel"], algorithmic_bytes=wl["bytes"]))
     else:
         tops = wl["ops"] / sec / 1e12
         peak = MFMA_PEAK_TOPS[wl["dtype"]]
         unit = "TOP/s" if wl["dtype"] == "i8" else "TFLOP/s"
-        out.update(value=wl["ops"] / (wall_ms * 1e-3) / 1e12, unit=unit,
+        out.update(value=wl["ops"] / wall_sec / 1e12, unit=unit,
                    roofline=dict(bound="mfma", achieved=tops, peak=peak, unit=unit, frac=tops / peak, traffic=None,
                                  kernel=wl["kernel"], ops=wl["ops"]))
     out["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get(key)
+    out["peak_kind"] = "hbm" if wl["bound"] == "hbm" else wl["dtype"]
     for buf in _flatten(wl["keep"]):
         buf.free()
     return out
@@ -545,6 +639,40 @@ def main():
     lib.skl_hip_set_pointer_mode(1)  # device pointers only: no per-call pointer queries
 
     head = measure(lib, args.workload, args.steps, args.warmup)
+    results = {args.workload: head}
+
+    def measured(key):
+        """The record of workload `key`, measured once; None (and an entry in `failed`) if it cannot be."""
+        if key not in results and key not in failed:
+            try:
+                results[key] = measure(lib, key)
+            except Exception as e:  # a failing extra must not hide the headline
+                failed[key] = str(e)
+        return results.get(key)
+
+    def with_measured_peak(rec):
+        """roofline of `rec` plus the ceiling measured on this device for its kind and the fraction of that."""
+        roof = dict(rec["roofline"])
+        probe = measured(MEASURED_PEAK_OF[rec["peak_kind"]]) if rec["peak_kind"] in MEASURED_PEAK_OF else None
+        if probe and not rec["workload"].startswith("peak_"):
+            roof["measured_peak"] = {"value": probe["roofline"]["achieved"], "unit": probe["roofline"]["unit"],
+                                     "workload": probe["workload"], "what": probe["name"]}
+            roof["frac_of_measured"] = roof["achieved"] / probe["roofline"]["achieved"]
+        return roof
+
+    failed = {}
+    roofline = with_measured_peak(head)
+    if not args.no_extra:
+        table = {}
+        for label, key in CONFIG_TABLE.items():
+            r = measured(key)
+            if r is None:
+                table[label] = {"error": failed[key]}
+                continue
+            roof = with_measured_peak(r)
+            table[label] = {"workload": key, "ms": r["event_ms_per_call"], "achieved": roof["achieved"], "unit": roof["unit"],
+                            "bound": roof["bound"], "frac": roof["frac"], "frac_of_measured": roof.get("frac_of_measured")}
+        roofline["configs"] = table
     result = {
         "metric": METRIC,
         "value": head["value"],
@@ -559,21 +687,23 @@ def main():
         "dtype": head["dtype"],
         "data": "synthetic",
         "config": {"workload": head["name"], "key": head["workload"], "resident": "HBM",
+                   "calls_per_step": head["calls_per_step"], "event_us_per_call": head["event_ms_per_call"] * 1e3,
                    "weight_buffers_rotated": 8 if args.workload == "gemv_i8" else 1},
-        "roofline": head["roofline"],
+        "roofline": roofline,
     }
     if not args.no_extra:
         extra = []
         for key in WORKLOADS:
             if key == args.workload:
                 continue
-            try:
-                r = measure(lib, key)
-                extra.append({"workload": r["workload"], "name": r["name"], "value": r["value"], "unit": r["unit"],
-                              "ms_per_step": r["ms_per_step"], "steps": r["steps"], "dtype": r["dtype"],
-                              "roofline": r["roofline"]})
-            except Exception as e:  # a failing extra must not hide the headline
-                extra.append({"workload": key, "error": str(e)})
+            r = measured(key)
+            if r is None:
+                extra.append({"workload": key, "error": failed[key]})
+                continue
+            extra.append({"workload": r["workload"], "name": r["name"], "value": r["value"], "unit": r["unit"],
+                          "ms_per_step": r["ms_per_step"], "steps": r["steps"], "calls_per_step": r["calls_per_step"],
+                          "event_us_per_call": r["event_ms_per_call"] * 1e3, "dtype": r["dtype"],
+                          "roofline": with_measured_peak(r)})
         result["extra"] = extra
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()

@@ -6,9 +6,10 @@
  * (cited as `path:line` below the reference checkout) and only changes the
  * ISA suffix of the name to `gfx950`: dimensions and strides are `size_t` in
  * ELEMENTS, alpha and beta have C's element type, all functions return void,
- * buffers are owned by the caller, C is always read (`C = alpha*A*B + beta*C`,
- * and `C = beta*C` when k == 0), elements outside the addressed set are never
- * written. Pointers may be all device-accessible (asynchronous launch on the
+ * buffers are owned by the caller, `C = alpha*A*B + beta*C` (and `C = beta*C`
+ * when k == 0; beta == 0 initialises a floating-point C without reading it
+ * unless skl_hip_set_beta_zero_mode asks for the reference's evaluation, see
+ * skl-hip.h), elements outside the addressed set are never written. Pointers may be all device-accessible (asynchronous launch on the
  * current stream) or all ordinary host memory (staged, synchronous); see
  * skl-hip.h. Errors are reported through skl_hip_last_error().
  *
@@ -69,11 +70,12 @@ void skl_gemm_f8e5m2rc_f8e5m2rc_f32rc_gfx950(size_t m, size_t n, size_t k, float
 void skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
                                              size_t rsa, size_t csa, const uint8_t *b, size_t rsb,
                                              size_t csb, float beta, float *c, size_t rsc, size_t csc);
-/* ref/gemm/gemm_f32rc_f32rc_f32rc.h:44. Served by the any-stride kernel (no matrix-core path). */
+/* ref/gemm/gemm_f32rc_f32rc_f32rc.h:44. Vector ALUs (the result is defined operation by operation): the
+ * register-tiled kernel, or the any-stride kernel for tiny or oddly blocked problems. */
 void skl_gemm_f32rc_f32rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const float *a, size_t rsa,
                                        size_t csa, const float *b, size_t rsb, size_t csb, float beta,
                                        float *c, size_t rsc, size_t csc);
-/* ref/gemm/gemm_f64rc_f64rc_f64rc.h:44. Served by the any-stride kernel. */
+/* ref/gemm/gemm_f64rc_f64rc_f64rc.h:44. Register-tiled or any-stride kernel, like f32. */
 void skl_gemm_f64rc_f64rc_f64rc_gfx950(size_t m, size_t n, size_t k, double alpha, const double *a,
                                        size_t rsa, size_t csa, const double *b, size_t rsb, size_t csb,
                                        double beta, double *c, size_t rsc, size_t csc);
@@ -106,7 +108,7 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f64rcprc_f64rcprc_f64rcprc_gfx950, double, dou
  * compiler does for a target without half arithmetic, i.e. how the reference's scalar library computes
  * on a general-purpose host); hardware with native half arithmetic rounds the product as well and may
  * differ in the last place, inside the reference's own bound (test/gemm/gemm_f16rcprc_f16rcprc_f16rcprc.c:157).
- * Served by the any-stride kernel.
+ * Register-tiled or any-stride kernel, like f32.
  * ref/gemm/gemm_f16rc_f16rc_f16rc.h:44 */
 void skl_gemm_f16rc_f16rc_f16rc_gfx950(size_t m, size_t n, size_t k, skl_f16_t alpha, const skl_f16_t *a,
                                        size_t rsa, size_t csa, const skl_f16_t *b, size_t rsb, size_t csb,

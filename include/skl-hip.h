@@ -64,6 +64,21 @@ int skl_hip_synchronize(void);
 
 void skl_hip_set_pointer_mode(int mode);
 int skl_hip_get_pointer_mode(void);
+
+/* What a GEMM call with beta == 0 does with a floating-point C (per calling thread).
+ * SKL_HIP_BETA_ZERO_INITIALISES (default): the call initialises C, which is what the reference gives beta == 0
+ *   for (src/gemm/README.md:43, "accumulation (beta=1) and initialization (beta=0)"): the old C is not read,
+ *   except where alpha*A*B is an exact zero, whose sign it decides. The result has the bits of the reference's
+ *   for every finite C; an Inf or NaN in C - or whatever uninitialised memory holds - is overwritten.
+ * SKL_HIP_BETA_ZERO_AS_REFERENCE: beta*C + alpha*A*B is evaluated as the reference's routines evaluate it
+ *   (ref/gemm/gemm_bf16rc_bf16rc_f32rc.c:21): the old C is read and multiplied by zero, so an Inf or NaN in it
+ *   makes the result NaN, exactly where the reference's result is NaN. Costs the read of C (8192^3 fp8: 256 MiB,
+ *   about a quarter on top of the call).
+ * Integer GEMMs give the same result either way and never read C when beta == 0; f64 GEMMs always read it. */
+#define SKL_HIP_BETA_ZERO_INITIALISES 0
+#define SKL_HIP_BETA_ZERO_AS_REFERENCE 1
+void skl_hip_set_beta_zero_mode(int mode);
+int skl_hip_get_beta_zero_mode(void);
 /* 1 if `ptr` is device-accessible, 0 if it is ordinary host memory. */
 int skl_hip_pointer_is_device(const void *ptr);
 
@@ -83,6 +98,18 @@ void skl_hip_event_destroy(void *event);
 int skl_hip_event_record(void *event);
 /* Waits for `stop`, returns milliseconds between the two events (negative on error). */
 float skl_hip_event_elapsed_ms(void *start, void *stop);
+
+/* The two ceilings a report prices kernels against, measured on the device (both enqueue one kernel on the
+ * current stream; time them with the events above).
+ * skl_hip_probe_hbm_read: a plain read of `bytes` (a multiple of 16, 16-byte aligned) with 128-bit non-temporal
+ *   loads, eight in flight per lane: what streaming kernels could reach at best on that many bytes.
+ * skl_hip_probe_mfma: `iters` rounds of eight independent 32 x 32 matrix-core instructions per wave on register
+ *   operands, two workgroups of four waves on every compute unit - kind 0: int8 32x32x32, 1: bf16 32x32x16,
+ *   2: fp8 E4M3 32x32x64; random_operands != 0 fills the operand registers with pseudo-random values (the clock
+ *   the chip sustains depends on the operand values), else every element is the same value. Returns the number of
+ *   operations (two per multiply-add) of the launch, 0 on error. */
+int skl_hip_probe_hbm_read(const void *src, size_t bytes);
+double skl_hip_probe_mfma(int kind, int random_operands, int iters);
 
 /* Name and compute-unit count of the current device (for reports). */
 int skl_hip_device_info(char *name, size_t name_len, int *compute_units, int *clock_mhz);

@@ -421,10 +421,21 @@ static void gemm_on_device(const skl_gemm_desc *d) {
   skl_hip_launch_gemm_generic(d);
 }
 
-static void gemm_run(const skl_gemm_desc *d, const char *who) {
+/* The kinds whose alpha and beta travel as a float (F16H: widened). */
+static int scalars_are_float(int dt) { return dt != SKL_DT_I8 && dt != SKL_DT_F64; }
+
+static void gemm_run(const skl_gemm_desc *in, const char *who) {
+  skl_gemm_desc with_mode = *in;
+  const skl_gemm_desc *d = &with_mode;
   const size_t M = d->m0 * d->m1, N = d->n0 * d->n1, K = d->k0 * d->k1;
   int where;
   if (M == 0 || N == 0) return; /* nothing is addressed */
+  if (scalars_are_float(d->ta)) { /* beta carries the thread's choice of what beta == 0 means (skl_launch.h) */
+    const float beta = in->beta.f;
+    memset(&with_mode.beta, 0, sizeof with_mode.beta);
+    with_mode.beta.fz.value = beta;
+    with_mode.beta.fz.skip_c_read = skl_hip_get_beta_zero_mode() != SKL_HIP_BETA_ZERO_AS_REFERENCE;
+  }
   where = classify(K ? d->a : NULL, K ? d->b : NULL, d->c, who);
   if (where < 0) return;
   if (d->bias || d->max) { /* the fused operands must be of the same kind as C */

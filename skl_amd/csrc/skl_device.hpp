@@ -32,21 +32,23 @@ static inline unsigned skl_div_up(size_t a, size_t b) { return (unsigned)((a + b
 // products and a sum, each rounded on its own (the translation units are built
 // with -ffp-contract=off); int32 wraps.
 //
-// beta == 0 is the initialising call (src/gemm/README.md:43 of the reference:
-// "accumulation (beta=1) and initialization (beta=0)"). There beta*C is a zero
-// whose sign is all the old value contributes, and the sign matters only when
-// alpha*acc is itself a zero: the old value is read for exactly those
-// elements. Results are bit-identical to the reference's for every finite C;
-// an Inf or NaN in C, which the reference would turn into NaN, is overwritten.
+// beta == 0 initialises C (src/gemm/README.md:43 of the reference: "accumulation (beta=1) and initialization
+// (beta=0)"): there beta*C is a zero whose sign is all the old value contributes, and the sign matters only when
+// alpha*acc is itself a zero - the old value is read for exactly those elements. The result has the reference's
+// bits for every finite C; an Inf or NaN in C, which ref/gemm/gemm_bf16rc_bf16rc_f32rc.c:21 (beta*c evaluated
+// whatever beta is) turns into NaN, is overwritten. A caller that wants the reference's result there too asks
+// for it (skl_hip_set_beta_zero_mode(SKL_HIP_BETA_ZERO_AS_REFERENCE)): beta then arrives without
+// fz.skip_c_read and C is read and combined whatever beta is. int32: 0 * c is 0 for every c, so C is never read
+// with beta == 0. f64 has no room for the switch next to the value: always read.
 // ---------------------------------------------------------------------------
 template <typename T>
-__device__ __forceinline__ bool skl_beta_is_zero(skl_scalar beta);
+__device__ __forceinline__ bool skl_beta_is_zero(skl_scalar beta);  // "C need not be read"
 template <>
 __device__ __forceinline__ bool skl_beta_is_zero<int>(skl_scalar beta) { return beta.i == 0; }
 template <>
-__device__ __forceinline__ bool skl_beta_is_zero<float>(skl_scalar beta) { return beta.f == 0.0f; }
+__device__ __forceinline__ bool skl_beta_is_zero<float>(skl_scalar beta) { return beta.fz.skip_c_read != 0 && beta.f == 0.0f; }
 template <>
-__device__ __forceinline__ bool skl_beta_is_zero<double>(skl_scalar beta) { return beta.d == 0.0; }
+__device__ __forceinline__ bool skl_beta_is_zero<double>(skl_scalar) { return false; }  // no room for the switch: always read
 
 __device__ __forceinline__ int skl_combine(int acc, int old, skl_scalar alpha, skl_scalar beta) {
   return (int)((unsigned)beta.i * (unsigned)old + (unsigned)alpha.i * (unsigned)acc);

@@ -69,4 +69,25 @@ __device__ __forceinline__ unsigned decode_ofp8_bits(unsigned code) {
   return sign | ((e + 127u - (unsigned)F::kBias) << 23) | (m << (23 - F::kMant));
 }
 
+// Eight OFP8 bytes (two dwords, ascending) as eight f16 values. Exact: every E4M3 and E5M2 value is an f16 value
+// (E5M2 is f16 cut to its top byte, E4M3 has fewer exponent and significand bits than f16), subnormal codes included.
+template <bool IS_E5M2>
+__device__ __forceinline__ auto widen8_to_f16(unsigned lo, unsigned hi) {
+  typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+  typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+  v2h p[4];
+  if constexpr (IS_E5M2) {
+    p[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(lo, 1.0f, false);
+    p[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(lo, 1.0f, true);
+    p[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(hi, 1.0f, false);
+    p[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(hi, 1.0f, true);
+  } else {
+    p[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false);
+    p[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, true);
+    p[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, false);
+    p[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, true);
+  }
+  return v8h{p[0].x, p[0].y, p[1].x, p[1].y, p[2].x, p[2].y, p[3].x, p[3].y};
+}
+
 }  // namespace skl_fp8

@@ -33,6 +33,7 @@
 #include <utility>
 
 #include "skl_device.hpp"
+#include "skl_fp8.hpp"
 
 namespace {
 
@@ -158,6 +159,44 @@ SKL_F8_MMA(SKL_DT_F8E4M3, SKL_DT_F8E4M3, 0, 0)
 SKL_F8_MMA(SKL_DT_F8E5M2, SKL_DT_F8E5M2, 1, 1)
 SKL_F8_MMA(SKL_DT_F8E4M3, SKL_DT_F8E5M2, 0, 1)
 SKL_F8_MMA(SKL_DT_F8E5M2, SKL_DT_F8E4M3, 1, 0)
+
+// OCP fp8 operands multiplied exactly: the bytes are widened to f16 in registers (every E4M3 / E5M2 value is an
+// f16 value) and two f16 instructions take 32 bytes of K - exact products, fp32 sums, which is what the reference's
+// error bound assumes. The fp8 instructions above align the products of one instruction to a common exponent and
+// keep about 12 bits below the largest; that is inside the bound only once K is a few thousand (the bound grows
+// with K, the instruction's error does not), so short K runs here, at the f16 rate.
+template <int TA, int TB>
+struct MmaF8Exact {
+  static constexpr int KB = 32;  // bytes of K per step: a 16-byte fragment per lane, like int8
+  using Frag = v4i;
+  struct Ready {
+    v8h lo, hi;
+  };
+  template <int DT>
+  __device__ static Ready widen(v4i f) {
+    constexpr bool e5m2 = DT == SKL_DT_F8E5M2;
+    return Ready{skl_fp8::widen8_to_f16<e5m2>((unsigned)f.x, (unsigned)f.y), skl_fp8::widen8_to_f16<e5m2>((unsigned)f.z, (unsigned)f.w)};
+  }
+  __device__ static Ready prep_a(v4i f) { return widen<TA>(f); }
+  __device__ static Ready prep_b(v4i f) { return widen<TB>(f); }
+  __device__ static v16f run(const Ready &a, const Ready &b, v16f c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.lo, b.lo, c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.hi, b.hi, c, 0, 0, 0);
+  }
+};
+// K up to which the fp8 kinds run on MmaF8Exact: the reference's bound 2((1 + 2^-24)^(K+2) - 1) passes the fp8
+// instructions' 2^-11.9 at K = 2193.
+constexpr size_t kF8ExactMaxK = 2304;
+
+// A fragment as the multiply wants it: widened where the operand kind asks for that, else as it was read.
+template <typename M, typename F>
+__device__ __forceinline__ auto prep_a(F f) {
+  if constexpr (requires { M::prep_a(f); }) return M::prep_a(f); else return f;
+}
+template <typename M, typename F>
+__device__ __forceinline__ auto prep_b(F f) {
+  if constexpr (requires { M::prep_b(f); }) return M::prep_b(f); else return f;
+}
 
 // ---------------------------------------------------------------------------
 // LDS tile geometry of one operand: ROWS along M or N, 128 bytes of K.
@@ -331,15 +370,15 @@ __device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, un
   tn = in_group / rows;
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED>
+template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED, bool EXACT = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaArgs p) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   using KA = Kind<TA>;
-  using M = Mma<TA, TB>;
+  using M = typename std::conditional<EXACT, MmaF8Exact<TA, TB>, Mma<TA, TB>>::type;
   using Acc = typename KA::Acc;
   using AccElem = decltype(Acc{}.x);
   constexpr int ES = KA::ES;
-  constexpr int KB = KA::KB;                    // bytes of K per MFMA
+  constexpr int KB = EXACT ? 32 : KA::KB;       // bytes of K per MFMA step
   constexpr int FRB = KB / 2;                   // fragment bytes per lane
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
   constexpr int MI = WM / 32, NI = WN / 32;     // MFMA blocks per wave
@@ -414,10 +453,18 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
       // down next to their uses (with one wave per SIMD nothing else would
       // hide their latency).
       __builtin_amdgcn_sched_barrier(0);
+      {
+        decltype(prep_a<M>(fa[cur][0])) wa[MI];
+        decltype(prep_b<M>(fb[cur][0])) wb[NI];
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
+        for (int i = 0; i < MI; ++i) wa[i] = prep_a<M>(fa[cur][i]);
 #pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = M::run(fa[cur][i], fb[cur][j], acc[i][j]);
+        for (int j = 0; j < NI; ++j) wb[j] = prep_b<M>(fb[cur][j]);
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+          for (int j = 0; j < NI; ++j) acc[i][j] = M::run(wa[i], wb[j], acc[i][j]);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     la.stash(na, ra);
@@ -1095,12 +1142,12 @@ inline unsigned splits_for(size_t tiles, size_t slices, size_t m, size_t n) {
   return (unsigned)(want < 1 ? 1 : want);
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED>
+template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED, bool EXACT = false>
 int launch_one(const MfmaArgs &args) {
   constexpr int ES = Kind<TA>::ES;
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int lds = 2 * (Tile<ES, BM, A_KC, NT>::kBytes + Tile<ES, BN, B_KC, NT>::kBytes);
-  auto kernel = gemm_mfma_kernel<TA, TB, A_KC, B_KC, BM, BN, WAVES_M, WAVES_N, GUARDED>;
+  auto kernel = gemm_mfma_kernel<TA, TB, A_KC, B_KC, BM, BN, WAVES_M, WAVES_N, GUARDED, EXACT>;
   static bool configured = false;  // per instantiation; racing threads would set the same value
   if (!configured) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -1144,6 +1191,15 @@ template <int TA, int TB, bool A_KC, bool B_KC>
 int launch_tile(const MfmaArgs &p) {
   constexpr int ES = Kind<TA>::ES;
   constexpr size_t kRing128FromTiles = 96;
+  constexpr bool kFp8 = TA == SKL_DT_F8E4M3 || TA == SKL_DT_F8E5M2;
+  if constexpr (kFp8) {
+    // short K: exact products (see MmaF8Exact), on the bounds-checked kernel whatever the shape
+    if (p.k <= kF8ExactMaxK) {
+      if (skl_div_up(p.m, 128) * (size_t)skl_div_up(p.n, 128) < 64)
+        return launch_one<TA, TB, A_KC, B_KC, 64, 64, 2, 2, true, true>(p);
+      return launch_one<TA, TB, A_KC, B_KC, 128, 128, 2, 4, true, true>(p);
+    }
+  }
   // The streaming kernel takes problems that its tiles divide evenly: 256 x 256 tiles when those
   // can fill the 256 compute units, 256 x 128 tiles for the sizes below that; everything else runs
   // on the small, bounds-checked kernel.
@@ -1248,6 +1304,7 @@ extern "C" int skl_hip_gemm_mfma_padded_plan(const skl_gemm_canon *g, size_t *mp
   if (!(g->ta == g->tb || (fp8a && fp8b)) || ((uintptr_t)g->c & 3) != 0) return 0;
   const size_t es = (g->ta == SKL_DT_BF16 || g->ta == SKL_DT_F16) ? 2 : 1;
   if (streams_in_place(g, es)) return 0;
+  if (fp8a && g->k <= kF8ExactMaxK) return 0;  // short K: the exact fp8 product, which the streaming kernel does not have
   const size_t tiles_m = (g->m + 255) / 256;
   int tile_cols = 0;
   if (tiles_m * ((g->n + 255) / 256) >= 200) tile_cols = 256;

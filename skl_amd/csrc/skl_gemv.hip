@@ -47,6 +47,7 @@
 #include <type_traits>
 
 #include "skl_device.hpp"
+#include "skl_fp8.hpp"
 
 namespace {
 
@@ -100,8 +101,9 @@ struct GemvArgs {
   size_t y_s;   // elements
   size_t n, k;
   skl_scalar alpha, beta;
-  void *acc;
-  unsigned *tickets;
+  void *acc;         // integer kinds: one zero-initialised 64-bit slot per column
+  unsigned *tickets; // floating point: one zero-initialised counter per strip ...
+  float *planes;     // ... and `slabs` planes of n sums (the stream's workspace)
   unsigned tiles, slabs;
 };
 
@@ -134,19 +136,74 @@ __device__ __forceinline__ float widen16(unsigned bits16, bool is_bf16) {
 }
 
 
+// Sum over the eight lanes of a row of 16 that share a column group (same lane parity), in every lane:
+// three DPP rotations inside the row, no LDS crossbar. A fixed order, also for floats.
+__device__ __forceinline__ int sum_over_row_groups(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x128 /* row_ror:8 */, 0xF, 0xF, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x124 /* row_ror:4 */, 0xF, 0xF, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x122 /* row_ror:2 */, 0xF, 0xF, false);
+  return v;
+}
+
+__device__ __forceinline__ float sum_over_row_groups(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xF, 0xF, false));
+  return v;
+}
+
+// Floating-point sums of the workgroups that share columns. Each workgroup leaves its sums in its own plane of
+// `planes` (element `idx` of plane `slab`, planes `plane_elems` apart) with stores that go through to memory, waits
+// until they have been performed and takes a ticket; the workgroup that draws the last ticket reads every plane
+// back - with read-modify-write atomics, which are performed where the stores went and never see a stale cache
+// line - and adds them in slab order: the same bits on every run, whichever workgroup finishes last. Returns
+// true in that workgroup, with the total of the caller's element in `total`. `mine` says whether the calling
+// thread owns an element at all; every thread of the workgroup must call.
+__device__ __forceinline__ bool ordered_sum_over_slabs(float *planes, size_t plane_elems, size_t idx, unsigned slab,
+                                                       unsigned slabs, unsigned *ticket, unsigned *ticket_s, bool mine,
+                                                       float sum, float &total) {
+  if (mine) __hip_atomic_store(planes + (size_t)slab * plane_elems + idx, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been performed
+  __syncthreads();
+  if (threadIdx.x == 0) *ticket_s = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (*ticket_s != slabs - 1) return false;
+  if (threadIdx.x == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
+  if (mine) {
+    // eight planes are requested before the first is used; the sum still runs over the planes in order
+    unsigned *words = reinterpret_cast<unsigned *>(planes) + idx;
+    float t = 0.0f;
+    for (unsigned q0 = 0; q0 < slabs; q0 += 8) {
+      unsigned v[8];
+#pragma unroll
+      for (unsigned u = 0; u < 8; ++u)
+        v[u] = q0 + u < slabs ? __hip_atomic_fetch_or(words + (size_t)(q0 + u) * plane_elems, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+#pragma unroll
+      for (unsigned u = 0; u < 8; ++u)
+        if (q0 + u < slabs) t = (q0 + u == 0) ? __uint_as_float(v[u]) : __fadd_rn(t, __uint_as_float(v[u]));
+    }
+    total = t;
+  }
+  return true;
+}
+
 // LOADS: 128-bit loads in flight per lane = rows of B (K-packed layout: groups of four rows) a lane takes.
+// Lane pairs read 32 adjacent bytes of a row and the eight row groups of a wave sit inside each row of 16 lanes
+// (column lane = pair member + 2 * row of 16), so that the lanes that share columns are summed with DPP rotations
+// and only one partial sum per wave and column goes through LDS.
 template <int MODE, int LOADS>
 __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
   using Md = Mode<MODE>;
   constexpr int kKPerLaneL = LOADS * Md::kKPerLoad, kKPerGroupL = kPartials * kKPerLaneL;
   using Acc = typename Md::Acc;
   constexpr int kCols = Md::kCols;
-  __shared__ Acc red[kPartials][Md::kTileCols + 4];
+  __shared__ Acc red[kWaves][Md::kTileCols + 4];
   __shared__ unsigned ticket_s;
 
   const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int cl = lane % kColLanes, rl = lane / kColLanes;
+  const int cl = (lane & 1) + 2 * (lane >> 4), rl = (lane >> 1) & 7;
   const int part = wave * kRowLanes + rl;
   const size_t k0 = (size_t)slab * kKPerGroupL + (size_t)part * kKPerLaneL;
   const size_t col = (size_t)tile * Md::kTileCols + (size_t)cl * kCols;
@@ -154,6 +211,14 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
   Acc acc[kCols];
 #pragma unroll
   for (int j = 0; j < kCols; ++j) acc[j] = 0;
+
+  // The thread that will write column tile_col0 + threadIdx.x asks for its old value now, so that it is there
+  // when the sums are: no memory round trip behind the last byte of B.
+  const size_t tile_col0 = (size_t)tile * Md::kTileCols;
+  const bool owner = threadIdx.x < Md::kTileCols && tile_col0 + threadIdx.x < p.n;
+  Acc *yv = reinterpret_cast<Acc *>(p.y);
+  const bool y_is_read = !skl_beta_is_zero<Acc>(p.beta);
+  Acc y_old = 0;
 
   if (col < p.n && k0 < p.k) {
     // All of the lane's loads are requested before anything is consumed.
@@ -170,6 +235,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
       else
         rows[r] = make_uint4(0, 0, 0, 0);
     }
+    if (owner && y_is_read) y_old = yv[(tile_col0 + threadIdx.x) * p.y_s];
     if constexpr (MODE == kI8RowMajor || MODE == kI8K4) {
       // x as packed bytes, four k per dword; k at or beyond K contributes zero.
       constexpr int kWords = kKPerLaneL / 4;
@@ -260,24 +326,32 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
         }
       }
     }
+  } else if (owner && y_is_read) {
+    y_old = yv[(tile_col0 + threadIdx.x) * p.y_s];
   }
-  // The workgroup's partial sums meet in LDS.
+  // The eight row groups of a wave are summed in registers (every lane takes part); the first hands the wave's
+  // sums to LDS, where the eight waves meet.
 #pragma unroll
-  for (int j = 0; j < kCols; ++j) red[part][cl * kCols + j] = acc[j];
+  for (int j = 0; j < kCols; ++j) acc[j] = sum_over_row_groups(acc[j]);
+  if (rl == 0) {
+#pragma unroll
+    for (int j = 0; j < kCols; ++j) red[wave][cl * kCols + j] = acc[j];
+  }
   __syncthreads();
-  const size_t tile_col0 = (size_t)tile * Md::kTileCols;
-  const bool owner = threadIdx.x < Md::kTileCols && tile_col0 + threadIdx.x < p.n;
   Acc sum = 0;
   if (owner) {
+    sum = red[0][threadIdx.x];
 #pragma unroll
-    for (int w = 0; w < kPartials; ++w) sum += red[w][threadIdx.x];
+    for (int w = 1; w < kWaves; ++w) sum += red[w][threadIdx.x];
   }
-  Acc *yv = reinterpret_cast<Acc *>(p.y);
+  // `total` is complete: the alpha/beta step with the old value that was asked for at the start (the initialising
+  // mode reads it only now, and only where alpha * total is a zero).
+  auto finish = [&](Acc total) {
+    Acc *y = yv + (tile_col0 + threadIdx.x) * p.y_s;
+    *y = y_is_read ? skl_combine(total, y_old, p.alpha, p.beta) : skl_initialise(total, y, p.alpha, p.beta);
+  };
   if (p.slabs == 1) {  // the strip is complete inside this workgroup
-    if (owner) {
-      Acc *y = yv + (tile_col0 + threadIdx.x) * p.y_s;
-      skl_update(sum, y, p.alpha, p.beta);
-    }
+    if (owner) finish(sum);
     return;
   }
   if constexpr (std::is_same<Acc, int>::value) {
@@ -291,27 +365,14 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
       const unsigned long long now = atomicAdd(slot, mine) + mine;
       if ((unsigned)now == p.slabs) {
         __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
-        Acc *y = yv + j * p.y_s;
-        skl_update((int)(unsigned)(now >> 32), y, p.alpha, p.beta);
+        finish((int)(unsigned)(now >> 32));
       }
     }
   } else {
-    Acc *scratch = reinterpret_cast<Acc *>(p.acc);
-    if (owner) atomicAdd(&scratch[tile_col0 + threadIdx.x], sum);
-    // Wait until this wave's atomics have been performed, then take a ticket.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    if (threadIdx.x == 0) ticket_s = atomicAdd(&p.tickets[tile], 1u);
-    __syncthreads();
-    if (ticket_s != p.slabs - 1) return;
-    if (owner) {
-      const size_t j = tile_col0 + threadIdx.x;
-      const Acc total = atomicExch(&scratch[j], (Acc)0);  // read the total and leave zero behind
-      Acc *y = yv + j * p.y_s;
-      skl_update(total, y, p.alpha, p.beta);
-    }
-    if (threadIdx.x == 0) atomicExch(&p.tickets[tile], 0u);
+    float total = 0.0f;
+    if (ordered_sum_over_slabs(p.planes, p.n, tile_col0 + threadIdx.x, slab, p.slabs, &p.tickets[tile], &ticket_s,
+                               owner, sum, total) && owner)
+      finish(total);
   }
 }
 
@@ -338,26 +399,11 @@ struct GemvRowsArgs {
   size_t y_row, y_s;
   size_t n, k;
   skl_scalar alpha, beta;
-  void *acc;       // MR * n 64-bit slots (floating point: fp32 values in the same region), zero between calls
-  unsigned *tickets;
+  void *acc;       // int8: MR * n 64-bit slots, zero between calls
+  unsigned *tickets;  // floating point: one counter per strip, zero between calls ...
+  float *planes;      // ... and `slabs` planes of MR * n sums (the stream's workspace)
   unsigned tiles, slabs;
 };
-
-// Sum over the eight lanes of a row of 16 that share a column group (same lane parity), in every lane:
-// three DPP rotations inside the row, no LDS crossbar.
-__device__ __forceinline__ int sum_over_row_groups(int v) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0x128 /* row_ror:8 */, 0xF, 0xF, false);
-  v += __builtin_amdgcn_update_dpp(0, v, 0x124 /* row_ror:4 */, 0xF, 0xF, false);
-  v += __builtin_amdgcn_update_dpp(0, v, 0x122 /* row_ror:2 */, 0xF, 0xF, false);
-  return v;
-}
-
-__device__ __forceinline__ float sum_over_row_groups(float v) {
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, false));
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, false));
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xF, 0xF, false));
-  return v;
-}
 
 constexpr int kRowChunk = 4;  // rows of A multiplied per pass over the loaded bytes of B: 64 sums per lane
 
@@ -543,28 +589,15 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
       }
     }
   } else {
-    // fp32 sums between workgroups, then a ticket per strip, as in the M = 1 kernel
-    float *scratch = reinterpret_cast<float *>(p.acc);
-#pragma unroll
-    for (int q = 0; q < kPasses; ++q) {
-      const int i = row0 + kRowStep * q;
-      if (valid && i < MR) atomicAdd(&scratch[(size_t)i * p.n + j], sum[q]);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    if (threadIdx.x == 0) ticket_s = atomicAdd(&p.tickets[tile], 1u);
-    __syncthreads();
-    if (ticket_s != p.slabs - 1) return;
-#pragma unroll
-    for (int q = 0; q < kPasses; ++q) {
-      const int i = row0 + kRowStep * q;
-      if (valid && i < MR) {
-        const float total = atomicExch(&scratch[(size_t)i * p.n + j], 0.0f);  // read the total and leave zero behind
-        skl_update(total, yv + (size_t)i * p.y_row + j * p.y_s, p.alpha, p.beta);
-      }
-    }
-    if (threadIdx.x == 0) atomicExch(&p.tickets[tile], 0u);
+    // one plane of sums per workgroup of the strip, added in slab order by the one that finishes last, as in the
+    // M = 1 kernel (at most three rows of A here: one element per thread)
+    static_assert(kPasses == 1 || kInt, "the floating-point kinds take at most kRowStep rows");
+    const int i = row0;
+    const bool mine = valid && i < MR;
+    float total = 0.0f;
+    if (ordered_sum_over_slabs(p.planes, (size_t)MR * p.n, (size_t)i * p.n + j, slab, p.slabs, &p.tickets[tile], &ticket_s,
+                               mine, sum[0], total) && mine)
+      skl_update(total, yv + (size_t)i * p.y_row + j * p.y_s, p.alpha, p.beta);
   }
 }
 
@@ -756,21 +789,17 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
         acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, xa[it]), __builtin_bit_cast(v8h, bw),
                                                         acc[c], 0, 0, 0);
       } else {
-        // 8 bytes of K per lane and instruction: the lane's 16 k in two halves, A's bytes split the same way
-        const long a_lo = (long)(((unsigned long long)(unsigned)xa[it].y << 32) | (unsigned)xa[it].x);
-        const long a_hi = (long)(((unsigned long long)(unsigned)xa[it].w << 32) | (unsigned)xa[it].z);
-        const long b_lo = (long)(((unsigned long long)t[1][c] << 32) | t[0][c]);
-        const long b_hi = (long)(((unsigned long long)t[3][c] << 32) | t[2][c]);
-        if constexpr (MODE == kF8E4M3) {
-          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a_lo, b_lo, acc[c], 0, 0, 0);
-          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a_hi, b_hi, acc[c], 0, 0, 0);
-        } else if constexpr (MODE == kF8E5M2) {
-          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(a_lo, b_lo, acc[c], 0, 0, 0);
-          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(a_hi, b_hi, acc[c], 0, 0, 0);
-        } else {  // E4M3 A, E5M2 B
-          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(a_lo, b_lo, acc[c], 0, 0, 0);
-          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_bf8(a_hi, b_hi, acc[c], 0, 0, 0);
-        }
+        // OCP fp8: both operands are widened to f16 in registers - every E4M3 and E5M2 value is an f16 value - and
+        // multiplied by the f16 instruction: exact products, fp32 sums, so the reference's own error bound holds.
+        // (The fp8 instructions align the products of one instruction to a common exponent and drop what falls
+        // about 12 bits below the largest: more than that bound allows when K is small. The conversions cost one
+        // VALU operation per two bytes, which this kernel has to spare.) 8 k per lane and instruction: the lane's
+        // 16 k in two halves, A's bytes split the same way.
+        constexpr bool a_e5m2 = MODE == kF8E5M2, b_e5m2 = MODE != kF8E4M3;
+        acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(skl_fp8::widen8_to_f16<a_e5m2>((unsigned)xa[it].x, (unsigned)xa[it].y),
+                                                        skl_fp8::widen8_to_f16<b_e5m2>(t[0][c], t[1][c]), acc[c], 0, 0, 0);
+        acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(skl_fp8::widen8_to_f16<a_e5m2>((unsigned)xa[it].z, (unsigned)xa[it].w),
+                                                        skl_fp8::widen8_to_f16<b_e5m2>(t[2][c], t[3][c]), acc[c], 0, 0, 0);
       }
     }
   }
@@ -989,6 +1018,10 @@ int launch(const skl_gemm_canon *g, const Reduction &red) {
     skl_hip_record_error(-2, "gemv: grid too large");
     return -2;
   }
+  p.planes = nullptr;
+  if constexpr (!std::is_same<typename Md::Acc, int>::value) {
+    if (p.slabs > 1 && !(p.planes = (float *)skl_workspace((size_t)p.slabs * p.n * sizeof(float)))) return -4;
+  }
   if (loads == 16)
     gemv_kernel<MODE, 16><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
   else
@@ -1021,6 +1054,10 @@ int launch_rows(const skl_gemm_canon *g, const Reduction &red) {
   if (grid > 0x7FFFFFFFu) {
     skl_hip_record_error(-2, "gemv: grid too large");
     return -2;
+  }
+  p.planes = nullptr;
+  if constexpr (MODE != kI8RowMajor) {
+    if (p.slabs > 1 && !(p.planes = (float *)skl_workspace((size_t)p.slabs * MR * p.n * sizeof(float)))) return -4;
   }
   gemv_rows_kernel<MR, MODE><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
   return skl_check_launch("gemv_rows");

@@ -30,10 +30,17 @@ enum {
   SKL_DT_F16H = 7 /* f16 operands with an f16 accumulator and an f16 C; any-stride kernel only */
 };
 
+/* alpha or beta in C's type. With a float in `f`, `skip_c_read` shares the 8 bytes: set on beta (by the host
+ * layer, unless skl_hip_set_beta_zero_mode asked for the reference's evaluation) it lets a kernel leave C unread
+ * when beta is zero. */
 typedef union {
   int32_t i;
   float f;
   double d;
+  struct {
+    float value;
+    uint32_t skip_c_read;
+  } fz;
 } skl_scalar;
 
 /* The fully general blocked GEMM of the reference (the `rcprc` form): element

@@ -50,6 +50,7 @@ DeviceState g_devices[kMaxDevices];
 
 thread_local hipStream_t t_stream = nullptr;
 thread_local int t_pointer_mode = SKL_HIP_POINTERS_AUTO;
+thread_local int t_beta_zero_mode = SKL_HIP_BETA_ZERO_INITIALISES;
 thread_local int t_error = SKL_HIP_OK;
 thread_local char t_error_text[256] = "no error";
 
@@ -244,6 +245,11 @@ void skl_hip_set_pointer_mode(int mode) {
   t_pointer_mode = (mode == SKL_HIP_POINTERS_DEVICE) ? SKL_HIP_POINTERS_DEVICE : SKL_HIP_POINTERS_AUTO;
 }
 int skl_hip_get_pointer_mode(void) { return t_pointer_mode; }
+
+void skl_hip_set_beta_zero_mode(int mode) {
+  t_beta_zero_mode = (mode == SKL_HIP_BETA_ZERO_AS_REFERENCE) ? SKL_HIP_BETA_ZERO_AS_REFERENCE : SKL_HIP_BETA_ZERO_INITIALISES;
+}
+int skl_hip_get_beta_zero_mode(void) { return t_beta_zero_mode; }
 
 int skl_hip_pointer_is_device(const void *ptr) {
   if (t_pointer_mode == SKL_HIP_POINTERS_DEVICE) return 1;

@@ -188,6 +188,8 @@ RUNTIME = {
     "skl_hip_synchronize": (ctypes.c_int, ""),
     "skl_hip_set_pointer_mode": (None, "i"),
     "skl_hip_get_pointer_mode": (ctypes.c_int, ""),
+    "skl_hip_set_beta_zero_mode": (None, "i"),
+    "skl_hip_get_beta_zero_mode": (ctypes.c_int, ""),
     "skl_hip_pointer_is_device": (ctypes.c_int, "p"),
     "skl_hip_last_error": (ctypes.c_int, ""),
     "skl_hip_last_error_string": (ctypes.c_char_p, ""),
@@ -197,6 +199,8 @@ RUNTIME = {
     "skl_hip_event_record": (ctypes.c_int, "p"),
     "skl_hip_event_elapsed_ms": (ctypes.c_float, "pp"),
     "skl_hip_device_info": (ctypes.c_int, "pzpp"),
+    "skl_hip_probe_hbm_read": (ctypes.c_int, "pz"),
+    "skl_hip_probe_mfma": (ctypes.c_double, "iii"),
 }
 
 

@@ -310,15 +310,12 @@ def case_args(case, a, b, c):
     return case.rcprc_args(a, b, c)
 
 
-#: The fp8 matrix-core instructions of gfx950 align the products of one
-#: instruction to a common exponent before adding them and keep about 12 bits
-#: below the largest term (measured: error <= 2^-11.9 * sum|a||b| for both
-#: v_mfma_f32_32x32x64_f8f6f4 and v_mfma_f32_32x32x16_fp8_fp8, already at K = 2).
-#: The reference's fp32-accumulation bound is therefore widened by this term
-#: (with a factor two of margin for several instructions adding into one
-#: accumulator) for fp8 inputs on the GPU; the relative Frobenius bound 1e-3 is
-#: unchanged.
-FP8_MFMA_REL = 2.0 ** -10
+#: Allowance on top of the reference's elementwise bound for fp8 operands: none. Up to K = 2304 the fp8 kinds are
+#: multiplied exactly (bytes widened to f16, f16 matrix-core instructions, fp32 sums - the arithmetic the bound
+#: assumes); beyond that the fp8 instructions are used, whose error (products of one instruction aligned to a
+#: common exponent, about 12 bits kept below the largest: <= 2^-11.9 * sum|a||b|) is inside the bound
+#: 2((1 + 2^-24)^(K+2) - 1) * sum|a||b| from K = 2193 on.
+FP8_MFMA_REL = 0.0
 
 
 def assert_fp_gemm_close(case, a, b, c_before, c_after, frob_tol=1e-3, extra_rel=0.0):

@@ -137,42 +137,137 @@ def test_f32_f64_bit_identical_to_the_checker(gpu):
                 assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (ta, mode)
 
 
-@pytest.mark.parametrize("ta,m,n,k", (("bf16", 130, 200, 64), ("f8e4m3", 256, 256, 128), ("f16", 512, 2048 + 128, 256),
-                                       ("f32", 33, 47, 17), ("f64", 20, 31, 9), ("f16h", 21, 30, 19),
-                                       ("bf16", 1, 4096, 512)))
-def test_beta_zero_initialises_c(gpu, ta, m, n, k):
-    """beta == 0 is the initialising call. The old C then contributes nothing but the sign of an exact
-    zero (beta*c is a signed zero, and it only shows when alpha*acc is a zero too), so the result must
-    equal the checker's bit for bit wherever it is a zero - rows of A are zeroed to make such elements,
-    C holds both signs - and an Inf or NaN in C must be overwritten exactly as a finite value is."""
+BETA_ZERO_SHAPES = (
+    # ta, m, n, k, what serves it
+    ("bf16", 130, 200, 64, "64 x 64 bounds-checked tiles"),
+    ("f8e4m3", 256, 256, 128, "bounds-checked tiles"),
+    ("f16", 512, 2048 + 128, 256, "streaming kernel"),
+    ("bf16", 128, 256, 4096, "bounds-checked tiles with K shared between workgroups"),
+    ("bf16", 256, 8192, 4096, "streaming kernel with K shared between two workgroups (too long for the checker)"),
+    ("f32", 33, 47, 17, "any-stride kernel"),
+    ("f32", 256, 192, 64, "register-tiled kernel"),
+    ("f64", 20, 31, 9, "any-stride kernel"),
+    ("f16h", 21, 30, 19, "any-stride kernel"),
+    ("bf16", 1, 4096, 512, "M = 1, one workgroup per strip"),
+    ("bf16", 1, 4096, 2048, "M = 1, four workgroups per strip"),
+    ("f8e4m3", 1, 2048, 4096, "M = 1, fp8"),
+    ("f16", 2, 1024, 2048, "two rows, fp32 multiply-adds"),
+    ("f8e4m3", 4, 2048, 2048, "four rows on the matrix cores (second pass adds the planes)"),
+)
+
+
+def _spoil(c, m, n, rows):
+    """Inf and NaN planted in rows `rows` of a row-major m x n C."""
+    spoiled = c.copy()
+    if len(rows):
+        view = spoiled.reshape(m, n)
+        view[rows[::3], ::5] = np.nan
+        view[rows[1::3], 1::7] = np.inf
+        view[rows[2::3], 2::11] = -np.inf
+    return spoiled
+
+
+@pytest.mark.parametrize("ta,m,n,k,what", BETA_ZERO_SHAPES)
+def test_beta_zero_as_the_reference_evaluates_it(gpu, ta, m, n, k, what):
+    """skl_hip_set_beta_zero_mode(SKL_HIP_BETA_ZERO_AS_REFERENCE): beta == 0 still evaluates beta*C + alpha*acc
+    (ref/gemm/gemm_bf16rc_bf16rc_f32rc.c:21). An Inf or NaN in C gives NaN exactly where the checker gives NaN, every
+    other element has the bits of the same call on a clean C (which the table tests check against the bound), and
+    where alpha*acc is an exact zero - rows of A are zeroed to make such elements, C holds both signs - the sign of
+    the result is the checker's."""
+    gpu.skl_hip_set_beta_zero_mode(1)
+    try:
+        assert gpu.skl_hip_get_beta_zero_mode() == 1
+        _beta_zero_as_reference(gpu, ta, m, n, k)
+    finally:
+        gpu.skl_hip_set_beta_zero_mode(0)
+
+
+def _beta_zero_as_reference(gpu, ta, m, n, k):
     rng = np.random.default_rng(77)
     for alpha, beta in ((-1.5, 0.0), (2.0, -0.0)):
         case = rowmajor_case(ta, m, n, k, alpha, beta)
         a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
-        zero_rows = sorted(set((0, m // 2, m - 1)))
+        zero_rows = sorted(set((0, m // 2, m - 1))) if m > 2 else []
         for i in zero_rows:
             a[i * k:(i + 1) * k] = 0
-        want = run_oracle_gemm(case, a, b, c)
-        spoiled = c.copy()
         live = np.ones(m, dtype=bool)
         live[zero_rows] = False
-        rows = np.flatnonzero(live)
-        if rows.size:
-            view = spoiled.reshape(m, n)
-            view[rows[::3], ::5] = np.nan
-            view[rows[1::3], 1::7] = np.inf
-            view[rows[2::3], 2::11] = -np.inf
+        spoiled = _spoil(c, m, n, np.flatnonzero(live))
+        nan_want = ~np.isfinite(spoiled.astype(np.float64))  # 0 * Inf and 0 * NaN are NaN, and NaN + x is NaN
+        assert nan_want.sum() > 0
+        checker = m * n * k <= 1 << 30  # the checker's scalar loop takes seconds beyond that
+        if checker:
+            want = run_oracle_gemm(case, a, b, c)
+            assert np.array_equal(np.isnan(run_oracle_gemm(case, a, b, spoiled).astype(np.float64)), nan_want)
         for mode in MODES:
             got = run_gemm(gpu, "rc", case, a, b, c, mode)
             again = run_gemm(gpu, "rc", case, a, b, spoiled, mode)
-            for i in zero_rows:
+            for i in zero_rows if checker else ():
                 row = slice(i * n, (i + 1) * n)
                 assert np.array_equal(got[row].view(np.uint8), want[row].view(np.uint8)), (ta, mode, alpha, i)
-            assert np.all(np.isfinite(again)), (ta, mode, alpha)
-            if m > 1:  # the M = 1 path sums with floating-point atomics: not the same bits from run to run
-                assert np.array_equal(got.view(np.uint8), again.view(np.uint8)), (ta, mode, alpha)
+            nan_got = np.isnan(again.astype(np.float64))
+            assert np.array_equal(nan_got, nan_want), (ta, mode, alpha, int(nan_got.sum()), int(nan_want.sum()))
+            assert np.array_equal(got[~nan_want].view(np.uint8), again[~nan_want].view(np.uint8)), (ta, mode, alpha)
             if ta in ("f32", "f64", "f16h"):
                 assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (ta, mode, alpha)
+                assert np.array_equal(again[~nan_want].view(np.uint8), want[~nan_want].view(np.uint8)), (ta, mode, alpha)
+
+
+@pytest.mark.parametrize("ta,m,n,k,what", BETA_ZERO_SHAPES)
+def test_beta_zero_initialises_c(gpu, ta, m, n, k, what):
+    """The default: beta == 0 is the initialising call (src/gemm/README.md:43). The old C contributes nothing but the
+    sign of an exact zero, so an Inf or NaN in C is overwritten exactly as a finite value is, and every result has
+    the bits of the reference-evaluation mode's result on a clean C. (f64: C is always read.)"""
+    if ta == "f64":
+        pytest.skip("f64 GEMMs always read C")
+    rng = np.random.default_rng(78)
+    case = rowmajor_case(ta, m, n, k, -1.5, 0.0)
+    a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+    zero_rows = sorted(set((0, m // 2, m - 1))) if m > 2 else []
+    for i in zero_rows:
+        a[i * k:(i + 1) * k] = 0
+    live = np.ones(m, dtype=bool)
+    live[zero_rows] = False
+    spoiled = _spoil(c, m, n, np.flatnonzero(live))
+    assert gpu.skl_hip_get_beta_zero_mode() == 0
+    for mode in MODES:
+        gpu.skl_hip_set_beta_zero_mode(1)
+        try:
+            reference_mode = run_gemm(gpu, "rc", case, a, b, c, mode)
+        finally:
+            gpu.skl_hip_set_beta_zero_mode(0)
+        got = run_gemm(gpu, "rc", case, a, b, c, mode)
+        again = run_gemm(gpu, "rc", case, a, b, spoiled, mode)
+        assert np.all(np.isfinite(again.astype(np.float64))), (ta, mode)
+        assert np.array_equal(got.view(np.uint8), again.view(np.uint8)), (ta, mode)
+        assert np.array_equal(got.view(np.uint8), reference_mode.view(np.uint8)), (ta, mode)
+
+
+@pytest.mark.parametrize("ta,tb", (("f8e4m3", "f8e4m3"), ("f8e5m2", "f8e5m2"), ("f8e4m3", "f8e5m2")))
+@pytest.mark.parametrize("a_rowmajor", (True, False))
+def test_fp8_short_k_is_multiplied_exactly(gpu, ta, tb, a_rowmajor):
+    """Up to K = 2304 the fp8 kinds run with the bytes widened to f16 and exact products. One-hot rows of A (1.0 at
+    position p_i): row i of C is row p_i of B as the format defines it, every finite code, subnormal ones included,
+    whichever lane, k-step half and instruction of the pair its k falls into. Then random operands: the
+    reference's elementwise bound with nothing added, at a K where the fp8 instructions would exceed it."""
+    m, n, k = 96, 256, 160
+    one = 0x38 if ta == "f8e4m3" else 0x3C
+    table = support.decode_table(tb)
+    finite_codes = np.flatnonzero(np.isfinite(table)).astype(np.uint8)  # 0 * Inf would spoil whole columns
+    b = finite_codes[(np.arange(k * n) * 7 + np.arange(k * n) // n) % finite_codes.size].astype(np.uint8)
+    assert set(b.tolist()) == set(finite_codes.tolist())
+    a = np.zeros(m * k, np.uint8)
+    pos = [(i * 37 + 5) % k for i in range(m)]
+    for i in range(m):
+        a[(i * k + pos[i]) if a_rowmajor else (pos[i] * m + i)] = one
+    case = (rowmajor_case if a_rowmajor else colmajor_a_case)(ta, m, n, k, 1.0, 0.0, tb=tb)
+    got = run_gemm(gpu, "rc", case, a, b, np.zeros(m * n, np.float32), "device").reshape(m, n)
+    for i in range(m):
+        assert np.array_equal(got[i].astype(np.float64), table[b[pos[i] * n:(pos[i] + 1) * n]]), (ta, tb, i)
+    for (mm, nn, kk) in ((200, 300, 64), (384, 512, 2304)):
+        case = (rowmajor_case if a_rowmajor else colmajor_a_case)(ta, mm, nn, kk, 1.5, -0.5, tb=tb)
+        a, b, c = case.make_inputs(mm + kk)
+        support.assert_fp_gemm_close(case, a, b, c, run_gemm(gpu, "rc", case, a, b, c, "device"))
 
 
 FUSED_SHAPES = (
