@@ -167,6 +167,17 @@ SKL_GFX950_DECLARE_FUSED_RCPRC(skl_gemm_fused_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_g
  * src/gemm/gemm_i8_i8_i32_zve32x.h:50, src/gemm/gemm_i8_i8_i32_zve32x_x390.h:50 */
 void skl_gemm_i8_i8_i32_gfx950(size_t m, size_t n, size_t k, int32_t alpha, const int8_t *a, size_t rsa,
                                const int8_t *b, size_t rsb, int32_t beta, int32_t *c, size_t rsc);
+/* skl_gemm_i8_i8_i32_gfx950 for callers that cannot allocate device memory: code under HIP graph capture, serving
+ * loops and harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments and the same
+ * result, bit for bit, but only for decode calls - 1 <= m <= 8, all pointers device-accessible (they are not
+ * queried), k > 0, n a multiple of 16, b and rsb multiples of 16 bytes, a 4-byte aligned with rsa a multiple of 4
+ * when m > 1 - and only while m * n <= 65536: the sums that workgroups share live in a static 512 KiB array on
+ * each GPU instead of a block the library allocates. Anything else records SKL_HIP_ERR_BAD_ARGUMENT and does
+ * nothing. The call itself allocates, frees and queries nothing (skl_hip_init on the device beforehand also
+ * keeps the one address lookup out of it). All such calls on one GPU share that array: calls that overlap on the
+ * device - different streams, or the branches of one graph - race. */
+void skl_gemm_i8_i8_i32_noalloc_gfx950(size_t m, size_t n, size_t k, int32_t alpha, const int8_t *a, size_t rsa,
+                                       const int8_t *b, size_t rsb, int32_t beta, int32_t *c, size_t rsc);
 /* src/gemm/gemm_bf16_bf16_f32_zvfbfwma.h:49, src/gemm/gemm_bf16_bf16_f32_zvfbfwma_x390.h:49 */
 void skl_gemm_bf16_bf16_f32_gfx950(size_t m, size_t n, size_t k, float alpha, const skl_bf16_t *a,
                                    size_t rsa, const skl_bf16_t *b, size_t rsb, float beta, float *c,

@@ -576,6 +576,21 @@ DEFINE_GEMM_ROWMAJOR(skl_gemm_f32_f32_f32_gfx950, skl_gemm_f32rc_f32rc_f32rc_gfx
 DEFINE_GEMM_ROWMAJOR(skl_gemm_f64_f64_f64_gfx950, skl_gemm_f64rc_f64rc_f64rc_gfx950, double, double)
 DEFINE_GEMM_ROWMAJOR(skl_gemm_f16_f16_f16_gfx950, skl_gemm_f16rc_f16rc_f16rc_gfx950, skl_f16_t, skl_f16_t)
 
+/* The row-major int8 GEMM for callers that cannot allocate: decode shapes only, device pointers only, nothing
+ * allocated, queried or freed on the way (see include/skl-gfx950.h). */
+void skl_gemm_i8_i8_i32_noalloc_gfx950(size_t m, size_t n, size_t k, int32_t alpha, const int8_t *a, size_t rsa,
+                                       const int8_t *b, size_t rsb, int32_t beta, int32_t *c, size_t rsc) {
+  skl_gemm_desc d = {SKL_DT_I8, SKL_DT_I8, 1, 1, 1, m, n, k, a, 0, 0, rsa, 1, b, 0, 0, rsb, 1,
+                     c, 0, 0, rsc, 1, {.i = alpha}, {.i = beta}, NULL, NULL};
+  skl_gemm_canon g;
+  if (m == 0 || n == 0) return;
+  if (!canonicalize(&d, &g)) {
+    skl_hip_record_error(SKL_HIP_ERR_BAD_ARGUMENT, __func__);
+    return;
+  }
+  skl_hip_launch_gemv_noalloc(&g);
+}
+
 /* column-major A: the rc form with rsa = 1
  * (src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:38-48) */
 #define DEFINE_GEMM_COLMAJOR_A(NAME, RC, TA_T, TC_T)                                               \

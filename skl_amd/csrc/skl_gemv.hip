@@ -46,8 +46,17 @@
 
 #include <type_traits>
 
+#include <mutex>
+
 #include "skl_device.hpp"
 #include "skl_fp8.hpp"
+
+// Scratch of the entry point that allocates nothing (skl_gemm_i8_i8_i32_noalloc_gfx950, at the end of this file):
+// the 64-bit sum + count slots of the int8 kernels in a static array of a fixed size instead of the block the
+// library allocates per stream. Each GPU the library runs on holds its own copy until the process ends. The
+// array is zero when the module is loaded, and every kernel puts the slots it used back to zero.
+constexpr size_t kNoAllocSlots = size_t(1) << 16;  // 512 KiB
+static __device__ __align__(256) unsigned long long scratch[kNoAllocSlots];
 
 namespace {
 
@@ -1350,4 +1359,54 @@ extern "C" int skl_hip_launch_gemv_kc(const skl_gemm_canon *g) {
     case kF8E5M2: return launch_kc_of<kF8E5M2>(g);
     default: return launch_kc_of<kF8Mixed>(g);
   }
+}
+
+// ---------------------------------------------------------------------------
+// The entry point that allocates nothing: int8 decode calls (1 to 8 rows of A against a row-major B) on the same
+// kernels as skl_hip_launch_gemv / skl_hip_launch_gemv_rows, with the static array at the top of this file as the
+// slots. The array's name is only a handle on the host; its address on a device comes from hipGetSymbolAddress,
+// asked once per device (skl_hip_init does it, else the first call here) and kept.
+// ---------------------------------------------------------------------------
+namespace {
+constexpr int kNoAllocMaxDevices = 16;
+unsigned long long *g_noalloc_slots[kNoAllocMaxDevices];  // per device: where `scratch` lives there
+std::mutex g_noalloc_mutex;
+
+unsigned long long *noalloc_slots_of_current_device() {
+  int dev = 0;
+  if (skl_check_hip(hipGetDevice(&dev), "hipGetDevice") != 0) return nullptr;
+  if (dev < 0 || dev >= kNoAllocMaxDevices) {
+    skl_hip_record_error(-2, "noalloc: device index beyond 15");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+  if (!g_noalloc_slots[dev]) {
+    void *ptr = nullptr;
+    if (skl_check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "noalloc: address of the static scratch") != 0)
+      return nullptr;
+    g_noalloc_slots[dev] = static_cast<unsigned long long *>(ptr);
+  }
+  return g_noalloc_slots[dev];
+}
+}  // namespace
+
+extern "C" int skl_hip_noalloc_setup(void) { return noalloc_slots_of_current_device() ? 0 : -2; }
+
+extern "C" size_t skl_hip_noalloc_max_sums(void) { return kNoAllocSlots; }
+
+extern "C" int skl_hip_launch_gemv_noalloc(const skl_gemm_canon *g) {
+  if (g->ta != SKL_DT_I8 || g->tb != SKL_DT_I8 || g->m < 1 || g->m > (size_t)kMaxRows ||
+      (g->m == 1 ? !skl_hip_gemv_supported(g, 0) : !skl_hip_gemv_rows_supported(g))) {
+    skl_hip_record_error(-2, "noalloc: not an int8 decode call (1 to 8 rows of A contiguous in K, row-major B with "
+                             "16-byte aligned rows, N a multiple of 16, K > 0)");
+    return -2;
+  }
+  if (g->m * g->n > kNoAllocSlots) {
+    skl_hip_record_error(-2, "noalloc: M * N exceeds the 65536 sums of the static scratch");
+    return -2;
+  }
+  Reduction red;
+  red.acc = noalloc_slots_of_current_device();
+  if (!red.acc) return -2;
+  return g->m == 1 ? launch<kI8RowMajor>(g, red) : launch_rows_of<kI8RowMajor>(g, red);
 }

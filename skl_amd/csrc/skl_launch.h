@@ -118,6 +118,13 @@ int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g, int layout);
 int skl_hip_gemv_kc_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
 
+/* int8 decode calls (1 <= M <= 8, row-major B) on the M == 1 / few-rows kernels with a static device array as the
+ * shared sums: no allocation, at most skl_hip_noalloc_max_sums() elements of C. skl_hip_noalloc_setup() looks the
+ * array's address on the current device up (once per device; the launch does it itself where it was not called). */
+int skl_hip_noalloc_setup(void);
+size_t skl_hip_noalloc_max_sums(void);
+int skl_hip_launch_gemv_noalloc(const skl_gemm_canon *g);
+
 /* A block of scratch memory of the current stream and device for operands copied into another layout ahead of a
  * launch (grows on demand, NULL when the device has no room; apart from the workspace of the split reductions). */
 void *skl_hip_operand_scratch(size_t bytes);

@@ -163,6 +163,8 @@ int skl_hip_init(int device) {
   }
   int rc = skl_check_hip(hipSetDevice(device), "hipSetDevice");
   if (rc != 0) return rc;
+  rc = skl_hip_noalloc_setup();  // the static scratch of the entry point that allocates nothing, on this device
+  if (rc != 0) return rc;
   return skl_workspace(1) ? SKL_HIP_OK : SKL_HIP_ERR_WORKSPACE;
 }
 
