@@ -127,17 +127,39 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, 
  * src/gemm/README.md:141-146 tells users to approximate by tiling the output. The reference keeps its
  * fused kernels private (SKL_FUNC_PRIVATE), so these entry points have no public prototype to mirror;
  * they take the argument list of the rc / rcprc form plus the descriptor.
- * For every addressed element (i, j), j the logical column:
+ * For every addressed element (i, j), (i, j) the logical row and column:
  *     v = beta*C(i,j) + alpha*(A*B)(i,j)        as in the plain GEMM, beta == 0 included
  *     v = v + bias[j]                            if bias != NULL (one rounded addition; int32 wraps)
- *     C(i,j) = v
+ *     v = v > 0 ? v : 0                          if activation == SKL_GFX950_ACT_RELU (a NaN becomes 0)
+ *     C(i,j) = v                                 unless q_only
+ *     Q(i,j) = clamp(rne((float)v * s_j) + q_zero, -128, 127)      if q != NULL: the requantised int8 copy,
+ *                                                at q[i*rsq + j*csq]; s_j = q_scale[j] with q_scale_per_column, else
+ *                                                q_scale[0]; (float)v rounds an int32 to nearest even, the product is
+ *                                                one fp32 multiplication, rne() rounds it to the nearest integer, ties
+ *                                                to even (a NaN counts as 0, values beyond int32 as its ends)
  *     *max = v  if v > *max                      if max != NULL (a NaN never replaces the maximum;
  *                                                the sign of a zero maximum is unspecified)
- * bias points to n = n1*n0 values of C's type, max to one; both must be memory of the same kind as C
- * (device or host), must not overlap C, and *max must not be NaN on entry. ep == NULL: the plain GEMM. */
+ * Bias and maximum are the steps of the reference's fused kernels; activation and requantisation are what
+ * src/gemm/README.md:46-47 names as the operations callers would fuse next ("requantization and activation
+ * functions") and leaves to them - the reference has no routine for either, the rules above define them here.
+ * bias points to n = n1*n0 values of C's type, max to one, q_scale to n floats or one; all of them and q must be
+ * memory of the same kind as C (device or host) and must not overlap C or each other; *max must not be NaN on
+ * entry; q_zero lies in [-128, 127]. With q_only the call still reads C when beta asks for it. Members left zero
+ * (e.g. by a designated initialiser that names only bias and max) switch their step off. ep == NULL: the plain GEMM. */
+#define SKL_GFX950_ACT_NONE 0
+#define SKL_GFX950_ACT_RELU 1
+/* Every step off: `skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE; ep.bias = ...;` is valid C and C++. */
+#define SKL_GFX950_EPILOGUE_NONE {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 typedef struct skl_gfx950_epilogue {
   const void *bias;
   void *max;
+  int activation;
+  int q_scale_per_column;
+  int q_only;
+  int32_t q_zero;
+  int8_t *q;
+  size_t rsq, csq;
+  const float *q_scale;
 } skl_gfx950_epilogue_t;
 
 #define SKL_GFX950_DECLARE_FUSED_RC(NAME, TA, TC)                                                    \

@@ -461,6 +461,36 @@ FUSED_RCPRC(f16rcprc_f16rcprc_f32rcprc, uint16_t, float)
 FUSED_RCPRC(f8e4m3rcprc_f8e4m3rcprc_f32rcprc, uint8_t, float)
 FUSED_RCPRC(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, float)
 
+/*
+ * The two steps src/gemm/README.md:46-47 names as what callers fuse behind a GEMM ("requantization and activation
+ * functions") and for which the reference has no routine: the rules are the ones include/skl-gfx950.h states for
+ * skl_gfx950_epilogue_t, restated here over a C that already holds the alpha/beta (and bias) result. They sit
+ * between the bias and the maximum, so a test composes: plain GEMM, bias, these, maximum.
+ *   activation 1:  v = v > 0 ? v : 0     (a NaN becomes 0), written back to C
+ *   q != NULL:     Q(i,j) = clamp(rne((float)v * s_j) + zero, -128, 127), one fp32 product, rne to the nearest
+ *                  integer with ties to even; a NaN counts as 0, values beyond int32 as its ends
+ */
+static int8_t requantised(float v, float scale, int32_t zero) {
+  const float r = nearbyintf(v * scale); /* the default rounding mode: to nearest, ties to even */
+  int64_t t = isnan(r) ? 0 : r >= 2147483648.0f ? INT32_MAX : r <= -2147483648.0f ? INT32_MIN : (int64_t)r;
+  t += zero;
+  return (int8_t)(t < -128 ? -128 : t > 127 ? 127 : t);
+}
+#define ACT_REQUANT(SUFFIX, TC)                                                                     \
+  void skl_oracle_act_requant_##SUFFIX(size_t m, size_t n, TC *c, size_t rsc, size_t csc, int activation, \
+                                       int8_t *q, size_t rsq, size_t csq, const float *q_scale,     \
+                                       int per_column, int32_t q_zero) {                            \
+    for (size_t i = 0; i < m; ++i)                                                                  \
+      for (size_t j = 0; j < n; ++j) {                                                              \
+        TC v = c[i * rsc + j * csc];                                                                \
+        if (activation == 1) v = v > 0 ? v : 0;                                                     \
+        c[i * rsc + j * csc] = v;                                                                   \
+        if (q) q[i * rsq + j * csq] = requantised((float)v, q_scale[per_column ? j : 0], q_zero);   \
+      }                                                                                             \
+  }
+ACT_REQUANT(i32, int32_t)
+ACT_REQUANT(f32, float)
+
 /* ======================================================================== */
 /* Widening helpers                                                          */
 /* ======================================================================== */

@@ -128,6 +128,15 @@ SKL_ORACLE_PFUSED_DECL(f16rcprc_f16rcprc_f32rcprc, uint16_t, float)
 SKL_ORACLE_PFUSED_DECL(f8e4m3rcprc_f8e4m3rcprc_f32rcprc, uint8_t, float)
 SKL_ORACLE_PFUSED_DECL(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, float)
 
+/* Activation and requantised int8 copy over an m x n strided C that holds the alpha/beta (+ bias) result: the
+ * steps between bias and maximum of skl_gfx950_epilogue_t (include/skl-gfx950.h). The reference has no routine
+ * for them (src/gemm/README.md:46-47 leaves them to callers); tests/test_oracle_gemm.py pins these against
+ * hand-worked values and an independent numpy formulation. q may be NULL. */
+void skl_oracle_act_requant_i32(size_t m, size_t n, int32_t *c, size_t rsc, size_t csc, int activation, int8_t *q,
+                                size_t rsq, size_t csq, const float *q_scale, int per_column, int32_t q_zero);
+void skl_oracle_act_requant_f32(size_t m, size_t n, float *c, size_t rsc, size_t csc, int activation, int8_t *q,
+                                size_t rsq, size_t csq, const float *q_scale, int per_column, int32_t q_zero);
+
 /* Widening helpers used to build fp64 comparison operands on the host. */
 void skl_oracle_widen_bf16_f64(double *dst, const uint16_t *src, size_t n);
 void skl_oracle_widen_f16_f64(double *dst, const uint16_t *src, size_t n);

@@ -52,13 +52,24 @@ def _as_pointer(x):
 
 class Epilogue:
     """Fused-epilogue operands of the `skl_gemm_fused_*` entry points: `bias` (n values of C's
-    type) and `max` (one value of C's type), each a DeviceBuffer, a numpy array or None."""
+    type), `max` (one value of C's type), `activation` (ACT_NONE / ACT_RELU) and the requantised
+    copy `q` (int8, element (i, j) at `i * rsq + j * csq`) made with `q_scale` (one float32, or n
+    of them with `q_scale_per_column`) and `q_zero`; `q_only` leaves C unwritten. Every operand
+    is a DeviceBuffer, a numpy array or None."""
 
-    def __init__(self, bias=None, max=None):
-        self.bias, self.max = bias, max
+    ACT_NONE, ACT_RELU = 0, 1
+
+    def __init__(self, bias=None, max=None, activation=0, q=None, rsq=0, csq=0, q_scale=None,
+                 q_scale_per_column=False, q_zero=0, q_only=False):
+        self.bias, self.max, self.activation = bias, max, activation
+        self.q, self.rsq, self.csq, self.q_scale = q, rsq, csq, q_scale
+        self.q_scale_per_column, self.q_zero, self.q_only = q_scale_per_column, q_zero, q_only
 
     def as_struct(self):
-        return signatures.EpilogueStruct(_as_pointer(self.bias), _as_pointer(self.max))
+        return signatures.EpilogueStruct(_as_pointer(self.bias), _as_pointer(self.max), int(self.activation),
+                                         int(bool(self.q_scale_per_column)), int(bool(self.q_only)), int(self.q_zero),
+                                         _as_pointer(self.q), int(self.rsq), int(self.csq),
+                                         _as_pointer(self.q_scale))
 
 
 def _wrap(raw, sig):

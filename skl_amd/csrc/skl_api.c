@@ -144,6 +144,7 @@ static int canonicalize(const skl_gemm_desc *d, skl_gemm_canon *g) {
   g->beta = d->beta;
   g->bias = d->bias;
   g->max = d->max;
+  g->rq = d->rq;
   if (!flat_k(d->k0, d->k1, d->csa0, d->csa1, &g->a_sk)) return 0;
   if (!flat_k(d->k0, d->k1, d->rsb0, d->rsb1, &g->b_sk)) return 0;
   if (!block64(d->m0, d->m1, d->rsa0, d->rsa1, &g->a_s0, &g->a_s1)) return 0;
@@ -335,6 +336,7 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   h.c_row_shift = h.c_col_shift = 6;
   h.alpha = d->alpha, h.beta = d->beta;
   h.bias = d->bias, h.max = d->max;
+  h.rq = d->rq;
   /* C in power-of-two blocks (the 4 x 4 blocks of that format) can be updated where it is by the matrix-core
    * kernels. Small blocks make their stores short (16 bytes per 4 x 4 block row), so that pays when C would
    * otherwise travel three times (unpack, update, pack: 8192^3 in 4 x 4 blocks 890 against 1048 us), not when an
@@ -359,7 +361,7 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
             skl_hip_launch_unpack(4, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, M, N, h.c, N, 1) == 0);
   }
   if (done) done = gemm_fast_path(&h, fused, 1);
-  if (done && !c_in_place)
+  if (done && !c_in_place && !d->rq.q_only) /* with q_only the result went to the requantised copy alone */
     done = skl_hip_launch_pack(4, M, N, h.c, N, 1, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, 0) == 0;
   skl_hip_sequence_end();
   return done;
@@ -393,7 +395,7 @@ static int k4_in_row_chunks(const skl_gemm_desc *d) {
 
 static void gemm_on_device(const skl_gemm_desc *d) {
   skl_gemm_canon g;
-  const int fused = d->bias != NULL || d->max != NULL; /* the M = 1 kernels have no fused steps */
+  const int fused = d->bias != NULL || d->max != NULL || d->rq.act != 0 || d->rq.q != NULL; /* the M = 1 kernels have no fused steps */
   if (d->k0 * d->k1 != 0 && d->ta <= SKL_DT_F8E5M2) {
     if (!fused && canonicalize_k4(d, &g, 0) && skl_hip_gemv_supported(&g, 1)) {
       skl_hip_launch_gemv(&g, 1);
@@ -438,8 +440,21 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
   }
   where = classify(K ? d->a : NULL, K ? d->b : NULL, d->c, who);
   if (where < 0) return;
+  if ((d->rq.act != SKL_GFX950_ACT_NONE && d->rq.act != SKL_GFX950_ACT_RELU) ||
+      (d->rq.q && (!d->rq.q_scale || d->rq.q_zero < -128 || d->rq.q_zero > 127))) {
+    skl_hip_record_error(SKL_HIP_ERR_BAD_ARGUMENT, who);
+    return;
+  }
   if (d->bias || d->max) { /* the fused operands must be of the same kind as C */
     const int extra = classify(d->bias, d->max, NULL, who);
+    if (extra < 0) return;
+    if (extra != where) {
+      skl_hip_record_error(SKL_HIP_ERR_MIXED_POINTERS, who);
+      return;
+    }
+  }
+  if (d->rq.q) {
+    const int extra = classify(d->rq.q, d->rq.q_scale, NULL, who);
     if (extra < 0) return;
     if (extra != where) {
       skl_hip_record_error(SKL_HIP_ERR_MIXED_POINTERS, who);
@@ -461,12 +476,18 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
     const size_t esc = c_elem_size(d->ta);
     void *da = stage_in(d->a, na * esa), *db = stage_in(d->b, nb * esb), *dc = stage_in(d->c, nc * esc);
     void *dbias = d->bias ? stage_in(d->bias, N * esc) : NULL, *dmax = d->max ? stage_in(d->max, esc) : NULL;
-    if ((na && !da) || (nb && !db) || !dc || (d->bias && !dbias) || (d->max && !dmax)) {
+    /* the requantised copy: its whole span travels both ways, like C's */
+    const size_t nq = d->rq.q ? (M - 1) * d->rq.rsq + (N - 1) * d->rq.csq + 1 : 0;
+    void *dq = d->rq.q ? stage_in(d->rq.q, nq) : NULL;
+    void *dqs = d->rq.q ? stage_in(d->rq.q_scale, (d->rq.q_per_column ? N : 1) * sizeof(float)) : NULL;
+    if ((na && !da) || (nb && !db) || !dc || (d->bias && !dbias) || (d->max && !dmax) || (d->rq.q && (!dq || !dqs))) {
       skl_hip_free(da);
       skl_hip_free(db);
       skl_hip_free(dc);
       skl_hip_free(dbias);
       skl_hip_free(dmax);
+      skl_hip_free(dq);
+      skl_hip_free(dqs);
       return;
     }
     dd.a = da;
@@ -474,9 +495,14 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
     dd.c = dc;
     dd.bias = dbias;
     dd.max = dmax;
+    dd.rq.q = dq;
+    dd.rq.q_scale = dqs;
     gemm_on_device(&dd);
     skl_hip_memcpy_d2h(d->c, dc, nc * esc);
     if (dmax) skl_hip_memcpy_d2h(d->max, dmax, esc);
+    if (dq) skl_hip_memcpy_d2h(d->rq.q, dq, nq);
+    skl_hip_free(dq);
+    skl_hip_free(dqs);
     skl_hip_free(da);
     skl_hip_free(db);
     skl_hip_free(dc);
@@ -495,7 +521,7 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
             const TA_T *b, size_t rsb, size_t csb, TC_T beta, TC_T *c, size_t rsc, size_t csc) {   \
     skl_gemm_desc d = {DTA, DTB, 1,   1,   1,   m,    n,    k,   a,    0, 0, rsa, csa,             \
                        b,   0,   0,   rsb, csb, c,    0,    0,   rsc,  csc, {SC(alpha)}, {SC(beta)}, \
-                       NULL, NULL};                                                                \
+                       NULL, NULL, {0}};                                                           \
     gemm_run(&d, #NAME);                                                                           \
   }
 
@@ -518,7 +544,7 @@ DEFINE_GEMM_RC(skl_gemm_f16rc_f16rc_f16rc_gfx950, skl_f16_t, skl_f16_t, SKL_DT_F
             size_t csc0, size_t rsc1, size_t csc1) {                                               \
     skl_gemm_desc d = {DT,   DT,   m0,   n0,   k0,   m1,   n1,   k1,   a,    rsa0, csa0, rsa1, csa1, \
                        b,    rsb0, csb0, rsb1, csb1, c,    rsc0, csc0, rsc1, csc1, {SC(alpha)},    \
-                       {SC(beta)}, NULL, NULL};                                                    \
+                       {SC(beta)}, NULL, NULL, {0}};                                               \
     gemm_run(&d, #NAME);                                                                           \
   }
 
@@ -531,6 +557,11 @@ DEFINE_GEMM_RCPRC(skl_gemm_f32rcprc_f32rcprc_f32rcprc_gfx950, float, float, SKL_
 DEFINE_GEMM_RCPRC(skl_gemm_f64rcprc_f64rcprc_f64rcprc_gfx950, double, double, SKL_DT_F64, SCALAR_f64)
 DEFINE_GEMM_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, skl_f16_t, SKL_DT_F16H, SCALAR_f32)
 
+static skl_requant requant_of(const skl_gfx950_epilogue_t *ep) {
+  skl_requant rq = {ep->activation, ep->q_scale_per_column != 0, ep->q_only != 0 && ep->q != NULL, ep->q_zero, ep->q, ep->rsq, ep->csq, ep->q_scale};
+  return rq;
+}
+
 /* The same two forms with the fused steps of `ep` behind the alpha/beta step; ep == NULL is the plain GEMM. */
 #define DEFINE_GEMM_FUSED_RC(NAME, TA_T, TC_T, DT, SC)                                             \
   void NAME(size_t m, size_t n, size_t k, TC_T alpha, const TA_T *a, size_t rsa, size_t csa,       \
@@ -538,7 +569,8 @@ DEFINE_GEMM_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, skl_f16
             const skl_gfx950_epilogue_t *ep) {                                                     \
     skl_gemm_desc d = {DT,  DT,  1,   1,   1,   m,    n,    k,   a,    0, 0, rsa, csa,             \
                        b,   0,   0,   rsb, csb, c,    0,    0,   rsc,  csc, {SC(alpha)}, {SC(beta)}, \
-                       ep ? ep->bias : NULL, ep ? ep->max : NULL};                                 \
+                       ep ? ep->bias : NULL, ep ? ep->max : NULL, {0}};                            \
+    if (ep) d.rq = requant_of(ep);                                                                 \
     gemm_run(&d, #NAME);                                                                           \
   }
 #define DEFINE_GEMM_FUSED_RCPRC(NAME, TA_T, TC_T, DT, SC)                                          \
@@ -548,7 +580,8 @@ DEFINE_GEMM_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, skl_f16
             size_t csc0, size_t rsc1, size_t csc1, const skl_gfx950_epilogue_t *ep) {              \
     skl_gemm_desc d = {DT,   DT,   m0,   n0,   k0,   m1,   n1,   k1,   a,    rsa0, csa0, rsa1, csa1, \
                        b,    rsb0, csb0, rsb1, csb1, c,    rsc0, csc0, rsc1, csc1, {SC(alpha)},    \
-                       {SC(beta)}, ep ? ep->bias : NULL, ep ? ep->max : NULL};                     \
+                       {SC(beta)}, ep ? ep->bias : NULL, ep ? ep->max : NULL, {0}};                \
+    if (ep) d.rq = requant_of(ep);                                                                 \
     gemm_run(&d, #NAME);                                                                           \
   }
 DEFINE_GEMM_FUSED_RC(skl_gemm_fused_i8rc_i8rc_i32rc_gfx950, int8_t, int32_t, SKL_DT_I8, SCALAR_i32)
@@ -581,7 +614,7 @@ DEFINE_GEMM_ROWMAJOR(skl_gemm_f16_f16_f16_gfx950, skl_gemm_f16rc_f16rc_f16rc_gfx
 void skl_gemm_i8_i8_i32_noalloc_gfx950(size_t m, size_t n, size_t k, int32_t alpha, const int8_t *a, size_t rsa,
                                        const int8_t *b, size_t rsb, int32_t beta, int32_t *c, size_t rsc) {
   skl_gemm_desc d = {SKL_DT_I8, SKL_DT_I8, 1, 1, 1, m, n, k, a, 0, 0, rsa, 1, b, 0, 0, rsb, 1,
-                     c, 0, 0, rsc, 1, {.i = alpha}, {.i = beta}, NULL, NULL};
+                     c, 0, 0, rsc, 1, {.i = alpha}, {.i = beta}, NULL, NULL, {0}};
   skl_gemm_canon g;
   if (m == 0 || n == 0) return;
   if (!canonicalize(&d, &g)) {
@@ -635,7 +668,7 @@ void skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4_gfx950(size_t m1, size_t n1, size_t k1
                                                  const int8_t *b, size_t rsb1, int32_t *c, size_t rsc1,
                                                  bool accum) {
   skl_gemm_desc d = {SKL_DT_I8, SKL_DT_I8, 4, 4, 8, m1, n1, k1, a, 8, 1, rsa1, 32, b, 4, 1, rsb1, 32,
-                     c, 4, 1, rsc1, 16, {.i = 1}, {.i = accum ? 1 : 0}, NULL, NULL};
+                     c, 4, 1, rsc1, 16, {.i = 1}, {.i = accum ? 1 : 0}, NULL, NULL, {0}};
   gemm_run(&d, __func__);
 }
 

@@ -120,16 +120,16 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(skl_gemm_desc d, unsi
     skl_update((float)acc, alias, d.alpha, d.beta);
     *c = (_Float16)wide;
   } else {
-    skl_update(acc, c, d.alpha, d.beta);
     if constexpr (std::is_same<Acc, int32_t>::value || std::is_same<Acc, float>::value) {
-      if (d.bias || d.max) {  // fused steps behind the alpha/beta step
-        Acc v = *c;
-        if (d.bias) {
-          v = skl_add_bias(v, reinterpret_cast<const Acc *>(d.bias)[j]);
-          *c = v;
-        }
-        if (d.max && v > skl_lowest<Acc>()) skl_atomic_max(reinterpret_cast<Acc *>(d.max), v);
-      }
+      // the alpha/beta step, then the fused steps: bias, activation, C, requantised copy, maximum
+      Acc v = skl_beta_is_zero<Acc>(d.beta) ? skl_initialise(acc, c, d.alpha, d.beta) : skl_combine(acc, *c, d.alpha, d.beta);
+      if (d.bias) v = skl_add_bias(v, reinterpret_cast<const Acc *>(d.bias)[j]);
+      v = skl_activate(v, d.rq.act);
+      if (!d.rq.q_only) *c = v;
+      skl_emit_requantised(d.rq, v, i, j);
+      if (d.max && v > skl_lowest<Acc>()) skl_atomic_max(reinterpret_cast<Acc *>(d.max), v);
+    } else {
+      skl_update(acc, c, d.alpha, d.beta);
     }
   }
 }

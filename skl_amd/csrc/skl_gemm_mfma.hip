@@ -63,6 +63,7 @@ struct MfmaArgs {
   skl_scalar alpha, beta;
   const char *bias;  // fused epilogue: per-column addend and running maximum of C's type, or null
   char *max;
+  skl_requant rq;    // ... activation and requantised int8 copy
   unsigned tiles_m, tiles_n;
   // Split along K (bounds-checked kernel only): workgroup b works on tile b % (tiles_m * tiles_n) and on the
   // slices [split * slices_per_split, ...) with split = b / (tiles_m * tiles_n); splits > 1 stores the raw
@@ -71,21 +72,40 @@ struct MfmaArgs {
   char *partial;
 };
 
-// The fused steps behind the alpha/beta step, for one lane: bias of the lane's column, running maximum.
-template <typename T>
+// The fused steps behind the alpha/beta step, for one lane: bias of the lane's column, activation, running maximum,
+// requantised copy.
+// EXTRA: with the activation and the requantised copy (kernels are instantiated with and without: the two steps cost
+// code in every one of a lane's 128 stores, which calls without them should not carry).
+template <typename T, bool EXTRA = false>
 struct FusedSteps {
   const T *bias;
   T *max;
+  const skl_requant rq;
   T bias_j, running;
+  size_t col;
   __device__ explicit FusedSteps(const MfmaArgs &p)
-      : bias(reinterpret_cast<const T *>(p.bias)), max(reinterpret_cast<T *>(p.max)), bias_j(0), running(skl_lowest<T>()) {}
-  __device__ __forceinline__ void column(size_t col) {
-    if (bias) bias_j = bias[col];
+      : bias(reinterpret_cast<const T *>(p.bias)), max(reinterpret_cast<T *>(p.max)), rq(p.rq), bias_j(0), running(skl_lowest<T>()), col(0) {}
+  __device__ __forceinline__ void column(size_t c) {
+    col = c;
+    if (bias) bias_j = bias[c];
   }
   __device__ __forceinline__ T apply(T v) {
     if (bias) v = skl_add_bias(v, bias_j);
+    if constexpr (EXTRA) v = skl_activate(v, rq.act);
     if (max && v > running) running = v;
     return v;
+  }
+  // The element of logical row `row` in the current column: the steps, then C (written once and not read again: a
+  // non-temporal store keeps it out of the operands' caches) and the requantised copy.
+  __device__ __forceinline__ void put(T v, T *dst, size_t row) {
+    v = apply(v);
+    if constexpr (EXTRA) {
+      if (!rq.q_only) __builtin_nontemporal_store(v, dst);
+      skl_emit_requantised(rq, v, row, col);
+    } else {
+      (void)row;
+      __builtin_nontemporal_store(v, dst);
+    }
   }
   // Every lane of the wave calls this once, after its last element.
   __device__ __forceinline__ void finish() {
@@ -370,7 +390,7 @@ __device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, un
   tn = in_group / rows;
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED, bool EXACT = false>
+template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED, bool EXACT = false, bool EXTRA = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaArgs p) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   using KA = Kind<TA>;
@@ -500,7 +520,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
   // element). C is written once and not read again: non-temporal stores keep it out of the operands' caches.
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
   const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
-  FusedSteps<AccElem> fused(p);
+  FusedSteps<AccElem, EXTRA> fused(p);
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
@@ -517,9 +537,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
           const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block (blocks have a multiple of 4 rows)
           out[i][g] = c + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 + col_off;
         }
-      auto in_range = [&](int i, int r) {
-        return !GUARDED || m0 + wm + (i0 + i) * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3) < p.m;
-      };
+      auto row_of = [&](int i, int r) { return m0 + wm + (i0 + i) * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); };
+      auto in_range = [&](int i, int r) { return !GUARDED || row_of(i, r) < p.m; };
       if (init) {
 #pragma unroll
         for (int i = 0; i < kEpilogueBatch; ++i)
@@ -527,7 +546,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
           for (int r = 0; r < 16; ++r)
             if (in_range(i, r)) {
               AccElem *dst = out[i][r >> 2] + (r & 3) * p.rsc0;
-              __builtin_nontemporal_store(fused.apply(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta)), dst);
+              fused.put(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst, row_of(i, r));
             }
       } else {
         AccElem old[kEpilogueBatch][16];
@@ -540,7 +559,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
 #pragma unroll
           for (int r = 0; r < 16; ++r)
             if (in_range(i, r))
-              __builtin_nontemporal_store(fused.apply(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta)), out[i][r >> 2] + (r & 3) * p.rsc0);
+              fused.put(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][r >> 2] + (r & 3) * p.rsc0, row_of(i, r));
       }
     }
   }
@@ -1019,8 +1038,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             AccElem *dst = out[i][r >> 2] + (r & 3) * p.rsc0;
-            if (inside(i, r))
-              __builtin_nontemporal_store(fused.apply(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta)), dst);
+            if (inside(i, r)) fused.put(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst, first_row[i][r >> 2] + (r & 3));
           }
       } else {
         AccElem old[kEpilogueBatch][16];
@@ -1033,7 +1051,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 #pragma unroll
           for (int r = 0; r < 16; ++r)
             if (inside(i, r))
-              __builtin_nontemporal_store(fused.apply(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta)), out[i][r >> 2] + (r & 3) * p.rsc0);
+              fused.put(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][r >> 2] + (r & 3) * p.rsc0, first_row[i][r >> 2] + (r & 3));
       }
     }
   }
@@ -1067,15 +1085,12 @@ __global__ void __launch_bounds__(256) gemm_split_reduce_kernel(MfmaArgs p) {
   }
   T *c = reinterpret_cast<T *>(p.c) + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 +
          (col >> p.ccs) * p.csc1 + (col & ((size_t(1) << p.ccs) - 1)) * p.csc0;
-  skl_update(sum, c, p.alpha, p.beta);
-  if (p.bias || p.max) {
-    T v = *c;
-    if (p.bias) {
-      v = skl_add_bias(v, reinterpret_cast<const T *>(p.bias)[col]);
-      *c = v;
-    }
-    if (p.max && v > skl_lowest<T>()) skl_atomic_max(reinterpret_cast<T *>(p.max), v);
-  }
+  T v = skl_beta_is_zero<T>(p.beta) ? skl_initialise(sum, c, p.alpha, p.beta) : skl_combine(sum, *c, p.alpha, p.beta);
+  if (p.bias) v = skl_add_bias(v, reinterpret_cast<const T *>(p.bias)[col]);
+  v = skl_activate(v, p.rq.act);
+  if (!p.rq.q_only) *c = v;
+  skl_emit_requantised(p.rq, v, row, col);
+  if (p.max && v > skl_lowest<T>()) skl_atomic_max(reinterpret_cast<T *>(p.max), v);
 }
 
 struct SequenceGuard {
@@ -1142,12 +1157,15 @@ inline unsigned splits_for(size_t tiles, size_t slices, size_t m, size_t n) {
   return (unsigned)(want < 1 ? 1 : want);
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED, bool EXACT = false>
+template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED, bool EXACT = false, bool EXTRA = false>
 int launch_one(const MfmaArgs &args) {
+  if constexpr (!EXTRA) {  // calls with an activation or a requantised copy take the kernels that carry those steps
+    if (args.rq.act || args.rq.q) return launch_one<TA, TB, A_KC, B_KC, BM, BN, WAVES_M, WAVES_N, GUARDED, EXACT, true>(args);
+  }
   constexpr int ES = Kind<TA>::ES;
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int lds = 2 * (Tile<ES, BM, A_KC, NT>::kBytes + Tile<ES, BN, B_KC, NT>::kBytes);
-  auto kernel = gemm_mfma_kernel<TA, TB, A_KC, B_KC, BM, BN, WAVES_M, WAVES_N, GUARDED, EXACT>;
+  auto kernel = gemm_mfma_kernel<TA, TB, A_KC, B_KC, BM, BN, WAVES_M, WAVES_N, GUARDED, EXACT, EXTRA>;
   static bool configured = false;  // per instantiation; racing threads would set the same value
   if (!configured) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -1203,7 +1221,8 @@ int launch_tile(const MfmaArgs &p) {
   // The streaming kernel takes problems that its tiles divide evenly: 256 x 256 tiles when those
   // can fill the 256 compute units, 256 x 128 tiles for the sizes below that; everything else runs
   // on the small, bounds-checked kernel.
-  if (p.m % 256 == 0 && (p.k * ES) % 128 == 0) {
+  const bool extra_steps = p.rq.act || p.rq.q;  // activation / requantised copy: on the bounds-checked kernels only
+  if (!extra_steps && p.m % 256 == 0 && (p.k * ES) % 128 == 0) {
     const size_t tiles_m = p.m / 256;
     if (p.n % 256 == 0 && tiles_m * (p.n / 256) >= 200) {
       // A last round that would fill at most half of the 256 compute units is run as 256 x 128 tiles
@@ -1217,6 +1236,8 @@ int launch_tile(const MfmaArgs &p) {
         tail.b = p.b + (head_cols / 64) * p.b_s1 * ES;
         tail.c = p.c + (head_cols >> p.ccs) * p.csc1 * sizeof(float);  // whole blocks; C elements are 4 bytes for every kind
         if (p.bias) tail.bias = p.bias + head_cols * sizeof(float);
+        if (p.rq.q) tail.rq.q = p.rq.q + head_cols * p.rq.csq;
+        if (p.rq.q && p.rq.q_per_column) tail.rq.q_scale = p.rq.q_scale + head_cols;
         const int rc = launch_ring<TA, TB, A_KC, B_KC, 256>(head);
         return rc != 0 ? rc : launch_ring<TA, TB, A_KC, B_KC, 128>(tail);
       }
@@ -1304,6 +1325,7 @@ extern "C" int skl_hip_gemm_mfma_padded_plan(const skl_gemm_canon *g, size_t *mp
   if (!(g->ta == g->tb || (fp8a && fp8b)) || ((uintptr_t)g->c & 3) != 0) return 0;
   const size_t es = (g->ta == SKL_DT_BF16 || g->ta == SKL_DT_F16) ? 2 : 1;
   if (streams_in_place(g, es)) return 0;
+  if (g->rq.act || g->rq.q) return 0;  // the streaming kernel has no activation / requantisation steps
   if (fp8a && g->k <= kF8ExactMaxK) return 0;  // short K: the exact fp8 product, which the streaming kernel does not have
   const size_t tiles_m = (g->m + 255) / 256;
   int tile_cols = 0;
@@ -1339,6 +1361,7 @@ extern "C" int skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile
   p.crs = g->c_row_shift, p.ccs = g->c_col_shift;
   p.alpha = g->alpha, p.beta = g->beta;
   p.bias = (const char *)g->bias, p.max = (char *)g->max;
+  p.rq = g->rq;
   p.tiles_m = p.tiles_n = 0;
   p.splits = 1, p.slices_per_split = 0, p.partial = nullptr;
   switch (g->ta * 8 + g->tb) {
@@ -1373,6 +1396,7 @@ extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
   p.crs = g->c_row_shift, p.ccs = g->c_col_shift;
   p.alpha = g->alpha, p.beta = g->beta;
   p.bias = (const char *)g->bias, p.max = (char *)g->max;
+  p.rq = g->rq;
   p.tiles_m = p.tiles_n = 0;
   p.splits = 1, p.slices_per_split = 0, p.partial = nullptr;
   switch (g->ta * 8 + g->tb) {

@@ -215,7 +215,7 @@ int launch_sized(const skl_gemm_canon *g) {
 }  // namespace
 
 extern "C" int skl_hip_gemm_tiled_supported(const skl_gemm_canon *g) {
-  if (g->ta != g->tb || g->bias || g->max || g->c_row_shift != 6 || g->c_col_shift != 6) return 0;
+  if (g->ta != g->tb || g->bias || g->max || g->rq.act || g->rq.q || g->c_row_shift != 6 || g->c_col_shift != 6) return 0;
   if (g->ta != SKL_DT_F32 && g->ta != SKL_DT_F64 && g->ta != SKL_DT_F16H) return 0;
   return g->m != 0 && g->n != 0 && g->k != 0;
 }

@@ -669,6 +669,7 @@ struct GemvMfmaArgs {
   float *planes;        // floating point: slabs planes of m x n raw sums
   const float *bias;    // floating point: fused steps of the second pass, or null
   float *max;
+  skl_requant rq;       // ... activation, requantised int8 copy
 };
 
 __global__ void __launch_bounds__(256) gemv_mfma_scale_c_kernel(GemvMfmaArgs p) {
@@ -697,15 +698,12 @@ __global__ void __launch_bounds__(256) gemv_mfma_add_planes_kernel(GemvMfmaArgs 
   }
   const size_t col = idx % p.n;
   float *c = reinterpret_cast<float *>(p.c) + (idx / p.n) * p.c_row + col * p.c_s;
-  skl_update(sum, c, p.alpha, p.beta);
-  if (p.bias || p.max) {
-    float v = *c;
-    if (p.bias) {
-      v = skl_add_bias(v, p.bias[col]);
-      *c = v;
-    }
-    if (p.max && v > skl_lowest<float>()) skl_atomic_max(p.max, v);
-  }
+  float v = skl_beta_is_zero<float>(p.beta) ? skl_initialise(sum, c, p.alpha, p.beta) : skl_combine(sum, *c, p.alpha, p.beta);
+  if (p.bias) v = skl_add_bias(v, p.bias[col]);
+  v = skl_activate(v, p.rq.act);
+  if (!p.rq.q_only) *c = v;
+  skl_emit_requantised(p.rq, v, idx / p.n, col);
+  if (p.max && v > skl_lowest<float>()) skl_atomic_max(p.max, v);
 }
 
 template <int MODE>
@@ -1216,7 +1214,7 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int lay
   if (mode < 0) return 0;
   if (mode == kI8K4) {
     // B(4P + p, j) at P * b_sk + 4 j + p; 2 to 16 rows (no other kernel reads this layout with more than one row)
-    if (g->c_row_shift != 6 || g->c_col_shift != 6 || g->bias || g->max) return 0;
+    if (g->c_row_shift != 6 || g->c_col_shift != 6 || g->bias || g->max || g->rq.act || g->rq.q) return 0;
     if (g->m < 2 || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;
     if ((g->k % 16) != 0 || (g->n % 4) != 0 || g->k * g->n < (size_t(1) << 20)) return 0;
     if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % 16) != 0) return 0;
@@ -1235,7 +1233,7 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int lay
   if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % piece) != 0) return 0;
   if (g->b_s0 != 1 || !aligned16(g->b) || (g->b_sk % piece) != 0 || (g->b_s1 % piece) != 0) return 0;
   if (g->csc1 != 64 * g->csc0) return 0;
-  if (mode == kI8RowMajor && (g->bias || g->max)) return 0;  // the fused steps ride on the second pass (floating point)
+  if (mode == kI8RowMajor && (g->bias || g->max || g->rq.act || g->rq.q)) return 0;  // the fused steps ride on the second pass (floating point)
   // floating point: one plane of raw sums per 512 k, inside the workspace's usual 64 MiB
   const size_t slabs = (g->k + MfmaShape<1>::kKPerGroup - 1) / MfmaShape<1>::kKPerGroup;
   static_assert(MfmaShape<1>::kKPerGroup == MfmaShape<2>::kKPerGroup, "one group length for every floating-point kind");
@@ -1320,6 +1318,7 @@ extern "C" int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g, int layout
   p.planes = nullptr;
   p.bias = (const float *)g->bias;
   p.max = (float *)g->max;
+  p.rq = g->rq;
   switch (mode) {
     case kI8RowMajor: return launch_mfma_rows<kI8RowMajor>(p);
     case kI8K4: return launch_mfma_rows<kI8K4>(p);

@@ -43,6 +43,18 @@ typedef union {
   } fz;
 } skl_scalar;
 
+/* Further fused steps behind bias (see skl_gfx950_epilogue_t in include/skl-gfx950.h): an activation and a
+ * requantised int8 copy of the result. All zero / NULL: nothing. */
+typedef struct {
+  int act;             /* 0 none, 1 max(v, 0) */
+  int q_per_column;    /* q_scale holds one factor per logical column, else one in all */
+  int q_only;          /* the result goes to q alone, C is not written */
+  int32_t q_zero;
+  int8_t *q;           /* Q(i, j) at q[i*rsq + j*csq], (i, j) the logical row and column; NULL: no requantised output */
+  size_t rsq, csq;
+  const float *q_scale;
+} skl_requant;
+
 /* The fully general blocked GEMM of the reference (the `rcprc` form): element
  * (I,i ; P,p) of A is at a + I*rsa1 + P*csa1 + i*rsa0 + p*csa0, and likewise
  * for B (rows = k, columns = n) and C. Strides are in elements. */
@@ -61,6 +73,7 @@ typedef struct {
    * the alpha/beta step; *max of C's type is raised to the largest element written. */
   const void *bias;
   void *max;
+  skl_requant rq;
 } skl_gemm_desc;
 
 /* Canonical form served by the matrix-core kernels: flat in K, blocked by 64
@@ -83,6 +96,7 @@ typedef struct {
   skl_scalar alpha, beta;
   const void *bias; /* as in skl_gemm_desc */
   void *max;
+  skl_requant rq;
 } skl_gemm_canon;
 
 int skl_hip_launch_gemm_generic(const skl_gemm_desc *d);

@@ -48,7 +48,9 @@ int main(void) {
       want[i * LDC + j] = -2 * want[i * LDC + j] + 3 * acc + bias[j];
       if (want[i * LDC + j] > want_top) want_top = want[i * LDC + j];
     }
-  skl_gfx950_epilogue_t ep = {bias, &top};
+  skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE;
+  ep.bias = bias;
+  ep.max = &top;
   skl_gemm_fused_i8rc_i8rc_i32rc_gfx950(M, N, K, 3, a, LDA, 1, b, LDB, 1, -2, c, LDC, 1, &ep);
   bad |= check_error("fused int8 GEMM");
   if (memcmp(c, want, sizeof(int32_t) * M * LDC) != 0 || top != want_top) {

@@ -62,28 +62,37 @@ def run_gemm(lib, kind, case, a, b, c, mode):
     return out
 
 
-def run_fused_gemm(lib, kind, case, a, b, c, bias, mx, mode):
+def run_fused_gemm(lib, kind, case, a, b, c, bias, mx, mode, activation=0, requant=None):
     """Runs `skl_gemm_fused_*` (kind "rc" or "rcprc"); returns (C's whole buffer, *max) afterwards.
-    `bias` / `mx` are arrays of C's type (n values / one value) or None."""
-    def call(a_, b_, c_, bias_, mx_):
+    `bias` / `mx` are arrays of C's type (n values / one value) or None. `requant` = dict(q=<int8 buffer>,
+    rsq, csq, scale=<float32 array>, per_column, zero, only) asks for the requantised copy, whose buffer
+    afterwards is returned as a third value."""
+    rq = requant or {}
+
+    def call(a_, b_, c_, bias_, mx_, q_, scale_):
         name, args = gemm_entry_args(kind, case, a_, b_, c_)
         fused = name.replace("skl_gemm_", "skl_gemm_fused_")
-        getattr(lib, fused)(*args, skl_amd.Epilogue(bias_, mx_))
+        getattr(lib, fused)(*args, skl_amd.Epilogue(bias_, mx_, activation=activation, q=q_, rsq=rq.get("rsq", 0),
+                                                    csq=rq.get("csq", 0), q_scale=scale_,
+                                                    q_scale_per_column=rq.get("per_column", False),
+                                                    q_zero=rq.get("zero", 0), q_only=rq.get("only", False)))
 
+    q, scale = rq.get("q"), rq.get("scale")
     if mode == "host":
-        out, mo = c.copy(), None if mx is None else mx.copy()
-        call(a, b, out, bias, mo)
+        out, mo, qo = c.copy(), None if mx is None else mx.copy(), None if q is None else q.copy()
+        call(a, b, out, bias, mo, qo, scale)
         skl_amd.check_error()
-        return out, mo
-    bufs = [DeviceBuffer.from_array(x) if x is not None else None for x in (a, b, c, bias, mx)]
+        return (out, mo) if requant is None else (out, mo, qo)
+    bufs = [DeviceBuffer.from_array(x) if x is not None else None for x in (a, b, c, bias, mx, q, scale)]
     call(*bufs)
     _finish(lib)
     out = bufs[2].download(c.dtype, c.size)
     mo = None if mx is None else bufs[4].download(mx.dtype, mx.size)
+    qo = None if q is None else bufs[5].download(q.dtype, q.size)
     for d in bufs:
         if d is not None:
             d.free()
-    return out, mo
+    return (out, mo) if requant is None else (out, mo, qo)
 
 
 def run_inout(lib, name, build_args, src, dst, mode):

@@ -58,7 +58,7 @@ def test_headers_compile_as_c99_c11_and_cxx(tmp_path):
     src = tmp_path / "use.c"
     src.write_text('#include "skl-gfx950-compat.h"\n'
                    'int probe(void) {\n'
-                   '  skl_gfx950_epilogue_t ep = {0, 0};\n'
+                   '  skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE;\n'
                    '  skl_gemm_i8_i8_i32_zve32x_x390(0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0);\n'
                    '  skl_gemm_fused_i8rc_i8rc_i32rc_gfx950(0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, &ep);\n'
                    '  return (int)skl_get_ete_xsfmmbase();\n'

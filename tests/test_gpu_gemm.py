@@ -329,6 +329,123 @@ def test_fused_epilogue(gpu, ta, m, n, k, what):
     assert top[0] == high[0]
 
 
+EXTRA_STEP_SHAPES = (
+    # m, n, k, beta, what serves it
+    (130, 200, 64, 1, "64 x 64 bounds-checked tiles"),
+    (300, 1100, 96, 0, "128 x 128 bounds-checked tiles"),
+    (512, 768, 256, 1, "whole 256 x 128 tiles: still the bounds-checked kernels, which carry the steps"),
+    (1000, 1100, 520, 0, "ragged and large enough for padded copies: must stay on the bounds-checked kernels"),
+    (16, 4096, 4096, 1, "a decode batch"),
+    (40, 300, 8192, 1, "K shared between workgroups: the steps ride on the pass that adds the shares"),
+    (1, 4096, 512, 0, "M = 1"),
+)
+
+
+@pytest.mark.parametrize("m,n,k,beta,what", EXTRA_STEP_SHAPES)
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f8e4m3"))
+def test_fused_activation_and_requantised_copy(gpu, ta, m, n, k, beta, what):
+    """Activation and the requantised int8 copy (include/skl-gfx950.h, fused section), which follow the bias and
+    precede the maximum. The fused call without them is the anchor for C (bit for bit: same kernel family, same
+    summation - the plain steps are checked against the checker elsewhere); C, Q and *max must then be exactly what
+    the rules make of that C: relu in C's type, Q = clamp(rne((float)v * s_j) + zero). Row-major and transposed Q,
+    one scale and one per column, both kinds of memory, and q_only, which must leave C alone."""
+    rng = np.random.default_rng(m * 11 + n + k)
+    case = rowmajor_case(ta, m, n, k, alpha=1, beta=beta)
+    a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+    if case.is_int:
+        bias = rng.integers(-1 << 12, 1 << 12, n).astype(np.int32)
+        start = np.array([-(1 << 31)], np.int32)
+    else:
+        bias = rng.uniform(-4, 4, n).astype(np.float32)
+        start = np.array([-np.inf], np.float32)
+    spread = float(np.abs(run_fused_gemm(gpu, "rc", case, a, b, c, None, None, "device")[0].astype(np.float64)).max())
+    scales = (rng.uniform(0.5, 2.0, n) * 100.0 / max(spread, 1e-3)).astype(np.float32)  # some values saturate
+    layouts = ((n + 3, 1), (1, m + 5))  # (rsq, csq)
+    for mode in MODES:
+        anchor, _ = run_fused_gemm(gpu, "rc", case, a, b, c, bias, None, mode)
+        for act, per_column, (rsq, csq), zero, only in ((1, True, layouts[0], 3, False), (0, False, layouts[1], -7, False),
+                                                        (1, False, layouts[0], 0, True)):
+            q0 = np.full((m - 1) * rsq + (n - 1) * csq + 1, 0x55, np.int8)
+            rq = dict(q=q0, rsq=rsq, csq=csq, scale=scales if per_column else scales[:1], per_column=per_column,
+                      zero=zero, only=only)
+            got, top, q = run_fused_gemm(gpu, "rc", case, a, b, c, bias, start, mode, activation=act, requant=rq)
+            want_c, want_top, want_q = fused_expectation(case, anchor, None, start, activation=act, requant=rq)
+            tag = (ta, what, mode, act, per_column, rsq, only)
+            assert np.array_equal(q, want_q), tag
+            if only:
+                assert np.array_equal(got.view(np.uint8), c.view(np.uint8)), tag
+            else:
+                assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8)), tag
+            assert top[0] == want_top[0], tag
+            assert len(np.unique(want_q)) > 20, "a degenerate scale would test nothing"
+        # the activation alone
+        got, top = run_fused_gemm(gpu, "rc", case, a, b, c, bias, start, mode, activation=1)
+        want_c, want_top = fused_expectation(case, anchor, None, start, activation=1)
+        assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8)) and top[0] == want_top[0], (ta, what, mode)
+
+
+def test_fused_extra_steps_blocked_form_any_strides_and_refusals(gpu):
+    """The rcprc form addresses Q by the logical row and column; odd blocks and strides take the any-stride
+    kernel. Descriptors the header rules out are refused before anything runs."""
+    rng = np.random.default_rng(15)
+    for ta in ("i8", "f16"):
+        case = support.GemmCase(ta, None, 2, 3, m0=3, n0=4, k0=5, m1=5, n1=3, k1=4, rsa0=5, csa0=1, rsa1=100, csa1=15,
+                                rsb0=4, csb0=1, rsb1=20, csb1=90, rsc0=1, csc0=3, rsc1=12, csc1=64)
+        a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+        m, n = case.m0 * case.m1, case.n0 * case.n1
+        bias = (rng.integers(-99, 99, n).astype(np.int32) if case.is_int else rng.uniform(-4, 4, n).astype(np.float32))
+        start = np.array([-(1 << 31)], np.int32) if case.is_int else np.array([-np.inf], np.float32)
+        scales = rng.uniform(0.01, 0.05, n).astype(np.float32) * (1.0 if case.is_int else 20.0)
+        for mode in MODES:
+            anchor, _ = run_fused_gemm(gpu, "rcprc", case, a, b, c, bias, None, mode)
+            rq = dict(q=np.full(m * 40, 9, np.int8), rsq=40, csq=2, scale=scales, per_column=True, zero=-1)
+            got, top, q = run_fused_gemm(gpu, "rcprc", case, a, b, c, bias, start, mode, activation=1, requant=rq)
+            want_c, want_top, want_q = fused_expectation(case, anchor, None, start, activation=1, requant=rq)
+            assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8)), (ta, mode)
+            assert np.array_equal(q, want_q) and top[0] == want_top[0], (ta, mode)
+    # the 4 x 8 by 8 x 4 block format: through copies of A and B, C where it lies (accumulating) or through a
+    # row-major scratch matrix (beta == 0)
+    from test_oracle_gemm import block4x8x4_case
+    for accum in (True, False):
+        case = block4x8x4_case(32, 40, 16, accum=accum)
+        a, b, c = case.make_inputs(77)
+        m, n = 128, 160
+        bias = rng.integers(-999, 999, n).astype(np.int32)
+        start = np.array([-(1 << 31)], np.int32)
+        plain = run_oracle_gemm(case, a, b, c)
+        rq = dict(q=np.full(m * n, 9, np.int8), rsq=n, csq=1, scale=np.array([1 / 64.0], np.float32), zero=4)
+        got, top, q = run_fused_gemm(gpu, "rcprc", case, a, b, c, bias, start, "device", activation=1, requant=rq)
+        want_c, want_top, want_q = fused_expectation(case, plain, bias, start, activation=1, requant=rq)
+        assert np.array_equal(got, want_c) and np.array_equal(q, want_q) and top[0] == want_top[0], accum
+        rq["only"] = True
+        got, top, q = run_fused_gemm(gpu, "rcprc", case, a, b, c, bias, start, "device", activation=1, requant=rq)
+        assert np.array_equal(got, c) and np.array_equal(q, want_q) and top[0] == want_top[0], accum
+    case = rowmajor_case("i8", 8, 8, 8, alpha=1, beta=0)
+    a, b, c = case.make_inputs(1)
+    q0, one = np.zeros(64, np.int8), np.ones(1, np.float32)
+    for bad in (dict(q=q0, rsq=8, csq=1, scale=None), dict(q=q0, rsq=8, csq=1, scale=one, zero=128),
+                dict(q=q0, rsq=8, csq=1, scale=one, zero=-129)):
+        run_fused_gemm_expecting_refusal(gpu, case, a, b, c, requant=bad)
+    run_fused_gemm_expecting_refusal(gpu, case, a, b, c, activation=2)
+    # a Q in memory of the other kind than C
+    dq = skl_amd.DeviceBuffer.from_array(q0)
+    try:
+        run_fused_gemm_expecting_refusal(gpu, case, a, b, c, requant=dict(q=dq, rsq=8, csq=1, scale=one))
+    finally:
+        dq.free()
+
+
+def run_fused_gemm_expecting_refusal(gpu, case, a, b, c, activation=0, requant=None):
+    before = c.copy()
+    rq = requant or {}
+    gpu.skl_gemm_fused_i8rc_i8rc_i32rc_gfx950(
+        case.m1, case.n1, case.k1, 1, a, case.rsa1, 1, b, case.rsb1, 1, 0, c, case.rsc1, 1,
+        skl_amd.Epilogue(None, None, activation=activation, q=rq.get("q"), rsq=rq.get("rsq", 0), csq=rq.get("csq", 0),
+                         q_scale=rq.get("scale"), q_zero=rq.get("zero", 0)))
+    assert gpu.skl_hip_last_error() != 0, (activation, requant)  # reading clears it
+    assert np.array_equal(c, before)
+
+
 def test_fused_epilogue_blocked_form_and_null_descriptor(gpu):
     """The rcprc form indexes the bias by the logical column (block * n0 + column in the block); a call
     without descriptor operands is the plain GEMM. Odd blocks and strides: the any-stride kernel."""

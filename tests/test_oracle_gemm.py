@@ -239,19 +239,46 @@ def test_f32_to_f16_rounding_matches_numpy():
 FUSED_TYPES = ("i8", "bf16", "f16", "f8e4m3", "f8e5m2")
 
 
-def fused_expectation(case, plain, bias, max_in):
+def requantised(v, scale, zero):
+    """clamp(rne((float)v * s) + zero, -128, 127) of include/skl-gfx950.h, in numpy and by another route than the
+    checker's C: the product of two fp32 values is exact in fp64, so rounding it to fp32 once is the one fp32
+    multiplication; np.rint rounds ties to even; a NaN counts as 0, values beyond int32 as its ends."""
+    with np.errstate(invalid="ignore", over="ignore"):
+        prod = (np.asarray(v).astype(np.float32).astype(np.float64) * np.asarray(scale, np.float32).astype(np.float64)
+                ).astype(np.float32)
+        r = np.rint(prod.astype(np.float64))
+    r = np.where(np.isnan(r), 0.0, np.clip(r, -2147483648.0, 2147483647.0))
+    return np.clip(r.astype(np.int64) + int(zero), -128, 127).astype(np.int8)
+
+
+def fused_expectation(case, plain, bias, max_in, activation=0, requant=None):
     """C and *max after the fused steps, from the plain GEMM's result: the bias of the logical column
-    added in C's arithmetic (one fp32 addition / int32 wrap), the maximum over what was written."""
+    added in C's arithmetic (one fp32 addition / int32 wrap), the activation, the maximum over what was
+    written. With `requant` = dict(q=<int8 buffer before the call>, rsq, csq, scale=<1 or n floats>,
+    per_column, zero, only) a third value follows: the int8 buffer afterwards (and C stays `plain`'s
+    memory where `only` says it is not written)."""
     oc = support.blocked_offsets(case.m1, case.n1, case.m0, case.n0, case.rsc0, case.csc0, case.rsc1, case.csc1)
     want = plain.copy()
     if bias is not None:
         with np.errstate(over="ignore"):
             want[oc] = (plain[oc] + bias[None, :]).astype(plain.dtype)
+    if activation == 1:
+        v = want[oc]
+        want[oc] = np.where(v > 0, v, 0).astype(plain.dtype)
     top = None
     if max_in is not None:
         written = want[oc]
-        top = np.array([max(max_in[0], written.max())], dtype=plain.dtype)
-    return want, top
+        with np.errstate(invalid="ignore"):
+            best = written[written > max_in[0]]
+        top = np.array([best.max() if best.size else max_in[0]], dtype=plain.dtype)
+    if requant is None:
+        return want, top
+    m, n = oc.shape
+    q = requant["q"].copy()
+    scale = requant["scale"][None, :] if requant.get("per_column") else requant["scale"][0]
+    oq = np.arange(m)[:, None] * requant["rsq"] + np.arange(n)[None, :] * requant["csq"]
+    q[oq] = requantised(want[oc], scale, requant.get("zero", 0))
+    return want, top, q
 
 
 @pytest.mark.parametrize("ta", FUSED_TYPES)
@@ -289,6 +316,70 @@ def test_fused_steps_follow_the_plain_gemm(ta):
                     assert mx[0] == top[0], (ta, blocked, use_bias)
                 else:
                     assert mx[0] == start[0]
+
+
+def test_requantisation_rule_on_worked_values():
+    """The checker's requantisation and activation (oracle/skl_oracle.c, skl_oracle_act_requant_*) against values
+    worked by hand from the rule in include/skl-gfx950.h - ties go to the even integer, the zero point is added
+    after rounding, both ends saturate, an int32 is rounded to fp32 before it is scaled, a NaN counts as 0 - and
+    against the numpy formulation above on random values, per-call and per-column scales, strided Q."""
+    o = oracle()
+    half = np.array([0.5], np.float32)
+
+    def run(values, scale, zero=0, act=0, per_column=0, suffix="f32"):
+        c = np.array(values, np.float32 if suffix == "f32" else np.int32).reshape(1, -1)
+        q = np.full(c.size, 99, np.int8)
+        getattr(o, "skl_oracle_act_requant_" + suffix)(1, c.size, c, c.size, 1, act, q, c.size, 1,
+                                                       np.asarray(scale, np.float32), per_column, zero)
+        return c[0], q
+
+    # x * 0.5 = 0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5: ties to even
+    assert list(run([1, 3, 5, 7, -1, -3, -5], half)[1]) == [0, 2, 2, 4, 0, -2, -2]
+    assert list(run([1, 3, 5, 7, -1, -3, -5], half, suffix="i32")[1]) == [0, 2, 2, 4, 0, -2, -2]
+    # the zero point is added after rounding, and the sum saturates: 2.5 -> 2 (+3 = 5); 300 -> 127; -300 -> -128
+    assert list(run([5, 600, -600, 250], half, zero=3)[1]) == [5, 127, -128, 127]
+    assert list(run([250, 252, -260], half, zero=-3)[1]) == [122, 123, -128]
+    # NaN -> 0 (+ zero); infinities and values beyond int32 end at the ends of int8 whatever the zero point
+    assert list(run([np.nan, np.inf, -np.inf, 3e38, -3e38, 4e9, -4e9], [1.0], zero=-128)[1]) == [-128, 127, -128, 127, -128, 127, -128]
+    assert list(run([np.nan, -4e9], [1.0], zero=127)[1]) == [127, -128]
+    # int32 -> fp32 rounds to nearest even before the product: 2^24 + 1 -> 2^24, 2^24 + 3 -> 2^24 + 4;
+    # times 2^-20: 16 and 16.000004 -> 16
+    assert list(run([(1 << 24) + 1, (1 << 24) + 3, 100 << 20, -(101 << 20)], [2.0 ** -20], suffix="i32")[1]) == [16, 16, 100, -101]
+    # relu before the requantisation, and written back to C; a NaN becomes 0
+    c, q = run([-4.0, 6.0, np.nan, -0.0], [1.0], act=1)
+    assert list(q) == [0, 6, 0, 0] and list(c[:2]) == [0.0, 6.0] and c[2] == 0.0 and c[3] == 0.0
+    c, q = run([-7, 9], [1.0], act=1, suffix="i32")
+    assert list(c) == [0, 9] and list(q) == [0, 9]
+    # per-column scales
+    assert list(run([10, 10, 10], [1.0, 0.25, 3.0], per_column=1)[1]) == [10, 2, 30]
+
+    rng = np.random.default_rng(77)
+    for suffix, dt in (("i32", np.int32), ("f32", np.float32)):
+        for per_column in (0, 1):
+            m, n, rsc, rsq, csq = 13, 29, 31, 3, 47
+            if dt is np.int32:
+                c = rng.integers(-1 << 31, 1 << 31, m * rsc, dtype=np.int64).astype(np.int32)
+                scale = (rng.uniform(0.5, 2.0, n) * 2.0 ** rng.integers(-30, -20, n)).astype(np.float32)
+            else:
+                c = (rng.standard_normal(m * rsc) * 300).astype(np.float32)
+                scale = rng.uniform(0.01, 2.0, n).astype(np.float32)
+            c[::17] = (c[::17] // 2) * 2  # some exact ties with a scale of 0.5
+            if not per_column:
+                scale = scale[:1]
+            for act in (0, 1):
+                for zero in (0, -128, 127, 5):
+                    got_c, q = c.copy(), np.full(m * rsq + n * csq, 77, np.int8)
+                    getattr(o, "skl_oracle_act_requant_" + suffix)(m, n, got_c, rsc, 1, act, q, rsq, csq, scale,
+                                                                   per_column, zero)
+                    oc = np.arange(m)[:, None] * rsc + np.arange(n)[None, :]
+                    want_c = c.copy()
+                    if act:
+                        want_c[oc] = np.where(c[oc] > 0, c[oc], 0)
+                    assert np.array_equal(got_c, want_c)
+                    want_q = np.full(m * rsq + n * csq, 77, np.int8)
+                    oq = np.arange(m)[:, None] * rsq + np.arange(n)[None, :] * csq
+                    want_q[oq] = requantised(want_c[oc], scale[None, :] if per_column else scale[0], zero)
+                    assert np.array_equal(q, want_q), (suffix, per_column, act, zero)
 
 
 def block4x8x4_case(m1, n1, k1, rsa1=None, rsb1=None, rsc1=None, accum=False):
