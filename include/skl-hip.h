@@ -36,6 +36,9 @@ extern "C" {
 #define SKL_HIP_ERR_BAD_ARGUMENT (-2)
 #define SKL_HIP_ERR_NO_DEVICE (-3)
 #define SKL_HIP_ERR_WORKSPACE (-4)
+/* Advisory: the calling thread's stream has no scratch slot on this device (32 other streams hold one). The call
+ * that recorded it has still completed, on kernels that need no scratch memory. See skl_hip_release_stream(). */
+#define SKL_HIP_ERR_STREAM_SLOTS (-5)
 
 /* Pointer-classification modes for skl_hip_set_pointer_mode(). */
 #define SKL_HIP_POINTERS_AUTO 0   /* ask the HIP runtime about every pointer (default) */
@@ -47,6 +50,12 @@ extern "C" {
 int skl_hip_init(int device);
 /* Releases every scratch block of every device and stream. Outstanding work is waited for. */
 void skl_hip_shutdown(void);
+/* Gives back the scratch blocks a stream holds on the current device (up to 64 MiB of workspace, 32.5 MiB of
+ * sums and counters, operand copies) and its slot: call it before destroying a stream that made calls into the
+ * library. Waits for the stream's work; no call may be issued on the stream meanwhile. A device keeps at most 32
+ * streams with scratch of their own - a call on a further stream records SKL_HIP_ERR_STREAM_SLOTS and runs on the
+ * kernels that need no scratch memory. Returns 0 or an error. */
+int skl_hip_release_stream(void *stream);
 
 void *skl_hip_malloc(size_t bytes);
 void skl_hip_free(void *ptr);

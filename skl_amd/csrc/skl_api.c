@@ -181,13 +181,21 @@ static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g, int rows) 
   return 1;
 }
 
-/* The streaming kernels in the order they are tried; 1 if one of them took the problem. */
+/* What became of a problem offered to a kernel: TAKEN (launched), DECLINED (not its kind of problem: the next kernel
+ * is tried) or FAILED (an error is recorded, nothing more is tried). A launcher that could not get its scratch
+ * memory returns SKL_HIP_ERR_WORKSPACE before it has launched anything: that counts as DECLINED, so the call ends
+ * on a kernel that needs no scratch, and the allocation error is withdrawn once one has taken it. */
+enum { DECLINED = 0, TAKEN = 1, FAILED = -1 };
+static int outcome(int rc) { return rc == 0 ? TAKEN : rc == SKL_HIP_ERR_WORKSPACE ? DECLINED : FAILED; }
+
+/* The streaming kernels in the order they are tried. */
 static int gemv_on_device(const skl_gemm_canon *g) {
-  if (skl_hip_gemv_kc_supported(g)) return skl_hip_launch_gemv_kc(g), 1;
-  if (g->m == 1 && skl_hip_gemv_supported(g, 0)) return skl_hip_launch_gemv(g, 0), 1;
-  if (skl_hip_gemv_mfma_rows_supported(g, 0)) return skl_hip_launch_gemv_mfma_rows(g, 0), 1;
-  if (skl_hip_gemv_rows_supported(g)) return skl_hip_launch_gemv_rows(g), 1;
-  return 0;
+  int r = DECLINED;
+  if (skl_hip_gemv_kc_supported(g) && (r = outcome(skl_hip_launch_gemv_kc(g))) != DECLINED) return r;
+  if (g->m == 1 && skl_hip_gemv_supported(g, 0) && (r = outcome(skl_hip_launch_gemv(g, 0))) != DECLINED) return r;
+  if (skl_hip_gemv_mfma_rows_supported(g, 0) && (r = outcome(skl_hip_launch_gemv_mfma_rows(g, 0))) != DECLINED) return r;
+  if (skl_hip_gemv_rows_supported(g) && (r = outcome(skl_hip_launch_gemv_rows(g))) != DECLINED) return r;
+  return DECLINED;
 }
 
 static int gemv_would_take(const skl_gemm_canon *g) {
@@ -220,24 +228,30 @@ static void transposed_view(const skl_gemm_canon *g, skl_gemm_canon *t) {
   t->c_col_shift = g->c_row_shift;
 }
 
-/* Offers `g` to every kernel but the any-stride one; 1 if one of them takes it. With `launch` == 0 only asks. */
+/* Offers `g` to the streaming kernels, as it is and with the roles of A and B exchanged. With `launch` == 0 only
+ * asks (TAKEN: one of them would take it). */
 static int gemv_paths(const skl_gemm_canon *g, int launch) {
   skl_gemm_canon t;
-  if (launch ? gemv_on_device(g) : gemv_would_take(g)) return 1;
+  int r = launch ? gemv_on_device(g) : gemv_would_take(g);
+  if (r != DECLINED) return r;
   if (g->n <= 8 && g->n < g->m) {
     transposed_view(g, &t);
-    if (launch ? gemv_on_device(&t) : gemv_would_take(&t)) return 1;
+    r = launch ? gemv_on_device(&t) : gemv_would_take(&t);
   }
-  return 0;
+  return r;
 }
 
+/* Streaming kernels, then the matrix-core tile kernels. */
 static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
-  if (!fused && gemv_paths(g, launch)) return 1;
+  int r = DECLINED;
+  if (!fused && (r = gemv_paths(g, launch)) != DECLINED) return r;
   /* the decode-batch kernel of the floating-point kinds applies the fused steps itself, so that a call gives the
    * same bits with and without them */
-  if (fused && skl_hip_gemv_mfma_rows_supported(g, 0)) return launch ? (skl_hip_launch_gemv_mfma_rows(g, 0), 1) : 1;
-  if (skl_hip_gemm_mfma_supported(g)) return launch ? (skl_hip_launch_gemm_mfma(g), 1) : 1;
-  return 0;
+  if (fused && skl_hip_gemv_mfma_rows_supported(g, 0) &&
+      (r = launch ? outcome(skl_hip_launch_gemv_mfma_rows(g, 0)) : TAKEN) != DECLINED)
+    return r;
+  if (skl_hip_gemm_mfma_supported(g)) return launch ? outcome(skl_hip_launch_gemm_mfma(g)) : TAKEN;
+  return DECLINED;
 }
 
 /* An operand in a layout that none of the kernels reads - a leading dimension that is not a multiple of 16 bytes,
@@ -248,8 +262,8 @@ static int gemm_with_realigned_operands(const skl_gemm_canon *g, int fused) {
   const size_t esa = elem_size(g->ta), esb = elem_size(g->tb);
   const size_t kpa = (g->k * esa + 15) / 16 * 16 / esa, kpb = (g->k * esb + 15) / 16 * 16 / esb;
   const size_t bytes_a = (g->m * kpa * esa + 255) / 256 * 256, bytes_b = g->n * kpb * esb;
-  int which, done;
-  if (esa > 2 || esb > 2 || g->m * g->n * g->k < ((size_t)1 << 18)) return 0;
+  int which, r;
+  if (esa > 2 || esb > 2 || g->m * g->n * g->k < ((size_t)1 << 18)) return DECLINED;
   for (which = 1; which <= 3; ++which) { /* 1: B, 2: A, 3: both */
     skl_gemm_canon h = *g;
     const int copy_a = (which & 2) != 0, copy_b = (which & 1) != 0;
@@ -262,24 +276,24 @@ static int gemm_with_realigned_operands(const skl_gemm_canon *g, int fused) {
       h.b = (const void *)(uintptr_t)256;
       h.b_sk = 1, h.b_s0 = kpb, h.b_s1 = SKL_TE * kpb;
     }
-    if (!gemm_fast_path(&h, fused, 0)) continue;
+    if (gemm_fast_path(&h, fused, 0) != TAKEN) continue;
     skl_hip_sequence_begin();
     scratch = skl_hip_operand_scratch((copy_a ? bytes_a : 0) + (copy_b ? bytes_b : 0));
-    done = scratch != NULL;
-    if (done && copy_a) {
-      done = skl_hip_launch_realign((int)esa, g->m, g->k, g->a, SKL_TE, g->a_s0, g->a_s1, 1, 0, g->a_sk, scratch, kpa) == 0;
+    r = scratch != NULL ? TAKEN : DECLINED; /* no memory for the copies: a kernel that needs none */
+    if (r == TAKEN && copy_a) {
+      r = outcome(skl_hip_launch_realign((int)esa, g->m, g->k, g->a, SKL_TE, g->a_s0, g->a_s1, 1, 0, g->a_sk, scratch, kpa));
       h.a = scratch;
       scratch += bytes_a;
     }
-    if (done && copy_b) {
-      done = skl_hip_launch_realign((int)esb, g->n, g->k, g->b, SKL_TE, g->b_s0, g->b_s1, 1, 0, g->b_sk, scratch, kpb) == 0;
+    if (r == TAKEN && copy_b) {
+      r = outcome(skl_hip_launch_realign((int)esb, g->n, g->k, g->b, SKL_TE, g->b_s0, g->b_s1, 1, 0, g->b_sk, scratch, kpb));
       h.b = scratch;
     }
-    if (done) done = gemm_fast_path(&h, fused, 1);
+    if (r == TAKEN) r = gemm_fast_path(&h, fused, 1); /* C is untouched so far: DECLINED still lets another kernel run */
     skl_hip_sequence_end();
-    return done;
+    return r;
   }
-  return 0;
+  return DECLINED;
 }
 
 /* Ragged or misaligned problems large enough for the streaming kernel: A and B copied into scratch memory padded
@@ -291,22 +305,24 @@ static int gemm_padded_to_tiles(const skl_gemm_canon *g) {
   const size_t esa = elem_size(g->ta), esb = elem_size(g->tb);
   skl_gemm_canon h = *g;
   char *scratch;
-  int done;
-  if (!tile_cols) return 0;
+  int r;
+  if (!tile_cols) return DECLINED;
   skl_hip_sequence_begin();
   scratch = skl_hip_operand_scratch(mp * kp * esa + np * kp * esb);
-  done = scratch != NULL &&
-         skl_hip_launch_realign((int)esa, g->m, g->k, g->a, SKL_TE, g->a_s0, g->a_s1, 1, 0, g->a_sk, scratch, kp) == 0 &&
-         skl_hip_launch_realign((int)esb, g->n, g->k, g->b, SKL_TE, g->b_s0, g->b_s1, 1, 0, g->b_sk,
-                                scratch + mp * kp * esa, kp) == 0;
-  if (done) {
+  r = scratch != NULL ? TAKEN : DECLINED;
+  if (r == TAKEN)
+    r = outcome(skl_hip_launch_realign((int)esa, g->m, g->k, g->a, SKL_TE, g->a_s0, g->a_s1, 1, 0, g->a_sk, scratch, kp));
+  if (r == TAKEN)
+    r = outcome(skl_hip_launch_realign((int)esb, g->n, g->k, g->b, SKL_TE, g->b_s0, g->b_s1, 1, 0, g->b_sk,
+                                       scratch + mp * kp * esa, kp));
+  if (r == TAKEN) {
     h.a = scratch, h.a_sk = 1, h.a_s0 = kp, h.a_s1 = SKL_TE * kp;
     h.b = scratch + mp * kp * esa, h.b_sk = 1, h.b_s0 = kp, h.b_s1 = SKL_TE * kp;
     h.k = kp;
-    done = skl_hip_launch_gemm_mfma_padded(&h, tile_cols) == 0;
+    r = outcome(skl_hip_launch_gemm_mfma_padded(&h, tile_cols));
   }
   skl_hip_sequence_end();
-  return done;
+  return r;
 }
 
 /* Any other blocking (the 4x8 / 8x4 / 4x4 blocks of src/gemm/packed-gemm.md:270-298, blocks of 32, ...): A and B
@@ -323,8 +339,8 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   const int c_is_read = !(d->ta == SKL_DT_I8 && d->beta.i == 0);
   skl_gemm_canon h;
   char *scratch;
-  int done, c_in_place;
-  if (esa > 2 || esb > 2 || M * N * K < ((size_t)1 << 18)) return 0;
+  int r, c_in_place;
+  if (esa > 2 || esb > 2 || M * N * K < ((size_t)1 << 18)) return DECLINED;
   memset(&h, 0, sizeof h);
   h.ta = d->ta, h.tb = d->tb;
   h.m = M, h.n = N, h.k = K;
@@ -347,24 +363,25 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
     h.rsc0 = N, h.rsc1 = SKL_TE * N, h.csc0 = 1, h.csc1 = SKL_TE;
     h.c_row_shift = h.c_col_shift = 6;
   }
-  if (!gemm_fast_path(&h, fused, 0)) return 0;
+  if (gemm_fast_path(&h, fused, 0) != TAKEN) return DECLINED;
   skl_hip_sequence_begin();
   scratch = skl_hip_operand_scratch(bytes_a + bytes_b + (c_in_place ? 0 : M * N * 4));
-  done = scratch != NULL;
-  if (done) {
+  r = scratch != NULL ? TAKEN : DECLINED;
+  if (r == TAKEN) {
     h.a = scratch, h.b = scratch + bytes_a;
     if (!c_in_place) h.c = scratch + bytes_a + bytes_b;
-    done = skl_hip_launch_realign((int)esa, M, K, d->a, d->m0, d->rsa0, d->rsa1, d->k0, d->csa0, d->csa1, scratch, kpa) == 0 &&
-           skl_hip_launch_realign((int)esb, N, K, d->b, d->n0, d->csb0, d->csb1, d->k0, d->rsb0, d->rsb1,
-                                  scratch + bytes_a, kpb) == 0 &&
-           (c_in_place || !c_is_read ||
-            skl_hip_launch_unpack(4, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, M, N, h.c, N, 1) == 0);
+    r = outcome(skl_hip_launch_realign((int)esa, M, K, d->a, d->m0, d->rsa0, d->rsa1, d->k0, d->csa0, d->csa1, scratch, kpa));
   }
-  if (done) done = gemm_fast_path(&h, fused, 1);
-  if (done && !c_in_place && !d->rq.q_only) /* with q_only the result went to the requantised copy alone */
-    done = skl_hip_launch_pack(4, M, N, h.c, N, 1, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, 0) == 0;
+  if (r == TAKEN)
+    r = outcome(skl_hip_launch_realign((int)esb, N, K, d->b, d->n0, d->csb0, d->csb1, d->k0, d->rsb0, d->rsb1,
+                                       scratch + bytes_a, kpb));
+  if (r == TAKEN && !c_in_place && c_is_read)
+    r = outcome(skl_hip_launch_unpack(4, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, M, N, h.c, N, 1));
+  if (r == TAKEN) r = gemm_fast_path(&h, fused, 1); /* the caller's C is untouched until this has launched */
+  if (r == TAKEN && !c_in_place && !d->rq.q_only) /* with q_only the result went to the requantised copy alone */
+    r = outcome(skl_hip_launch_pack(4, M, N, h.c, N, 1, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, 0)) == TAKEN ? TAKEN : FAILED;
   skl_hip_sequence_end();
-  return done;
+  return r;
 }
 
 /* K-packed B with more rows of A than one call of the decode-batch kernel takes: chunks of 16 rows, one pass over
@@ -373,54 +390,59 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
 static int k4_in_row_chunks(const skl_gemm_desc *d) {
   skl_gemm_canon g;
   int launch;
-  if (d->ta != SKL_DT_I8 || d->k0 != 4 || d->m0 != 1 || d->m1 <= 16 || d->m1 > 112) return 0;
+  if (d->ta != SKL_DT_I8 || d->k0 != 4 || d->m0 != 1 || d->m1 <= 16 || d->m1 > 112) return DECLINED;
   for (launch = 0; launch < 2; ++launch) {
     size_t i;
+    /* A chunk that fails after others have run would leave C half updated: the one thing a chunk may lack, the
+     * scratch of the single-row kernel, is reserved before the first is launched. */
+    if (launch && d->m1 % 16 == 1 && skl_hip_gemv_reserve_scratch() != 0) return DECLINED;
     for (i = 0; i < d->m1; i += 16) {
       skl_gemm_desc part = *d;
+      int rc = 0;
       part.m1 = d->m1 - i < 16 ? d->m1 - i : 16;
       part.a = (const char *)d->a + i * d->rsa1;
       part.c = (char *)d->c + 4 * i * d->rsc1;
       if (part.m1 == 1) {
-        if (!canonicalize_k4(&part, &g, 0) || !skl_hip_gemv_supported(&g, 1)) return 0;
-        if (launch) skl_hip_launch_gemv(&g, 1);
+        if (!canonicalize_k4(&part, &g, 0) || !skl_hip_gemv_supported(&g, 1)) return DECLINED;
+        if (launch) rc = skl_hip_launch_gemv(&g, 1);
       } else {
-        if (!canonicalize_k4(&part, &g, 1) || !skl_hip_gemv_mfma_rows_supported(&g, 1)) return 0;
-        if (launch) skl_hip_launch_gemv_mfma_rows(&g, 1);
+        if (!canonicalize_k4(&part, &g, 1) || !skl_hip_gemv_mfma_rows_supported(&g, 1)) return DECLINED;
+        if (launch) rc = skl_hip_launch_gemv_mfma_rows(&g, 1);
+      }
+      if (rc != 0) return FAILED; /* a launch error of the device: recorded, C is not to be relied on */
+    }
+  }
+  return TAKEN;
+}
+
+/* 0, or nonzero when no kernel could be launched (the error is recorded). */
+static int gemm_on_device(const skl_gemm_desc *d) {
+  skl_gemm_canon g;
+  const int fused = d->bias != NULL || d->max != NULL || d->rq.act != 0 || d->rq.q != NULL; /* the M = 1 kernels have no fused steps */
+  int r = DECLINED;
+  if (d->k0 * d->k1 != 0 && d->ta <= SKL_DT_F8E5M2) {
+    if (!fused && canonicalize_k4(d, &g, 0) && skl_hip_gemv_supported(&g, 1)) r = outcome(skl_hip_launch_gemv(&g, 1));
+    if (r == DECLINED && !fused && canonicalize_k4(d, &g, 1) && skl_hip_gemv_mfma_rows_supported(&g, 1))
+      r = outcome(skl_hip_launch_gemv_mfma_rows(&g, 1));
+    if (r == DECLINED && !fused) r = k4_in_row_chunks(d);
+    if (r == DECLINED) {
+      if (canonicalize(d, &g)) {
+        if (!fused) r = gemv_paths(&g, 1);
+        if (r == DECLINED) r = gemm_padded_to_tiles(&g);
+        if (r == DECLINED) r = gemm_fast_path(&g, fused, 1);
+        if (r == DECLINED) r = gemm_with_realigned_operands(&g, fused);
+      } else {
+        r = gemm_through_copies(d, fused);
       }
     }
   }
-  return 1;
-}
-
-static void gemm_on_device(const skl_gemm_desc *d) {
-  skl_gemm_canon g;
-  const int fused = d->bias != NULL || d->max != NULL || d->rq.act != 0 || d->rq.q != NULL; /* the M = 1 kernels have no fused steps */
-  if (d->k0 * d->k1 != 0 && d->ta <= SKL_DT_F8E5M2) {
-    if (!fused && canonicalize_k4(d, &g, 0) && skl_hip_gemv_supported(&g, 1)) {
-      skl_hip_launch_gemv(&g, 1);
-      return;
-    }
-    if (!fused && canonicalize_k4(d, &g, 1) && skl_hip_gemv_mfma_rows_supported(&g, 1)) {
-      skl_hip_launch_gemv_mfma_rows(&g, 1);
-      return;
-    }
-    if (!fused && k4_in_row_chunks(d)) return;
-    if (canonicalize(d, &g)) {
-      if (!fused && gemv_paths(&g, 1)) return;
-      if (gemm_padded_to_tiles(&g)) return;
-      if (gemm_fast_path(&g, fused, 1)) return;
-      if (gemm_with_realigned_operands(&g, fused)) return;
-    } else if (gemm_through_copies(d, fused)) {
-      return;
-    }
-  }
-  if (d->k0 * d->k1 != 0 && !fused && canonicalize(d, &g) && skl_hip_gemm_tiled_supported(&g) &&
-      g.m * g.n * g.k >= ((size_t)1 << 15)) {
-    skl_hip_launch_gemm_tiled(&g);
-    return;
-  }
-  skl_hip_launch_gemm_generic(d);
+  if (r == DECLINED && d->k0 * d->k1 != 0 && !fused && canonicalize(d, &g) && skl_hip_gemm_tiled_supported(&g) &&
+      g.m * g.n * g.k >= ((size_t)1 << 15))
+    r = outcome(skl_hip_launch_gemm_tiled(&g));
+  if (r == DECLINED) r = outcome(skl_hip_launch_gemm_generic(d)); /* needs no scratch memory */
+  /* a kernel further down the list ran in place of one that could not get its scratch memory: the call succeeded */
+  if (r == TAKEN) skl_hip_withdraw_error(SKL_HIP_ERR_WORKSPACE);
+  return r == TAKEN ? 0 : -1;
 }
 
 /* The kinds whose alpha and beta travel as a float (F16H: widened). */
@@ -462,7 +484,7 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
     }
   }
   if (where == 1) {
-    gemm_on_device(d);
+    (void)gemm_on_device(d);
     return;
   }
   {
@@ -497,10 +519,11 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
     dd.max = dmax;
     dd.rq.q = dq;
     dd.rq.q_scale = dqs;
-    gemm_on_device(&dd);
-    skl_hip_memcpy_d2h(d->c, dc, nc * esc);
-    if (dmax) skl_hip_memcpy_d2h(d->max, dmax, esc);
-    if (dq) skl_hip_memcpy_d2h(d->rq.q, dq, nq);
+    if (gemm_on_device(&dd) == 0) { /* after a failure the caller's memory stays as it was */
+      skl_hip_memcpy_d2h(d->c, dc, nc * esc);
+      if (dmax) skl_hip_memcpy_d2h(d->max, dmax, esc);
+      if (dq) skl_hip_memcpy_d2h(d->rq.q, dq, nq);
+    }
     skl_hip_free(dq);
     skl_hip_free(dqs);
     skl_hip_free(da);

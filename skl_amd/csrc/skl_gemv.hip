@@ -1389,6 +1389,11 @@ unsigned long long *noalloc_slots_of_current_device() {
 }
 }  // namespace
 
+extern "C" int skl_hip_gemv_reserve_scratch(void) {
+  Reduction red;
+  return reduction_scratch(&red) ? 0 : -4;  // SKL_HIP_ERR_WORKSPACE
+}
+
 extern "C" int skl_hip_noalloc_setup(void) { return noalloc_slots_of_current_device() ? 0 : -2; }
 
 extern "C" size_t skl_hip_noalloc_max_sums(void) { return kNoAllocSlots; }

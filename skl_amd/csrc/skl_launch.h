@@ -138,6 +138,8 @@ int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
 int skl_hip_noalloc_setup(void);
 size_t skl_hip_noalloc_max_sums(void);
 int skl_hip_launch_gemv_noalloc(const skl_gemm_canon *g);
+/* Makes sure the current stream has the sums-and-counters block of the single-row kernels; 0 or SKL_HIP_ERR_WORKSPACE. */
+int skl_hip_gemv_reserve_scratch(void);
 
 /* A block of scratch memory of the current stream and device for operands copied into another layout ahead of a
  * launch (grows on demand, NULL when the device has no room; apart from the workspace of the split reductions). */
@@ -171,6 +173,8 @@ int skl_hip_launch_cvt_f4_f8e4m3(uint8_t *dst, const uint8_t *src, size_t n);
 
 /* Error recording shared by both layers. */
 void skl_hip_record_error(int code, const char *what);
+/* Forgets the calling thread's recorded error if it is `code` (a failure that a later step of the same call made good). */
+void skl_hip_withdraw_error(int code);
 
 #ifdef __cplusplus
 }

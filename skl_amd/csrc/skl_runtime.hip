@@ -33,8 +33,8 @@ struct StreamState {
   size_t zeroed_bytes = 0;
 };
 
-// Streams with scratch of their own per device; every further stream shares the last entry (calls on those
-// streams must then not overlap on the device).
+// Streams with scratch of their own per device. A further stream gets none (its calls run on the kernels that need
+// no scratch and an error is recorded) until skl_hip_release_stream() has given a slot back.
 constexpr size_t kMaxStreamStates = 32;
 
 struct DeviceState {
@@ -55,6 +55,10 @@ thread_local int t_error = SKL_HIP_OK;
 thread_local char t_error_text[256] = "no error";
 
 }  // namespace
+
+extern "C" void skl_hip_withdraw_error(int code) {
+  if (t_error == code) t_error = SKL_HIP_OK;
+}
 
 extern "C" void skl_hip_record_error(int code, const char *what) {
   if (code == SKL_HIP_OK || t_error != SKL_HIP_OK) return;  // keep the first error until it is read
@@ -105,15 +109,18 @@ DeviceState *current_device_state() {
   return &g_devices[dev];
 }
 
-// Under g_mutex: the scratch of the calling thread's stream on this device.
-StreamState &current_stream_state(DeviceState &st) {
+// Under g_mutex: the scratch of the calling thread's stream on this device; nullptr when every slot belongs to
+// another stream (two streams on one slot would mix their partial sums and counters).
+StreamState *current_stream_state(DeviceState &st) {
   for (StreamState &s : st.streams)
-    if (s.stream == t_stream) return s;
-  if (st.streams.size() < kMaxStreamStates) {
-    st.streams.emplace_back();
-    st.streams.back().stream = t_stream;
+    if (s.stream == t_stream) return &s;
+  if (st.streams.size() >= kMaxStreamStates) {
+    skl_hip_record_error(SKL_HIP_ERR_STREAM_SLOTS, "scratch memory: 32 streams hold a slot on this device - release one (skl_hip_release_stream)");
+    return nullptr;
   }
-  return st.streams.back();
+  st.streams.emplace_back();
+  st.streams.back().stream = t_stream;
+  return &st.streams.back();
 }
 
 }  // namespace
@@ -122,21 +129,28 @@ void *skl_workspace(size_t bytes) {
   DeviceState *st = current_device_state();
   if (!st) return nullptr;
   std::lock_guard<std::mutex> lock(g_mutex);
-  return grow(*st, current_stream_state(*st).workspace, bytes, kWorkspaceBytes, "skl_workspace", true);
+  StreamState *ss = current_stream_state(*st);
+  return ss ? grow(*st, ss->workspace, bytes, kWorkspaceBytes, "skl_workspace", true) : nullptr;
 }
 
 void *skl_zeroed_scratch(size_t bytes) {
   DeviceState *st = current_device_state();
   if (!st) return nullptr;
   std::lock_guard<std::mutex> lock(g_mutex);
-  StreamState &ss = current_stream_state(*st);
+  StreamState *slot = current_stream_state(*st);
+  if (!slot) return nullptr;
+  StreamState &ss = *slot;
   if (ss.zeroed) {
     if (bytes <= ss.zeroed_bytes) return ss.zeroed;
     skl_hip_record_error(SKL_HIP_ERR_BAD_ARGUMENT, "skl_zeroed_scratch: size differs from the first request");
     return nullptr;
   }
   void *p = nullptr;
-  if (skl_check_hip(hipMalloc(&p, bytes), "zeroed scratch") != 0) return nullptr;
+  if (hipMalloc(&p, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    skl_hip_record_error(SKL_HIP_ERR_WORKSPACE, "zeroed scratch");
+    return nullptr;
+  }
   // Cleared on the stream that will use it, and finished before any other stream can be handed the block.
   if (skl_check_hip(hipMemsetAsync(p, 0, bytes, t_stream), "zeroed scratch clear") != 0 ||
       skl_check_hip(hipStreamSynchronize(t_stream), "zeroed scratch clear") != 0) {
@@ -173,7 +187,28 @@ void *skl_hip_operand_scratch(size_t bytes) {
   if (!st) return nullptr;
   std::lock_guard<std::mutex> lock(g_mutex);
   // not recorded as an error: the caller falls back to a kernel that needs no copy
-  return grow(*st, current_stream_state(*st).operands, bytes, kOperandBytes, "skl_hip_operand_scratch", false);
+  StreamState *ss = current_stream_state(*st);
+  return ss ? grow(*st, ss->operands, bytes, kOperandBytes, "skl_hip_operand_scratch", false) : nullptr;
+}
+
+int skl_hip_release_stream(void *stream) {
+  DeviceState *st = current_device_state();
+  if (!st) return SKL_HIP_ERR_NO_DEVICE;
+  // The stream's work may still use the blocks: wait for it before they go (outside the lock; the caller has
+  // promised not to issue more work on the stream meanwhile).
+  int rc = skl_check_hip(hipStreamSynchronize((hipStream_t)stream), "skl_hip_release_stream");
+  if (rc != 0) return rc;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (size_t i = 0; i < st->streams.size(); ++i) {
+    StreamState &s = st->streams[i];
+    if (s.stream != (hipStream_t)stream) continue;
+    if (s.workspace.ptr) (void)hipFree(s.workspace.ptr);
+    if (s.operands.ptr) (void)hipFree(s.operands.ptr);
+    if (s.zeroed) (void)hipFree(s.zeroed);
+    st->streams.erase(st->streams.begin() + (long)i);
+    break;
+  }
+  return SKL_HIP_OK;
 }
 
 void skl_hip_sequence_begin(void) { g_sequence.lock(); }

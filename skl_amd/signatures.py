@@ -195,6 +195,7 @@ RUNTIME = {
     "skl_hip_set_beta_zero_mode": (None, "i"),
     "skl_hip_get_beta_zero_mode": (ctypes.c_int, ""),
     "skl_hip_pointer_is_device": (ctypes.c_int, "p"),
+    "skl_hip_release_stream": (ctypes.c_int, "p"),
     "skl_hip_last_error": (ctypes.c_int, ""),
     "skl_hip_last_error_string": (ctypes.c_char_p, ""),
     "skl_hip_te": (ctypes.c_size_t, ""),

@@ -33,9 +33,10 @@ static int g_nranges;
 static long g_checked, g_launches;
 static int g_failures;
 /* how often each stand-in ran: the summary shows which routes of the dispatch the cases reached */
-enum { P_GENERIC, P_TILED, P_MFMA, P_PADDED, P_GEMV, P_GEMV_K4, P_ROWS, P_MFMA_ROWS, P_MFMA_ROWS_K4, P_KC, P_REALIGN, P_PACK, P_UNPACK, P_CVT, P_COUNT };
+enum { P_GENERIC, P_TILED, P_MFMA, P_PADDED, P_GEMV, P_GEMV_K4, P_ROWS, P_MFMA_ROWS, P_MFMA_ROWS_K4, P_KC, P_REALIGN, P_PACK, P_UNPACK, P_CVT, P_SCARCE, P_COUNT };
 static const char *const kPathNames[P_COUNT] = {"any-stride", "register-tiled", "matrix-core", "padded tiles", "GEMV", "GEMV K-packed", "few rows",
-                                                "decode batch", "decode batch K-packed", "dot-product GEMV", "operand copy", "pack", "unpack", "cvt"};
+                                                "decode batch", "decode batch K-packed", "dot-product GEMV", "operand copy", "pack", "unpack", "cvt",
+                                                "declined: no scratch"};
 static long g_path[P_COUNT];
 
 static void range_add(const void *p, size_t bytes, int device) {
@@ -217,6 +218,23 @@ static void gemm_over_canon(const skl_gemm_canon *g, int layout, const char *who
 }
 
 /* ------------------------------------------------------------------ the redirected GPU layer */
+/* Scratch memory runs out: every kernel that would use some reports so before launching anything, as the real
+ * launchers do, and the copies of operands get no memory either. The call must then end on a kernel that needs
+ * none, with the right result and no error left recorded. */
+static int g_scarce;
+#define SCARCE(what)                                          \
+  do {                                                        \
+    if (g_scarce) {                                           \
+      ++g_path[P_SCARCE];                                     \
+      skl_hip_record_error(SKL_HIP_ERR_WORKSPACE, what);      \
+      return SKL_HIP_ERR_WORKSPACE;                           \
+    }                                                         \
+  } while (0)
+int __wrap_skl_hip_gemv_reserve_scratch(void) {
+  SCARCE("reserve (stand-in)");
+  return 0;
+}
+
 #define EXPECT(cond, what) \
   do {                     \
     if (!(cond)) fail(what); \
@@ -234,12 +252,14 @@ int __wrap_skl_hip_launch_gemm_tiled(const skl_gemm_canon *g) {
   return 0;
 }
 int __wrap_skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
+  SCARCE("matrix-core GEMM (stand-in)");
   EXPECT(skl_hip_gemm_mfma_supported(g), "matrix-core GEMM handed a problem it does not support");
   ++g_path[P_MFMA];
   gemm_over_canon(g, 0, "matrix-core GEMM");
   return 0;
 }
 int __wrap_skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile_cols) {
+  SCARCE("padded GEMM (stand-in)");
   const size_t es = esize(g->ta);
   EXPECT(tile_cols == 256 || tile_cols == 128, "padded GEMM: tile width");
   EXPECT(g->a_sk == 1 && g->b_sk == 1 && (g->k * es) % 128 == 0, "padded GEMM: K not padded to whole slice pairs");
@@ -252,24 +272,28 @@ int __wrap_skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile_col
   return 0;
 }
 int __wrap_skl_hip_launch_gemv(const skl_gemm_canon *g, int layout) {
+  SCARCE("GEMV (stand-in)");
   EXPECT(skl_hip_gemv_supported(g, layout), "GEMV handed a problem it does not support");
   ++g_path[layout ? P_GEMV_K4 : P_GEMV];
   gemm_over_canon(g, layout, "GEMV");
   return 0;
 }
 int __wrap_skl_hip_launch_gemv_rows(const skl_gemm_canon *g) {
+  SCARCE("few-rows GEMV (stand-in)");
   EXPECT(skl_hip_gemv_rows_supported(g), "few-rows GEMV handed a problem it does not support");
   ++g_path[P_ROWS];
   gemm_over_canon(g, 0, "few-rows GEMV");
   return 0;
 }
 int __wrap_skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g, int layout) {
+  SCARCE("decode batch (stand-in)");
   EXPECT(skl_hip_gemv_mfma_rows_supported(g, layout), "decode-batch kernel handed a problem it does not support");
   ++g_path[layout ? P_MFMA_ROWS_K4 : P_MFMA_ROWS];
   gemm_over_canon(g, layout, "decode-batch kernel");
   return 0;
 }
 int __wrap_skl_hip_launch_gemv_kc(const skl_gemm_canon *g) {
+  SCARCE("dot-product GEMV (stand-in)");
   EXPECT(skl_hip_gemv_kc_supported(g), "dot-product GEMV handed a problem it does not support");
   ++g_path[P_KC];
   gemm_over_canon(g, 0, "dot-product GEMV");
@@ -405,6 +429,7 @@ int __wrap_skl_hip_pointer_is_device(const void *p) {
 static void *g_operand_scratch;
 static size_t g_operand_scratch_bytes;
 void *__wrap_skl_hip_operand_scratch(size_t bytes) {
+  if (g_scarce) return NULL; /* not an error: the caller goes on to a kernel that needs no copy */
   if (bytes > g_operand_scratch_bytes) { /* like the library's block: grows, the address may change */
     if (g_operand_scratch) {
       range_remove(g_operand_scratch);
@@ -715,6 +740,9 @@ int main(int argc, char **argv) {
       default: run_gemm_case(device_pointers); break;
     }
   }
+  g_scarce = 1;
+  for (int t = 0; t < cases / 4 && !g_failures; ++t) run_gemm_case((int)(rnd() % 2));
+  g_scarce = 0;
   if (!g_failures && argc <= 2) run_large_cases();  /* with a seed: random cases only */
   if (g_nranges != (g_operand_scratch ? 1 : 0)) fail("a buffer of the host layer was not released");
   printf("%s: %d cases, %ld launches carried out, %ld address ranges checked\n", g_failures ? "host layer check FAILED" : "host layer ok",

@@ -494,6 +494,54 @@ def test_few_tiles_long_k_shares_k_between_workgroups(gpu, ta, m, n, k):
     assert top[0] == want_top[0]
 
 
+def test_stream_slots_run_out_and_come_back(gpu):
+    """A device keeps scratch memory for 32 streams. A call on a further stream still gives the right result - on a
+    kernel that needs no scratch - and records the advisory SKL_HIP_ERR_STREAM_SLOTS; once a stream has been
+    released (skl_hip_release_stream), the same call runs without a word."""
+    import ctypes as ct
+    from skl_amd import DeviceBuffer
+
+    hip = ct.CDLL("libamdhip64.so.7")
+    hip.hipStreamCreate.restype = hip.hipStreamDestroy.restype = ct.c_int
+    case = rowmajor_case("i8", 1, 2048, 4096, alpha=1, beta=0)   # a GEMV: its workgroups meet in the stream's scratch
+    a, b, c = case.make_inputs(4242)
+    want = run_oracle_gemm(case, a, b, c)
+    da, db, dc = DeviceBuffer.from_array(a), DeviceBuffer.from_array(b), DeviceBuffer.from_array(c)
+    streams, codes = [], []
+    gpu.skl_hip_set_pointer_mode(1)
+
+    def call_on(stream):
+        gpu.skl_hip_set_stream(stream.value)
+        gpu.skl_hip_memcpy_h2d(dc, c, c.nbytes)
+        gpu.skl_gemm_i8_i8_i32_gfx950(1, 2048, 4096, 1, da, case.rsa1, db, case.rsb1, 0, dc, case.rsc1)
+        assert gpu.skl_hip_synchronize() == 0
+        code = gpu.skl_hip_last_error()
+        assert np.array_equal(dc.download(c.dtype, c.size), want), (len(streams), code)
+        return code
+
+    try:
+        for _ in range(34):   # other tests of this process may hold a few slots already
+            stream = ct.c_void_p()
+            assert hip.hipStreamCreate(ct.byref(stream)) == 0
+            streams.append(stream)
+            codes.append(call_on(stream))
+            if codes[-1] != 0:
+                break
+        assert codes[-1] == -5 and all(code == 0 for code in codes[:-1]), codes
+        assert call_on(streams[-1]) == -5           # and again: nothing was claimed meanwhile
+        assert gpu.skl_hip_release_stream(streams[0].value) == 0
+        assert call_on(streams[-1]) == 0            # the freed slot is this stream's now
+    finally:
+        gpu.skl_hip_set_stream(None)
+        gpu.skl_hip_set_pointer_mode(0)
+        for stream in streams:
+            gpu.skl_hip_release_stream(stream.value)
+            hip.hipStreamDestroy(stream)
+        for d in (da, db, dc):
+            d.free()
+        gpu.skl_hip_last_error()
+
+
 def test_mixed_e4m3_e5m2(gpu):
     for (m, n, k) in ((13, 21, 37), (128, 192, 256)):
         case = rowmajor_case("f8e4m3", m, n, k, 1.0, 0.0, tb="f8e5m2")
@@ -702,6 +750,7 @@ def test_host_threads_on_streams_of_their_own(gpu):
                 for d in trio:
                     d.free()
             if stream:
+                gpu.skl_hip_release_stream(stream.value)
                 hip.hipStreamDestroy(stream)
 
     threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]

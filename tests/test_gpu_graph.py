@@ -86,6 +86,7 @@ def test_decode_loop_replays_from_a_graph(gpu):
             hip.hipGraphExecDestroy(executable)
         if graph:
             hip.hipGraphDestroy(graph)
+        gpu.skl_hip_release_stream(stream.value)
         hip.hipStreamDestroy(stream)
         for d in w + y + [wt, w16, wb, x, xs, a16, xb, yt, ys, y16, yb]:
             d.free()
