@@ -14,33 +14,35 @@
 // the arithmetic is ref/gemm/gemm_i8rc_i8rc_i32rc.c:10-26 with m = 1.
 //
 // Work decomposition (row-major B, int8): a lane owns 16 consecutive columns
-// (one 128-bit load per row) and ROWS_PER_LANE consecutive rows; eight lanes
-// cover one 128-byte line of a row and the eight lane-groups of a wave take
-// different row ranges, so a workgroup streams a 128-column strip of
-// kRowsPerGroup rows with every load instruction touching eight full lines and
-// all loads of a wave in flight before the first use. Four rows at a time are
-// transposed in registers (v_perm_b32) so that v_dot4_i32_i8 multiplies four
-// k-values of one column with four packed x bytes. The 32 partial sums per
-// column of a workgroup meet in LDS; the few workgroups that share a column
-// strip (K / kRowsPerGroup of them) meet in a zero-initialised int32 accumulator
-// in device memory through relaxed device-scope atomics (integer adds: exact in
-// any order). The slot is 64 bits wide: the sum lives in the high word and an
-// arrival count in the low word, one atomic add carries both and returns the
-// previous value, so the lane whose add completes the count knows the total,
-// applies alpha and beta, writes y and puts the slot back to zero - one round
-// trip to memory after the last byte of B has arrived. (The floating-point
-// modes cannot fold a count into the sum: there a ticket counter per strip
-// tells the workgroup that arrives last to read the totals back. Only atomics
-// carry data between workgroups, so ordering needs no cache write-back: a wait
-// for the workgroup's outstanding atomics before the ticket is taken is enough;
-// a device-scope fence would flush the whole L2 and costs ten times the kernel.)
+// (one 128-bit load per row) and ROWS_PER_LANE consecutive rows; a pair of lanes
+// reads 32 adjacent bytes of a row, the four pairs of a wave that sit at the same
+// place in the four rows of 16 lanes cover one 128-byte line, and the eight row
+// groups of a wave sit inside each row of 16 lanes. A workgroup (eight waves)
+// streams a 128-column strip of kRowsPerGroup rows with all loads of every lane
+// in flight before the first use. Four rows at a time are transposed in
+// registers (v_perm_b32) so that v_dot4_i32_i8 multiplies four k-values of one
+// column with four packed x bytes. The eight row groups of a wave are summed in
+// registers with three DPP rotations; one partial sum per wave and column goes
+// through LDS. The few workgroups that share a column strip (K / kRowsPerGroup
+// of them) meet in a zero-initialised accumulator in device memory through
+// relaxed device-scope atomics (integer adds: exact in any order). The slot is
+// 64 bits wide: the sum lives in the high word and an arrival count in the low
+// word, one atomic add carries both and returns the previous value, so the lane
+// whose add completes the count knows the total, applies alpha and beta - the
+// old y was asked for when the kernel started - writes y and puts the slot back
+// to zero: one round trip to memory after the last byte of B has arrived.
+// Floating-point sums depend on their order, so those modes do not add into a
+// shared slot: every workgroup stores its sums to a plane of its own, and the
+// one that draws the last ticket of the strip adds the planes in slab order
+// (ordered_sum_over_slabs): the same bits on every run. Ordering needs no cache
+// write-back: a wait for the workgroup's own stores before the ticket is taken
+// is enough; a device-scope fence would flush the whole L2 and costs ten times
+// the kernel.
 //
 // The same skeleton serves more operand kinds: OCP fp8 weights and x (E4M3, E5M2 and E4M3 x with E5M2
 // weights; a lane owns 16 columns, the hardware conversions decode to fp32), bf16 and f16 weights
-// (a lane owns 8 columns, fp32 accumulation with v_fma, fp32 atomics between
-// workgroups - the summation order then varies from run to run, within the
-// reference's tolerance) and the K-packed int8 layout of the dot4 entry point
-// (B(4P+p, j) at P*rsb1 + 4j + p: a 128-bit load holds four columns times four
+// (a lane owns 8 columns, fp32 accumulation with v_fma) and the K-packed int8 layout of the dot4
+// entry point (B(4P+p, j) at P*rsb1 + 4j + p: a 128-bit load holds four columns times four
 // k, which v_dot4_i32_i8 consumes without any byte shuffling).
 #include <hip/hip_runtime.h>
 
@@ -395,7 +397,8 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
 // out inside each row of 16 lanes, so their sums are combined with three DPP rotations; the eight waves
 // meet in LDS, and the workgroups of a strip meet in one 64-bit slot per (row, column) like the M = 1 kernel.
 // The floating-point kinds (bf16, f16, fp8) run on the same skeleton: a loaded row of B is widened once and
-// multiplied with the x value of every row, fp32 sums, fp32 atomics and a ticket between workgroups.
+// multiplied with the x value of every row, fp32 sums; between workgroups the sums travel in planes that the
+// last workgroup of a strip adds in slab order, as in the M = 1 kernel (the same bits on every run).
 // ---------------------------------------------------------------------------
 constexpr int kMaxRows = 8;
 
@@ -628,11 +631,13 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
 // arithmetic wraps, so beta*c + alpha*s1 + alpha*s2 + ... equals beta*c + alpha*(s1 + s2 + ...) bit for bit.
 // (Partial sums in planes and a second kernel that adds them: 19 us for 16 x 4096 x 11008; 64-bit atomics that
 // carry an arrival count like the M = 1 kernel's: 19 us; this: 15 us, and 13 us for 5 rows.)
-// OCP fp8 (E4M3, E5M2, E4M3 A with E5M2 B) runs on the same skeleton with v_mfma_f32_16x16x32_{fp8,bf8}_{fp8,bf8}
-// (8 bytes of K per lane: two instructions per column and block). Floating-point sums depend on their order and
-// the reference's epilogue rounds beta*c + alpha*acc in one place, so here each workgroup stores its raw sums to
-// its own plane of the stream's workspace and a second kernel adds the planes in order, applies alpha / beta and
-// the fused steps: deterministic, at the accuracy of the fp8 matrix-core instructions like the tile kernels.
+// OCP fp8 (E4M3, E5M2, E4M3 A with E5M2 B) runs on the same skeleton: every E4M3 / E5M2 value is an f16 value, so
+// the bytes are widened in registers (exactly) and multiplied with v_mfma_f32_16x16x32_f16, whose products are
+// exact and whose sums are fp32 - the fp8 matrix-core instructions drop bits below the largest product of an
+// instruction, and here the arithmetic is free (8 values of K per lane and instruction: two per column and block).
+// Floating-point sums depend on their order and the reference's epilogue rounds beta*c + alpha*acc in one place, so
+// here each workgroup stores its raw sums to its own plane of the stream's workspace and a second kernel adds the
+// planes in order, applies alpha / beta and the fused steps: deterministic.
 // bf16 / f16: a 128-bit load holds 8 columns and v_mfma_f32_16x16x32_{bf16,f16} wants 8 consecutive k per lane, so a
 // lane loads 8 rows of 8 columns and transposes 8 x 8 halfwords (one v_perm_b32 per dword of the result); 16 lanes
 // cover 128 columns, the four lane groups 32 rows, a wave takes four such blocks. Raw sums in planes like fp8.

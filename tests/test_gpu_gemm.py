@@ -30,6 +30,11 @@ def check(gpu, kind, case, seed, mode):
     if case.is_int or case.ta == "f16h":  # the half-accumulating GEMM is defined operation by operation
         want = run_oracle_gemm(case, a, b, c)
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (kind, vars(case))
+        if case.ta == "f16h":
+            # Bit-identity holds against the reference as compiled for x86 (product in float, one rounding to half per
+            # step); hardware with half arithmetic rounds the product too. What every evaluation must meet is the
+            # reference test's own bound (P = 11, test/gemm/gemm_f16rcprc_f16rcprc_f16rcprc.c:157): applied as well.
+            support.assert_fp_gemm_close(case, a, b, c, got, frob_tol=None)
     else:
         fp8 = case.ta.startswith("f8")
         support.assert_fp_gemm_close(case, a, b, c, got, extra_rel=support.FP8_MFMA_REL if fp8 else 0.0)
