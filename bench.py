@@ -190,19 +190,22 @@ def wl_gemv_p4x1c(lib, rng):
                 name="int8 GEMV 1x4096x11008 (W in the p4x1c K-packed layout, beta=0)", kernel="gemv_kernel<int8 K-packed>")
 
 
-def wl_small_batch_p4x1c(lib, rng):
-    """Decode with a batch of 16 against the same prepacked weights: the K-packed B read in place, no transposes."""
-    m, k, n, nbuf = 16, 4096, 11008, 8
-    w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
-    x = DeviceBuffer.from_array(rand_i8(rng, m * k))
-    y = DeviceBuffer(4 * m * n)
+def _wl_small_batch_p4x1c(m):
+    """Decode with a batch of m rows against the same prepacked weights: the K-packed B read in place, no transposes."""
+    def build(lib, rng):
+        k, n, nbuf = 4096, 11008, 8
+        w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+        x = DeviceBuffer.from_array(rand_i8(rng, m * k))
+        y = DeviceBuffer(4 * m * n)
 
-    def step(i):
-        lib.skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(m, n, k // 4, 1, x, k, 4, w[i % nbuf], 4 * n, 0, y, n)
+        def step(i):
+            lib.skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(m, n, k // 4, 1, x, k, 4, w[i % nbuf], 4 * n, 0, y, n)
 
-    return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
-                name="int8 GEMM 16x4096x11008 (W in the p4x1c K-packed layout, decode with a batch of 16)",
-                kernel="gemv_mfma_scale_c_kernel + gemv_mfma_rows_kernel<int8 K-packed>")
+        kernel = "gemv_mfma_rows_kernel<int8 K-packed>" if m <= 16 else "gemv_k4_rowgroups_kernel"
+        return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
+                    name=f"int8 GEMM {m}x4096x11008 (W in the p4x1c K-packed layout, decode with a batch of {m})",
+                    kernel="gemv_mfma_scale_c_kernel + " + kernel)
+    return build
 
 
 def wl_gemv_bf16(lib, rng):
@@ -474,7 +477,10 @@ WORKLOADS = {
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 10, 2, 64),
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 10, 2, 64),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 10, 2, 64),
-    "gemm_i8_p4x1c_16x4096x11008": (wl_small_batch_p4x1c, 10, 2, 64),
+    "gemm_i8_p4x1c_16x4096x11008": (_wl_small_batch_p4x1c(16), 10, 2, 64),
+    "gemm_i8_p4x1c_32x4096x11008": (_wl_small_batch_p4x1c(32), 10, 2, 32),
+    "gemm_i8_p4x1c_112x4096x11008": (_wl_small_batch_p4x1c(112), 10, 2, 32),
+    "gemm_i8_p4x1c_512x4096x11008": (_wl_small_batch_p4x1c(512), 5, 1, 8),
     "gemm_f8e4m3_16x4096x11008": (wl_small_batch_f8, 10, 2, 64),
     "gemm_bf16_8x4096x11008": (wl_small_batch_bf16, 10, 2, 32),
     "peak_mfma_i8_random": (_wl_peak_mfma(0, "i8", 1), 3, 1, 1),

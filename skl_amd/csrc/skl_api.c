@@ -152,11 +152,11 @@ static int canonicalize(const skl_gemm_desc *d, skl_gemm_canon *g) {
   return canonicalize_c(d, g, 0);
 }
 
-/* The K4-interleaved int8 layout of the dot4 entry point: one row of A (`rows` == 0), or up to 16 rows that are
- * contiguous in K and lie in one block of C's rows. */
+/* The K4-interleaved int8 layout of the dot4 entry point: one row of A (`rows` == 0), or 2 to 128 rows that are
+ * contiguous in K. */
 static int canonicalize_k4(const skl_gemm_desc *d, skl_gemm_canon *g, int rows) {
   if (d->ta != SKL_DT_I8 || d->k0 != 4 || d->n0 != 1) return 0;
-  if (rows ? (d->m0 != 1 || d->m1 < 2 || d->m1 > 16) : d->m0 * d->m1 != 1) return 0;
+  if (rows ? (d->m0 != 1 || d->m1 < 2 || d->m1 > 128) : d->m0 * d->m1 != 1) return 0;
   if (d->rsb0 != 1 || d->csb1 != 4 || d->csa0 != 1) return 0;
   if (!(d->k1 == 1 || d->csa1 == 4)) return 0;
   memset(g, 0, sizeof *g);
@@ -384,22 +384,23 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   return r;
 }
 
-/* K-packed B with more rows of A than one call of the decode-batch kernel takes: chunks of 16 rows, one pass over
- * B each. Up to 112 rows that is cheaper than copying B into a layout the tile kernels read (17 x 4096 x 11008:
- * 126 us on copies). Every chunk is checked before the first is launched. */
+/* K-packed B with more rows of A than one call of the decode-batch kernel takes (128): chunks of 128 rows, one pass
+ * over B each. Up to 1024 rows that is cheaper than copying B into a layout the tile kernels read (the byte-wise
+ * copy of 4096 x 11008 out of its groups of four k alone costs about 100 us). Every chunk is checked before the
+ * first is launched. */
 static int k4_in_row_chunks(const skl_gemm_desc *d) {
   skl_gemm_canon g;
   int launch;
-  if (d->ta != SKL_DT_I8 || d->k0 != 4 || d->m0 != 1 || d->m1 <= 16 || d->m1 > 112) return DECLINED;
+  if (d->ta != SKL_DT_I8 || d->k0 != 4 || d->m0 != 1 || d->m1 <= 128 || d->m1 > 1024) return DECLINED;
   for (launch = 0; launch < 2; ++launch) {
     size_t i;
     /* A chunk that fails after others have run would leave C half updated: the one thing a chunk may lack, the
      * scratch of the single-row kernel, is reserved before the first is launched. */
-    if (launch && d->m1 % 16 == 1 && skl_hip_gemv_reserve_scratch() != 0) return DECLINED;
-    for (i = 0; i < d->m1; i += 16) {
+    if (launch && d->m1 % 128 == 1 && skl_hip_gemv_reserve_scratch() != 0) return DECLINED;
+    for (i = 0; i < d->m1; i += 128) {
       skl_gemm_desc part = *d;
       int rc = 0;
-      part.m1 = d->m1 - i < 16 ? d->m1 - i : 16;
+      part.m1 = d->m1 - i < 128 ? d->m1 - i : 128;
       part.a = (const char *)d->a + i * d->rsa1;
       part.c = (char *)d->c + 4 * i * d->rsc1;
       if (part.m1 == 1) {

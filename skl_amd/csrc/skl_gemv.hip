@@ -849,6 +849,100 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
 
 
 // ---------------------------------------------------------------------------
+// 17 to 128 rows of int8 A against the K-packed B: the kernel above with RG groups of 16 rows. B's bytes are loaded
+// once and stay in registers while the row groups take their turns (a pass over B per 16 rows, as chunked calls of
+// the kernel above cost, is what this saves: 112 x 4096 x 11008 took 110 us in seven passes). The A fragment of a
+// row group - 16 bytes per lane and block, from L2 - is requested two groups ahead; the sums of a group (16
+// registers) go through the same LDS block as above, one group at a time, and meet the other workgroups' in C.
+// ---------------------------------------------------------------------------
+constexpr int kK4MaxRowGroups = 8;
+
+template <int RG>
+__global__ void __launch_bounds__(kMfmaWaves * 64, 2) gemv_k4_rowgroups_kernel(GemvMfmaArgs p) {
+  using Sh = MfmaShape<1, true>;
+  constexpr int LC = Sh::kLaneCols, LR = Sh::kLaneRows, ITERS = Sh::kIters;
+  static_assert(LC == 4 && LR == 4, "four columns x four k per 128-bit load");
+  typedef int v4i __attribute__((ext_vector_type(4)));
+  extern __shared__ __attribute__((aligned(16))) int mfma_red_raw[];
+  int(*red)[16][Sh::kPitch] = reinterpret_cast<int(*)[16][Sh::kPitch]>(mfma_red_raw);
+  const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int jl = lane & 15, g = lane >> 4;
+  const size_t col = (size_t)tile * Sh::kTileCols + (size_t)jl * LC;
+  const size_t kwave = ((size_t)slab * kMfmaWaves + wave) * (Sh::kBlockK * ITERS);
+  const bool col_ok = col < p.n;  // n is a multiple of four
+  const char *bp = p.b + col * 4;
+
+  uint4 rows[ITERS][LR];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * 16;
+#pragma unroll
+    for (int r = 0; r < LR; ++r) {
+      if (col_ok && k0 + (size_t)r * 4 < p.k)
+        rows[it][r] = stream_load(bp + (k0 / 4 + r) * p.b_sk);
+      else
+        rows[it][r] = make_uint4(0, 0, 0, 0);
+    }
+  }
+  // The lane's 16 k of row 16 rg + jl, for each of the wave's blocks; zeros beyond M and K.
+  auto fragment_of = [&](int rg, v4i(&xa)[ITERS]) {
+    const size_t row = (size_t)rg * 16 + jl;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * 16;
+      if (row < p.m && k0 < p.k)
+        xa[it] = *reinterpret_cast<const v4i *>(p.a + row * p.a_row + k0);
+      else
+        xa[it] = v4i{0, 0, 0, 0};
+    }
+  };
+  v4i xa[3][ITERS];
+  fragment_of(0, xa[0]);
+  if constexpr (RG > 1) fragment_of(1, xa[1]);
+  constexpr int kRowStep = kMfmaWaves * 64 / Sh::kTileCols;  // 4
+  const int tc = threadIdx.x % Sh::kTileCols;
+  const size_t j = (size_t)tile * Sh::kTileCols + tc;
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) {
+    if (rg + 2 < RG) fragment_of(rg + 2, xa[(rg + 2) % 3]);
+    if ((size_t)rg * 16 >= p.m) break;  // the same for every thread of the workgroup
+    v4i acc[LC];
+#pragma unroll
+    for (int c = 0; c < LC; ++c) acc[c] = v4i{0, 0, 0, 0};
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const unsigned t[4][4] = {{rows[it][0].x, rows[it][0].y, rows[it][0].z, rows[it][0].w},
+                                {rows[it][1].x, rows[it][1].y, rows[it][1].z, rows[it][1].w},
+                                {rows[it][2].x, rows[it][2].y, rows[it][2].z, rows[it][2].w},
+                                {rows[it][3].x, rows[it][3].y, rows[it][3].z, rows[it][3].w}};
+#pragma unroll
+      for (int c = 0; c < LC; ++c) {
+        const v4i bw = {(int)t[0][c], (int)t[1][c], (int)t[2][c], (int)t[3][c]};
+        acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[rg % 3][it], bw, acc[c], 0, 0, 0);
+      }
+    }
+    // acc[c][r] is row 16 rg + 4 g + r of C, column 4 jl + c of the tile.
+    if (rg > 0) __syncthreads();  // the previous group's sums have been read
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      *reinterpret_cast<v4i *>(&red[wave][4 * g + r][LC * jl]) = v4i{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+    __syncthreads();
+    if (j < p.n) {
+      for (size_t i = threadIdx.x / Sh::kTileCols; i < 16; i += kRowStep) {
+        const size_t row = (size_t)rg * 16 + i;
+        if (row >= p.m) break;
+        unsigned sum = 0;
+#pragma unroll
+        for (int w = 0; w < kMfmaWaves; ++w) sum += (unsigned)red[w][i][tc];
+        (void)__hip_atomic_fetch_add(p.c + row * p.c_row + j * p.c_s, (int)((unsigned)p.alpha.i * sum), __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // B with K contiguous (column j is K consecutive elements, columns a fixed distance apart - how a linear
 // layer's weight [out][in] is stored): every output is a dot product over contiguous memory. A wave owns
 // two or four columns and walks K one KiB (64 lanes x 16 bytes) at a time, kKcUnroll KiB per column in
@@ -1218,9 +1312,9 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int lay
   const int mode = mode_of(g, layout);
   if (mode < 0) return 0;
   if (mode == kI8K4) {
-    // B(4P + p, j) at P * b_sk + 4 j + p; 2 to 16 rows (no other kernel reads this layout with more than one row)
+    // B(4P + p, j) at P * b_sk + 4 j + p; 2 to 128 rows (no other kernel reads this layout with more than one row)
     if (g->c_row_shift != 6 || g->c_col_shift != 6 || g->bias || g->max || g->rq.act || g->rq.q) return 0;
-    if (g->m < 2 || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;
+    if (g->m < 2 || g->m > (size_t)(16 * kK4MaxRowGroups) || g->k == 0 || g->n == 0) return 0;
     if ((g->k % 16) != 0 || (g->n % 4) != 0 || g->k * g->n < (size_t(1) << 20)) return 0;
     if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % 16) != 0) return 0;
     if (!aligned16(g->b) || (g->b_sk % 16) != 0) return 0;
@@ -1274,6 +1368,23 @@ int launch_mfma_rows(const GemvMfmaArgs &args) {
       gemv_mfma_scale_c_kernel<<<(unsigned)cells, 256, 0, skl_current_stream()>>>(p);
       int rc = skl_check_launch("gemv_mfma_scale_c");
       if (rc != 0) return rc;
+    }
+    if constexpr (MODE == kI8K4) {
+      if (p.m > (size_t)kMfmaMaxRows) {  // more than one group of 16 rows: one pass over B for all of them
+        constexpr unsigned threads = kMfmaWaves * 64;
+        static_assert(kMfmaLds <= 64 * 1024, "fits the default LDS limit of a launch");
+        hipStream_t st = skl_current_stream();
+        switch ((p.m + 15) / 16) {
+          case 2: gemv_k4_rowgroups_kernel<2><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+          case 3: gemv_k4_rowgroups_kernel<3><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+          case 4: gemv_k4_rowgroups_kernel<4><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+          case 5: gemv_k4_rowgroups_kernel<5><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+          case 6: gemv_k4_rowgroups_kernel<6><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+          case 7: gemv_k4_rowgroups_kernel<7><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+          default: gemv_k4_rowgroups_kernel<8><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+        }
+        return skl_check_launch("gemv_k4_rowgroups");
+      }
     }
     kernel<<<(unsigned)grid, kMfmaWaves * 64, kMfmaLds, skl_current_stream()>>>(p);
     return skl_check_launch("gemv_mfma_rows");
