@@ -176,6 +176,24 @@ def wl_small_batch_f8(lib, rng):
                 kernel="gemv_mfma_rows_kernel<fp8 E4M3> + gemv_mfma_add_planes_kernel")
 
 
+def _wl_ofp4(m):
+    """Decode against OFP4 (E2M1) weights stored column by column: the weights cross HBM at half a byte per element.
+    16 buffers rotated (22.5 MB each) so that the stream exceeds the last-level cache."""
+    def build(lib, rng):
+        k, n, nbuf = 4096, 11008, 16
+        w = [DeviceBuffer.from_array(rng.integers(0, 256, size=k * n // 2, dtype=np.uint8)) for _ in range(nbuf)]
+        x = DeviceBuffer.from_array(rng.integers(8, 127, size=m * k, dtype=np.uint8))
+        y = DeviceBuffer(4 * m * n)
+
+        def step(i):
+            lib.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(m, n, k, 1.0, x, k, 1, w[i % nbuf], k, 0.0, y, n, 1)
+
+        return dict(fn=step, bytes=k * n // 2 + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="f4e2m1", keep=(w, x, y),
+                    name=f"E4M3 x OFP4 GEMM {m}x4096x11008 (4-bit weights, columns contiguous in K, beta=0)",
+                    kernel="gemv_f4_kernel")
+    return build
+
+
 def wl_gemv_p4x1c(lib, rng):
     """Config 2 with W prepacked in the K-packed dot4 layout (B(4P+p, j) at P*rsb1 + 4j + p): same bytes."""
     k, n, nbuf = 4096, 11008, 8
@@ -471,6 +489,8 @@ WORKLOADS = {
     "gemv_i8_p4x1c": (wl_gemv_p4x1c, 10, 2, 128),
     "gemv_bf16": (wl_gemv_bf16, 10, 2, 64),
     "gemv_f8e4m3": (wl_gemv_f8, 10, 2, 128),
+    "gemv_f8e4m3_f4_1x4096x11008": (_wl_ofp4(1), 10, 2, 128),
+    "gemm_f8e4m3_f4_16x4096x11008": (_wl_ofp4(16), 10, 2, 128),
     "gemv_i8_1x8192x28672": (wl_gemv_large, 10, 2, 32),
     "gemv_i8_kcontig": (wl_gemv_kc, 10, 2, 128),
     "gemv_bf16_kcontig": (wl_gemv_kc_bf16, 10, 2, 64),

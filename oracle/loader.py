@@ -28,6 +28,7 @@ _EXTRA_ORACLE = {
     "skl_oracle_widen_f16_f64": (None, "ppz"),
     "skl_oracle_widen_f8e4m3_f64": (None, "ppz"),
     "skl_oracle_widen_f8e5m2_f64": (None, "ppz"),
+    "skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle": (None, "zzzfpzzpzfpzz"),
     # (m, n, c, rsc, csc, activation, q, rsq, csq, q_scale, per_column, q_zero)
     "skl_oracle_act_requant_i32": (None, "zzpzzipzzpii"),
     "skl_oracle_act_requant_f32": (None, "zzpzzipzzpii"),

@@ -9,6 +9,7 @@
 #include "skl_oracle.h"
 
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 /* ======================================================================== */
@@ -353,6 +354,19 @@ GEMM_RCPRC(bf16rcprc_bf16rcprc_f32rcprc, uint16_t, uint16_t, float, skl_oracle_b
            skl_oracle_bf16_to_f32)
 GEMM_RCPRC(f16rcprc_f16rcprc_f32rcprc, uint16_t, uint16_t, float, skl_oracle_f16_to_f32,
            skl_oracle_f16_to_f32)
+/* No GEMM over 4-bit operands exists in the reference: its users convert OFP4 weights with skl_cvt_f4e2m1_f8e4m3
+ * (ref/cvt/cvt_ofp4.c:59-68) and call the fp8 GEMM (ref/gemm/gemm_f8e4m3rc_f8e4m3rc_f32rc.c). This is that
+ * composition, for a B stored column by column: 4-bit value number j * ldb + p of `b` is B(p, j). */
+void skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa,
+                                            size_t csa, const uint8_t *b, size_t ldb, float beta, float *c, size_t rsc,
+                                            size_t csc) {
+  const size_t values = (n && k) ? (n - 1) * ldb + k : 0;
+  uint8_t *b8 = (uint8_t *)malloc(values ? values : 1);
+  skl_cvt_f4e2m1_f8e4m3_oracle(b8, b, values);
+  skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_oracle(m, n, k, alpha, a, rsa, csa, b8, 1, ldb, beta, c, rsc, csc);
+  free(b8);
+}
+
 GEMM_RCPRC(f8e4m3rcprc_f8e4m3rcprc_f32rcprc, uint8_t, uint8_t, float,
            skl_oracle_f8e4m3_to_f32, skl_oracle_f8e4m3_to_f32)
 GEMM_RCPRC(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, uint8_t, float,

@@ -115,6 +115,12 @@ void skl_gemm_f16rcprc_f16rcprc_f16rcprc_oracle(size_t m0, size_t n0, size_t k0,
                                                 size_t csb0, size_t rsb1, size_t csb1, float beta, uint16_t *c,
                                                 size_t rsc0, size_t csc0, size_t rsc1, size_t csc1);
 
+/* E4M3 A times OFP4 B stored column by column: the reference's conversion (ref/cvt/cvt_ofp4.c:59-68) followed by its
+ * fp8 GEMM with rsb = 1, csb = ldb. */
+void skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa,
+                                            size_t csa, const uint8_t *b, size_t ldb, float beta, float *c, size_t rsc,
+                                            size_t csc);
+
 /* GEMM + fused bias / maximum steps (src/gemm/fused-kernel-API.md:159-207); bias and max may be NULL. */
 #define SKL_ORACLE_FUSED_DECL(NAME, TA, TC)                                                        \
   void skl_gemm_fused_##NAME##_oracle(size_t m, size_t n, size_t k, TC alpha, const TA *a, size_t rsa, \

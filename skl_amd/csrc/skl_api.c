@@ -648,6 +648,68 @@ void skl_gemm_i8_i8_i32_noalloc_gfx950(size_t m, size_t n, size_t k, int32_t alp
   skl_hip_launch_gemv_noalloc(&g);
 }
 
+/* E4M3 A times OFP4 (E2M1) B, columns of B contiguous in K, two values per byte (see include/skl-gfx950.h). The
+ * result is defined as the reference's conversion of B to E4M3 followed by its fp8 GEMM with rsb = 1, csb = ldb.
+ * Decode shapes stream the 4-bit weights through the kernel that multiplies them as they are; everything else
+ * converts B once into scratch memory of the stream and runs the fp8 GEMM on that. */
+static int f4_gemm_on_device(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa, size_t csa,
+                             const uint8_t *b, size_t ldb, skl_scalar beta, float *c, size_t rsc, size_t csc) {
+  const skl_scalar alpha_s = {.f = alpha};
+  int rc;
+  if (k != 0 && skl_hip_gemv_f4_supported(m, n, k, a, rsa, csa, b, ldb))
+    return skl_hip_launch_gemv_f4(m, n, k, alpha_s, a, rsa, csa, b, ldb, beta, c, rsc, csc);
+  {
+    const size_t values = k ? (n - 1) * ldb + k : 0; /* 4-bit values from B's first to its last, gaps included */
+    uint8_t *b8 = NULL;
+    skl_gemm_desc d = {SKL_DT_F8E4M3, SKL_DT_F8E4M3, 1, 1, 1, m, n, k, a, 0, 0, rsa, csa, NULL, 0, 0, 1, ldb,
+                       c, 0, 0, rsc, csc, {.f = alpha}, beta, NULL, NULL, {0}};
+    skl_hip_sequence_begin(); /* the converted B travels from one launch to the next through the stream's scratch */
+    if (values) {
+      b8 = (uint8_t *)skl_hip_converted_scratch(values);
+      if (!b8) {
+        skl_hip_sequence_end();
+        return SKL_HIP_ERR_WORKSPACE;
+      }
+      rc = skl_hip_launch_cvt_f4_f8e4m3(b8, b, values);
+      if (rc != 0) {
+        skl_hip_sequence_end();
+        return rc;
+      }
+    }
+    d.b = b8;
+    rc = gemm_on_device(&d);
+    skl_hip_sequence_end();
+    return rc;
+  }
+}
+
+void skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa, size_t csa,
+                                           const uint8_t *b, size_t ldb, float beta, float *c, size_t rsc, size_t csc) {
+  skl_scalar beta_s;
+  int where;
+  if (m == 0 || n == 0) return; /* nothing is addressed */
+  memset(&beta_s, 0, sizeof beta_s);
+  beta_s.fz.value = beta;
+  beta_s.fz.skip_c_read = skl_hip_get_beta_zero_mode() != SKL_HIP_BETA_ZERO_AS_REFERENCE;
+  where = classify(k ? a : NULL, k ? b : NULL, c, __func__);
+  if (where < 0) return;
+  if (where == 1) {
+    (void)f4_gemm_on_device(m, n, k, alpha, a, rsa, csa, b, ldb, beta_s, c, rsc, csc);
+    return;
+  }
+  {
+    const size_t na = k ? (m - 1) * rsa + (k - 1) * csa + 1 : 0, nb = k ? ((n - 1) * ldb + k + 1) / 2 : 0;
+    const size_t nc = (m - 1) * rsc + (n - 1) * csc + 1;
+    void *da = stage_in(a, na), *db = stage_in(b, nb), *dc = stage_in(c, nc * sizeof(float));
+    if ((!na || da) && (!nb || db) && dc &&
+        f4_gemm_on_device(m, n, k, alpha, (const uint8_t *)da, rsa, csa, (const uint8_t *)db, ldb, beta_s, (float *)dc, rsc, csc) == 0)
+      skl_hip_memcpy_d2h(c, dc, nc * sizeof(float)); /* C's whole span: the elements in its stride gaps come back unchanged */
+    skl_hip_free(da);
+    skl_hip_free(db);
+    skl_hip_free(dc);
+  }
+}
+
 /* column-major A: the rc form with rsa = 1
  * (src/gemm/gemm_i8c_i8_i32_xsfmm32a8i.h:38-48) */
 #define DEFINE_GEMM_COLMAJOR_A(NAME, RC, TA_T, TC_T)                                               \

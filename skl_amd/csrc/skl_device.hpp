@@ -34,9 +34,10 @@ static inline unsigned skl_div_up(size_t a, size_t b) { return (unsigned)((a + b
 //
 // beta == 0 initialises C (src/gemm/README.md:43 of the reference: "accumulation (beta=1) and initialization
 // (beta=0)"): there beta*C is a zero whose sign is all the old value contributes, and the sign matters only when
-// alpha*acc is itself a zero - the old value is read for exactly those elements. The result has the reference's
-// bits for every finite C; an Inf or NaN in C, which ref/gemm/gemm_bf16rc_bf16rc_f32rc.c:21 (beta*c evaluated
-// whatever beta is) turns into NaN, is overwritten. A caller that wants the reference's result there too asks
+// alpha*acc is itself a zero - the old value is read for exactly those elements, and only its sign bit is used.
+// The result has the reference's bits for every finite C; an Inf or NaN in C, which
+// ref/gemm/gemm_bf16rc_bf16rc_f32rc.c:21 (beta*c evaluated whatever beta is) turns into NaN, is overwritten
+// everywhere (so C may be uninitialised memory). A caller that wants the reference's result there too asks
 // for it (skl_hip_set_beta_zero_mode(SKL_HIP_BETA_ZERO_AS_REFERENCE)): beta then arrives without
 // fz.skip_c_read and C is read and combined whatever beta is. int32: 0 * c is 0 for every c, so C is never read
 // with beta == 0. f64 has no room for the switch next to the value: always read.
@@ -60,17 +61,20 @@ __device__ __forceinline__ double skl_combine(double acc, double old, skl_scalar
   return __dadd_rn(__dmul_rn(beta.d, old), __dmul_rn(alpha.d, acc));
 }
 
-// The beta == 0 case; `c` is dereferenced only where alpha*acc is a zero.
+// The beta == 0 case; `c` is dereferenced only where alpha*acc is a zero, and only for its sign: beta*c is the zero
+// whose sign is the product of the two signs (what 0 * c is for every finite c).
 __device__ __forceinline__ int skl_initialise(int acc, const int *, skl_scalar alpha, skl_scalar) {
   return (int)((unsigned)alpha.i * (unsigned)acc);
 }
 __device__ __forceinline__ float skl_initialise(float acc, const float *c, skl_scalar alpha, skl_scalar beta) {
   const float x = __fmul_rn(alpha.f, acc);
-  return x == 0.0f ? __fadd_rn(__fmul_rn(beta.f, *c), x) : x;
+  return x == 0.0f ? __fadd_rn(__uint_as_float((__float_as_uint(*c) ^ __float_as_uint(beta.f)) & 0x80000000u), x) : x;
 }
 __device__ __forceinline__ double skl_initialise(double acc, const double *c, skl_scalar alpha, skl_scalar beta) {
   const double x = __dmul_rn(alpha.d, acc);
-  return x == 0.0 ? __dadd_rn(__dmul_rn(beta.d, *c), x) : x;
+  if (x != 0.0) return x;
+  const unsigned long long sign = (unsigned long long)(__double_as_longlong(*c) ^ __double_as_longlong(beta.d)) & 0x8000000000000000ull;
+  return __dadd_rn(__longlong_as_double((long long)sign), x);
 }
 
 template <typename T>

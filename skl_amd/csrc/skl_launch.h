@@ -138,12 +138,20 @@ int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
 int skl_hip_noalloc_setup(void);
 size_t skl_hip_noalloc_max_sums(void);
 int skl_hip_launch_gemv_noalloc(const skl_gemm_canon *g);
+/* E4M3 A (1 to 16 rows, K contiguous) times OFP4 B (columns contiguous in K, two values per byte, `ldb` elements
+ * apart): skl_gemv_f4.hip. */
+int skl_hip_gemv_f4_supported(size_t m, size_t n, size_t k, const void *a, size_t rsa, size_t csa, const void *b, size_t ldb);
+int skl_hip_launch_gemv_f4(size_t m, size_t n, size_t k, skl_scalar alpha, const void *a, size_t rsa, size_t csa, const void *b,
+                           size_t ldb, skl_scalar beta, float *c, size_t rsc, size_t csc);
 /* Makes sure the current stream has the sums-and-counters block of the single-row kernels; 0 or SKL_HIP_ERR_WORKSPACE. */
 int skl_hip_gemv_reserve_scratch(void);
 
 /* A block of scratch memory of the current stream and device for operands copied into another layout ahead of a
  * launch (grows on demand, NULL when the device has no room; apart from the workspace of the split reductions). */
 void *skl_hip_operand_scratch(size_t bytes);
+/* A third block, for an operand converted to another element type ahead of a GEMM that may copy operands itself
+ * (into the block above). NULL, with the error recorded, when there is no room. */
+void *skl_hip_converted_scratch(size_t bytes);
 /* Brackets a sequence of launches that hands data from one kernel to the next through the stream's scratch memory
  * (operand copies, partial sums), so that sequences of different host threads do not interleave on a stream.
  * Recursive. */

@@ -29,6 +29,7 @@ struct StreamState {
   Scratch workspace;       // partial sums of the split reductions (never more than kWorkspaceBytes are asked for)
   Scratch operands;        // copies of operands in another layout; apart from the workspace so that a launch which
                            // uses the workspace keeps the copies it was given
+  Scratch converted;       // an operand converted to another element type ahead of a GEMM that may itself copy operands
   void *zeroed = nullptr;  // block that is zero between launches (sums and counters shared by workgroups)
   size_t zeroed_bytes = 0;
 };
@@ -204,11 +205,20 @@ int skl_hip_release_stream(void *stream) {
     if (s.stream != (hipStream_t)stream) continue;
     if (s.workspace.ptr) (void)hipFree(s.workspace.ptr);
     if (s.operands.ptr) (void)hipFree(s.operands.ptr);
+    if (s.converted.ptr) (void)hipFree(s.converted.ptr);
     if (s.zeroed) (void)hipFree(s.zeroed);
     st->streams.erase(st->streams.begin() + (long)i);
     break;
   }
   return SKL_HIP_OK;
+}
+
+void *skl_hip_converted_scratch(size_t bytes) {
+  DeviceState *st = current_device_state();
+  if (!st) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  StreamState *ss = current_stream_state(*st);
+  return ss ? grow(*st, ss->converted, bytes, kOperandBytes, "skl_hip_converted_scratch", true) : nullptr;
 }
 
 void skl_hip_sequence_begin(void) { g_sequence.lock(); }
@@ -229,6 +239,7 @@ void skl_hip_shutdown(void) {
       for (StreamState &s : st.streams) {
         if (s.workspace.ptr) (void)hipFree(s.workspace.ptr);
         if (s.operands.ptr) (void)hipFree(s.operands.ptr);
+        if (s.converted.ptr) (void)hipFree(s.converted.ptr);
         if (s.zeroed) (void)hipFree(s.zeroed);
       }
       for (void *p : st.retired) (void)hipFree(p);

@@ -221,8 +221,9 @@ def _beta_zero_as_reference(gpu, ta, m, n, k):
 @pytest.mark.parametrize("ta,m,n,k,what", BETA_ZERO_SHAPES)
 def test_beta_zero_initialises_c(gpu, ta, m, n, k, what):
     """The default: beta == 0 is the initialising call (src/gemm/README.md:43). The old C contributes nothing but the
-    sign of an exact zero, so an Inf or NaN in C is overwritten exactly as a finite value is, and every result has
-    the bits of the reference-evaluation mode's result on a clean C. (f64: C is always read.)"""
+    sign of an exact zero, so an Inf or NaN in C is overwritten exactly as a finite value is - also in the rows whose
+    products are exact zeros, where the old sign is all that is read - and every result has the bits of the
+    reference-evaluation mode's result on a clean C. (f64: C is always read.)"""
     if ta == "f64":
         pytest.skip("f64 GEMMs always read C")
     rng = np.random.default_rng(78)
@@ -234,6 +235,10 @@ def test_beta_zero_initialises_c(gpu, ta, m, n, k, what):
     live = np.ones(m, dtype=bool)
     live[zero_rows] = False
     spoiled = _spoil(c, m, n, np.flatnonzero(live))
+    for i in zero_rows:  # the zero rows too: NaN and Inf that keep the sign of the value they replace
+        row = spoiled.reshape(m, n)[i]
+        row[::2] = np.copysign(np.nan, row[::2])
+        row[1::4] = np.copysign(np.inf, row[1::4])
     assert gpu.skl_hip_get_beta_zero_mode() == 0
     for mode in MODES:
         gpu.skl_hip_set_beta_zero_mode(1)

@@ -1,0 +1,102 @@
+"""GPU parity of the GEMM over OFP4 (E2M1) weights, skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950: the reference has no
+such routine - its users convert the weights (skl_cvt_f4e2m1_f8e4m3, ref/cvt/cvt_ofp4.c:59-68) and call the fp8 GEMM
+(ref/gemm/gemm_f8e4m3rc_f8e4m3rc_f32rc.h:48). The result must lie inside that GEMM's own bound
+(test/gemm/gemm_f8rcprc_f8rcprc_f32rcprc.c:132-204, no allowance on top) around the exact product of the decoded
+operands, on the kernel that streams the 4-bit weights (1 to 16 rows: matrix-core FP4 format for long K, f16
+instructions on widened operands up to K = 2304) and on the route through a converted copy."""
+import numpy as np
+import pytest
+
+import ofp4_support as f4
+import skl_amd
+import support
+from gpu_support import MODES, _finish
+from skl_amd import DeviceBuffer
+
+pytestmark = pytest.mark.gpu
+
+
+def run(lib, case, a, b4, c, mode, m, n, k, ldb):
+    args = lambda a_, b_, c_: (m, n, k, case.alpha, a_, case.rsa1, case.csa1, b_, ldb, case.beta, c_, case.rsc1, case.csc1)
+    if mode == "host":
+        out = c.copy()
+        lib.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(*args(a, b4, out))
+        skl_amd.check_error()
+        return out
+    da, db, dc = DeviceBuffer.from_array(a), DeviceBuffer.from_array(b4), DeviceBuffer.from_array(c)
+    lib.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(*args(da, db, dc))
+    _finish(lib)
+    out = dc.download(c.dtype, c.size)
+    for d in (da, db, dc):
+        d.free()
+    return out
+
+
+SHAPES = (
+    # m, n, k, ldb, rsa, what
+    (1, 11008, 4096, 4096, None, "decode, FP4 operand format of the matrix cores"),
+    (16, 1000, 4352, 4384, 4368, "16 rows, n off the 16-column groups, K off the chunk of 1024"),
+    (3, 500, 2304, 2304, None, "longest K multiplied exactly (operands widened to f16)"),
+    (7, 48, 2336, 2336, None, "shortest K on the FP4 format"),
+    (5, 48, 32, 32, None, "one piece of K"),
+    (1, 17, 64, 96, None, "a last group of one column"),
+    (17, 300, 512, 512, None, "more than 16 rows: through the converted copy"),
+    (300, 260, 1000, 1000, None, "a GEMM: through the converted copy"),
+    (4, 64, 100, 101, None, "K off 32 and an odd column distance (columns start inside a byte): converted copy"),
+    (2, 40, 64, 64, 67, "rows of A off 16 bytes: converted copy"),
+)
+
+
+@pytest.mark.parametrize("m,n,k,ldb,rsa,what", SHAPES)
+def test_ofp4_weights(gpu, m, n, k, ldb, rsa, what):
+    for i, (alpha, beta) in enumerate(((1.0, 0.0), (1.5, -0.5))):
+        case, a, b4, b8, c = f4.make_problem(700 + m + n + i, m, n, k, ldb, alpha, beta, rsa=rsa, rsc=n + 3)
+        for mode in MODES:
+            got = run(gpu, case, a, b4, c, mode, m, n, k, ldb)
+            support.assert_fp_gemm_close(case, a, b8, c, got)
+            assert np.array_equal(got.view(np.uint32), run(gpu, case, a, b4, c, mode, m, n, k, ldb).view(np.uint32)), what
+
+
+@pytest.mark.parametrize("k", (2304, 2560))
+def test_every_position_and_code_is_read_back(gpu, k):
+    """A row of A that is 1.0 at one k and zero elsewhere reads B(k, :) back exactly: every position of a 256-k chunk
+    (16 rows per call), every E2M1 code, both kernel variants (k = 2304: f16 instructions, 2560: FP4 format). This
+    is what fixes which nibble is which k and that A's and B's lanes hold the same k."""
+    n = 64
+    rng = np.random.default_rng(k)
+    codes = rng.integers(0, 16, size=n * k, dtype=np.uint8)
+    codes[:16 * k:k + 1] = np.arange(16)          # and every code at least once on a diagonal
+    b4 = f4.pack_nibbles(codes)
+    table = f4.E2M1_VALUES[codes].reshape(n, k)
+    for base in (0, k - 256):
+        for p0 in range(0, 256, 16):
+            a = np.zeros(16 * k, np.uint8)
+            pos = base + p0 + np.arange(16)
+            a[np.arange(16) * k + pos] = 0x38      # 1.0
+            case = f4.f8_case(16, n, k, k, 1.0, 0.0)
+            got = run(gpu, case, a, b4, np.full(16 * n, np.nan, np.float32), "device", 16, n, k, k).reshape(16, n)
+            assert np.array_equal(got.astype(np.float64), table[:, pos].T), (k, base, p0)
+
+
+def test_ofp4_edges(gpu):
+    """K = 0 scales C; empty problems touch nothing; a NaN in C is overwritten by beta == 0 (the library's default)
+    and kept by the reference's evaluation of 0 * C when that is asked for; mixed pointers are refused."""
+    case, a, b4, b8, c = f4.make_problem(9, 4, 32, 64, 64, 2.0, 3.0)
+    got = run(gpu, case, a, b4, c, "device", 4, 32, 0, 64)
+    assert np.array_equal(got, (np.float32(3.0) * c).astype(np.float32))
+    assert np.array_equal(run(gpu, case, a, b4, c, "device", 0, 32, 64, 64), c)
+    spoiled = c.copy()
+    spoiled[5] = np.nan
+    case0 = f4.f8_case(4, 32, 64, 64, 1.0, 0.0)
+    got = run(gpu, case0, a, b4, spoiled, "device", 4, 32, 64, 64)
+    support.assert_fp_gemm_close(case0, a, b8, c, got)
+    gpu.skl_hip_set_beta_zero_mode(1)
+    try:
+        got = run(gpu, case0, a, b4, spoiled, "device", 4, 32, 64, 64)
+        assert np.isnan(got[5]) and not np.isnan(np.delete(got, 5)).any()
+    finally:
+        gpu.skl_hip_set_beta_zero_mode(0)
+    d = DeviceBuffer.from_array(a)
+    gpu.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(4, 32, 64, 1.0, d, 64, 1, b4, 64, 0.0, c.copy(), 32, 1)
+    assert gpu.skl_hip_last_error() == -1
+    d.free()

@@ -318,6 +318,38 @@ def test_fused_steps_follow_the_plain_gemm(ta):
                     assert mx[0] == start[0]
 
 
+def test_ofp4_gemm_is_the_conversion_followed_by_the_fp8_gemm():
+    """The checker's GEMM over OFP4 weights (oracle/skl_oracle.c: the reference's conversion, ref/cvt/cvt_ofp4.c:59-68,
+    then its fp8 GEMM) against the same GEMM on a B converted by the format's value table in numpy: bit for bit, odd
+    and even column distances, ragged everything; and against the exact product where every sum is exact."""
+    import ofp4_support as f4
+    o = oracle()
+    # the table itself: the checker's conversion of all 16 codes, and their values
+    got = np.zeros(16, np.uint8)
+    o.skl_cvt_f4e2m1_f8e4m3_oracle(got, f4.pack_nibbles(np.arange(16)), 16)
+    assert np.array_equal(got, f4.E2M1_AS_E4M3)
+    assert np.array_equal(support.decode_table("f8e4m3")[f4.E2M1_AS_E4M3], f4.E2M1_VALUES)
+    for i, (m, n, k, ldb, alpha, beta) in enumerate(((3, 5, 7, 7, 1.0, 0.0), (4, 6, 33, 40, 1.5, -0.5), (1, 9, 64, 65, 2.0, 1.0),
+                                                     (17, 3, 100, 101, 1.0, 0.0), (2, 2, 0, 4, 3.0, 2.0))):
+        case, a, b4, b8, c = f4.make_problem(50 + i, m, n, k, ldb, alpha, beta, rsa=k + 3, rsc=n + 2)
+        got = c.copy()
+        o.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle(m, n, k, alpha, a, case.rsa1, 1, b4, ldb, beta, got, case.rsc1, 1)
+        want = run_oracle_gemm(case, a, b8, c)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (m, n, k, ldb)
+        if k:
+            support.assert_fp_gemm_close(case, a, b8, c, got)
+    # exact sums: A in {1, 2, 4}, K = 64: every partial sum is a small multiple of 0.5
+    m, n, k = 5, 11, 64
+    rng = np.random.default_rng(3)
+    a = rng.choice(np.array([0x38, 0x40, 0x48], np.uint8), m * k)
+    codes = rng.integers(0, 16, n * k, dtype=np.uint8)
+    got = np.zeros(m * n, np.float32)
+    o.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle(m, n, k, 1.0, a, k, 1, f4.pack_nibbles(codes), k, 0.0, got, n, 1)
+    A = support.decode_table("f8e4m3")[a].reshape(m, k)
+    B = f4.E2M1_VALUES[codes].reshape(n, k).T
+    assert np.array_equal(got.reshape(m, n).astype(np.float64), A @ B)
+
+
 def test_requantisation_rule_on_worked_values():
     """The checker's requantisation and activation (oracle/skl_oracle.c, skl_oracle_act_requant_*) against values
     worked by hand from the rule in include/skl-gfx950.h - ties go to the even integer, the zero point is added
