@@ -273,6 +273,26 @@ def wl_gemm_i8_8192(lib, rng):
                   8192, 1, lambda n: rand_i8(rng, n), lambda n: rand_i8(rng, n), 1, 0, np.int32, "i8")
 
 
+def wl_gemm_i8_8192_requantised(lib, rng):
+    """A quantised layer: int8 in, ReLU, int8 out (per-column scales), the int32 C never written (q_only)."""
+    import skl_amd
+    m = n = k = 8192
+    a, b = DeviceBuffer.from_array(rand_i8(rng, m * k)), DeviceBuffer.from_array(rand_i8(rng, k * n))
+    c = DeviceBuffer(16)  # not written
+    q = DeviceBuffer(m * n)
+    bias = DeviceBuffer.from_array(rng.integers(-1000, 1000, n).astype(np.int32))
+    scales = DeviceBuffer.from_array((rng.uniform(0.5, 2.0, n) / (74.0 * 74.0 * 90.0 * 0.4)).astype(np.float32))
+    ep = skl_amd.Epilogue(bias, None, activation=skl_amd.Epilogue.ACT_RELU, q=q, rsq=n, csq=1, q_scale=scales,
+                          q_scale_per_column=True, q_zero=-128, q_only=True)
+
+    def step(i):
+        lib.skl_gemm_fused_i8rc_i8rc_i32rc_gfx950(m, n, k, 1, a, k, 1, b, n, 1, 0, c, n, 1, ep)
+
+    return dict(fn=step, bytes=m * k + k * n + m * n, ops=2 * m * n * k, bound="mfma", dtype="i8", keep=(a, b, c, q, bias, scales),
+                name="int8 GEMM 8192^3 with bias, ReLU and requantised int8 output only (q_only)",
+                kernel="gemm_mfma_ring_kernel<int8, EXTRA>")
+
+
 def wl_gemm_i8_4000(lib, rng):
     """Ragged M, N, K: A and B are copied into tile-padded scratch memory, the streaming kernel runs on the copies."""
     d = _dense(lib, rng, "int8 GEMM 4000^3 (row-major, alpha=1, beta=0; ragged: runs on tile-padded copies)",
@@ -510,6 +530,7 @@ WORKLOADS = {
     "peak_mfma_bf16_random": (_wl_peak_mfma(1, "bf16", 1), 3, 1, 1),
     "peak_mfma_bf16_constant": (_wl_peak_mfma(1, "bf16", 0), 3, 1, 1),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2, 1),
+    "gemm_i8_8192_requantised": (wl_gemm_i8_8192_requantised, 10, 2, 1),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2, 1),
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2, 1),
     "gemm_f8e4m3_8192_rowmajor_a": (wl_gemm_f8_layout(True, False), 10, 2, 1),

@@ -90,18 +90,25 @@ __device__ __forceinline__ int skl_add_bias(int v, int b) { return (int)((unsign
 __device__ __forceinline__ float skl_add_bias(float v, float b) { return __fadd_rn(v, b); }
 
 // The activation step: 0 none, 1 max(v, 0) (a NaN becomes 0, like `v > 0 ? v : 0`).
-__device__ __forceinline__ int skl_activate(int v, int act) { return (act == 1 && v < 0) ? 0 : v; }
+__device__ __forceinline__ int skl_activate(int v, int act) {
+  const int floor = act == 1 ? 0 : (int)0x80000000;  // uniform: one max per element
+  return v < floor ? floor : v;
+}
 __device__ __forceinline__ float skl_activate(float v, int act) { return act == 1 ? (v > 0.0f ? v : 0.0f) : v; }
 
 // The requantised int8 value of v: round-to-nearest-even of (float)v * scale as an integer (a NaN counts as 0, values
 // beyond int32 as its ends), plus the zero point, clamped to [-128, 127].
-__device__ __forceinline__ int8_t skl_requantise(float v, float scale, int zero) {
-  float r = __builtin_rintf(__fmul_rn(v, scale));
+__device__ __forceinline__ int skl_requantise_int(float v, float scale, int zero) {
+  const float r = __builtin_rintf(__fmul_rn(v, scale));
+  int t;
+  // the hardware's conversion is the rule itself: a NaN gives 0, values beyond int32 its ends (the C cast leaves
+  // both undefined)
+  asm("v_cvt_i32_f32 %0, %1" : "=v"(t) : "v"(r));
   // The zero point lies in [-128, 127], so anything beyond +-512 ends at the same end of int8 as the int32 ends would.
-  r = (r != r) ? 0.0f : r > 512.0f ? 512.0f : r < -512.0f ? -512.0f : r;
-  const int t = (int)r + zero;
-  return (int8_t)(t < -128 ? -128 : t > 127 ? 127 : t);
+  t = (t < -512 ? -512 : t > 512 ? 512 : t) + zero;
+  return t < -128 ? -128 : t > 127 ? 127 : t;
 }
+__device__ __forceinline__ int8_t skl_requantise(float v, float scale, int zero) { return (int8_t)skl_requantise_int(v, scale, zero); }
 // Element (row, col) of the requantised output, if there is one.
 template <typename T>
 __device__ __forceinline__ void skl_emit_requantised(const skl_requant &rq, T v, size_t row, size_t col) {

@@ -75,36 +75,75 @@ struct MfmaArgs {
 // The fused steps behind the alpha/beta step, for one lane: bias of the lane's column, activation, running maximum,
 // requantised copy.
 // EXTRA: with the activation and the requantised copy (kernels are instantiated with and without: the two steps cost
-// code in every one of a lane's 128 stores, which calls without them should not carry).
-template <typename T, bool EXTRA = false>
+// code in every one of a lane's 128 stores, which calls without them should not carry). 1: any descriptor, decided
+// element by element at run time. 2 and 3: for kernels that hand every lane's elements to rows4() with all lanes
+// active - a row-major copy on 4-byte boundaries, written as dwords, without (2, q_only) or with (3) C; no
+// branches inside the epilogue, which with 128 accumulators live is what keeps the registers from spilling (the
+// run-time form in the streaming kernel: 240 spilled registers, an 8192^3 call 45 % longer).
+template <typename T, int EXTRA = 0>
 struct FusedSteps {
   const T *bias;
   T *max;
   const skl_requant rq;
   T bias_j, running;
   size_t col;
+  float q_scale_j;  // EXTRA: the current column's scale
   __device__ explicit FusedSteps(const MfmaArgs &p)
-      : bias(reinterpret_cast<const T *>(p.bias)), max(reinterpret_cast<T *>(p.max)), rq(p.rq), bias_j(0), running(skl_lowest<T>()), col(0) {}
+      : bias(reinterpret_cast<const T *>(p.bias)), max(reinterpret_cast<T *>(p.max)), rq(p.rq), bias_j(0), running(skl_lowest<T>()), col(0),
+        q_scale_j(0.0f) {}
+  // What a descriptor must look like for modes 2 and 3.
+  __host__ __device__ static bool dword_copy(const skl_requant &r) {
+    return r.q && r.csq == 1 && (r.rsq & 3) == 0 && ((uintptr_t)r.q & 3) == 0;
+  }
   __device__ __forceinline__ void column(size_t c) {
     col = c;
     if (bias) bias_j = bias[c];
+    if constexpr (EXTRA >= 2) q_scale_j = rq.q_scale[rq.q_per_column ? c : 0];
+    if constexpr (EXTRA == 1) {
+      if (rq.q) q_scale_j = rq.q_scale[rq.q_per_column ? c : 0];
+    }
   }
   __device__ __forceinline__ T apply(T v) {
     if (bias) v = skl_add_bias(v, bias_j);
-    if constexpr (EXTRA) v = skl_activate(v, rq.act);
+    if constexpr (EXTRA != 0) v = skl_activate(v, rq.act);
     if (max && v > running) running = v;
     return v;
   }
   // The element of logical row `row` in the current column: the steps, then C (written once and not read again: a
-  // non-temporal store keeps it out of the operands' caches) and the requantised copy.
-  __device__ __forceinline__ void put(T v, T *dst, size_t row) {
+  // non-temporal store keeps it out of the operands' caches) and, in mode 1, the requantised copy. Returns what
+  // was written.
+  __device__ __forceinline__ T put(T v, T *dst, size_t row) {
     v = apply(v);
-    if constexpr (EXTRA) {
+    if constexpr (EXTRA == 1) {
       if (!rq.q_only) __builtin_nontemporal_store(v, dst);
-      skl_emit_requantised(rq, v, row, col);
+      if (rq.q) rq.q[row * rq.rsq + col * rq.csq] = skl_requantise((float)v, q_scale_j, rq.q_zero);
     } else {
       (void)row;
-      __builtin_nontemporal_store(v, dst);
+      if constexpr (EXTRA != 2) __builtin_nontemporal_store(v, dst);
+    }
+    return v;
+  }
+  // Modes 2 and 3: the requantised copy of rows row0 .. row0 + 3 of the current column, v as put() returned them.
+  // A lane's four values are one column of a 4 x 4 block of bytes whose other columns its quad's lanes hold (four
+  // neighbouring columns, the first a multiple of four); the block is transposed across the quad (four broadcasts
+  // and three byte permutes per lane), and lane q stores row row0 + q of it as one dword - a quarter of the store
+  // instructions and address arithmetic of single bytes.
+  __device__ __forceinline__ void rows4(const T (&v)[4], size_t row0) {
+    if constexpr (EXTRA >= 2) {
+      unsigned packed = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) packed |= ((unsigned)skl_requantise_int((float)v[i], q_scale_j, rq.q_zero) & 0xFFu) << (8 * i);
+      const unsigned p0 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)packed, 0x00, 0xF, 0xF, true);  // quad_perm: lane 0 of the quad
+      const unsigned p1 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)packed, 0x55, 0xF, 0xF, true);
+      const unsigned p2 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)packed, 0xAA, 0xF, 0xF, true);
+      const unsigned p3 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)packed, 0xFF, 0xF, 0xF, true);
+      const unsigned q = threadIdx.x & 3u;
+      const unsigned sel = 0x0C0C0400u + q * 0x0101u;  // byte q of the second operand, byte q of the first, zeros
+      const unsigned lo = __builtin_amdgcn_perm(p1, p0, sel), hi = __builtin_amdgcn_perm(p3, p2, sel);
+      const unsigned out = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+      *reinterpret_cast<unsigned *>(rq.q + (row0 + q) * rq.rsq + (col - q)) = out;
+    } else {
+      (void)v, (void)row0;
     }
   }
   // Every lane of the wave calls this once, after its last element.
@@ -520,7 +559,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
   // element). C is written once and not read again: non-temporal stores keep it out of the operands' caches.
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
   const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
-  FusedSteps<AccElem, EXTRA> fused(p);
+  FusedSteps<AccElem, EXTRA ? 1 : 0> fused(p);
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
@@ -760,7 +799,7 @@ constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // EDGE: the operands are copies padded to whole tiles, C is not - its last tile rows / columns end at p.m / p.n and
 // the epilogue touches nothing beyond them.
-template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false>
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0>
 __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   using KA = Kind<TA>;
   using M = Mma<TA, TB>;
@@ -1012,7 +1051,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   // Epilogue, as in the kernel above: old values requested kEpilogueBatch blocks at a time, non-temporal stores.
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
   const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
-  FusedSteps<AccElem> fused(p);
+  FusedSteps<AccElem, EXTRA> fused(p);
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     const size_t col = n0 + wn + j * 32 + (lane & 31);
@@ -1032,13 +1071,21 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
           out[i][g] = c + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 + col_off;
         }
       auto inside = [&](int i, int r) { return !EDGE || first_row[i][r >> 2] + (r & 3) < p.m; };
+      // Four consecutive rows at a time: what put() wrote goes on to the requantised copy (rows4) while it is
+      // still in registers.
       if (init) {
 #pragma unroll
         for (int i = 0; i < kEpilogueBatch; ++i)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            AccElem *dst = out[i][r >> 2] + (r & 3) * p.rsc0;
-            if (inside(i, r)) fused.put(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst, first_row[i][r >> 2] + (r & 3));
+          for (int g = 0; g < 4; ++g) {
+            AccElem four[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int r = 4 * g + q;
+              AccElem *dst = out[i][g] + q * p.rsc0;
+              four[q] = inside(i, r) ? fused.put(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst, first_row[i][g] + q) : AccElem(0);
+            }
+            fused.rows4(four, first_row[i][g]);
           }
       } else {
         AccElem old[kEpilogueBatch][16];
@@ -1049,9 +1096,17 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 #pragma unroll
         for (int i = 0; i < kEpilogueBatch; ++i)
 #pragma unroll
-          for (int r = 0; r < 16; ++r)
-            if (inside(i, r))
-              fused.put(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][r >> 2] + (r & 3) * p.rsc0, first_row[i][r >> 2] + (r & 3));
+          for (int g = 0; g < 4; ++g) {
+            AccElem four[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int r = 4 * g + q;
+              four[q] = inside(i, r) ? fused.put(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][g] + q * p.rsc0,
+                                                 first_row[i][g] + q)
+                                     : AccElem(0);
+            }
+            fused.rows4(four, first_row[i][g]);
+          }
       }
     }
   }
@@ -1101,10 +1156,19 @@ struct SequenceGuard {
 
 constexpr size_t kRingMinSlicesPerSplit = 64;  // below 8 KiB of K per row the pass over the planes costs what the split saves
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false>
+// The int8 streaming kernels for whole tiles also exist with the activation and requantisation steps, for a copy
+// that can be written as dwords (a quantised layer's int8 output at a quarter of C's bytes); every other call with
+// those steps goes to the bounds-checked kernels.
+template <int TA>
+constexpr bool kRingCarriesExtraSteps = TA == SKL_DT_I8;
+
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0>
 int launch_ring(const MfmaArgs &args) {
+  if constexpr (EXTRA == 0 && kRingCarriesExtraSteps<TA> && !EDGE) {
+    if (args.rq.q) return args.rq.q_only ? launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 2>(args) : launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 3>(args);
+  }
   constexpr int lds = kRingStages * (256 + BN) * kRingSlice;
-  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE>;
+  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE, EXTRA>;
   static bool configured = false;
   if (!configured) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -1221,7 +1285,8 @@ int launch_tile(const MfmaArgs &p) {
   // The streaming kernel takes problems that its tiles divide evenly: 256 x 256 tiles when those
   // can fill the 256 compute units, 256 x 128 tiles for the sizes below that; everything else runs
   // on the small, bounds-checked kernel.
-  const bool extra_steps = p.rq.act || p.rq.q;  // activation / requantised copy: on the bounds-checked kernels only
+  // activation / requantised copy: on the streaming kernel only int8 with a copy that goes out as dwords
+  const bool extra_steps = (p.rq.act || p.rq.q) && !(kRingCarriesExtraSteps<TA> && FusedSteps<int, 2>::dword_copy(p.rq));
   if (!extra_steps && p.m % 256 == 0 && (p.k * ES) % 128 == 0) {
     const size_t tiles_m = p.m / 256;
     if (p.n % 256 == 0 && tiles_m * (p.n / 256) >= 200) {
@@ -1325,7 +1390,7 @@ extern "C" int skl_hip_gemm_mfma_padded_plan(const skl_gemm_canon *g, size_t *mp
   if (!(g->ta == g->tb || (fp8a && fp8b)) || ((uintptr_t)g->c & 3) != 0) return 0;
   const size_t es = (g->ta == SKL_DT_BF16 || g->ta == SKL_DT_F16) ? 2 : 1;
   if (streams_in_place(g, es)) return 0;
-  if (g->rq.act || g->rq.q) return 0;  // the streaming kernel has no activation / requantisation steps
+  if (g->rq.act || g->rq.q) return 0;  // the streaming kernel over padded copies has no activation / requantisation steps
   if (fp8a && g->k <= kF8ExactMaxK) return 0;  // short K: the exact fp8 product, which the streaming kernel does not have
   const size_t tiles_m = (g->m + 255) / 256;
   int tile_cols = 0;

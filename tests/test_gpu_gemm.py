@@ -343,7 +343,9 @@ EXTRA_STEP_SHAPES = (
     # m, n, k, beta, what serves it
     (130, 200, 64, 1, "64 x 64 bounds-checked tiles"),
     (300, 1100, 96, 0, "128 x 128 bounds-checked tiles"),
-    (512, 768, 256, 1, "whole 256 x 128 tiles: still the bounds-checked kernels, which carry the steps"),
+    (512, 768, 256, 1, "whole tiles, too few for the streaming kernel"),
+    (2048, 2048, 128, 1, "streaming kernel, 256 x 128 tiles (int8 with a row-major copy; everything else: bounds-checked kernels)"),
+    (2048, 9216, 128, 0, "streaming kernel, 256 x 256 tiles and a second launch of 256 x 128 on the last columns (int8)"),
     (1000, 1100, 520, 0, "ragged and large enough for padded copies: must stay on the bounds-checked kernels"),
     (16, 4096, 4096, 1, "a decode batch"),
     (40, 300, 8192, 1, "K shared between workgroups: the steps ride on the pass that adds the shares"),
@@ -370,7 +372,7 @@ def test_fused_activation_and_requantised_copy(gpu, ta, m, n, k, beta, what):
         start = np.array([-np.inf], np.float32)
     spread = float(np.abs(run_fused_gemm(gpu, "rc", case, a, b, c, None, None, "device")[0].astype(np.float64)).max())
     scales = (rng.uniform(0.5, 2.0, n) * 100.0 / max(spread, 1e-3)).astype(np.float32)  # some values saturate
-    layouts = ((n + 3, 1), (1, m + 5))  # (rsq, csq)
+    layouts = ((n + 4, 1), (1, m + 5))  # (rsq, csq); row-major rows on 4-byte boundaries: the streaming kernel writes them as dwords (int8)
     for mode in MODES:
         anchor, _ = run_fused_gemm(gpu, "rc", case, a, b, c, bias, None, mode)
         for act, per_column, (rsq, csq), zero, only in ((1, True, layouts[0], 3, False), (0, False, layouts[1], -7, False),
