@@ -140,7 +140,8 @@ def _wl_small_batch(m):
         def step(i):
             lib.skl_gemm_i8_i8_i32_gfx950(m, n, k, 1, x, k, w[i % nbuf], n, 0, y, n)
 
-        kernel = "gemv_rows_kernel" if m <= 3 else "gemv_mfma_scale_c_kernel + gemv_mfma_rows_kernel"
+        kernel = ("gemv_rows_kernel" if m <= 3 else "gemv_mfma_scale_c_kernel + gemv_mfma_rows_kernel" if m <= 16 else
+                  "gemm_mfma_kernel (K shared between workgroups) + gemm_split_reduce_kernel")
         return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
                     name=f"int8 GEMM {m}x4096x11008 (decode with a batch of {m}: still a stream over W)", kernel=kernel)
     return build
@@ -517,6 +518,8 @@ WORKLOADS = {
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 10, 2, 64),
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 10, 2, 64),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 10, 2, 64),
+    "gemm_i8_32x4096x11008": (_wl_small_batch(32), 10, 2, 64),
+    "gemm_i8_64x4096x11008": (_wl_small_batch(64), 10, 2, 32),
     "gemm_i8_p4x1c_16x4096x11008": (_wl_small_batch_p4x1c(16), 10, 2, 64),
     "gemm_i8_p4x1c_32x4096x11008": (_wl_small_batch_p4x1c(32), 10, 2, 32),
     "gemm_i8_p4x1c_112x4096x11008": (_wl_small_batch_p4x1c(112), 10, 2, 32),
