@@ -33,9 +33,9 @@ static int g_nranges;
 static long g_checked, g_launches;
 static int g_failures;
 /* how often each stand-in ran: the summary shows which routes of the dispatch the cases reached */
-enum { P_GENERIC, P_TILED, P_MFMA, P_PADDED, P_GEMV, P_GEMV_K4, P_ROWS, P_MFMA_ROWS, P_MFMA_ROWS_K4, P_KC, P_REALIGN, P_PACK, P_UNPACK, P_CVT, P_SCARCE, P_COUNT };
+enum { P_GENERIC, P_TILED, P_MFMA, P_PADDED, P_GEMV, P_GEMV_K4, P_ROWS, P_MFMA_ROWS, P_MFMA_ROWS_K4, P_KC, P_REALIGN, P_PACK, P_UNPACK, P_CVT, P_F4, P_SCARCE, P_COUNT };
 static const char *const kPathNames[P_COUNT] = {"any-stride", "register-tiled", "matrix-core", "padded tiles", "GEMV", "GEMV K-packed", "few rows",
-                                                "decode batch", "decode batch K-packed", "dot-product GEMV", "operand copy", "pack", "unpack", "cvt",
+                                                "decode batch", "decode batch K-packed", "dot-product GEMV", "operand copy", "pack", "unpack", "cvt", "4-bit weights",
                                                 "declined: no scratch"};
 static long g_path[P_COUNT];
 
@@ -129,12 +129,24 @@ static void store_c(int dt, void *c, size_t i, double v) {
 static double scalar_of(int dt, skl_scalar s) { return dt == SKL_DT_I8 ? s.i : dt == SKL_DT_F64 ? s.d : s.f; }
 
 /* ------------------------------------------------------------------ plain loops over the two descriptors */
-static void bias_and_max(int dt, void *c, size_t idx, size_t j, const void *bias, void *max) {
-  if (!bias && !max) return;
-  double v = load_c(dt, c, idx);
-  if (bias) {
-    v += load_c(dt, bias, j);
-    store_c(dt, c, idx, v);
+/* The fused steps behind the alpha/beta step for element (i, j) of value v (include/skl-gfx950.h): bias, activation,
+ * C unless q_only, the requantised copy, the maximum. Scales are powers of two and values small integers here, so
+ * double arithmetic gives the float result exactly. */
+static void fused_steps(int dt, void *c, size_t idx, size_t i, size_t j, double v, const void *bias, void *max, const skl_requant *rq,
+                        const char *who) {
+  if (bias) v += load_c(dt, bias, j);
+  if (rq->act == 1 && !(v > 0)) v = 0;
+  if (!rq->q_only) store_c(dt, c, idx, v);
+  if (rq->q) {
+    const size_t at = i * rq->rsq + j * rq->csq;
+    double r;
+    long t;
+    must_own(rq->q, at, at, 1, who);
+    must_own(rq->q_scale, rq->q_per_column ? j : 0, rq->q_per_column ? j : 0, sizeof(float), who);
+    if (g_failures) return;
+    r = nearbyint(v * (double)rq->q_scale[rq->q_per_column ? j : 0]);
+    t = (long)(r > 1e9 ? 1e9 : r < -1e9 ? -1e9 : r) + rq->q_zero;
+    rq->q[at] = (int8_t)(t < -128 ? -128 : t > 127 ? 127 : t);
   }
   if (max && v > load_c(dt, max, 0)) store_c(dt, max, 0, v);
 }
@@ -155,7 +167,7 @@ static void gemm_over_desc(const skl_gemm_desc *d, int check, const char *who) {
       for (size_t J = 0; J < d->n1; ++J)
         for (size_t j = 0; j < d->n0; ++j) {
           double acc = 0;
-          if (d->ta == SKL_DT_I8 && d->k0 == 1) { /* the common case without the per-element dispatch */
+          if (d->ta == SKL_DT_I8 && d->k0 == 1 && d->k1 != 0) { /* the common case without the per-element dispatch (K = 0: A and B may be null) */
             const int8_t *ap = (const int8_t *)d->a + I * d->rsa1 + i * d->rsa0, *bp = (const int8_t *)d->b + J * d->csb1 + j * d->csb0;
             long sum = 0;
             for (size_t P = 0; P < d->k1; ++P) sum += (long)ap[P * d->csa1] * bp[P * d->rsb1];
@@ -167,8 +179,8 @@ static void gemm_over_desc(const skl_gemm_desc *d, int check, const char *who) {
                        load_elem(d->tb, d->b, P * d->rsb1 + J * d->csb1 + p * d->rsb0 + j * d->csb0);
           }
           const size_t idx = I * d->rsc1 + J * d->csc1 + i * d->rsc0 + j * d->csc0;
-          store_c(d->ta, d->c, idx, beta * load_c(d->ta, d->c, idx) + alpha * acc);
-          bias_and_max(d->ta, d->c, idx, J * d->n0 + j, d->bias, d->max);
+          fused_steps(d->ta, d->c, idx, I * d->m0 + i, J * d->n0 + j, beta * load_c(d->ta, d->c, idx) + alpha * acc, d->bias, d->max, &d->rq,
+                      who);
         }
 }
 
@@ -207,8 +219,7 @@ static void gemm_over_canon(const skl_gemm_canon *g, int layout, const char *who
       const size_t idx = (i >> g->c_row_shift) * g->rsc1 + (i & rmask) * g->rsc0 + (j >> g->c_col_shift) * g->csc1 + (j & cmask) * g->csc0;
       if (idx > c_max) c_max = idx;
       if (g->k == 0 && i == 0 && j == 0) must_own(g->c, 0, 0, esc, who);
-      store_c(g->ta, g->c, idx, beta * load_c(g->ta, g->c, idx) + alpha * acc);
-      bias_and_max(g->ta, g->c, idx, j, g->bias, g->max);
+      fused_steps(g->ta, g->c, idx, i, j, beta * load_c(g->ta, g->c, idx) + alpha * acc, g->bias, g->max, &g->rq, who);
     }
   if (g->k) {
     must_own(g->a, 0, a_max, esa, who);
@@ -398,8 +409,44 @@ int __wrap_skl_hip_launch_cvt_f8_bf16(int fmt, uint16_t *dst, const uint8_t *src
   (void)fmt;
   return cvt_spans(dst, 2 * n, src, n, "cvt fp8 -> bf16");
 }
+/* E2M1 code -> the E4M3 byte of the same value (ref/cvt/cvt_ofp4.c:59-68 is exact) */
+static const uint8_t kE2M1AsE4M3[16] = {0x00, 0x30, 0x38, 0x3C, 0x40, 0x44, 0x48, 0x4C, 0x80, 0xB0, 0xB8, 0xBC, 0xC0, 0xC4, 0xC8, 0xCC};
+static unsigned nibble_of(const uint8_t *b, size_t i) { return (i & 1) ? (unsigned)(b[i / 2] >> 4) : (unsigned)(b[i / 2] & 0xF); }
 int __wrap_skl_hip_launch_cvt_f4_f8e4m3(uint8_t *dst, const uint8_t *src, size_t n) {
-  return cvt_spans(dst, n, src, (n + 1) / 2, "cvt fp4 -> fp8");
+  const int rc = cvt_spans(dst, n, src, (n + 1) / 2, "cvt fp4 -> fp8");
+  if (!g_failures) /* the GEMM over 4-bit weights multiplies what this writes */
+    for (size_t i = 0; i < n; ++i) dst[i] = kE2M1AsE4M3[nibble_of(src, i)];
+  return rc;
+}
+int __wrap_skl_hip_launch_gemv_f4(size_t m, size_t n, size_t k, skl_scalar alpha, const void *a, size_t rsa, size_t csa, const void *b,
+                                  size_t ldb, skl_scalar beta, float *c, size_t rsc, size_t csc) {
+  const char *who = "4-bit-weight decode kernel";
+  EXPECT(skl_hip_gemv_f4_supported(m, n, k, a, rsa, csa, b, ldb), "4-bit-weight decode kernel handed a problem it does not support");
+  ++g_launches, ++g_path[P_F4];
+  must_own(a, 0, (m - 1) * rsa + (k - 1) * csa, 1, who);
+  must_own(b, 0, ((n - 1) * ldb + k - 1) / 2, 1, who);
+  must_own(c, 0, (m - 1) * rsc + (n - 1) * csc, sizeof(float), who);
+  if (g_failures) return 0;
+  for (size_t i = 0; i < m; ++i)
+    for (size_t j = 0; j < n; ++j) {
+      double acc = 0;
+      for (size_t p = 0; p < k; ++p)
+        acc += f8_value(((const uint8_t *)a)[i * rsa + p * csa], 4) * f8_value(kE2M1AsE4M3[nibble_of((const uint8_t *)b, j * ldb + p)], 4);
+      c[i * rsc + j * csc] = (float)((double)beta.f * c[i * rsc + j * csc] + (double)alpha.f * acc);
+    }
+  return 0;
+}
+static void *g_converted_scratch;
+void *__wrap_skl_hip_converted_scratch(size_t bytes) {
+  if (g_scarce) return NULL;
+  if (g_converted_scratch) {
+    range_remove(g_converted_scratch);
+    free(g_converted_scratch);
+  }
+  g_converted_scratch = malloc(bytes ? bytes : 1);
+  range_add(g_converted_scratch, bytes ? bytes : 1, 1);
+  memset(g_converted_scratch, 0xEE, bytes);
+  return g_converted_scratch;
 }
 
 /* "device" memory is host memory the registry knows as device memory */
@@ -495,19 +542,37 @@ static const int kKinds[][2] = {{SKL_DT_I8, SKL_DT_I8},         {SKL_DT_BF16, SK
                                 {SKL_DT_F32, SKL_DT_F32},       {SKL_DT_F64, SKL_DT_F64},       {SKL_DT_F16H, SKL_DT_F16H}};
 
 /* One blocked GEMM through the entry point of its kind. */
-static void call_blocked(skl_gemm_desc *d) {
+static void call_blocked(skl_gemm_desc *d, const skl_gfx950_epilogue_t *ep) {
   switch (d->ta) {
     case SKL_DT_I8:
+      if (ep) {
+        skl_gemm_fused_i8rcprc_i8rcprc_i32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.i, d->a, d->rsa0, d->csa0, d->rsa1,
+                                                 d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.i, d->c, d->rsc0, d->csc0,
+                                                 d->rsc1, d->csc1, ep);
+        break;
+      }
       skl_gemm_i8rcprc_i8rcprc_i32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.i, d->a, d->rsa0, d->csa0, d->rsa1,
                                                d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.i, d->c, d->rsc0, d->csc0,
                                                d->rsc1, d->csc1);
       break;
     case SKL_DT_BF16:
+      if (ep) {
+        skl_gemm_fused_bf16rcprc_bf16rcprc_f32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.f, d->a, d->rsa0, d->csa0, d->rsa1,
+                                                     d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.f, d->c, d->rsc0,
+                                                     d->csc0, d->rsc1, d->csc1, ep);
+        break;
+      }
       skl_gemm_bf16rcprc_bf16rcprc_f32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.f, d->a, d->rsa0, d->csa0, d->rsa1,
                                                    d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.f, d->c, d->rsc0,
                                                    d->csc0, d->rsc1, d->csc1);
       break;
     case SKL_DT_F16:
+      if (ep) {
+        skl_gemm_fused_f16rcprc_f16rcprc_f32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.f, d->a, d->rsa0, d->csa0, d->rsa1,
+                                                   d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.f, d->c, d->rsc0, d->csc0,
+                                                   d->rsc1, d->csc1, ep);
+        break;
+      }
       skl_gemm_f16rcprc_f16rcprc_f32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.f, d->a, d->rsa0, d->csa0, d->rsa1,
                                                  d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.f, d->c, d->rsc0, d->csc0,
                                                  d->rsc1, d->csc1);
@@ -518,11 +583,23 @@ static void call_blocked(skl_gemm_desc *d) {
                                                 d->beta.f, d->c, d->rsc1, d->csc1);
         break;
       }
+      if (ep) {
+        skl_gemm_fused_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.f, d->a, d->rsa0, d->csa0,
+                                                         d->rsa1, d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.f, d->c,
+                                                         d->rsc0, d->csc0, d->rsc1, d->csc1, ep);
+        break;
+      }
       skl_gemm_f8e4m3rcprc_f8e4m3rcprc_f32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.f, d->a, d->rsa0, d->csa0,
                                                        d->rsa1, d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.f, d->c,
                                                        d->rsc0, d->csc0, d->rsc1, d->csc1);
       break;
     case SKL_DT_F8E5M2:
+      if (ep) {
+        skl_gemm_fused_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.f, d->a, d->rsa0, d->csa0,
+                                                         d->rsa1, d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.f, d->c,
+                                                         d->rsc0, d->csc0, d->rsc1, d->csc1, ep);
+        break;
+      }
       skl_gemm_f8e5m2rcprc_f8e5m2rcprc_f32rcprc_gfx950(d->m0, d->n0, d->k0, d->m1, d->n1, d->k1, d->alpha.f, d->a, d->rsa0, d->csa0,
                                                        d->rsa1, d->csa1, d->b, d->rsb0, d->csb0, d->rsb1, d->csb1, d->beta.f, d->c,
                                                        d->rsc0, d->csc0, d->rsc1, d->csc1);
@@ -611,20 +688,97 @@ static int run_gemm_case(int device_pointers) {
     memcpy(want.ptr, c.ptr, nc * esc);
     d.a = a.ptr, d.b = b.ptr, d.c = c.ptr;
     set_scalars(&d, small(), rnd() % 3 ? small() : 0);
+    /* A third of the calls of the kinds that have them go through the fused entry points with a random descriptor:
+     * bias, maximum, activation, a requantised copy in either orientation with one scale or one per column, q_only. */
+    const int fusable = ta == tb && (ta == SKL_DT_I8 || ta == SKL_DT_BF16 || ta == SKL_DT_F16 || ta == SKL_DT_F8E4M3 || ta == SKL_DT_F8E5M2);
+    const int fused = fusable && rnd() % 3 == 0;
+    const size_t M = d.m0 * d.m1, N = d.n0 * d.n1;
+    skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE;
+    buf_t bias = {0}, top = {0}, q = {0}, scales = {0}, want_q = {0}, want_top = {0};
+    size_t nq = 0;
+    if (fused) {
+      static const float kScales[4] = {0.25f, 0.5f, 1.0f, 2.0f};
+      if (rnd() % 2) {
+        bias = new_buf(N * esc, device_pointers);
+        for (size_t j = 0; j < N; ++j) store_c(ta, bias.ptr, j, small());
+        ep.bias = bias.ptr;
+      }
+      if (rnd() % 2) {
+        top = new_buf(esc, device_pointers), want_top = new_buf(esc, 0);
+        store_c(ta, top.ptr, 0, -1000), store_c(ta, want_top.ptr, 0, -1000);
+        ep.max = top.ptr;
+      }
+      ep.activation = (int)(rnd() % 2);
+      if (rnd() % 2) {
+        const size_t pad = rnd() % 5;
+        if (rnd() % 2) ep.rsq = N + pad, ep.csq = 1; else ep.rsq = 1, ep.csq = M + pad;
+        nq = (M - 1) * ep.rsq + (N - 1) * ep.csq + 1;
+        q = new_buf(nq, device_pointers), want_q = new_buf(nq, 0);
+        memset(q.ptr, 0x5A, nq), memset(want_q.ptr, 0x5A, nq);
+        ep.q = (int8_t *)q.ptr;
+        ep.q_scale_per_column = (int)(rnd() % 2);
+        scales = new_buf((ep.q_scale_per_column ? N : 1) * sizeof(float), device_pointers);
+        for (size_t j = 0; j < (ep.q_scale_per_column ? N : 1); ++j) ((float *)scales.ptr)[j] = kScales[rnd() % 4];
+        ep.q_scale = (const float *)scales.ptr;
+        ep.q_zero = small();
+        ep.q_only = rnd() % 3 == 0;
+      }
+    }
     {
       skl_gemm_desc ref = d;
       ref.c = want.ptr;
-      gemm_over_desc(&ref, 0, "reference loops");
+      ref.bias = ep.bias;
+      ref.max = want_top.ptr;
+      ref.rq.act = ep.activation, ref.rq.q_per_column = ep.q_scale_per_column, ref.rq.q_only = ep.q_only && ep.q, ref.rq.q_zero = ep.q_zero;
+      ref.rq.q = (int8_t *)want_q.ptr, ref.rq.rsq = ep.rsq, ref.rq.csq = ep.csq, ref.rq.q_scale = ep.q_scale;
+      { /* the reference loops read bias and scales where the caller put them: known to the registry either way */
+        gemm_over_desc(&ref, 0, "reference loops");
+      }
     }
-    call_blocked(&d);
+    call_blocked(&d, fused ? &ep : NULL);
     if (skl_hip_last_error() != 0) fail(skl_hip_last_error_string());
-    if (memcmp(want.ptr, c.ptr, nc * esc) != 0) {
-      fprintf(stderr, "FAIL: GEMM result differs: kind %d/%d form %d blocks %zu %zu %zu x %zu %zu %zu, %s pointers\n", ta, tb, form, d.m0,
-              d.n0, d.k0, d.m1, d.n1, d.k1, device_pointers ? "device" : "host");
+    if (memcmp(want.ptr, c.ptr, nc * esc) != 0 || (nq && memcmp(want_q.ptr, q.ptr, nq) != 0) ||
+        (top.ptr && memcmp(want_top.ptr, top.ptr, esc) != 0)) {
+      fprintf(stderr, "FAIL: GEMM result differs: kind %d/%d form %d blocks %zu %zu %zu x %zu %zu %zu, %s pointers, fused %d (act %d, q %d, q_only %d)\n",
+              ta, tb, form, d.m0, d.n0, d.k0, d.m1, d.n1, d.k1, device_pointers ? "device" : "host", fused, ep.activation, ep.q != NULL, ep.q_only);
       ++g_failures;
     }
     drop_buf(a), drop_buf(b), drop_buf(c), drop_buf(want);
+    if (bias.ptr) drop_buf(bias);
+    if (top.ptr) drop_buf(top), drop_buf(want_top);
+    if (q.ptr) drop_buf(q), drop_buf(want_q), drop_buf(scales);
   }
+  return g_failures;
+}
+
+/* E4M3 A times 4-bit B stored column by column: decode shapes on the kernel that reads the weights as they are,
+ * everything else through the converted copy and the fp8 GEMM's dispatch. */
+static int run_f4_case(int device_pointers) {
+  const size_t m = rnd() % 3 ? rnd_in(1, 16) : rnd_in(17, 40), n = rnd_in(1, 40);
+  const size_t k = rnd() % 8 == 0 ? 0 : rnd() % 2 ? 32 * rnd_in(1, 6) : rnd_in(1, 150);
+  const size_t ldb = rnd() % 2 ? (k + 31) / 32 * 32 + 32 * (rnd() % 2) : k + rnd() % 5, rsa = rnd() % 2 ? (k + 15) / 16 * 16 + 16 : k + rnd() % 3 + 1;
+  const size_t rsc = n + rnd() % 3, nib = k ? (n - 1) * ldb + k : 0;
+  buf_t a = new_buf(m * rsa, device_pointers), b = new_buf((nib + 1) / 2 + 1, device_pointers), c = new_buf(m * rsc * sizeof(float), device_pointers);
+  buf_t want = new_buf(m * rsc * sizeof(float), 0);
+  const float alpha = (float)small(), beta = rnd() % 3 ? (float)small() : 0.0f;
+  for (size_t i = 0; i < m * rsa; ++i) store_small(SKL_DT_F8E4M3, a.ptr, i, small());
+  for (size_t i = 0; i < b.bytes; ++i) ((uint8_t *)b.ptr)[i] = (uint8_t)rnd();
+  for (size_t i = 0; i < m * rsc; ++i) ((float *)c.ptr)[i] = (float)small();
+  memcpy(want.ptr, c.ptr, m * rsc * sizeof(float));
+  for (size_t i = 0; i < m; ++i)
+    for (size_t j = 0; j < n; ++j) {
+      double acc = 0;
+      for (size_t p = 0; p < k; ++p)
+        acc += f8_value(((const uint8_t *)a.ptr)[i * rsa + p], 4) * f8_value(kE2M1AsE4M3[nibble_of((const uint8_t *)b.ptr, j * ldb + p)], 4);
+      ((float *)want.ptr)[i * rsc + j] = (float)((double)beta * ((float *)want.ptr)[i * rsc + j] + (double)alpha * acc);
+    }
+  skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(m, n, k, alpha, (const uint8_t *)a.ptr, rsa, 1, (const uint8_t *)b.ptr, ldb, beta, (float *)c.ptr, rsc, 1);
+  if (skl_hip_last_error() != 0) fail(skl_hip_last_error_string());
+  if (memcmp(want.ptr, c.ptr, m * rsc * sizeof(float)) != 0) {
+    fprintf(stderr, "FAIL: 4-bit-weight GEMM differs: %zu x %zu x %zu, ldb %zu, rsa %zu, %s pointers\n", m, n, k, ldb, rsa, device_pointers ? "device" : "host");
+    ++g_failures;
+  }
+  drop_buf(a), drop_buf(b), drop_buf(c), drop_buf(want);
   return g_failures;
 }
 
@@ -693,7 +847,7 @@ static void run_rowmajor(int ta, size_t m, size_t n, size_t k, size_t pad_a, siz
   set_scalars(&d, alpha, beta);
   gemm_over_desc(&d, 0, "reference loops");
   d.c = c.ptr;
-  call_blocked(&d);
+  call_blocked(&d, NULL);
   if (skl_hip_last_error() != 0) fail(skl_hip_last_error_string());
   if (memcmp(want.ptr, c.ptr, c.bytes) != 0) fail(what);
   drop_buf(a), drop_buf(b), drop_buf(c), drop_buf(want);
@@ -730,13 +884,14 @@ static int run_large_cases(void) {
 }
 
 int main(int argc, char **argv) {
-  const int cases = argc > 1 ? atoi(argv[1]) : 600;
+  const int cases = argc > 1 ? atoi(argv[1]) : 900;
   if (argc > 2) g_rng ^= strtoull(argv[2], NULL, 0);
   for (int t = 0; t < cases && !g_failures; ++t) {
     const int device_pointers = (int)(rnd() % 2);
     switch (rnd() % 8) {
       case 0: run_pack_case(device_pointers); break;
       case 1: run_cvt_case(device_pointers); break;
+      case 2: run_f4_case(device_pointers); break;
       default: run_gemm_case(device_pointers); break;
     }
   }
@@ -744,7 +899,7 @@ int main(int argc, char **argv) {
   for (int t = 0; t < cases / 4 && !g_failures; ++t) run_gemm_case((int)(rnd() % 2));
   g_scarce = 0;
   if (!g_failures && argc <= 2) run_large_cases();  /* with a seed: random cases only */
-  if (g_nranges != (g_operand_scratch ? 1 : 0)) fail("a buffer of the host layer was not released");
+  if (g_nranges != (g_operand_scratch ? 1 : 0) + (g_converted_scratch ? 1 : 0)) fail("a buffer of the host layer was not released");
   printf("%s: %d cases, %ld launches carried out, %ld address ranges checked\n", g_failures ? "host layer check FAILED" : "host layer ok",
          cases, g_launches, g_checked);
   for (int q = 0; q < P_COUNT; ++q) printf("  %-24s %ld\n", kPathNames[q], g_path[q]);
