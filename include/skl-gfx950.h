@@ -143,6 +143,13 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, 
  *     v = beta*C(i,j) + alpha*(A*B)(i,j)        as in the plain GEMM, beta == 0 included
  *     v = v + bias[j]                            if bias != NULL (one rounded addition; int32 wraps)
  *     v = v > 0 ? v : 0                          if activation == SKL_GFX950_ACT_RELU (a NaN becomes 0)
+ *     v = v / (1 + exp(-v))                      if activation == SKL_GFX950_ACT_SILU, v * Phi(v) if SKL_GFX950_ACT_GELU:
+ *                                                floating-point C only; the values of the reference's
+ *                                                skl_silu_f32_ref (ref/sigmoid/sigmoid_f32.c:36-38) and skl_gelu_f32_ref
+ *                                                (ref/gelu/gelu_f32.c:12-22) to within the error its own vector kernels
+ *                                                are held to (test/sigmoid/sigmoid_f32_zve32f.c: 52 ulp;
+ *                                                test/gelu/skl_gelu_f32_zve32f.c: 4 ulp for v >= 0, 5 in [-1, 0),
+ *                                                62 in [-2, -1), unbounded below), a NaN stays a NaN
  *     C(i,j) = v                                 unless q_only
  *     Q(i,j) = clamp(rne((float)v * s_j) + q_zero, -128, 127)      if q != NULL: the requantised int8 copy,
  *                                                at q[i*rsq + j*csq]; s_j = q_scale[j] with q_scale_per_column, else
@@ -160,6 +167,8 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, 
  * (e.g. by a designated initialiser that names only bias and max) switch their step off. ep == NULL: the plain GEMM. */
 #define SKL_GFX950_ACT_NONE 0
 #define SKL_GFX950_ACT_RELU 1
+#define SKL_GFX950_ACT_SILU 2 /* floating-point C only */
+#define SKL_GFX950_ACT_GELU 3 /* floating-point C only */
 /* Every step off: `skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE; ep.bias = ...;` is valid C and C++. */
 #define SKL_GFX950_EPILOGUE_NONE {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 typedef struct skl_gfx950_epilogue {

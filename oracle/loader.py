@@ -29,6 +29,8 @@ _EXTRA_ORACLE = {
     "skl_oracle_widen_f8e4m3_f64": (None, "ppz"),
     "skl_oracle_widen_f8e5m2_f64": (None, "ppz"),
     "skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle": (None, "zzzfpzzpzfpzz"),
+    "skl_oracle_silu_f32": (ctypes.c_float, "f"),
+    "skl_oracle_gelu_f32": (ctypes.c_float, "f"),
     # (m, n, c, rsc, csc, activation, q, rsq, csq, q_scale, per_column, q_zero)
     "skl_oracle_act_requant_i32": (None, "zzpzzipzzpii"),
     "skl_oracle_act_requant_f32": (None, "zzpzzipzzpii"),
@@ -38,6 +40,8 @@ _RC = "zzz{s}pzzpzz{s}pzz"
 _RCPRC = "zzzzzz{s}pzzzzpzzzz{s}pzzzz"
 _HELPER_GEMMS = {}  # the f32 / f64 routines are part of the shared list
 #: scalar routines of the reference library
+#: (out, in, n) activations of the reference library, used to pin the checker's restatements
+_REF_UNARY = ("skl_silu_f32_ref", "skl_gelu_f32_ref")
 _REF_SCALARS = {
     "skl_cvt_f8e4m3_f32": (ctypes.c_float, "b"),
     "skl_cvt_f8e5m2_f32": (ctypes.c_float, "b"),
@@ -123,4 +127,7 @@ def load_ref():
         setattr(f, name, _wrap(signatures.bind(cdll, name, sig), sig))
     for name, (restype, sig) in _REF_SCALARS.items():
         setattr(f, name, _wrap(signatures.bind(cdll, name, sig, restype), sig))
+    for name in _REF_UNARY:
+        if hasattr(cdll, name):  # a library built before these sources joined the list lacks them
+            setattr(f, name, _wrap(signatures.bind(cdll, name, "ppz"), "ppz"))
     return f

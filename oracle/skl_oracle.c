@@ -481,6 +481,10 @@ FUSED_RCPRC(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, float)
  * skl_gfx950_epilogue_t, restated here over a C that already holds the alpha/beta (and bias) result. They sit
  * between the bias and the maximum, so a test composes: plain GEMM, bias, these, maximum.
  *   activation 1:  v = v > 0 ? v : 0     (a NaN becomes 0), written back to C
+ *   activation 2:  SiLU as ref/sigmoid/sigmoid_f32.c:10-28 evaluates skl_silu_f32_ref (beta = 1, y = x, no gate): the
+ *                  logistic in double, times x, rounded to float once          (floating point only)
+ *   activation 3:  GELU as ref/gelu/gelu_f32.c:12-22: fma(-|x|/2, erfc(|x|/sqrt 2), relu(x)) in double, rounded to
+ *                  float once                                                   (floating point only)
  *   q != NULL:     Q(i,j) = clamp(rne((float)v * s_j) + zero, -128, 127), one fp32 product, rne to the nearest
  *                  integer with ties to even; a NaN counts as 0, values beyond int32 as its ends
  */
@@ -490,6 +494,23 @@ static int8_t requantised(float v, float scale, int32_t zero) {
   t += zero;
   return (int8_t)(t < -128 ? -128 : t > 127 ? 127 : t);
 }
+float skl_oracle_silu_f32(float x) {
+  const double a = x;
+  double o = 1. / (1. + exp(-1.f * a)); /* beta = 1.f, as skl_silu_f32_ref passes it */
+  o *= x;
+  return (float)o;
+}
+float skl_oracle_gelu_f32(float x) {
+  const double sqrt2 = 0x1.6a09e667f3bcdp0;
+  const float b = (x > 0) ? x : -0.f;
+  const float h = -0.5f * fabsf(x);
+  const double e = erfc(-sqrt2 * h);
+  return (float)fma(h, e, b);
+}
+static int32_t activated_i32(int32_t v, int activation) { return activation == 1 ? (v > 0 ? v : 0) : v; }
+static float activated_f32(float v, int activation) {
+  return activation == 1 ? (v > 0 ? v : 0) : activation == 2 ? skl_oracle_silu_f32(v) : activation == 3 ? skl_oracle_gelu_f32(v) : v;
+}
 #define ACT_REQUANT(SUFFIX, TC)                                                                     \
   void skl_oracle_act_requant_##SUFFIX(size_t m, size_t n, TC *c, size_t rsc, size_t csc, int activation, \
                                        int8_t *q, size_t rsq, size_t csq, const float *q_scale,     \
@@ -497,7 +518,7 @@ static int8_t requantised(float v, float scale, int32_t zero) {
     for (size_t i = 0; i < m; ++i)                                                                  \
       for (size_t j = 0; j < n; ++j) {                                                              \
         TC v = c[i * rsc + j * csc];                                                                \
-        if (activation == 1) v = v > 0 ? v : 0;                                                     \
+        v = activated_##SUFFIX(v, activation);                                                      \
         c[i * rsc + j * csc] = v;                                                                   \
         if (q) q[i * rsq + j * csq] = requantised((float)v, q_scale[per_column ? j : 0], q_zero);   \
       }                                                                                             \

@@ -147,6 +147,8 @@ SKL_ORACLE_PFUSED_DECL(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, float)
  * steps between bias and maximum of skl_gfx950_epilogue_t (include/skl-gfx950.h). The reference has no routine
  * for them (src/gemm/README.md:46-47 leaves them to callers); tests/test_oracle_gemm.py pins these against
  * hand-worked values and an independent numpy formulation. q may be NULL. */
+float skl_oracle_silu_f32(float x); /* ref/sigmoid/sigmoid_f32.c:36-38 for one value */
+float skl_oracle_gelu_f32(float x); /* ref/gelu/gelu_f32.c:12-22 for one value */
 void skl_oracle_act_requant_i32(size_t m, size_t n, int32_t *c, size_t rsc, size_t csc, int activation, int8_t *q,
                                 size_t rsq, size_t csq, const float *q_scale, int per_column, int32_t q_zero);
 void skl_oracle_act_requant_f32(size_t m, size_t n, float *c, size_t rsc, size_t csc, int activation, int8_t *q,

@@ -52,12 +52,12 @@ def _as_pointer(x):
 
 class Epilogue:
     """Fused-epilogue operands of the `skl_gemm_fused_*` entry points: `bias` (n values of C's
-    type), `max` (one value of C's type), `activation` (ACT_NONE / ACT_RELU) and the requantised
+    type), `max` (one value of C's type), `activation` (ACT_NONE / ACT_RELU; floating-point C also ACT_SILU / ACT_GELU) and the requantised
     copy `q` (int8, element (i, j) at `i * rsq + j * csq`) made with `q_scale` (one float32, or n
     of them with `q_scale_per_column`) and `q_zero`; `q_only` leaves C unwritten. Every operand
     is a DeviceBuffer, a numpy array or None."""
 
-    ACT_NONE, ACT_RELU = 0, 1
+    ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU = 0, 1, 2, 3
 
     def __init__(self, bias=None, max=None, activation=0, q=None, rsq=0, csq=0, q_scale=None,
                  q_scale_per_column=False, q_zero=0, q_only=False):

@@ -463,7 +463,7 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
   }
   where = classify(K ? d->a : NULL, K ? d->b : NULL, d->c, who);
   if (where < 0) return;
-  if ((d->rq.act != SKL_GFX950_ACT_NONE && d->rq.act != SKL_GFX950_ACT_RELU) ||
+  if (d->rq.act < SKL_GFX950_ACT_NONE || d->rq.act > (d->ta == SKL_DT_I8 ? SKL_GFX950_ACT_RELU : SKL_GFX950_ACT_GELU) ||
       (d->rq.q && (!d->rq.q_scale || d->rq.q_zero < -128 || d->rq.q_zero > 127))) {
     skl_hip_record_error(SKL_HIP_ERR_BAD_ARGUMENT, who);
     return;

@@ -89,12 +89,39 @@ __device__ __forceinline__ void skl_update(T acc, T *c, skl_scalar alpha, skl_sc
 __device__ __forceinline__ int skl_add_bias(int v, int b) { return (int)((unsigned)v + (unsigned)b); }
 __device__ __forceinline__ float skl_add_bias(float v, float b) { return __fadd_rn(v, b); }
 
-// The activation step: 0 none, 1 max(v, 0) (a NaN becomes 0, like `v > 0 ? v : 0`).
+// The activation step: 0 none, 1 max(v, 0) (a NaN becomes 0, like `v > 0 ? v : 0`); integers have no other.
 __device__ __forceinline__ int skl_activate(int v, int act) {
   const int floor = act == 1 ? 0 : (int)0x80000000;  // uniform: one max per element
   return v < floor ? floor : v;
 }
-__device__ __forceinline__ float skl_activate(float v, int act) { return act == 1 ? (v > 0.0f ? v : 0.0f) : v; }
+// SiLU, x * logistic(x). ref/sigmoid/sigmoid_f32.c:10-28 evaluates 1 / (1 + exp(-x)) * x in double and rounds once;
+// here in fp32, arranged so that nothing cancels and nothing leaves the normal range before the last product:
+// below -17, 1 + e^x is 1 to beyond fp32 and the value is x e^x; below -80, where e^x is a denormal and would
+// carry only a few bits, e^(x + 64) is multiplied in first and e^-64 last. Within a few ulp of the reference's
+// value (its own vector kernels are tested to 52 ulp, test/sigmoid/sigmoid_f32_zve32f.c).
+__device__ __forceinline__ float skl_silu(float x) {
+  if (x < -17.0f) {
+    const bool deep = x < -80.0f;
+    const float r = x * expf(deep ? x + 64.0f : x);
+    return deep ? r * 1.6038108905486378e-28f : r;  // e^-64
+  }
+  return x / (1.0f + expf(-x));
+}
+// GELU, x Phi(x), in the reference's arrangement (ref/gelu/gelu_f32.c:12-22): an offset from the ReLU,
+// fma(-|x| / 2, erfc(|x| / sqrt 2), relu(x)) - nothing cancels on either side of zero. The reference evaluates erfc
+// and the fma in double; here fp32 (its own vector kernels are tested to 4 to 62 ulp by range,
+// test/gelu/skl_gelu_f32_zve32f.c).
+__device__ __forceinline__ float skl_gelu(float x) {
+  const float h = -0.5f * __builtin_fabsf(x);
+  const float e = erfcf(-1.41421356237309504880f * h);
+  return __builtin_fmaf(h, e, x > 0.0f ? x : -0.0f);
+}
+// 0 none, 1 ReLU, 2 SiLU, 3 GELU (floating point only).
+__device__ __forceinline__ float skl_activate(float v, int act) {
+  if (act == 0) return v;
+  if (act == 1) return v > 0.0f ? v : 0.0f;
+  return act == 2 ? skl_silu(v) : skl_gelu(v);
+}
 
 // The requantised int8 value of v: round-to-nearest-even of (float)v * scale as an integer (a NaN counts as 0, values
 // beyond int32 as its ends), plus the zero point, clamped to [-128, 127].

@@ -344,3 +344,33 @@ def assert_fp_gemm_close(case, a, b, c_before, c_after, frob_tol=1e-3, extra_rel
     assert np.array_equal(c_after[mask].view(np.uint8), c_before[mask].view(np.uint8)), \
         "elements outside the addressed C were modified"
     return float((err / (ref_bound + slack)).max()) if err.size else 0.0
+
+
+def ulp_error_f32(x, r):
+    """skl_abs_error_ulp_f32 of the reference's test driver (test/skl-test-driver.h:565-592): the distance between
+    x and the reference value r in units of ulp(r), denormal results counted in units of 2^-149."""
+    x, r = np.asarray(x, np.float32), np.asarray(r, np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        d = np.abs(x.astype(np.float64) - r.astype(np.float64))
+        _, e = np.frexp(r.astype(np.float64))
+        e = np.where((e < -125) | (r == 0), -125 - 24, e - 24)
+        err = np.ldexp(d, -e)
+    same = (x == r) | (np.isnan(x) & np.isnan(r))
+    bad = np.isinf(r) | np.isnan(x) | np.isnan(r)
+    return np.where(same, 0.0, np.where(bad, np.inf, err))
+
+
+def activation_reference(values, activation):
+    """skl_silu_f32_ref (2) / skl_gelu_f32_ref (3) through the checker's restatement, for a float32 array."""
+    v = np.ascontiguousarray(values, np.float32).copy().reshape(-1)
+    oracle().skl_oracle_act_requant_f32(1, v.size, v, v.size, 1, activation, None, 0, 0, None, 0, 0)
+    return v.reshape(np.shape(values))
+
+
+#: what the reference's own vector kernels are held to (test/sigmoid/sigmoid_f32_zve32f.c: 52 ulp on [-110, 18];
+#: test/gelu/skl_gelu_f32_zve32f.c, the tightest variant: 4 ulp for x >= 0, 5 in [-1, 0), 62 in [-2, -1), 1.7e7 below)
+def activation_ulp_bound(x, activation):
+    x = np.asarray(x, np.float64)
+    if activation == 2:
+        return np.full(x.shape, 52.0)
+    return np.where(x >= 0, 4.0, np.where(x >= -1, 5.0, np.where(x >= -2, 62.0, 1.7e7)))

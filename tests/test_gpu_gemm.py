@@ -396,6 +396,67 @@ def test_fused_activation_and_requantised_copy(gpu, ta, m, n, k, beta, what):
         assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8)) and top[0] == want_top[0], (ta, what, mode)
 
 
+@pytest.mark.parametrize("act", (2, 3))
+def test_silu_and_gelu_values(gpu, act):
+    """The activation alone: with alpha = 0 and beta = 1 the value it is applied to is C itself, so any fp32 value
+    can be put through it - the ranges of the reference's own tests (test/sigmoid/sigmoid_f32_zve32f.c: [-110, 18];
+    test/gelu/skl_gelu_f32_zve32f.c: [-14.356, 5.348]) densely, the far tails, zeros, infinities, NaN. The result must
+    be the reference routine's value (skl_silu_f32_ref / skl_gelu_f32_ref through the checker) within the error the
+    reference allows its own vector kernels, range by range; measured: well inside."""
+    rng = np.random.default_rng(act)
+    m, n, k = 256, 1024, 8
+    lo, hi = ((-110.0, 18.0), (-14.356, 5.348))[act - 2]
+    c = np.concatenate([rng.uniform(lo, hi, m * n - 70000), rng.uniform(-3, 3, 40000), rng.uniform(-1e-3, 1e-3, 29980),
+                        np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-40, -1e-40, -88.7, -103.9, -109.9, 88.8, 3e38, -3e38,
+                                  -17.0, -17.000002, -80.0, -80.00001, 1.0, -1.0, -2.0])]).astype(np.float32)
+    case = rowmajor_case("bf16", m, n, k, alpha=0.0, beta=1.0)
+    a, b, _ = case.make_inputs(1)
+    for mode in MODES:
+        got, _ = run_fused_gemm(gpu, "rc", case, a, b, c, None, None, mode, activation=act)
+        want = support.activation_reference(c, act)
+        err = support.ulp_error_f32(got, want)
+        finite = np.isfinite(want)
+        assert np.all(err[finite] <= support.activation_ulp_bound(c, act)[finite]), (act, mode, float(err[finite].max()))
+        assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(got[np.isinf(want)], want[np.isinf(want)])
+        inside = finite & (c >= (-80 if act == 2 else -1)) & (np.abs(want) > 1e-30)
+        assert err[inside].max() <= 4.0, (act, mode, float(err[inside].max()))   # where nothing underflows: a few ulp
+
+
+@pytest.mark.parametrize("ta,m,n,k,what", (
+    ("bf16", 300, 1100, 96, "bounds-checked tiles"),
+    ("f16", 2048, 2048, 128, "whole tiles: still the bounds-checked kernels, which carry the steps"),
+    ("f8e4m3", 40, 300, 8192, "K shared between workgroups: the pass that adds the shares"),
+    ("bf16", 16, 4096, 4096, "a decode batch: the pass that adds the planes"),
+    ("f8e5m2", 1, 2048, 512, "M = 1"),
+))
+def test_fused_silu_and_gelu(gpu, ta, m, n, k, what):
+    """SiLU and GELU behind alpha / beta and the bias on every kernel family: C must be the reference routine's value
+    of the fused call's own pre-activation C (the same call without an activation gives it bit for bit) within the
+    reference's bounds; the maximum is the largest value written, and the requantised copy is the rule applied to the
+    value written."""
+    from test_oracle_gemm import requantised
+    rng = np.random.default_rng(m + n + k)
+    case = rowmajor_case(ta, m, n, k, alpha=0.25, beta=1.0)
+    a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+    bias = rng.uniform(-2, 2, n).astype(np.float32)
+    start = np.array([-np.inf], np.float32)
+    scale = np.array([16.0], np.float32)
+    for mode in MODES:
+        anchor, _ = run_fused_gemm(gpu, "rc", case, a, b, c, bias, None, mode)
+        for act in (2, 3):
+            rq = dict(q=np.zeros(m * n, np.int8), rsq=n, csq=1, scale=scale, zero=-3)
+            got, top, q = run_fused_gemm(gpu, "rc", case, a, b, c, bias, start, mode, activation=act, requant=rq)
+            want = support.activation_reference(anchor, act)
+            err = support.ulp_error_f32(got, want)
+            assert np.all(err <= support.activation_ulp_bound(anchor, act)), (ta, what, mode, act, float(err.max()))
+            assert top[0] == got.max(), (ta, what, mode, act)
+            assert np.array_equal(q, requantised(got, scale[0], -3)), (ta, what, mode, act)
+    # integers have no such activation
+    icase = rowmajor_case("i8", 8, 8, 8, alpha=1, beta=0)
+    ia, ib, ic = icase.make_inputs(1)
+    run_fused_gemm_expecting_refusal(gpu, icase, ia, ib, ic, activation=2)
+
+
 def test_fused_extra_steps_blocked_form_any_strides_and_refusals(gpu):
     """The rcprc form addresses Q by the logical row and column; odd blocks and strides take the any-stride
     kernel. Descriptors the header rules out are refused before anything runs."""

@@ -265,6 +265,8 @@ def fused_expectation(case, plain, bias, max_in, activation=0, requant=None):
     if activation == 1:
         v = want[oc]
         want[oc] = np.where(v > 0, v, 0).astype(plain.dtype)
+    elif activation in (2, 3):
+        want[oc] = support.activation_reference(want[oc], activation)
     top = None
     if max_in is not None:
         written = want[oc]
@@ -348,6 +350,33 @@ def test_ofp4_gemm_is_the_conversion_followed_by_the_fp8_gemm():
     A = support.decode_table("f8e4m3")[a].reshape(m, k)
     B = f4.E2M1_VALUES[codes].reshape(n, k).T
     assert np.array_equal(got.reshape(m, n).astype(np.float64), A @ B)
+
+
+def test_silu_and_gelu_restate_the_reference():
+    """The checker's SiLU and GELU (oracle/skl_oracle.c) against the reference's own routines compiled from
+    ref/sigmoid/sigmoid_f32.c and ref/gelu/gelu_f32.c - bit for bit over the ranges of the reference's tests and the
+    special values - and, independently, against the closed forms in fp64 (scipy) and the identity f(x) - f(-x) = x."""
+    from scipy import special
+    rng = np.random.default_rng(12)
+    x = np.concatenate([rng.uniform(-110, 18, 100000), rng.uniform(-3, 3, 50000), rng.uniform(-15, 6, 50000)]).astype(np.float32)
+    x = np.concatenate([x, np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-40, -1e-40, -103.5, -88.7, 88.8, 3e38], np.float32)])
+    ref = support.ref()
+    for act, name in ((2, "skl_silu_f32_ref"), (3, "skl_gelu_f32_ref")):
+        got = support.activation_reference(x, act)
+        if ref is not None and hasattr(ref, name):
+            want = np.zeros_like(x)
+            getattr(ref, name)(want, x, x.size)
+            same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))  # a NaN's sign is the compiler's
+            assert same.all(), name
+        xd = x[:-11].astype(np.float64)
+        with np.errstate(over="ignore"):
+            closed = xd / (1 + np.exp(-xd)) if act == 2 else 0.5 * xd * special.erfc(-xd / np.sqrt(2))
+        assert support.ulp_error_f32(got[:-11], closed.astype(np.float32)).max() <= 1.0, name
+        pos = np.abs(x[:1000])
+        diff = support.activation_reference(pos, act).astype(np.float64) - support.activation_reference(-pos, act).astype(np.float64)
+        assert np.allclose(diff, pos, rtol=1e-6, atol=1e-30), name
+    assert support.activation_reference(np.array([0.0, -0.0], np.float32), 2).tolist() == [0.0, -0.0]
+    assert support.activation_reference(np.array([0.0], np.float32), 3)[0] == 0.0
 
 
 def test_requantisation_rule_on_worked_values():
