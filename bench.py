@@ -177,20 +177,26 @@ def wl_small_batch_f8(lib, rng):
                 kernel="gemv_mfma_rows_kernel<fp8 E4M3> + gemv_mfma_add_planes_kernel")
 
 
-def _wl_ofp4(m):
-    """Decode against OFP4 (E2M1) weights stored column by column: the weights cross HBM at half a byte per element.
-    16 buffers rotated (22.5 MB each) so that the stream exceeds the last-level cache."""
+def _wl_ofp4(m, mx=False):
+    """Decode against OFP4 (E2M1) weights stored column by column: the weights cross HBM at half a byte per element
+    (with `mx`: plus one E8M0 scale per 32 k, the OCP MXFP4 format). 16 buffers rotated (22.5 MB each) so that the
+    stream exceeds the last-level cache."""
     def build(lib, rng):
         k, n, nbuf = 4096, 11008, 16
         w = [DeviceBuffer.from_array(rng.integers(0, 256, size=k * n // 2, dtype=np.uint8)) for _ in range(nbuf)]
+        sc = [DeviceBuffer.from_array(rng.integers(120, 135, size=n * k // 32, dtype=np.uint8)) for _ in range(nbuf)] if mx else None
         x = DeviceBuffer.from_array(rng.integers(8, 127, size=m * k, dtype=np.uint8))
         y = DeviceBuffer(4 * m * n)
 
         def step(i):
-            lib.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(m, n, k, 1.0, x, k, 1, w[i % nbuf], k, 0.0, y, n, 1)
+            if mx:
+                lib.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_gfx950(m, n, k, 1.0, x, k, 1, w[i % nbuf], k, sc[i % nbuf], k // 32, 0.0, y, n, 1)
+            else:
+                lib.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(m, n, k, 1.0, x, k, 1, w[i % nbuf], k, 0.0, y, n, 1)
 
-        return dict(fn=step, bytes=k * n // 2 + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="f4e2m1", keep=(w, x, y),
-                    name=f"E4M3 x OFP4 GEMM {m}x4096x11008 (4-bit weights, columns contiguous in K, beta=0)",
+        return dict(fn=step, bytes=k * n // 2 + (k * n // 32 if mx else 0) + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm",
+                    dtype="f4e2m1", keep=(w, sc or [], x, y),
+                    name=f"E4M3 x {'MXFP4' if mx else 'OFP4'} GEMM {m}x4096x11008 (4-bit weights, columns contiguous in K, beta=0)",
                     kernel="gemv_f4_kernel")
     return build
 
@@ -512,6 +518,8 @@ WORKLOADS = {
     "gemv_f8e4m3": (wl_gemv_f8, 10, 2, 128),
     "gemv_f8e4m3_f4_1x4096x11008": (_wl_ofp4(1), 10, 2, 128),
     "gemm_f8e4m3_f4_16x4096x11008": (_wl_ofp4(16), 10, 2, 128),
+    "gemv_f8e4m3_mxf4_1x4096x11008": (_wl_ofp4(1, mx=True), 10, 2, 128),
+    "gemm_f8e4m3_mxf4_16x4096x11008": (_wl_ofp4(16, mx=True), 10, 2, 128),
     "gemv_i8_1x8192x28672": (wl_gemv_large, 10, 2, 32),
     "gemv_i8_kcontig": (wl_gemv_kc, 10, 2, 128),
     "gemv_bf16_kcontig": (wl_gemv_kc_bf16, 10, 2, 64),

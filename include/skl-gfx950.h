@@ -82,6 +82,17 @@ void skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950(size_t m, size_t n, size_t k, float
 void skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
                                             size_t rsa, size_t csa, const uint8_t *b, size_t ldb, float beta,
                                             float *c, size_t rsc, size_t csc);
+/* The same with OCP microscaling (MXFP4): every 32 consecutive k of a column share a scale 2^(s - 127), s = the
+ * E8M0 byte scales[j * lds + p / 32] (1 <= s <= 254; s == 127 everywhere or scales == NULL is the call above). The
+ * reference has no notion of block scales: the result is that of decoding both operands to fp32 - A by
+ * ref/cvt/cvt_ofp8.c:18-52, B's E2M1 values times their scales, all exact - and calling
+ * ref/gemm/gemm_f32rc_f32rc_f32rc.h:44 (sums in fp32), inside the error bound of the reference's fp8 GEMM test.
+ * Decode shapes (as above) stream the weights and hand the scales to the matrix cores one per lane and instruction;
+ * every other call converts both operands to bf16 (exact) into scratch memory and runs the bf16 GEMM. */
+void skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a,
+                                              size_t rsa, size_t csa, const uint8_t *b, size_t ldb,
+                                              const uint8_t *scales, size_t lds, float beta, float *c, size_t rsc,
+                                              size_t csc);
 /* ref/gemm/gemm_f32rc_f32rc_f32rc.h:44. Vector ALUs (the result is defined operation by operation): the
  * register-tiled kernel, or the any-stride kernel for tiny or oddly blocked problems. */
 void skl_gemm_f32rc_f32rc_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const float *a, size_t rsa,

@@ -29,6 +29,7 @@ _EXTRA_ORACLE = {
     "skl_oracle_widen_f8e4m3_f64": (None, "ppz"),
     "skl_oracle_widen_f8e5m2_f64": (None, "ppz"),
     "skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle": (None, "zzzfpzzpzfpzz"),
+    "skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_oracle": (None, "zzzfpzzpzpzfpzz"),
     "skl_oracle_silu_f32": (ctypes.c_float, "f"),
     "skl_oracle_gelu_f32": (ctypes.c_float, "f"),
     # (m, n, c, rsc, csc, activation, q, rsq, csq, q_scale, per_column, q_zero)

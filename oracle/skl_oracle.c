@@ -367,6 +367,27 @@ void skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle(size_t m, size_t n, size_t k, float 
   free(b8);
 }
 
+/* OCP microscaling on top: every 32 consecutive k of a column share the scale 2^(s - 127), s = scales[j * lds + p / 32].
+ * Nothing in the reference knows block scales; the definition is the reference's fp32 GEMM
+ * (ref/gemm/gemm_f32rc_f32rc_f32rc.c:9-24: acc += a * b in float, k ascending, then beta * c + alpha * acc) on the
+ * decoded operands - A by ref/cvt/cvt_ofp8.c:18-52, B's E2M1 values (ref/cvt/cvt_ofp4.c:18-48) times their scales,
+ * exact in float. scales == NULL: every scale is 1. */
+void skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_oracle(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa,
+                                              size_t csa, const uint8_t *b, size_t ldb, const uint8_t *scales, size_t lds,
+                                              float beta, float *c, size_t rsc, size_t csc) {
+  for (size_t i = 0; i < m; ++i)
+    for (size_t j = 0; j < n; ++j) {
+      float acc = 0.0f;
+      for (size_t p = 0; p < k; ++p) {
+        const size_t at = j * ldb + p;
+        const uint8_t nib = (at & 1u) ? (uint8_t)(b[at >> 1] >> 4) : (uint8_t)(b[at >> 1] & 0xFu);
+        const float w = skl_oracle_f4e2m1_to_f32(nib) * (scales ? ldexpf(1.0f, (int)scales[j * lds + p / 32] - 127) : 1.0f);
+        acc += skl_oracle_f8e4m3_to_f32(a[i * rsa + p * csa]) * w;
+      }
+      c[i * rsc + j * csc] = beta * c[i * rsc + j * csc] + alpha * acc;
+    }
+}
+
 GEMM_RCPRC(f8e4m3rcprc_f8e4m3rcprc_f32rcprc, uint8_t, uint8_t, float,
            skl_oracle_f8e4m3_to_f32, skl_oracle_f8e4m3_to_f32)
 GEMM_RCPRC(f8e5m2rcprc_f8e5m2rcprc_f32rcprc, uint8_t, uint8_t, float,

@@ -121,6 +121,12 @@ void skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle(size_t m, size_t n, size_t k, float 
                                             size_t csa, const uint8_t *b, size_t ldb, float beta, float *c, size_t rsc,
                                             size_t csc);
 
+/* ... with one E8M0 scale per 32 consecutive k of a column (OCP microscaling): the reference's fp32 GEMM on the decoded
+ * operands. scales may be NULL. */
+void skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_oracle(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa,
+                                              size_t csa, const uint8_t *b, size_t ldb, const uint8_t *scales, size_t lds,
+                                              float beta, float *c, size_t rsc, size_t csc);
+
 /* GEMM + fused bias / maximum steps (src/gemm/fused-kernel-API.md:159-207); bias and max may be NULL. */
 #define SKL_ORACLE_FUSED_DECL(NAME, TA, TC)                                                        \
   void skl_gemm_fused_##NAME##_oracle(size_t m, size_t n, size_t k, TC alpha, const TA *a, size_t rsa, \

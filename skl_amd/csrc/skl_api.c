@@ -653,61 +653,80 @@ void skl_gemm_i8_i8_i32_noalloc_gfx950(size_t m, size_t n, size_t k, int32_t alp
  * Decode shapes stream the 4-bit weights through the kernel that multiplies them as they are; everything else
  * converts B once into scratch memory of the stream and runs the fp8 GEMM on that. */
 static int f4_gemm_on_device(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa, size_t csa,
-                             const uint8_t *b, size_t ldb, skl_scalar beta, float *c, size_t rsc, size_t csc) {
+                             const uint8_t *b, size_t ldb, const uint8_t *scales, size_t lds, skl_scalar beta, float *c, size_t rsc,
+                             size_t csc) {
   const skl_scalar alpha_s = {.f = alpha};
   int rc;
   if (k != 0 && skl_hip_gemv_f4_supported(m, n, k, a, rsa, csa, b, ldb))
-    return skl_hip_launch_gemv_f4(m, n, k, alpha_s, a, rsa, csa, b, ldb, beta, c, rsc, csc);
+    return skl_hip_launch_gemv_f4(m, n, k, alpha_s, a, rsa, csa, b, ldb, scales, lds, beta, c, rsc, csc);
   {
     const size_t values = k ? (n - 1) * ldb + k : 0; /* 4-bit values from B's first to its last, gaps included */
-    uint8_t *b8 = NULL;
     skl_gemm_desc d = {SKL_DT_F8E4M3, SKL_DT_F8E4M3, 1, 1, 1, m, n, k, a, 0, 0, rsa, csa, NULL, 0, 0, 1, ldb,
                        c, 0, 0, rsc, csc, {.f = alpha}, beta, NULL, NULL, {0}};
-    skl_hip_sequence_begin(); /* the converted B travels from one launch to the next through the stream's scratch */
-    if (values) {
-      b8 = (uint8_t *)skl_hip_converted_scratch(values);
-      if (!b8) {
-        skl_hip_sequence_end();
-        return SKL_HIP_ERR_WORKSPACE;
-      }
-      rc = skl_hip_launch_cvt_f4_f8e4m3(b8, b, values);
-      if (rc != 0) {
-        skl_hip_sequence_end();
-        return rc;
-      }
+    skl_hip_sequence_begin(); /* the converted operands travel from one launch to the next through the stream's scratch */
+    if (values && !scales) { /* B as E4M3: exact */
+      uint8_t *b8 = (uint8_t *)skl_hip_converted_scratch(values);
+      rc = b8 ? skl_hip_launch_cvt_f4_f8e4m3(b8, b, values) : SKL_HIP_ERR_WORKSPACE;
+      d.b = b8;
+    } else if (values) { /* scaled values leave E4M3's range: both operands as bf16 (exact), then the bf16 GEMM */
+      const size_t span_a = (m - 1) * rsa + (k - 1) * csa + 1, bytes_a = (2 * span_a + 255) / 256 * 256;
+      char *block = (char *)skl_hip_converted_scratch(bytes_a + 2 * values);
+      rc = block ? skl_hip_launch_cvt_f8_bf16(SKL_DT_F8E4M3, (uint16_t *)block, a, span_a) : SKL_HIP_ERR_WORKSPACE;
+      if (rc == 0) rc = skl_hip_launch_cvt_mxf4_bf16((uint16_t *)(block + bytes_a), b, scales, lds, n, k, ldb);
+      d.ta = d.tb = SKL_DT_BF16;
+      d.a = block;
+      d.b = block ? block + bytes_a : NULL;
+    } else {
+      rc = 0;
     }
-    d.b = b8;
-    rc = gemm_on_device(&d);
+    if (rc == 0) rc = gemm_on_device(&d);
     skl_hip_sequence_end();
     return rc;
   }
 }
 
-void skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa, size_t csa,
-                                           const uint8_t *b, size_t ldb, float beta, float *c, size_t rsc, size_t csc) {
+static void f4_gemm_run(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa, size_t csa, const uint8_t *b, size_t ldb,
+                        const uint8_t *scales, size_t lds, float beta, float *c, size_t rsc, size_t csc, const char *who) {
   skl_scalar beta_s;
   int where;
   if (m == 0 || n == 0) return; /* nothing is addressed */
   memset(&beta_s, 0, sizeof beta_s);
   beta_s.fz.value = beta;
   beta_s.fz.skip_c_read = skl_hip_get_beta_zero_mode() != SKL_HIP_BETA_ZERO_AS_REFERENCE;
-  where = classify(k ? a : NULL, k ? b : NULL, c, __func__);
+  where = classify(k ? a : NULL, k ? b : NULL, c, who);
   if (where < 0) return;
+  if (k && scales && classify(scales, NULL, NULL, who) != where) {
+    skl_hip_record_error(SKL_HIP_ERR_MIXED_POINTERS, who);
+    return;
+  }
   if (where == 1) {
-    (void)f4_gemm_on_device(m, n, k, alpha, a, rsa, csa, b, ldb, beta_s, c, rsc, csc);
+    (void)f4_gemm_on_device(m, n, k, alpha, a, rsa, csa, b, ldb, scales, lds, beta_s, c, rsc, csc);
     return;
   }
   {
     const size_t na = k ? (m - 1) * rsa + (k - 1) * csa + 1 : 0, nb = k ? ((n - 1) * ldb + k + 1) / 2 : 0;
-    const size_t nc = (m - 1) * rsc + (n - 1) * csc + 1;
-    void *da = stage_in(a, na), *db = stage_in(b, nb), *dc = stage_in(c, nc * sizeof(float));
-    if ((!na || da) && (!nb || db) && dc &&
-        f4_gemm_on_device(m, n, k, alpha, (const uint8_t *)da, rsa, csa, (const uint8_t *)db, ldb, beta_s, (float *)dc, rsc, csc) == 0)
+    const size_t ns = (k && scales) ? (n - 1) * lds + (k + 31) / 32 : 0, nc = (m - 1) * rsc + (n - 1) * csc + 1;
+    void *da = stage_in(a, na), *db = stage_in(b, nb), *ds = stage_in(scales, ns), *dc = stage_in(c, nc * sizeof(float));
+    if ((!na || da) && (!nb || db) && (!ns || ds) && dc &&
+        f4_gemm_on_device(m, n, k, alpha, (const uint8_t *)da, rsa, csa, (const uint8_t *)db, ldb, (const uint8_t *)ds, lds, beta_s,
+                          (float *)dc, rsc, csc) == 0)
       skl_hip_memcpy_d2h(c, dc, nc * sizeof(float)); /* C's whole span: the elements in its stride gaps come back unchanged */
     skl_hip_free(da);
     skl_hip_free(db);
+    skl_hip_free(ds);
     skl_hip_free(dc);
   }
+}
+
+void skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa, size_t csa,
+                                           const uint8_t *b, size_t ldb, float beta, float *c, size_t rsc, size_t csc) {
+  f4_gemm_run(m, n, k, alpha, a, rsa, csa, b, ldb, NULL, 0, beta, c, rsc, csc, __func__);
+}
+
+void skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_gfx950(size_t m, size_t n, size_t k, float alpha, const uint8_t *a, size_t rsa, size_t csa,
+                                             const uint8_t *b, size_t ldb, const uint8_t *scales, size_t lds, float beta, float *c,
+                                             size_t rsc, size_t csc) {
+  f4_gemm_run(m, n, k, alpha, a, rsa, csa, b, ldb, scales, lds, beta, c, rsc, csc, __func__);
 }
 
 /* column-major A: the rc form with rsa = 1

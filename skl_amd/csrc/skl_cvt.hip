@@ -132,6 +132,27 @@ __global__ void __launch_bounds__(256) cvt_f4_f8e4m3_kernel(uint8_t *__restrict_
   }
 }
 
+// One thread per block of 32 k of a column: E2M1 values times the block's scale 2^(s - 127), as bf16 (exact: one
+// or two significant bits). Columns may start inside a byte (odd ldb): nibbles are addressed one by one.
+__global__ void __launch_bounds__(256) cvt_mxf4_bf16_kernel(uint16_t *__restrict__ dst, const uint8_t *__restrict__ src,
+                                                            const uint8_t *__restrict__ scales, size_t lds, size_t n, size_t k,
+                                                            size_t ldb) {
+  const size_t blocks_per_col = (k + 31) / 32;
+  const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n * blocks_per_col) return;
+  const size_t j = t / blocks_per_col, p0 = (t % blocks_per_col) * 32;
+  const float scale = __uint_as_float((unsigned)scales[j * lds + p0 / 32] << 23);
+  const size_t end = p0 + 32 < k ? p0 + 32 : k;
+  for (size_t p = p0; p < end; ++p) {
+    const size_t i = j * ldb + p;
+    const unsigned byte = src[i >> 1], nib = (i & 1) ? (byte >> 4) : (byte & 0xFu);
+    const unsigned e = (nib >> 1) & 3u, m = nib & 1u;
+    const float mag = e == 0 ? (m ? 0.5f : 0.0f) : __uint_as_float(((e + 126u) << 23) | (m << 22));
+    const float v = __fmul_rn((nib & 8u) ? -mag : mag, scale);
+    dst[i] = (uint16_t)(__float_as_uint(v) >> 16);
+  }
+}
+
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
 }  // namespace
@@ -172,6 +193,17 @@ int skl_hip_launch_cvt_f8_bf16(int fmt, uint16_t *dst, const uint8_t *src, size_
   else
     cvt_f8_bf16_kernel<E5M2><<<blocks, 256, 0, s>>>(dst, src, n, vec);
   return skl_check_launch("cvt_f8_bf16");
+}
+
+int skl_hip_launch_cvt_mxf4_bf16(uint16_t *dst, const uint8_t *src, const uint8_t *scales, size_t lds, size_t n, size_t k, size_t ldb) {
+  if (n == 0 || k == 0) return 0;
+  const size_t threads = n * ((k + 31) / 32), blocks = (threads + 255) / 256;
+  if (blocks > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "cvt_mxf4_bf16: too large");
+    return -2;
+  }
+  cvt_mxf4_bf16_kernel<<<(unsigned)blocks, 256, 0, skl_current_stream()>>>(dst, src, scales, lds, n, k, ldb);
+  return skl_check_launch("cvt_mxf4_bf16");
 }
 
 int skl_hip_launch_cvt_f4_f8e4m3(uint8_t *dst, const uint8_t *src, size_t n) {

@@ -142,7 +142,9 @@ int skl_hip_launch_gemv_noalloc(const skl_gemm_canon *g);
  * apart): skl_gemv_f4.hip. */
 int skl_hip_gemv_f4_supported(size_t m, size_t n, size_t k, const void *a, size_t rsa, size_t csa, const void *b, size_t ldb);
 int skl_hip_launch_gemv_f4(size_t m, size_t n, size_t k, skl_scalar alpha, const void *a, size_t rsa, size_t csa, const void *b,
-                           size_t ldb, skl_scalar beta, float *c, size_t rsc, size_t csc);
+                           size_t ldb, const uint8_t *scales, size_t lds, skl_scalar beta, float *c, size_t rsc, size_t csc);
+/* dst[j * ldb + p] (bf16) = E2M1 value number j * ldb + p of src times 2^(scales[j * lds + p / 32] - 127), for p < k, j < n. */
+int skl_hip_launch_cvt_mxf4_bf16(uint16_t *dst, const uint8_t *src, const uint8_t *scales, size_t lds, size_t n, size_t k, size_t ldb);
 /* Makes sure the current stream has the sums-and-counters block of the single-row kernels; 0 or SKL_HIP_ERR_WORKSPACE. */
 int skl_hip_gemv_reserve_scratch(void);
 

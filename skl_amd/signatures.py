@@ -165,6 +165,7 @@ def gfx950_only():
         sigs[name] = _panel(s)
     sigs["skl_gemm_i8_i8_i32_noalloc"] = _plain("i")              # decode calls without any allocation
     sigs["skl_gemm_f8e4m3rc_f4e2m1c_f32rc"] = "zzzfpzzpzfpzz"           # m n k alpha a rsa csa b ldb beta c rsc csc
+    sigs["skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc"] = "zzzfpzzpzpzfpzz"       # ... b ldb scales lds beta c rsc csc
     sigs["skl_gemm_i8rcp1x4_i8p4x1c_i32"] = "zzzipzzpzipz"
     sigs["skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4"] = "zzzpzpzpzB"   # m1 n1 k1 a rsa1 b rsb1 c rsc1 accum
     sigs["skl_pack_e8_e8p4x8"] = "zzpzpzb"                        # m n src rs dst rs1 pad

@@ -406,8 +406,15 @@ int __wrap_skl_hip_launch_cvt_bf16_f8(int fmt, int sat, uint8_t *dst, const uint
   return cvt_spans(dst, n, src, 2 * n, "cvt bf16 -> fp8");
 }
 int __wrap_skl_hip_launch_cvt_f8_bf16(int fmt, uint16_t *dst, const uint8_t *src, size_t n) {
-  (void)fmt;
-  return cvt_spans(dst, 2 * n, src, n, "cvt fp8 -> bf16");
+  const int rc = cvt_spans(dst, 2 * n, src, n, "cvt fp8 -> bf16");
+  if (!g_failures) /* the GEMM over scaled 4-bit weights multiplies what this writes (finite codes: exact) */
+    for (size_t i = 0; i < n; ++i) {
+      const float v = (float)f8_value(src[i], fmt == SKL_DT_F8E4M3 ? 4 : 5);
+      uint32_t bits;
+      memcpy(&bits, &v, 4);
+      dst[i] = (uint16_t)(bits >> 16);
+    }
+  return rc;
 }
 /* E2M1 code -> the E4M3 byte of the same value (ref/cvt/cvt_ofp4.c:59-68 is exact) */
 static const uint8_t kE2M1AsE4M3[16] = {0x00, 0x30, 0x38, 0x3C, 0x40, 0x44, 0x48, 0x4C, 0x80, 0xB0, 0xB8, 0xBC, 0xC0, 0xC4, 0xC8, 0xCC};
@@ -418,20 +425,39 @@ int __wrap_skl_hip_launch_cvt_f4_f8e4m3(uint8_t *dst, const uint8_t *src, size_t
     for (size_t i = 0; i < n; ++i) dst[i] = kE2M1AsE4M3[nibble_of(src, i)];
   return rc;
 }
+static double scale_of(const uint8_t *scales, size_t lds, size_t j, size_t p) { return scales ? ldexp(1.0, (int)scales[j * lds + p / 32] - 127) : 1.0; }
+int __wrap_skl_hip_launch_cvt_mxf4_bf16(uint16_t *dst, const uint8_t *src, const uint8_t *scales, size_t lds, size_t n, size_t k, size_t ldb) {
+  const char *who = "cvt scaled fp4 -> bf16";
+  ++g_launches, ++g_path[P_CVT];
+  must_own(dst, 0, (n - 1) * ldb + k - 1, 2, who);
+  must_own(src, 0, ((n - 1) * ldb + k - 1) / 2, 1, who);
+  must_own(scales, 0, (n - 1) * lds + (k - 1) / 32, 1, who);
+  if (g_failures) return 0;
+  for (size_t j = 0; j < n; ++j)
+    for (size_t p = 0; p < k; ++p) { /* exact in float, and a float with at most two significant bits is a bf16 */
+      const float v = (float)(f8_value(kE2M1AsE4M3[nibble_of(src, j * ldb + p)], 4) * scale_of(scales, lds, j, p));
+      uint32_t bits;
+      memcpy(&bits, &v, 4);
+      dst[j * ldb + p] = (uint16_t)(bits >> 16);
+    }
+  return 0;
+}
 int __wrap_skl_hip_launch_gemv_f4(size_t m, size_t n, size_t k, skl_scalar alpha, const void *a, size_t rsa, size_t csa, const void *b,
-                                  size_t ldb, skl_scalar beta, float *c, size_t rsc, size_t csc) {
+                                  size_t ldb, const uint8_t *scales, size_t lds, skl_scalar beta, float *c, size_t rsc, size_t csc) {
   const char *who = "4-bit-weight decode kernel";
   EXPECT(skl_hip_gemv_f4_supported(m, n, k, a, rsa, csa, b, ldb), "4-bit-weight decode kernel handed a problem it does not support");
   ++g_launches, ++g_path[P_F4];
   must_own(a, 0, (m - 1) * rsa + (k - 1) * csa, 1, who);
   must_own(b, 0, ((n - 1) * ldb + k - 1) / 2, 1, who);
   must_own(c, 0, (m - 1) * rsc + (n - 1) * csc, sizeof(float), who);
+  if (scales) must_own(scales, 0, (n - 1) * lds + (k - 1) / 32, 1, who);
   if (g_failures) return 0;
   for (size_t i = 0; i < m; ++i)
     for (size_t j = 0; j < n; ++j) {
       double acc = 0;
       for (size_t p = 0; p < k; ++p)
-        acc += f8_value(((const uint8_t *)a)[i * rsa + p * csa], 4) * f8_value(kE2M1AsE4M3[nibble_of((const uint8_t *)b, j * ldb + p)], 4);
+        acc += f8_value(((const uint8_t *)a)[i * rsa + p * csa], 4) * f8_value(kE2M1AsE4M3[nibble_of((const uint8_t *)b, j * ldb + p)], 4) *
+               scale_of(scales, lds, j, p);
       c[i * rsc + j * csc] = (float)((double)beta.f * c[i * rsc + j * csc] + (double)alpha.f * acc);
     }
   return 0;
@@ -758,27 +784,37 @@ static int run_f4_case(int device_pointers) {
   const size_t k = rnd() % 8 == 0 ? 0 : rnd() % 2 ? 32 * rnd_in(1, 6) : rnd_in(1, 150);
   const size_t ldb = rnd() % 2 ? (k + 31) / 32 * 32 + 32 * (rnd() % 2) : k + rnd() % 5, rsa = rnd() % 2 ? (k + 15) / 16 * 16 + 16 : k + rnd() % 3 + 1;
   const size_t rsc = n + rnd() % 3, nib = k ? (n - 1) * ldb + k : 0;
+  const int mx = (int)(rnd() % 2); /* with block scales 2^-2 .. 2^2: sums of small multiples of 1/8 stay exact */
+  const size_t lds = (k + 31) / 32 + rnd() % 2;
+  buf_t sc = new_buf(n * lds + 1, device_pointers);
   buf_t a = new_buf(m * rsa, device_pointers), b = new_buf((nib + 1) / 2 + 1, device_pointers), c = new_buf(m * rsc * sizeof(float), device_pointers);
   buf_t want = new_buf(m * rsc * sizeof(float), 0);
   const float alpha = (float)small(), beta = rnd() % 3 ? (float)small() : 0.0f;
   for (size_t i = 0; i < m * rsa; ++i) store_small(SKL_DT_F8E4M3, a.ptr, i, small());
   for (size_t i = 0; i < b.bytes; ++i) ((uint8_t *)b.ptr)[i] = (uint8_t)rnd();
+  for (size_t i = 0; i < sc.bytes; ++i) ((uint8_t *)sc.ptr)[i] = (uint8_t)(125 + rnd() % 5);
   for (size_t i = 0; i < m * rsc; ++i) ((float *)c.ptr)[i] = (float)small();
   memcpy(want.ptr, c.ptr, m * rsc * sizeof(float));
   for (size_t i = 0; i < m; ++i)
     for (size_t j = 0; j < n; ++j) {
       double acc = 0;
       for (size_t p = 0; p < k; ++p)
-        acc += f8_value(((const uint8_t *)a.ptr)[i * rsa + p], 4) * f8_value(kE2M1AsE4M3[nibble_of((const uint8_t *)b.ptr, j * ldb + p)], 4);
+        acc += f8_value(((const uint8_t *)a.ptr)[i * rsa + p], 4) * f8_value(kE2M1AsE4M3[nibble_of((const uint8_t *)b.ptr, j * ldb + p)], 4) *
+               scale_of(mx ? (const uint8_t *)sc.ptr : NULL, lds, j, p);
       ((float *)want.ptr)[i * rsc + j] = (float)((double)beta * ((float *)want.ptr)[i * rsc + j] + (double)alpha * acc);
     }
-  skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(m, n, k, alpha, (const uint8_t *)a.ptr, rsa, 1, (const uint8_t *)b.ptr, ldb, beta, (float *)c.ptr, rsc, 1);
+  if (mx)
+    skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_gfx950(m, n, k, alpha, (const uint8_t *)a.ptr, rsa, 1, (const uint8_t *)b.ptr, ldb, (const uint8_t *)sc.ptr,
+                                             lds, beta, (float *)c.ptr, rsc, 1);
+  else
+    skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(m, n, k, alpha, (const uint8_t *)a.ptr, rsa, 1, (const uint8_t *)b.ptr, ldb, beta, (float *)c.ptr, rsc, 1);
   if (skl_hip_last_error() != 0) fail(skl_hip_last_error_string());
   if (memcmp(want.ptr, c.ptr, m * rsc * sizeof(float)) != 0) {
-    fprintf(stderr, "FAIL: 4-bit-weight GEMM differs: %zu x %zu x %zu, ldb %zu, rsa %zu, %s pointers\n", m, n, k, ldb, rsa, device_pointers ? "device" : "host");
+    fprintf(stderr, "FAIL: 4-bit-weight GEMM differs: %zu x %zu x %zu, ldb %zu, rsa %zu, scales %d, %s pointers\n", m, n, k, ldb, rsa, mx,
+            device_pointers ? "device" : "host");
     ++g_failures;
   }
-  drop_buf(a), drop_buf(b), drop_buf(c), drop_buf(want);
+  drop_buf(a), drop_buf(b), drop_buf(c), drop_buf(want), drop_buf(sc);
   return g_failures;
 }
 

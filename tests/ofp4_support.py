@@ -34,3 +34,27 @@ def make_problem(seed, m, n, k, ldb, alpha=1.0, beta=0.0, **strides):
     codes = rng.integers(0, 16, size=max(nb, 1), dtype=np.uint8)
     c = rng.uniform(-1.0, 1.0, size=max(nc, 1)).astype(np.float32)
     return case, a, pack_nibbles(codes), E2M1_AS_E4M3[codes], c
+
+
+def make_mx_problem(seed, m, n, k, ldb, alpha=1.0, beta=0.0, **strides):
+    """make_problem plus block scales: (case, a, packed b, B as fp64 values (k x n), scales, lds, c). Scales within
+    2^-6 .. 2^6 so that nothing leaves fp32's comfortable range."""
+    case, a, b4, b8, c = make_problem(seed, m, n, k, ldb, alpha, beta, **strides)
+    rng = np.random.default_rng(seed + 1)
+    blocks = (k + 31) // 32
+    lds = blocks + int(rng.integers(0, 3))
+    scales = rng.integers(121, 134, size=max(n * lds, 1), dtype=np.uint8)
+    return case, a, b4, b8, scales, lds, c
+
+
+def mx_bound(case, a, b8, scales, lds, c, m, n, k, ldb):
+    """(exact fp64 result, elementwise bound of the reference's fp8 GEMM test) with B's values times their scales."""
+    A = support.decode_table("f8e4m3")[a[(np.arange(m)[:, None] * case.rsa1 + np.arange(k)[None, :] * case.csa1)]] if k else np.zeros((m, 0))
+    Bv = support.decode_table("f8e4m3")[b8[(np.arange(n)[None, :] * ldb + np.arange(k)[:, None])]] if k else np.zeros((0, n))
+    S = np.ldexp(1.0, scales[(np.arange(n)[None, :] * lds + (np.arange(k) // 32)[:, None])].astype(np.int64) - 127) if k else np.zeros((0, n))
+    B = Bv * S
+    oc = np.arange(m)[:, None] * case.rsc1 + np.arange(n)[None, :] * case.csc1
+    C = c[oc].astype(np.float64)
+    gamma = 2.0 * np.expm1((k + 2) * np.log1p(2.0 ** -24))
+    bound = gamma * (abs(case.alpha) * (np.abs(A) @ np.abs(B)) + abs(case.beta) * np.abs(C))
+    return case.alpha * (A @ B) + case.beta * C, bound, oc

@@ -16,19 +16,25 @@ from skl_amd import DeviceBuffer
 pytestmark = pytest.mark.gpu
 
 
-def run(lib, case, a, b4, c, mode, m, n, k, ldb):
-    args = lambda a_, b_, c_: (m, n, k, case.alpha, a_, case.rsa1, case.csa1, b_, ldb, case.beta, c_, case.rsc1, case.csc1)
+def run(lib, case, a, b4, c, mode, m, n, k, ldb, scales=None, lds=0):
+    def call(a_, b_, c_, s_):
+        if scales is None:
+            lib.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(m, n, k, case.alpha, a_, case.rsa1, case.csa1, b_, ldb, case.beta, c_, case.rsc1, case.csc1)
+        else:
+            lib.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_gfx950(m, n, k, case.alpha, a_, case.rsa1, case.csa1, b_, ldb, s_, lds, case.beta, c_,
+                                                         case.rsc1, case.csc1)
     if mode == "host":
         out = c.copy()
-        lib.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(*args(a, b4, out))
+        call(a, b4, out, scales)
         skl_amd.check_error()
         return out
-    da, db, dc = DeviceBuffer.from_array(a), DeviceBuffer.from_array(b4), DeviceBuffer.from_array(c)
-    lib.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(*args(da, db, dc))
+    bufs = [DeviceBuffer.from_array(x) if x is not None else None for x in (a, b4, c, scales)]
+    call(bufs[0], bufs[1], bufs[2], bufs[3])
     _finish(lib)
-    out = dc.download(c.dtype, c.size)
-    for d in (da, db, dc):
-        d.free()
+    out = bufs[2].download(c.dtype, c.size)
+    for d in bufs:
+        if d is not None:
+            d.free()
     return out
 
 
@@ -55,6 +61,45 @@ def test_ofp4_weights(gpu, m, n, k, ldb, rsa, what):
             got = run(gpu, case, a, b4, c, mode, m, n, k, ldb)
             support.assert_fp_gemm_close(case, a, b8, c, got)
             assert np.array_equal(got.view(np.uint32), run(gpu, case, a, b4, c, mode, m, n, k, ldb).view(np.uint32)), what
+
+
+@pytest.mark.parametrize("m,n,k,ldb,rsa,what", SHAPES)
+def test_mx_scaled_ofp4_weights(gpu, m, n, k, ldb, rsa, what):
+    """The same shapes with one E8M0 scale per 32 k of a column (OCP microscaling): inside the reference's
+    fp32-accumulation bound around the exact product of the decoded, scaled operands - the decode kernel hands the
+    scales to the matrix cores (or folds them into the bf16 widening up to K = 2304), the other shapes run the bf16
+    GEMM on exactly converted copies - and the same bits on a second run."""
+    for i, (alpha, beta) in enumerate(((1.0, 0.0), (1.5, -0.5))):
+        case, a, b4, b8, scales, lds, c = f4.make_mx_problem(800 + m + n + i, m, n, k, ldb, alpha, beta, rsa=rsa, rsc=n + 3)
+        exact, bound, oc = f4.mx_bound(case, a, b8, scales, lds, c, m, n, k, ldb)
+        for mode in MODES:
+            got = run(gpu, case, a, b4, c, mode, m, n, k, ldb, scales, lds)
+            err = np.abs(got[oc] - exact)
+            assert np.all(err <= bound + np.abs(exact) * 2.0 ** -22 + 1e-30), (what, mode, float((err / (bound + 1e-30)).max()))
+            mask = np.ones(c.size, bool)
+            mask[oc.ravel()] = False
+            assert np.array_equal(got[mask], c[mask]), "elements outside the addressed C were modified"
+            again = run(gpu, case, a, b4, c, mode, m, n, k, ldb, scales, lds)
+            assert np.array_equal(got.view(np.uint32), again.view(np.uint32)), what
+
+
+@pytest.mark.parametrize("k", (2304, 2560))
+def test_scales_reach_their_blocks(gpu, k):
+    """A row of A that is 1.0 at one k reads B(k, :) times its block's scale back exactly: every block of 32 k gets the
+    scale stored for it, in both kernel variants."""
+    n, lds = 48, k // 32 + 1
+    rng = np.random.default_rng(k + 1)
+    codes = rng.integers(1, 8, size=n * k, dtype=np.uint8)        # positive, non-zero values
+    scales = rng.integers(117, 138, size=n * lds, dtype=np.uint8)
+    b4 = f4.pack_nibbles(codes)
+    values = f4.E2M1_VALUES[codes].reshape(n, k) * np.ldexp(1.0, scales.reshape(n, lds)[:, :k // 32].astype(np.int64) - 127).repeat(32, axis=1)
+    for p0 in range(0, k, 16 * 32):
+        pos = np.minimum(p0 + np.arange(16) * 32 + (np.arange(16) * 7) % 32, k - 1)   # one k in each of 16 blocks
+        a = np.zeros(16 * k, np.uint8)
+        a[np.arange(16) * k + pos] = 0x38
+        case = f4.f8_case(16, n, k, k, 1.0, 0.0)
+        got = run(gpu, case, a, b4, np.zeros(16 * n, np.float32), "device", 16, n, k, k, scales, lds).reshape(16, n)
+        assert np.array_equal(got.astype(np.float64), values[:, pos].T), (k, p0)
 
 
 @pytest.mark.parametrize("k", (2304, 2560))

@@ -352,6 +352,42 @@ def test_ofp4_gemm_is_the_conversion_followed_by_the_fp8_gemm():
     assert np.array_equal(got.reshape(m, n).astype(np.float64), A @ B)
 
 
+def test_mx_scaled_ofp4_gemm_definition():
+    """The checker's GEMM over MXFP4 weights (oracle/skl_oracle.c): with every scale 2^0, or none, it is the
+    unscaled routine bit for bit (which is pinned against the reference's conversion + fp8 GEMM above); raising
+    every scale by one doubles every sum exactly; the result lies inside the reference's fp32-accumulation bound around
+    the exact product of the decoded, scaled operands; exact where the sums are."""
+    import ofp4_support as f4
+    o = oracle()
+    for i, (m, n, k, ldb) in enumerate(((3, 5, 70, 71), (4, 6, 64, 64), (2, 9, 200, 224), (1, 3, 31, 40))):
+        case, a, b4, b8, scales, lds, c = f4.make_mx_problem(90 + i, m, n, k, ldb, 1.5, -0.5, rsa=k + 3, rsc=n + 2)
+        plain, unit, none = c.copy(), c.copy(), c.copy()
+        o.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_oracle(m, n, k, 1.5, a, case.rsa1, 1, b4, ldb, -0.5, plain, case.rsc1, 1)
+        o.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_oracle(m, n, k, 1.5, a, case.rsa1, 1, b4, ldb, np.full_like(scales, 127), lds, -0.5, unit, case.rsc1, 1)
+        o.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_oracle(m, n, k, 1.5, a, case.rsa1, 1, b4, ldb, None, 0, -0.5, none, case.rsc1, 1)
+        assert np.array_equal(plain.view(np.uint32), unit.view(np.uint32)) and np.array_equal(plain.view(np.uint32), none.view(np.uint32))
+        got, twice = np.zeros_like(c), np.zeros_like(c)
+        o.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_oracle(m, n, k, 1.0, a, case.rsa1, 1, b4, ldb, scales, lds, 0.0, got, case.rsc1, 1)
+        o.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_oracle(m, n, k, 1.0, a, case.rsa1, 1, b4, ldb, scales + 1, lds, 0.0, twice, case.rsc1, 1)
+        assert np.array_equal(twice, 2 * got)
+        scaled = c.copy()
+        o.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_oracle(m, n, k, 1.5, a, case.rsa1, 1, b4, ldb, scales, lds, -0.5, scaled, case.rsc1, 1)
+        exact, bound, oc = f4.mx_bound(case, a, b8, scales, lds, c, m, n, k, ldb)
+        assert np.all(np.abs(scaled[oc] - exact) <= bound + np.abs(exact) * 2.0 ** -22)
+    # exact sums: A in {1, 2, 4}, scales 2^-2 .. 2^2, K = 64
+    m, n, k = 5, 11, 64
+    rng = np.random.default_rng(4)
+    a = rng.choice(np.array([0x38, 0x40, 0x48], np.uint8), m * k)
+    codes = rng.integers(0, 16, n * k, dtype=np.uint8)
+    scales = rng.integers(125, 130, size=n * 2, dtype=np.uint8)
+    got = np.zeros(m * n, np.float32)
+    o.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_oracle(m, n, k, 1.0, a, k, 1, f4.pack_nibbles(codes), k, scales, 2, 0.0, got, n, 1)
+    A = support.decode_table("f8e4m3")[a].reshape(m, k)
+    S = np.ldexp(1.0, scales.reshape(n, 2).astype(np.int64) - 127).repeat(32, axis=1)
+    B = (f4.E2M1_VALUES[codes].reshape(n, k) * S).T
+    assert np.array_equal(got.reshape(m, n).astype(np.float64), A @ B)
+
+
 def test_silu_and_gelu_restate_the_reference():
     """The checker's SiLU and GELU (oracle/skl_oracle.c) against the reference's own routines compiled from
     ref/sigmoid/sigmoid_f32.c and ref/gelu/gelu_f32.c - bit for bit over the ranges of the reference's tests and the
