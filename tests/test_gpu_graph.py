@@ -36,6 +36,12 @@ def test_decode_loop_replays_from_a_graph(gpu):
     x, xs, a16, xb = B(k), B(4 * k), B(16 * 4096), B(2 * k)
     y = [B(4 * n) for _ in range(layers)]
     yt, ys, y16, yb = B(4 * n), B(16 * n), B(64 * n), B(4 * n)
+    # MXFP4 weights stored [n][k] with one scale per 32 k, E4M3 activations in {1, 2, 4}: every sum is exact
+    import ofp4_support as f4
+    codes4 = rng.integers(0, 16, size=n * k, dtype=np.uint8)
+    hs4 = rng.integers(125, 130, size=n * (k // 32), dtype=np.uint8)
+    w4, s4, x4, y4 = B.from_array(f4.pack_nibbles(codes4)), B.from_array(hs4), B(k), B(4 * n)
+    W4 = f4.E2M1_VALUES[codes4].reshape(n, k) * np.ldexp(1.0, hs4.reshape(n, k // 32).astype(np.int64) - 127).repeat(32, axis=1)
 
     def enqueue():
         for l in range(layers):
@@ -44,13 +50,14 @@ def test_decode_loop_replays_from_a_graph(gpu):
         gpu.skl_gemm_i8_i8_i32_gfx950(4, n, k, 1, xs, k, w[0], n, 0, ys, n)
         gpu.skl_gemm_i8_i8_i32_gfx950(16, n, 4096, 1, a16, 4096, w16, n, 0, y16, n)
         gpu.skl_gemm_bf16_bf16_f32_gfx950(1, n, k, 1.0, xb, k, wb, n, 0.0, yb, n)
+        gpu.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_gfx950(1, n, k, 1.0, x4, k, 1, w4, k, s4, k // 32, 0.0, y4, n, 1)
 
     stream, graph, executable = ct.c_void_p(), ct.c_void_p(), ct.c_void_p()
     assert hip.hipStreamCreate(ct.byref(stream)) == 0
     gpu.skl_hip_set_pointer_mode(1)  # device pointers promised: no runtime queries inside the capture
     gpu.skl_hip_set_stream(stream.value)
     try:
-        for buf, nbytes in ((x, k), (xs, 4 * k), (a16, 16 * 4096), (xb, 2 * k)):
+        for buf, nbytes in ((x, k), (xs, 4 * k), (a16, 16 * 4096), (xb, 2 * k), (x4, k)):
             gpu.skl_hip_memset(buf, 0, nbytes)
         enqueue()  # eager once: creates the library's scratch blocks and configures the kernels
         assert gpu.skl_hip_synchronize() == 0
@@ -65,8 +72,9 @@ def test_decode_loop_replays_from_a_graph(gpu):
             hxs = rng.integers(-128, 128, (4, k), dtype=np.int8)
             ha = rng.integers(-128, 128, (16, 4096), dtype=np.int8)
             hb = support.ETYPES["bf16"].gen(rng, k)
-            x.upload(hx), xs.upload(hxs), a16.upload(ha), xb.upload(hb)
-            for t, count in [(t, n) for t in y] + [(yt, n), (ys, 4 * n), (y16, 16 * n), (yb, n)]:
+            hx4 = rng.choice(np.array([0x38, 0x40, 0x48], np.uint8), k)
+            x.upload(hx), xs.upload(hxs), a16.upload(ha), xb.upload(hb), x4.upload(hx4)
+            for t, count in [(t, n) for t in y] + [(yt, n), (ys, 4 * n), (y16, 16 * n), (yb, n), (y4, n)]:
                 gpu.skl_hip_memset(t, 0x5A, 4 * count)  # a replay must rewrite every output
             assert hip.hipGraphLaunch(executable, stream) == 0
             assert hip.hipStreamSynchronize(stream) == 0
@@ -79,6 +87,7 @@ def test_decode_loop_replays_from_a_graph(gpu):
             xv, wv = support.ETYPES["bf16"].widen(hb), support.ETYPES["bf16"].widen(hwb).reshape(k, n)
             bound = 2 * ((1 + 2.0 ** -24) ** (k + 2) - 1) * (np.abs(xv) @ np.abs(wv)) + 1e-30
             assert np.all(np.abs(yb.download(np.float32) - xv @ wv) <= bound), rep
+            assert np.array_equal(y4.download(np.float32).astype(np.float64), W4 @ support.decode_table("f8e4m3")[hx4]), rep
     finally:
         gpu.skl_hip_set_stream(None)
         gpu.skl_hip_set_pointer_mode(0)
@@ -88,7 +97,7 @@ def test_decode_loop_replays_from_a_graph(gpu):
             hip.hipGraphDestroy(graph)
         gpu.skl_hip_release_stream(stream.value)
         hip.hipStreamDestroy(stream)
-        for d in w + y + [wt, w16, wb, x, xs, a16, xb, yt, ys, y16, yb]:
+        for d in w + y + [wt, w16, wb, x, xs, a16, xb, yt, ys, y16, yb, w4, s4, x4, y4]:
             d.free()
     # the integer products used above are what the checker computes (one layer)
     case = rowmajor_case("i8", 1, n, k, alpha=1, beta=0)
