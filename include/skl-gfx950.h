@@ -167,6 +167,9 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, 
  *                                                q_scale[0]; (float)v rounds an int32 to nearest even, the product is
  *                                                one fp32 multiplication, rne() rounds it to the nearest integer, ties
  *                                                to even (a NaN counts as 0, values beyond int32 as its ends)
+ *                                                with q_format one of the fp8 codes below the byte is instead the OCP fp8
+ *                                                encoding of (float)v * s_j as skl_cvt_[sat_]f32_f8e4m3 / _f8e5m2
+ *                                                (ref/cvt/cvt_ofp8.c:174-242) produces it, q_zero unused
  *     *max = v  if v > *max                      if max != NULL (a NaN never replaces the maximum;
  *                                                the sign of a zero maximum is unspecified)
  * Bias and maximum are the steps of the reference's fused kernels; activation and requantisation are what
@@ -181,7 +184,12 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, 
 #define SKL_GFX950_ACT_SILU 2 /* floating-point C only */
 #define SKL_GFX950_ACT_GELU 3 /* floating-point C only */
 /* Every step off: `skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE; ep.bias = ...;` is valid C and C++. */
-#define SKL_GFX950_EPILOGUE_NONE {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
+#define SKL_GFX950_Q_INT8 0       /* what a byte of q holds: int8 by the rule above (default) */
+#define SKL_GFX950_Q_F8E4M3 1     /* OCP E4M3, overflow to the format's NaN like skl_cvt_f32_f8e4m3 */
+#define SKL_GFX950_Q_F8E4M3_SAT 2 /* ... saturating like skl_cvt_sat_f32_f8e4m3 */
+#define SKL_GFX950_Q_F8E5M2 3
+#define SKL_GFX950_Q_F8E5M2_SAT 4
+#define SKL_GFX950_EPILOGUE_NONE {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 typedef struct skl_gfx950_epilogue {
   const void *bias;
   void *max;
@@ -192,6 +200,7 @@ typedef struct skl_gfx950_epilogue {
   int8_t *q;
   size_t rsq, csq;
   const float *q_scale;
+  int q_format; /* SKL_GFX950_Q_* */
 } skl_gfx950_epilogue_t;
 
 #define SKL_GFX950_DECLARE_FUSED_RC(NAME, TA, TC)                                                    \

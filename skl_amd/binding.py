@@ -59,17 +59,19 @@ class Epilogue:
 
     ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU = 0, 1, 2, 3
 
+    Q_INT8, Q_F8E4M3, Q_F8E4M3_SAT, Q_F8E5M2, Q_F8E5M2_SAT = range(5)
+
     def __init__(self, bias=None, max=None, activation=0, q=None, rsq=0, csq=0, q_scale=None,
-                 q_scale_per_column=False, q_zero=0, q_only=False):
+                 q_scale_per_column=False, q_zero=0, q_only=False, q_format=0):
         self.bias, self.max, self.activation = bias, max, activation
         self.q, self.rsq, self.csq, self.q_scale = q, rsq, csq, q_scale
-        self.q_scale_per_column, self.q_zero, self.q_only = q_scale_per_column, q_zero, q_only
+        self.q_scale_per_column, self.q_zero, self.q_only, self.q_format = q_scale_per_column, q_zero, q_only, q_format
 
     def as_struct(self):
         return signatures.EpilogueStruct(_as_pointer(self.bias), _as_pointer(self.max), int(self.activation),
                                          int(bool(self.q_scale_per_column)), int(bool(self.q_only)), int(self.q_zero),
                                          _as_pointer(self.q), int(self.rsq), int(self.csq),
-                                         _as_pointer(self.q_scale))
+                                         _as_pointer(self.q_scale), int(self.q_format))
 
 
 def _wrap(raw, sig):

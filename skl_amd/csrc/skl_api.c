@@ -464,7 +464,8 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
   where = classify(K ? d->a : NULL, K ? d->b : NULL, d->c, who);
   if (where < 0) return;
   if (d->rq.act < SKL_GFX950_ACT_NONE || d->rq.act > (d->ta == SKL_DT_I8 ? SKL_GFX950_ACT_RELU : SKL_GFX950_ACT_GELU) ||
-      (d->rq.q && (!d->rq.q_scale || d->rq.q_zero < -128 || d->rq.q_zero > 127))) {
+      (d->rq.q && (!d->rq.q_scale || d->rq.q_zero < -128 || d->rq.q_zero > 127 || d->rq.q_fmt < SKL_GFX950_Q_INT8 ||
+                   d->rq.q_fmt > SKL_GFX950_Q_F8E5M2_SAT))) {
     skl_hip_record_error(SKL_HIP_ERR_BAD_ARGUMENT, who);
     return;
   }
@@ -582,7 +583,8 @@ DEFINE_GEMM_RCPRC(skl_gemm_f64rcprc_f64rcprc_f64rcprc_gfx950, double, double, SK
 DEFINE_GEMM_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, skl_f16_t, SKL_DT_F16H, SCALAR_f32)
 
 static skl_requant requant_of(const skl_gfx950_epilogue_t *ep) {
-  skl_requant rq = {ep->activation, ep->q_scale_per_column != 0, ep->q_only != 0 && ep->q != NULL, ep->q_zero, ep->q, ep->rsq, ep->csq, ep->q_scale};
+  skl_requant rq = {ep->activation, ep->q_scale_per_column != 0, ep->q_only != 0 && ep->q != NULL, ep->q_zero, ep->q, ep->rsq, ep->csq, ep->q_scale,
+                    ep->q_format};
   return rq;
 }
 

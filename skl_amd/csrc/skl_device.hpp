@@ -5,6 +5,7 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "skl_fp8.hpp"
 #include "skl_launch.h"
 
 // Stream the calling thread launches on (set through skl_hip_set_stream).
@@ -136,10 +137,19 @@ __device__ __forceinline__ int skl_requantise_int(float v, float scale, int zero
   return t < -128 ? -128 : t > 127 ? 127 : t;
 }
 __device__ __forceinline__ int8_t skl_requantise(float v, float scale, int zero) { return (int8_t)skl_requantise_int(v, scale, zero); }
+// The byte of the 8-bit copy for value v: int8 by the rule above, or the OCP fp8 encoding of v * scale exactly as the
+// conversion kernels produce it (ref/cvt/cvt_ofp8.c:174-242: one fp32 product, round to nearest even, saturating or
+// not) - a fused skl_cvt_[sat_]f32_f8e*.
+__device__ __forceinline__ int8_t skl_quantise(float v, float scale, int zero, int fmt) {
+  if (fmt == 0) return skl_requantise(v, scale, zero);
+  const unsigned bits = __float_as_uint(__fmul_rn(v, scale));
+  const bool sat = fmt == 2 || fmt == 4;
+  return (int8_t)(fmt <= 2 ? skl_fp8::encode_ofp8<skl_fp8::E4M3>(bits, sat) : skl_fp8::encode_ofp8<skl_fp8::E5M2>(bits, sat));
+}
 // Element (row, col) of the requantised output, if there is one.
 template <typename T>
 __device__ __forceinline__ void skl_emit_requantised(const skl_requant &rq, T v, size_t row, size_t col) {
-  if (rq.q) rq.q[row * rq.rsq + col * rq.csq] = skl_requantise((float)v, rq.q_scale[rq.q_per_column ? col : 0], rq.q_zero);
+  if (rq.q) rq.q[row * rq.rsq + col * rq.csq] = skl_quantise((float)v, rq.q_scale[rq.q_per_column ? col : 0], rq.q_zero, rq.q_fmt);
 }
 
 template <typename T>

@@ -93,7 +93,7 @@ struct FusedSteps {
         q_scale_j(0.0f) {}
   // What a descriptor must look like for modes 2 and 3.
   __host__ __device__ static bool dword_copy(const skl_requant &r) {
-    return r.q && r.csq == 1 && (r.rsq & 3) == 0 && ((uintptr_t)r.q & 3) == 0;
+    return r.q && r.q_fmt == 0 && r.csq == 1 && (r.rsq & 3) == 0 && ((uintptr_t)r.q & 3) == 0;
   }
   __device__ __forceinline__ void column(size_t c) {
     col = c;
@@ -116,7 +116,7 @@ struct FusedSteps {
     v = apply(v);
     if constexpr (EXTRA == 1) {
       if (!rq.q_only) __builtin_nontemporal_store(v, dst);
-      if (rq.q) rq.q[row * rq.rsq + col * rq.csq] = skl_requantise((float)v, q_scale_j, rq.q_zero);
+      if (rq.q) rq.q[row * rq.rsq + col * rq.csq] = skl_quantise((float)v, q_scale_j, rq.q_zero, rq.q_fmt);
     } else {
       (void)row;
       if constexpr (EXTRA != 2) __builtin_nontemporal_store(v, dst);

@@ -44,7 +44,7 @@ typedef union {
 } skl_scalar;
 
 /* Further fused steps behind bias (see skl_gfx950_epilogue_t in include/skl-gfx950.h): an activation and a
- * requantised int8 copy of the result. All zero / NULL: nothing. */
+ * requantised 8-bit copy of the result. All zero / NULL: nothing. */
 typedef struct {
   int act;             /* 0 none, 1 max(v, 0) */
   int q_per_column;    /* q_scale holds one factor per logical column, else one in all */
@@ -53,6 +53,8 @@ typedef struct {
   int8_t *q;           /* Q(i, j) at q[i*rsq + j*csq], (i, j) the logical row and column; NULL: no requantised output */
   size_t rsq, csq;
   const float *q_scale;
+  int q_fmt;           /* what a byte of q holds: 0 int8 (rounded, zero point, clamped); 1 / 2 OCP E4M3 without / with
+                          saturation, 3 / 4 E5M2 likewise (the fp32 -> fp8 conversion of the cvt family on v * scale) */
 } skl_requant;
 
 /* The fully general blocked GEMM of the reference (the `rcprc` form): element

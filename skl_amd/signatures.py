@@ -46,7 +46,7 @@ class EpilogueStruct(ctypes.Structure):
     _fields_ = [("bias", ctypes.c_void_p), ("max", ctypes.c_void_p), ("activation", ctypes.c_int),
                 ("q_scale_per_column", ctypes.c_int), ("q_only", ctypes.c_int), ("q_zero", ctypes.c_int32),
                 ("q", ctypes.c_void_p), ("rsq", ctypes.c_size_t), ("csq", ctypes.c_size_t),
-                ("q_scale", ctypes.c_void_p)]
+                ("q_scale", ctypes.c_void_p), ("q_format", ctypes.c_int)]
 
 
 def _rc(s):      # m n k alpha a rsa csa b rsb csb beta c rsc csc

@@ -82,6 +82,22 @@ static double f8_value(unsigned code, int ebits) { /* finite codes only */
   const double mag = e ? ldexp(1.0 + m / (double)(1 << mbits), e - bias) : ldexp(m / (double)(1 << mbits), 1 - bias);
   return (code & 0x80) ? -mag : mag;
 }
+/* x as an OCP fp8 code by search over the codes: the nearest value, a tie to the code with an even last bit, and one
+ * value beyond the largest (480 / 65536) standing for overflow, which gives the largest finite code when saturating,
+ * else E4M3's NaN without a sign or E5M2's infinity (ref/cvt/cvt_ofp8.c:97-172). Finite x only. */
+static uint8_t f8_encode(double x, int ebits, int sat) {
+  const unsigned top = ebits == 4 ? 0x7F : 0x7C;
+  const uint8_t sign = signbit(x) ? 0x80 : 0;
+  const double mag = fabs(x), beyond = ebits == 4 ? 480.0 : 65536.0;
+  unsigned best = 0;
+  double best_d = mag;
+  for (unsigned code = 1; code <= top; ++code) {
+    const double d = fabs((code == top ? beyond : f8_value(code, ebits)) - mag);
+    if (d < best_d || (d == best_d && !(code & 1))) best = code, best_d = d;
+  }
+  if (best == top || mag > beyond) return sat ? (uint8_t)(sign | (top - 1)) : ebits == 4 ? 0x7F : (uint8_t)(sign | 0x7C);
+  return (uint8_t)(sign | best);
+}
 static double load_elem(int dt, const void *base, size_t i) {
   switch (dt) {
     case SKL_DT_I8: return ((const int8_t *)base)[i];
@@ -144,9 +160,13 @@ static void fused_steps(int dt, void *c, size_t idx, size_t i, size_t j, double 
     must_own(rq->q, at, at, 1, who);
     must_own(rq->q_scale, rq->q_per_column ? j : 0, rq->q_per_column ? j : 0, sizeof(float), who);
     if (g_failures) return;
-    r = nearbyint(v * (double)rq->q_scale[rq->q_per_column ? j : 0]);
-    t = (long)(r > 1e9 ? 1e9 : r < -1e9 ? -1e9 : r) + rq->q_zero;
-    rq->q[at] = (int8_t)(t < -128 ? -128 : t > 127 ? 127 : t);
+    if (rq->q_fmt) {
+      rq->q[at] = (int8_t)f8_encode(v * (double)rq->q_scale[rq->q_per_column ? j : 0], rq->q_fmt <= 2 ? 4 : 5, rq->q_fmt == 2 || rq->q_fmt == 4);
+    } else {
+      r = nearbyint(v * (double)rq->q_scale[rq->q_per_column ? j : 0]);
+      t = (long)(r > 1e9 ? 1e9 : r < -1e9 ? -1e9 : r) + rq->q_zero;
+      rq->q[at] = (int8_t)(t < -128 ? -128 : t > 127 ? 127 : t);
+    }
   }
   if (max && v > load_c(dt, max, 0)) store_c(dt, max, 0, v);
 }
@@ -748,6 +768,7 @@ static int run_gemm_case(int device_pointers) {
         ep.q_scale = (const float *)scales.ptr;
         ep.q_zero = small();
         ep.q_only = rnd() % 3 == 0;
+        if (rnd() % 3 == 0) ep.q_format = 1 + (int)(rnd() % 4);
       }
     }
     {
@@ -756,7 +777,7 @@ static int run_gemm_case(int device_pointers) {
       ref.bias = ep.bias;
       ref.max = want_top.ptr;
       ref.rq.act = ep.activation, ref.rq.q_per_column = ep.q_scale_per_column, ref.rq.q_only = ep.q_only && ep.q, ref.rq.q_zero = ep.q_zero;
-      ref.rq.q = (int8_t *)want_q.ptr, ref.rq.rsq = ep.rsq, ref.rq.csq = ep.csq, ref.rq.q_scale = ep.q_scale;
+      ref.rq.q = (int8_t *)want_q.ptr, ref.rq.rsq = ep.rsq, ref.rq.csq = ep.csq, ref.rq.q_scale = ep.q_scale, ref.rq.q_fmt = ep.q_format;
       { /* the reference loops read bias and scales where the caller put them: known to the registry either way */
         gemm_over_desc(&ref, 0, "reference loops");
       }

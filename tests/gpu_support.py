@@ -65,7 +65,7 @@ def run_gemm(lib, kind, case, a, b, c, mode):
 def run_fused_gemm(lib, kind, case, a, b, c, bias, mx, mode, activation=0, requant=None):
     """Runs `skl_gemm_fused_*` (kind "rc" or "rcprc"); returns (C's whole buffer, *max) afterwards.
     `bias` / `mx` are arrays of C's type (n values / one value) or None. `requant` = dict(q=<int8 buffer>,
-    rsq, csq, scale=<float32 array>, per_column, zero, only) asks for the requantised copy, whose buffer
+    rsq, csq, scale=<float32 array>, per_column, zero, only, format) asks for the requantised copy, whose buffer
     afterwards is returned as a third value."""
     rq = requant or {}
 
@@ -75,7 +75,8 @@ def run_fused_gemm(lib, kind, case, a, b, c, bias, mx, mode, activation=0, requa
         getattr(lib, fused)(*args, skl_amd.Epilogue(bias_, mx_, activation=activation, q=q_, rsq=rq.get("rsq", 0),
                                                     csq=rq.get("csq", 0), q_scale=scale_,
                                                     q_scale_per_column=rq.get("per_column", False),
-                                                    q_zero=rq.get("zero", 0), q_only=rq.get("only", False)))
+                                                    q_zero=rq.get("zero", 0), q_only=rq.get("only", False),
+                                                    q_format=rq.get("format", 0)))
 
     q, scale = rq.get("q"), rq.get("scale")
     if mode == "host":

@@ -396,6 +396,38 @@ def test_fused_activation_and_requantised_copy(gpu, ta, m, n, k, beta, what):
         assert np.array_equal(got.view(np.uint8), want_c.view(np.uint8)) and top[0] == want_top[0], (ta, what, mode)
 
 
+@pytest.mark.parametrize("m,n,k,beta,what", EXTRA_STEP_SHAPES)
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f8e5m2"))
+def test_fused_fp8_copy(gpu, ta, m, n, k, beta, what):
+    """The 8-bit copy as OCP fp8 (q_format): each byte must be what the reference's fp32 -> fp8 conversion
+    (skl_cvt_[sat_]f32_f8e4m3 / _f8e5m2, ref/cvt/cvt_ofp8.c:174-198, through the checker) makes of the value written to
+    C times the column's scale, on every kernel family; the scales put a good part of the values beyond the format's
+    largest, so the saturating and the non-saturating rule differ, and (one scale per column) others among its subnormals."""
+    rng = np.random.default_rng(m * 13 + n + k)
+    case = rowmajor_case(ta, m, n, k, alpha=1, beta=beta)
+    a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+    bias = rng.integers(-1 << 12, 1 << 12, n).astype(np.int32) if case.is_int else rng.uniform(-4, 4, n).astype(np.float32)
+    for mode in MODES:
+        anchor, _ = run_fused_gemm(gpu, "rc", case, a, b, c, bias, None, mode)
+        spread = float(np.abs(anchor.astype(np.float64)).max())
+        for fmt, (rsq, csq), per_column, act, only in ((1, (n + 4, 1), True, 0, False), (2, (1, m + 3), False, 1, False),
+                                                       (3, (n, 1), False, 0, True), (4, (n + 1, 1), True, 1, False)):
+            largest = 448.0 if fmt <= 2 else 57344.0
+            base = largest * 1.25 / max(spread, 1e-3)   # the widest values land a quarter beyond the format's largest
+            scales = (base * np.exp2(rng.integers(-24, 4, n))).astype(np.float32) if per_column else np.array([base], np.float32)
+            q0 = np.full((m - 1) * rsq + (n - 1) * csq + 1, 0x55, np.int8)
+            rq = dict(q=q0, rsq=rsq, csq=csq, scale=scales, per_column=per_column, only=only, format=fmt)
+            got, _, q = run_fused_gemm(gpu, "rc", case, a, b, c, bias, None, mode, activation=act, requant=rq)
+            want_c, _, want_q = fused_expectation(case, anchor, None, None, activation=act, requant=rq)
+            tag = (ta, what, mode, fmt, per_column, rsq, only)
+            assert np.array_equal(q, want_q), tag
+            assert np.array_equal(got.view(np.uint8), (c if only else want_c).view(np.uint8)), tag
+            oq = np.arange(m)[:, None] * rsq + np.arange(n)[None, :] * csq
+            codes = want_q[oq].view(np.uint8) & 0x7F
+            beyond = {1: 0x7F, 2: 0x7E, 3: 0x7C, 4: 0x7B}[fmt]   # what a value past the largest becomes
+            assert np.count_nonzero(codes == beyond) > 0 and len(np.unique(codes)) > (40 if per_column else 3), tag
+
+
 @pytest.mark.parametrize("act", (2, 3))
 def test_silu_and_gelu_values(gpu, act):
     """The activation alone: with alpha = 0 and beta = 1 the value it is applied to is C itself, so any fp32 value
@@ -497,7 +529,8 @@ def test_fused_extra_steps_blocked_form_any_strides_and_refusals(gpu):
     a, b, c = case.make_inputs(1)
     q0, one = np.zeros(64, np.int8), np.ones(1, np.float32)
     for bad in (dict(q=q0, rsq=8, csq=1, scale=None), dict(q=q0, rsq=8, csq=1, scale=one, zero=128),
-                dict(q=q0, rsq=8, csq=1, scale=one, zero=-129)):
+                dict(q=q0, rsq=8, csq=1, scale=one, zero=-129), dict(q=q0, rsq=8, csq=1, scale=one, format=5),
+                dict(q=q0, rsq=8, csq=1, scale=one, format=-1)):
         run_fused_gemm_expecting_refusal(gpu, case, a, b, c, requant=bad)
     run_fused_gemm_expecting_refusal(gpu, case, a, b, c, activation=2)
     # a Q in memory of the other kind than C
@@ -514,7 +547,7 @@ def run_fused_gemm_expecting_refusal(gpu, case, a, b, c, activation=0, requant=N
     gpu.skl_gemm_fused_i8rc_i8rc_i32rc_gfx950(
         case.m1, case.n1, case.k1, 1, a, case.rsa1, 1, b, case.rsb1, 1, 0, c, case.rsc1, 1,
         skl_amd.Epilogue(None, None, activation=activation, q=rq.get("q"), rsq=rq.get("rsq", 0), csq=rq.get("csq", 0),
-                         q_scale=rq.get("scale"), q_zero=rq.get("zero", 0)))
+                         q_scale=rq.get("scale"), q_zero=rq.get("zero", 0), q_format=rq.get("format", 0)))
     assert gpu.skl_hip_last_error() != 0, (activation, requant)  # reading clears it
     assert np.array_equal(c, before)
 

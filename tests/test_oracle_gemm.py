@@ -239,13 +239,24 @@ def test_f32_to_f16_rounding_matches_numpy():
 FUSED_TYPES = ("i8", "bf16", "f16", "f8e4m3", "f8e5m2")
 
 
-def requantised(v, scale, zero):
+FP8_COPY_FORMATS = {1: "skl_cvt_f32_f8e4m3_oracle", 2: "skl_cvt_sat_f32_f8e4m3_oracle",
+                    3: "skl_cvt_f32_f8e5m2_oracle", 4: "skl_cvt_sat_f32_f8e5m2_oracle"}   # q_format -> the conversion it fuses
+
+
+def requantised(v, scale, zero, fmt=0):
     """clamp(rne((float)v * s) + zero, -128, 127) of include/skl-gfx950.h, in numpy and by another route than the
     checker's C: the product of two fp32 values is exact in fp64, so rounding it to fp32 once is the one fp32
-    multiplication; np.rint rounds ties to even; a NaN counts as 0, values beyond int32 as its ends."""
+    multiplication; np.rint rounds ties to even; a NaN counts as 0, values beyond int32 as its ends.
+    With an fp8 `fmt` the bytes are the checker's fp32 -> fp8 conversion (pinned to the reference's vectors in
+    test_oracle_cvt.py) of that same product (its own factor 1 changes nothing)."""
     with np.errstate(invalid="ignore", over="ignore"):
         prod = (np.asarray(v).astype(np.float32).astype(np.float64) * np.asarray(scale, np.float32).astype(np.float64)
                 ).astype(np.float32)
+        if fmt:
+            flat = np.ascontiguousarray(prod).ravel()
+            out = np.empty(flat.size, np.uint8)
+            getattr(oracle(), FP8_COPY_FORMATS[fmt])(out, flat, 1.0, flat.size)
+            return out.view(np.int8).reshape(prod.shape)
         r = np.rint(prod.astype(np.float64))
     r = np.where(np.isnan(r), 0.0, np.clip(r, -2147483648.0, 2147483647.0))
     return np.clip(r.astype(np.int64) + int(zero), -128, 127).astype(np.int8)
@@ -255,7 +266,7 @@ def fused_expectation(case, plain, bias, max_in, activation=0, requant=None):
     """C and *max after the fused steps, from the plain GEMM's result: the bias of the logical column
     added in C's arithmetic (one fp32 addition / int32 wrap), the activation, the maximum over what was
     written. With `requant` = dict(q=<int8 buffer before the call>, rsq, csq, scale=<1 or n floats>,
-    per_column, zero, only) a third value follows: the int8 buffer afterwards (and C stays `plain`'s
+    per_column, zero, only, format) a third value follows: the int8 buffer afterwards (and C stays `plain`'s
     memory where `only` says it is not written)."""
     oc = support.blocked_offsets(case.m1, case.n1, case.m0, case.n0, case.rsc0, case.csc0, case.rsc1, case.csc1)
     want = plain.copy()
@@ -279,7 +290,7 @@ def fused_expectation(case, plain, bias, max_in, activation=0, requant=None):
     q = requant["q"].copy()
     scale = requant["scale"][None, :] if requant.get("per_column") else requant["scale"][0]
     oq = np.arange(m)[:, None] * requant["rsq"] + np.arange(n)[None, :] * requant["csq"]
-    q[oq] = requantised(want[oc], scale, requant.get("zero", 0))
+    q[oq] = requantised(want[oc], scale, requant.get("zero", 0), requant.get("format", 0))
     return want, top, q
 
 
@@ -477,6 +488,29 @@ def test_requantisation_rule_on_worked_values():
                     oq = np.arange(m)[:, None] * rsq + np.arange(n)[None, :] * csq
                     want_q[oq] = requantised(want_c[oc], scale[None, :] if per_column else scale[0], zero)
                     assert np.array_equal(q, want_q), (suffix, per_column, act, zero)
+
+
+def test_fp8_copy_rule_on_worked_values():
+    """The fp8 forms of the 8-bit copy (q_format of include/skl-gfx950.h) as this file's tests expect them: worked
+    codes for both formats - exact values, the tie at the largest value (E4M3: 464 stays 448, its last bit is even;
+    E5M2: 61440 goes up and overflows), what lies beyond with and without saturation (E4M3's NaN carries no sign,
+    ref/cvt/cvt_ofp8.c:97-107), the smallest subnormal - and the product taken once in fp32 before the conversion
+    equal to the conversion given the scale itself."""
+    def codes(values, scale, fmt):
+        return list(requantised(np.array(values, np.float32), np.float32(scale), 0, fmt).view(np.uint8))
+
+    assert codes([1.0, 448.0, 464.0, 465.0, -500.0, 2.0 ** -9, -0.0], 1.0, 1) == [0x38, 0x7E, 0x7E, 0x7F, 0x7F, 0x01, 0x80]
+    assert codes([1.0, 448.0, 464.0, 465.0, -500.0, 2.0 ** -9, -0.0], 1.0, 2) == [0x38, 0x7E, 0x7E, 0x7E, 0xFE, 0x01, 0x80]
+    assert codes([1.0, 57344.0, 61439.0, 61440.0, -70000.0, 2.0 ** -16], 1.0, 3) == [0x3C, 0x7B, 0x7B, 0x7C, 0xFC, 0x01]
+    assert codes([1.0, 57344.0, 61439.0, 61440.0, -70000.0, 2.0 ** -16], 1.0, 4) == [0x3C, 0x7B, 0x7B, 0x7B, 0xFB, 0x01]
+    assert codes([2.0, 928.0, 930.0], 0.5, 1) == [0x38, 0x7E, 0x7F]   # the scale is applied first
+    rng = np.random.default_rng(8)
+    v = (rng.standard_normal(20000) * np.exp2(rng.integers(-20, 18, 20000))).astype(np.float32)
+    for fmt, name in FP8_COPY_FORMATS.items():
+        for scale in (0.37, 3.0, 2.0 ** -7):
+            direct = np.empty(v.size, np.uint8)
+            getattr(oracle(), name)(direct, v, scale, v.size)
+            assert np.array_equal(direct.view(np.int8), requantised(v, np.float32(scale), 0, fmt)), (fmt, scale)
 
 
 def block4x8x4_case(m1, n1, k1, rsa1=None, rsb1=None, rsc1=None, accum=False):
