@@ -280,6 +280,22 @@ def wl_gemm_i8_8192(lib, rng):
                   8192, 1, lambda n: rand_i8(rng, n), lambda n: rand_i8(rng, n), 1, 0, np.int32, "i8")
 
 
+def wl_gemm_i8_blocks_4x8x4(accum):
+    """The 4 x 8 by 8 x 4 block format (A in 4 x 8 blocks, B in 8 x 4, C in 4 x 4), 8192^3."""
+    def make(lib, rng):
+        m = n = k = 8192
+        a, b = DeviceBuffer.from_array(rand_i8(rng, m * k)), DeviceBuffer.from_array(rand_i8(rng, k * n))
+        c = DeviceBuffer.from_array(np.zeros(m * n, np.int32))
+
+        def step(i):
+            lib.skl_gemm_a1b01_i8p4x8_i8p8x4_i32p4x4_gfx950(m // 4, n // 4, k // 8, a, 4 * k, b, 8 * n, c, 4 * n, accum)
+
+        return dict(fn=step, bytes=m * k + k * n + 4 * m * n * (2 if accum else 1), ops=2 * m * n * k, bound="mfma", dtype="i8",
+                    keep=(a, b, c), name="int8 GEMM 8192^3 in 4x8 / 8x4 / 4x4 blocks" + (", accumulating" if accum else ""),
+                    kernel="copies + gemm_mfma_ring_kernel")
+    return make
+
+
 def wl_gemm_i8_8192_requantised(lib, rng):
     """A quantised layer: int8 in, ReLU, int8 out (per-column scales), the int32 C never written (q_only)."""
     import skl_amd
@@ -542,6 +558,8 @@ WORKLOADS = {
     "peak_mfma_bf16_constant": (_wl_peak_mfma(1, "bf16", 0), 3, 1, 1),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2, 1),
     "gemm_i8_8192_requantised": (wl_gemm_i8_8192_requantised, 10, 2, 1),
+    "gemm_i8_8192_blocks_4x8x4": (wl_gemm_i8_blocks_4x8x4(False), 10, 2, 1),
+    "gemm_i8_8192_blocks_4x8x4_accum": (wl_gemm_i8_blocks_4x8x4(True), 10, 2, 1),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2, 1),
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 10, 2, 1),
     "gemm_f8e4m3_8192_rowmajor_a": (wl_gemm_f8_layout(True, False), 10, 2, 1),

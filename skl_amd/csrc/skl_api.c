@@ -326,9 +326,9 @@ static int gemm_padded_to_tiles(const skl_gemm_canon *g) {
 }
 
 /* Any other blocking (the 4x8 / 8x4 / 4x4 blocks of src/gemm/packed-gemm.md:270-298, blocks of 32, ...): A and B
- * are copied into rows contiguous in K, C is unpacked into a row-major scratch matrix - also for beta == 0 when C is
- * floating point, since such a call still reads C where the product is an exact zero - multiplied there, and packed
- * back. M and N are
+ * are copied into rows contiguous in K; C is updated where it lies when the kernels can index its blocks (below),
+ * else unpacked into a row-major scratch matrix - also for beta == 0 when C is floating point, since such a call
+ * still reads C where the product is an exact zero - multiplied there, and packed back. M and N are
  * whole numbers of blocks, so packing writes exactly the elements the reference writes. */
 static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   const size_t M = d->m0 * d->m1, N = d->n0 * d->n1, K = d->k0 * d->k1;
@@ -354,10 +354,15 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   h.bias = d->bias, h.max = d->max;
   h.rq = d->rq;
   /* C in power-of-two blocks (the 4 x 4 blocks of that format) can be updated where it is by the matrix-core
-   * kernels. Small blocks make their stores short (16 bytes per 4 x 4 block row), so that pays when C would
-   * otherwise travel three times (unpack, update, pack: 8192^3 in 4 x 4 blocks 890 against 1048 us), not when an
-   * integer C with beta == 0 is only packed (998 against 913 us). */
-  c_in_place = c_is_read && canonicalize_c(d, &h, 1);
+   * kernels. Small blocks make the bounds-checked kernels' stores short (16 bytes per 4 x 4 block row), so that pays
+   * when C would otherwise travel three times (unpack, update, pack), not when an integer C with beta == 0 is only
+   * packed - unless the streaming kernel takes the problem and writes such blocks 16 bytes per lane (8192^3: no
+   * pack pass of 81 us). */
+  c_in_place = canonicalize_c(d, &h, 1);
+  if (c_in_place && !c_is_read) {
+    h.a = h.b = (const void *)(uintptr_t)256;
+    c_in_place = skl_hip_gemm_mfma_streams_c_quads(&h);
+  }
   if (!c_in_place) {
     h.c = (void *)(uintptr_t)256;
     h.rsc0 = N, h.rsc1 = SKL_TE * N, h.csc0 = 1, h.csc1 = SKL_TE;

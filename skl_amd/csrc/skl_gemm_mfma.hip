@@ -799,7 +799,9 @@ constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // EDGE: the operands are copies padded to whole tiles, C is not - its last tile rows / columns end at p.m / p.n and
 // the epilogue touches nothing beyond them.
-template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0>
+// CQUADS: an int32 C in small blocks with contiguous rows (the 4 x 4 blocks of src/gemm/packed-gemm.md:270-298, up to
+// 16 columns), no fused steps - see the epilogue.
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0, bool CQUADS = false>
 __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   using KA = Kind<TA>;
   using M = Mma<TA, TB>;
@@ -1048,6 +1050,64 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
     }
     return;
   }
+  if constexpr (CQUADS) {
+    // A lane holds four consecutive rows of one column, and with blocks of four columns a row of a block is 16
+    // bytes: stored as they are, a wave's stores are 16-byte runs 64 bytes apart (8192^3: 100 us more than a
+    // row-major C). The four lanes of a quad hold the four columns of those rows, so the 4 x 4 values are exchanged
+    // inside the quad - lane q ends up with row q's four columns - and every lane moves 16 bytes per instruction: a
+    // quad covers 64 contiguous bytes, lanes 0-31 eight neighbouring blocks.
+    static_assert(std::is_same<AccElem, int>::value && !EDGE && EXTRA == 0, "int32 C, whole tiles, no fused steps");
+    int *c = reinterpret_cast<int *>(p.c);
+    const bool init = p.beta.i == 0;
+    const int qd = lane & 3;
+    const size_t cmask = (size_t(1) << p.ccs) - 1, rmask = (size_t(1) << p.crs) - 1;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const size_t col4 = n0 + wn + j * 32 + (lane & 28);   // the quad's first column, a multiple of four
+      const size_t col_off = (col4 >> p.ccs) * p.csc1 + (col4 & cmask);
+#pragma unroll
+      for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
+        v4i *out[kEpilogueBatch][4];
+        v4i old[kEpilogueBatch][4];
+#pragma unroll
+        for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4 + qd;
+            out[i][g] = reinterpret_cast<v4i *>(c + (row >> p.crs) * p.rsc1 + (row & rmask) * p.rsc0 + col_off);
+          }
+        if (!init) {
+#pragma unroll
+          for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) old[i][g] = *out[i][g];
+        }
+#pragma unroll
+        for (int i = 0; i < kEpilogueBatch; ++i)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const Acc &t = acc[i0 + i][j];
+            v4i r;
+#define SKL_ROW_OF_QUAD(CC, CTRL)                                                                                    \
+  {                                                                                                                   \
+    const int b0 = __builtin_amdgcn_update_dpp(0, t[4 * g + 0], CTRL, 0xF, 0xF, true), b1 = __builtin_amdgcn_update_dpp(0, t[4 * g + 1], CTRL, 0xF, 0xF, true); \
+    const int b2 = __builtin_amdgcn_update_dpp(0, t[4 * g + 2], CTRL, 0xF, 0xF, true), b3 = __builtin_amdgcn_update_dpp(0, t[4 * g + 3], CTRL, 0xF, 0xF, true); \
+    r[CC] = qd == 0 ? b0 : qd == 1 ? b1 : qd == 2 ? b2 : b3;                                                          \
+  }
+            SKL_ROW_OF_QUAD(0, 0x00)   // quad_perm: every lane reads the quad's lane 0 - column 0 of the four rows
+            SKL_ROW_OF_QUAD(1, 0x55)
+            SKL_ROW_OF_QUAD(2, 0xAA)
+            SKL_ROW_OF_QUAD(3, 0xFF)
+#undef SKL_ROW_OF_QUAD
+            v4i v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = init ? skl_initialise(r[e], (const int *)nullptr, p.alpha, p.beta) : skl_combine(r[e], old[i][g][e], p.alpha, p.beta);
+            __builtin_nontemporal_store(v, out[i][g]);
+          }
+      }
+    }
+    return;
+  }
   // Epilogue, as in the kernel above: old values requested kEpilogueBatch blocks at a time, non-temporal stores.
   AccElem *c = reinterpret_cast<AccElem *>(p.c);
   const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
@@ -1162,13 +1222,23 @@ constexpr size_t kRingMinSlicesPerSplit = 64;  // below 8 KiB of K per row the p
 template <int TA>
 constexpr bool kRingCarriesExtraSteps = TA == SKL_DT_I8;
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0>
+// An int32 C the streaming kernel writes 16 bytes per lane: blocks of 4 to 16 columns with contiguous rows, a
+// multiple of four rows per block, everything on 16-byte boundaries, no fused steps.
+inline bool c_in_row_quads(const MfmaArgs &p) {
+  return !p.bias && !p.max && !p.rq.act && !p.rq.q && p.csc0 == 1 && p.ccs >= 2 && p.ccs <= 4 && p.crs >= 2 &&
+         (((uintptr_t)p.c | (p.rsc0 * 4) | (p.rsc1 * 4) | (p.csc1 * 4)) & 15) == 0;
+}
+
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0, bool CQUADS = false>
 int launch_ring(const MfmaArgs &args) {
   if constexpr (EXTRA == 0 && kRingCarriesExtraSteps<TA> && !EDGE) {
     if (args.rq.q) return args.rq.q_only ? launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 2>(args) : launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 3>(args);
   }
+  if constexpr (TA == SKL_DT_I8 && TB == SKL_DT_I8 && A_KC && B_KC && !EDGE && EXTRA == 0 && !CQUADS) {  // what copies of blocked operands look like
+    if (c_in_row_quads(args)) return launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 0, true>(args);
+  }
   constexpr int lds = kRingStages * (256 + BN) * kRingSlice;
-  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE, EXTRA>;
+  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE, EXTRA, CQUADS>;
   static bool configured = false;
   if (!configured) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -1371,6 +1441,23 @@ bool streams_in_place(const skl_gemm_canon *g, size_t es) {
   const size_t tiles_m = g->m / 256;
   return (g->n % 256 == 0 && tiles_m * (g->n / 256) >= 200) || (g->n % 128 == 0 && tiles_m * (g->n / 128) >= 96);
 }
+
+}  // namespace
+
+// Would the streaming kernel take this int8 problem as it lies and write its C 16 bytes per lane (C in blocks of 4
+// to 16 columns with contiguous rows)? Then a blocked C costs no more than a row-major one.
+extern "C" int skl_hip_gemm_mfma_streams_c_quads(const skl_gemm_canon *g) {
+  if (g->ta != SKL_DT_I8 || g->tb != SKL_DT_I8 || g->a_sk != 1 || g->b_sk != 1 || !streams_in_place(g, 1)) return 0;
+  MfmaArgs p;
+  p.c = (char *)g->c;
+  p.rsc0 = g->rsc0, p.csc0 = g->csc0, p.rsc1 = g->rsc1, p.csc1 = g->csc1;
+  p.crs = g->c_row_shift, p.ccs = g->c_col_shift;
+  p.bias = (const char *)g->bias, p.max = (char *)g->max;
+  p.rq = g->rq;
+  return c_in_row_quads(p);
+}
+
+namespace {
 
 template <int TA, int TB>
 int launch_padded(const MfmaArgs &p, size_t tile_cols) {

@@ -115,6 +115,9 @@ int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g);
  * width (256 / 128) and the padded extents when that pays, else 0; the launch takes the canonical description of the
  * copies (K contiguous, rows *kp apart, k == *kp) with the true m, n and C. */
 int skl_hip_gemm_mfma_padded_plan(const skl_gemm_canon *g, size_t *mp, size_t *np, size_t *kp);
+/* 1 when the streaming kernel would take this int8 problem where it lies and write its blocked C (4 to 16 columns
+ * per block, contiguous rows) 16 bytes per lane - as cheaply as a row-major C. */
+int skl_hip_gemm_mfma_streams_c_quads(const skl_gemm_canon *g);
 int skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile_cols);
 
 /* M == 1 streaming kernels: y[j*csc] = beta*y + alpha * sum_p x[p*x_sk] * B(p,j).

@@ -94,6 +94,56 @@ __global__ void __launch_bounds__(kThreads) realign_rows_kernel(const char *__re
   *reinterpret_cast<uint4 *>(dst + xx * pitch + off) = v;
 }
 
+// Source blocked along K with the block's k contiguous in runs of a whole number of 8-byte pieces (the 4 x 8 blocks
+// of src/gemm/packed-gemm.md:270-298: four rows of eight k in 32 bytes): one thread per 16-byte piece of a destination
+// row, gathered from 8-byte pieces of the source. The rows of one block of x0 rows are neighbouring threads, so a
+// wave reads whole lines of the source and writes 16-byte pieces that the next lanes continue.
+template <int ES>
+__global__ void __launch_bounds__(kThreads) realign_kruns_kernel(const char *__restrict__ src, char *__restrict__ dst, size_t x,
+                                                                 size_t kbytes, size_t pitch, RealignSource f, size_t lanes_x) {
+  const size_t pieces_per_row = pitch / 16;
+  const size_t idx = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  // lanes_x rows (a power of two dividing x0, at most 64) x pieces, rows fastest
+  const size_t in_group = idx % lanes_x, rest = idx / lanes_x;
+  const size_t piece = rest % pieces_per_row, xx = (rest / pieces_per_row) * lanes_x + in_group;
+  if (xx >= x) return;
+  const char *row = src + ((xx / f.x0) * f.s1 + (xx % f.x0) * f.s0) * ES;
+  uint2 half[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const size_t off = piece * 16 + 8 * h, p = off / ES;
+    half[h] = off < kbytes ? *reinterpret_cast<const uint2 *>(row + ((p / f.k0) * f.sk1 + (p % f.k0)) * ES) : make_uint2(0, 0);
+  }
+  *reinterpret_cast<uint4 *>(dst + xx * pitch + piece * 16) = make_uint4(half[0].x, half[0].y, half[1].x, half[1].y);
+}
+
+// 8-bit source in blocks of k0 k-rows of four contiguous x (the 8 x 4 blocks of src/gemm/packed-gemm.md:270-298):
+// a thread takes eight k-rows of one block - 32 contiguous bytes -, turns them into eight k-bytes for each of the
+// four x (byte permutes) and stores them to the four destination rows. Four neighbouring blocks along x and 64
+// k-groups per workgroup: a wave reads 128 contiguous bytes per k-group when the blocks lie side by side and writes
+// 128 contiguous bytes per destination row.
+__global__ void __launch_bounds__(kThreads) realign_x4_kernel(const char *__restrict__ src, char *__restrict__ dst, size_t x,
+                                                              size_t k, size_t pitch, RealignSource f, unsigned tiles_p) {
+  const size_t xb = (size_t)(blockIdx.x / tiles_p) * 4 + (threadIdx.x & 3);   // block of four x
+  const size_t kg = (size_t)(blockIdx.x % tiles_p) * 64 + (threadIdx.x >> 2);  // group of eight k
+  if (xb * 4 >= x || kg * 8 >= pitch) return;
+  unsigned v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (kg * 8 < k) {
+    const size_t p = kg * 8;
+    const uint4 *from = reinterpret_cast<const uint4 *>(src + xb * f.s1 + (p / f.k0) * f.sk1 + (p % f.k0) * 4);
+    const uint4 lo = from[0], hi = from[1];
+    v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const unsigned pick = 0x0C0C0000u | ((4u + c) << 8) | (unsigned)c;   // byte c of the low, then of the high operand
+    const unsigned k01 = __builtin_amdgcn_perm(v[1], v[0], pick), k23 = __builtin_amdgcn_perm(v[3], v[2], pick);
+    const unsigned k45 = __builtin_amdgcn_perm(v[5], v[4], pick), k67 = __builtin_amdgcn_perm(v[7], v[6], pick);
+    *reinterpret_cast<uint2 *>(dst + (xb * 4 + c) * pitch + kg * 8) =
+        make_uint2(__builtin_amdgcn_perm(k23, k01, 0x05040100u), __builtin_amdgcn_perm(k67, k45, 0x05040100u));
+  }
+}
+
 // Any other source (contiguous along x, blocked in K, no unit stride at all): a 64 x 64 tile is read with lanes
 // along the source's denser direction, kept in LDS with K contiguous (row pitch 64 elements + 4 bytes: lanes along
 // x hit distinct banks), and written as 16-byte pieces of the destination rows.
@@ -472,6 +522,27 @@ int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_
         }
         return skl_check_launch("realign_rows");
       }
+    }
+  }
+  if (k0 > 1 && sk0 == 1 && (k0 * es) % 8 == 0 && pitch % 16 == 0 && ((uintptr_t)dst & 15) == 0 && k % k0 == 0 &&
+      (((uintptr_t)src | (x0 > 1 ? s0 * es : 0) | (s1 * es) | (sk1 * es)) & 7) == 0) {
+    // K in blocks whose k are contiguous: 8-byte pieces
+    size_t lanes_x = 1;
+    while (lanes_x < 64 && x0 % (lanes_x * 2) == 0) lanes_x *= 2;
+    const size_t groups = (x + lanes_x - 1) / lanes_x, blocks = (groups * lanes_x * (pitch / 16) + kThreads - 1) / kThreads;
+    if (blocks <= 0x7FFFFFFFu) {
+      if (esize == 1) realign_kruns_kernel<1><<<(unsigned)blocks, kThreads, 0, st>>>((const char *)src, (char *)dst, x, k * es, pitch, f, lanes_x);
+      else realign_kruns_kernel<2><<<(unsigned)blocks, kThreads, 0, st>>>((const char *)src, (char *)dst, x, k * es, pitch, f, lanes_x);
+      return skl_check_launch("realign_kruns");
+    }
+  }
+  if (esize == 1 && x0 == 4 && s0 == 1 && sk0 == 4 && k0 % 8 == 0 && k % k0 == 0 && x % 4 == 0 && pitch % 8 == 0 &&
+      ((uintptr_t)dst & 7) == 0 && (((uintptr_t)src | s1 | sk1) & 15) == 0) {
+    // blocks of k0 k-rows of four contiguous x
+    const size_t tp = (pitch / 8 + 63) / 64, blocks = ((x / 4 + 3) / 4) * tp;
+    if (blocks <= 0x7FFFFFFFu) {
+      realign_x4_kernel<<<(unsigned)blocks, kThreads, 0, st>>>((const char *)src, (char *)dst, x, k, pitch, f, (unsigned)tp);
+      return skl_check_launch("realign_x4");
     }
   }
   if (pitch % 16 == 0 && ((uintptr_t)dst & 15) == 0) {

@@ -874,7 +874,10 @@ def test_block4x8x4_entry_point(gpu, mode):
     gaps between them; C = A*B and C += A*B; empty dimensions. Whole C buffer compared bit for bit."""
     from test_oracle_gemm import block4x8x4_case
     shapes = [(1, 1, 1, 0), (3, 2, 5, 7), (0, 2, 2, 0), (2, 0, 2, 0), (2, 2, 0, 0), (64, 96, 40, 0), (33, 50, 129, 48),
-              (256, 8, 64, 16)]
+              (256, 8, 64, 16),
+              # whole 256-row tiles: the streaming kernel, which writes the 4 x 4 blocks of C 16 bytes per lane (256 x 128
+              # and 256 x 256 tiles); with a gap that keeps block rows on 16-byte boundaries and one that does not
+              (512, 384, 32, 0), (512, 384, 16, 16), (512, 384, 16, 2), (1024, 832, 16, 0)]
     for i, (m1, n1, k1, gap) in enumerate(shapes):
         for accum in (False, True):
             case = block4x8x4_case(m1, n1, k1, 32 * k1 + gap, 32 * n1 + gap, 16 * n1 + gap, accum)
