@@ -280,6 +280,26 @@ def wl_gemm_i8_8192(lib, rng):
                   8192, 1, lambda n: rand_i8(rng, n), lambda n: rand_i8(rng, n), 1, 0, np.int32, "i8")
 
 
+def wl_gemm_f8_8192_f8_out(lib, rng):
+    """An fp8 layer feeding the next: E4M3 in, bias, E4M3 out (saturating, per-column scales), the fp32 C never written."""
+    import skl_amd
+    m = n = k = 8192
+    a, b = _fp8_operand(lib, rng, m * k, "f8e4m3"), _fp8_operand(lib, rng, k * n, "f8e4m3")
+    c = DeviceBuffer(4 * m * n)  # neither written nor, with beta == 0, read
+    q = DeviceBuffer(m * n)
+    bias = DeviceBuffer.from_array(rng.uniform(-1, 1, n).astype(np.float32))
+    scales = DeviceBuffer.from_array(rng.uniform(0.5, 2.0, n).astype(np.float32) / 64.0)
+    ep = skl_amd.Epilogue(bias, None, q=q, rsq=n, csq=1, q_scale=scales, q_scale_per_column=True, q_only=True,
+                          q_format=skl_amd.Epilogue.Q_F8E4M3_SAT)
+
+    def step(i):
+        lib.skl_gemm_fused_f8e4m3rc_f8e4m3rc_f32rc_gfx950(m, n, k, 1.0, a, k, 1, b, n, 1, 0.0, c, n, 1, ep)
+
+    return dict(fn=step, bytes=m * k + k * n + m * n, ops=2 * m * n * k, bound="mfma", dtype="f8", keep=(a, b, c, q, bias, scales),
+                name="fp8 E4M3 GEMM 8192^3 with bias and saturating E4M3 output only (q_only)",
+                kernel="gemm_mfma_ring_kernel<E4M3, EXTRA>")
+
+
 def wl_gemm_i8_blocks_4x8x4(accum):
     """The 4 x 8 by 8 x 4 block format (A in 4 x 8 blocks, B in 8 x 4, C in 4 x 4), 8192^3."""
     def make(lib, rng):
@@ -558,6 +578,7 @@ WORKLOADS = {
     "peak_mfma_bf16_constant": (_wl_peak_mfma(1, "bf16", 0), 3, 1, 1),
     "gemm_i8_8192": (wl_gemm_i8_8192, 10, 2, 1),
     "gemm_i8_8192_requantised": (wl_gemm_i8_8192_requantised, 10, 2, 1),
+    "gemm_f8e4m3_8192_f8_out": (wl_gemm_f8_8192_f8_out, 10, 2, 1),
     "gemm_i8_8192_blocks_4x8x4": (wl_gemm_i8_blocks_4x8x4(False), 10, 2, 1),
     "gemm_i8_8192_blocks_4x8x4_accum": (wl_gemm_i8_blocks_4x8x4(True), 10, 2, 1),
     "gemm_f8e4m3_8192": (wl_gemm_f8_8192, 10, 2, 1),

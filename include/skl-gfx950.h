@@ -170,6 +170,10 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, 
  *                                                with q_format one of the fp8 codes below the byte is instead the OCP fp8
  *                                                encoding of (float)v * s_j as skl_cvt_[sat_]f32_f8e4m3 / _f8e5m2
  *                                                (ref/cvt/cvt_ofp8.c:174-242) produces it, q_zero unused
+ *                                                with q_only C is not written; and with beta == 0 it is not read either
+ *                                                (the pointer need not address a matrix): where the product is an
+ *                                                exact zero a floating-point result then takes the sign that an old
+ *                                                C of +0 would give it
  *     *max = v  if v > *max                      if max != NULL (a NaN never replaces the maximum;
  *                                                the sign of a zero maximum is unspecified)
  * Bias and maximum are the steps of the reference's fused kernels; activation and requantisation are what
@@ -177,7 +181,7 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, 
  * functions") and leaves to them - the reference has no routine for either, the rules above define them here.
  * bias points to n = n1*n0 values of C's type, max to one, q_scale to n floats or one; all of them and q must be
  * memory of the same kind as C (device or host) and must not overlap C or each other; *max must not be NaN on
- * entry; q_zero lies in [-128, 127]. With q_only the call still reads C when beta asks for it. Members left zero
+ * entry; q_zero lies in [-128, 127]. With q_only the call still reads C when beta is not zero (or skl_hip_set_beta_zero_mode asked for the reference's evaluation of beta * C). Members left zero
  * (e.g. by a designated initialiser that names only bias and max) switch their step off. ep == NULL: the plain GEMM. */
 #define SKL_GFX950_ACT_NONE 0
 #define SKL_GFX950_ACT_RELU 1

@@ -325,6 +325,12 @@ static int gemm_padded_to_tiles(const skl_gemm_canon *g) {
   return r;
 }
 
+/* A floating-point call that writes only the 8-bit copy, with beta == 0: C is neither written nor read (gemm_run
+ * marks beta so; the kernels then take +0 for the old C where the product is an exact zero). */
+static int c_untouched(const skl_gemm_desc *d) {
+  return d->ta != SKL_DT_I8 && d->ta != SKL_DT_F64 && d->beta.fz.skip_c_read == SKL_C_UNTOUCHED;
+}
+
 /* Any other blocking (the 4x8 / 8x4 / 4x4 blocks of src/gemm/packed-gemm.md:270-298, blocks of 32, ...): A and B
  * are copied into rows contiguous in K; C is updated where it lies when the kernels can index its blocks (below),
  * else unpacked into a row-major scratch matrix - also for beta == 0 when C is floating point, since such a call
@@ -336,7 +342,7 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   const size_t kpa = (K * esa + 15) / 16 * 16 / esa, kpb = (K * esb + 15) / 16 * 16 / esb;
   const size_t bytes_a = (M * kpa * esa + 255) / 256 * 256, bytes_b = (N * kpb * esb + 255) / 256 * 256;
   /* an integer C with beta == 0 is not read at all; a floating-point one is, where the product is an exact zero */
-  const int c_is_read = !(d->ta == SKL_DT_I8 && d->beta.i == 0);
+  const int c_is_read = !(d->ta == SKL_DT_I8 && d->beta.i == 0) && !c_untouched(d);
   skl_gemm_canon h;
   char *scratch;
   int r, c_in_place;
@@ -454,6 +460,7 @@ static int gemm_on_device(const skl_gemm_desc *d) {
 /* The kinds whose alpha and beta travel as a float (F16H: widened). */
 static int scalars_are_float(int dt) { return dt != SKL_DT_I8 && dt != SKL_DT_F64; }
 
+
 static void gemm_run(const skl_gemm_desc *in, const char *who) {
   skl_gemm_desc with_mode = *in;
   const skl_gemm_desc *d = &with_mode;
@@ -465,6 +472,8 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
     memset(&with_mode.beta, 0, sizeof with_mode.beta);
     with_mode.beta.fz.value = beta;
     with_mode.beta.fz.skip_c_read = skl_hip_get_beta_zero_mode() != SKL_HIP_BETA_ZERO_AS_REFERENCE;
+    /* a call that writes only the 8-bit copy does not read C either when beta is zero: C need not be a matrix */
+    if (with_mode.beta.fz.skip_c_read && beta == 0.0f && in->rq.q && in->rq.q_only) with_mode.beta.fz.skip_c_read = SKL_C_UNTOUCHED;
   }
   where = classify(K ? d->a : NULL, K ? d->b : NULL, d->c, who);
   if (where < 0) return;
@@ -503,7 +512,8 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
     const size_t nc = span4(d->m1, d->rsc1, d->n1, d->csc1, d->m0, d->rsc0, d->n0, d->csc0);
     skl_gemm_desc dd = *d;
     const size_t esc = c_elem_size(d->ta);
-    void *da = stage_in(d->a, na * esa), *db = stage_in(d->b, nb * esb), *dc = stage_in(d->c, nc * esc);
+    const int untouched = c_untouched(d); /* then the caller's C need not exist: a stand-in that no kernel touches */
+    void *da = stage_in(d->a, na * esa), *db = stage_in(d->b, nb * esb), *dc = untouched ? skl_hip_malloc(16) : stage_in(d->c, nc * esc);
     void *dbias = d->bias ? stage_in(d->bias, N * esc) : NULL, *dmax = d->max ? stage_in(d->max, esc) : NULL;
     /* the requantised copy: its whole span travels both ways, like C's */
     const size_t nq = d->rq.q ? (M - 1) * d->rq.rsq + (N - 1) * d->rq.csq + 1 : 0;
@@ -527,7 +537,7 @@ static void gemm_run(const skl_gemm_desc *in, const char *who) {
     dd.rq.q = dq;
     dd.rq.q_scale = dqs;
     if (gemm_on_device(&dd) == 0) { /* after a failure the caller's memory stays as it was */
-      skl_hip_memcpy_d2h(d->c, dc, nc * esc);
+      if (!untouched) skl_hip_memcpy_d2h(d->c, dc, nc * esc);
       if (dmax) skl_hip_memcpy_d2h(d->max, dmax, esc);
       if (dq) skl_hip_memcpy_d2h(d->rq.q, dq, nq);
     }

@@ -41,7 +41,8 @@ static inline unsigned skl_div_up(size_t a, size_t b) { return (unsigned)((a + b
 // everywhere (so C may be uninitialised memory). A caller that wants the reference's result there too asks
 // for it (skl_hip_set_beta_zero_mode(SKL_HIP_BETA_ZERO_AS_REFERENCE)): beta then arrives without
 // fz.skip_c_read and C is read and combined whatever beta is. int32: 0 * c is 0 for every c, so C is never read
-// with beta == 0. f64 has no room for the switch next to the value: always read.
+// with beta == 0. f64 has no room for the switch next to the value: always read. A call that leaves C unwritten
+// (q_only) with beta == 0 does not touch C at all: the old C counts as +0 (skip_c_read == SKL_C_UNTOUCHED).
 // ---------------------------------------------------------------------------
 template <typename T>
 __device__ __forceinline__ bool skl_beta_is_zero(skl_scalar beta);  // "C need not be read"
@@ -69,7 +70,9 @@ __device__ __forceinline__ int skl_initialise(int acc, const int *, skl_scalar a
 }
 __device__ __forceinline__ float skl_initialise(float acc, const float *c, skl_scalar alpha, skl_scalar beta) {
   const float x = __fmul_rn(alpha.f, acc);
-  return x == 0.0f ? __fadd_rn(__uint_as_float((__float_as_uint(*c) ^ __float_as_uint(beta.f)) & 0x80000000u), x) : x;
+  const bool read_c = x == 0.0f && beta.fz.skip_c_read != SKL_C_UNTOUCHED;  // a call that does not write C does not read it either
+  const unsigned old = read_c ? __float_as_uint(*c) : 0u;
+  return x == 0.0f ? __fadd_rn(__uint_as_float((old ^ __float_as_uint(beta.f)) & 0x80000000u), x) : x;
 }
 __device__ __forceinline__ double skl_initialise(double acc, const double *c, skl_scalar alpha, skl_scalar beta) {
   const double x = __dmul_rn(alpha.d, acc);

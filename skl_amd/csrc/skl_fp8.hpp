@@ -49,6 +49,36 @@ __device__ __forceinline__ unsigned encode_ofp8(unsigned bits, bool sat) {
   return sign | mag;
 }
 
+// The same conversion with the format as values instead of a type, and without a branch: for epilogues that convert
+// their accumulators in place, where one code path serves both formats (the constants are uniform across the wave)
+// and a branch per element would cost registers next to 128 live accumulators. `fmt`: 1 / 2 E4M3 without / with
+// saturation, 3 / 4 E5M2 likewise.
+struct Ofp8Format {
+  int mant, bias, emin;
+  unsigned max, overflow_sign, overflow_code;
+  __host__ __device__ explicit Ofp8Format(int fmt) {
+    const bool e5 = fmt >= 3, sat = fmt == 2 || fmt == 4;
+    mant = e5 ? 2 : 3, bias = e5 ? 15 : 7, emin = e5 ? -14 : -6;
+    max = e5 ? 0x7Bu : 0x7Eu;
+    overflow_sign = (sat || e5) ? 0x80u : 0u;            // E4M3's overflow without saturation is the sign-less NaN
+    overflow_code = sat ? max : e5 ? 0x7Cu : 0x7Fu;
+  }
+};
+__host__ __device__ __forceinline__ unsigned encode_ofp8(unsigned bits, const Ofp8Format &f) {
+  const unsigned sign = (bits >> 24) & 0x80u, mag32 = bits & 0x7FFFFFFFu, field = mag32 >> 23;
+  const int e = field ? (int)field - 127 : -126;                             // fp32 subnormal: no hidden bit
+  const unsigned sig = field ? ((mag32 & 0x7FFFFFu) | 0x800000u) : mag32;
+  const int te = e > f.emin ? e : f.emin;
+  int shift = (te - f.mant) - (e - 23);
+  shift = shift > 31 ? 31 : shift;
+  unsigned q = sig >> shift;
+  const unsigned rem = sig & ((1u << shift) - 1u), half = 1u << (shift - 1);
+  q += (rem > half || (rem == half && (q & 1u))) ? 1u : 0u;
+  const unsigned mag = e < f.emin ? q : ((unsigned)(te + f.bias - 1) << f.mant) + q;   // inf / NaN: far beyond max
+  const unsigned finite = mag > f.max ? ((sign & f.overflow_sign) | f.overflow_code) : (sign | mag);
+  return mag32 > 0x7F800000u ? 0x7Fu : finite;
+}
+
 // OFP8 byte -> fp32 bit pattern. NaN codes give the sign-less quiet NaN.
 template <class F>
 __device__ __forceinline__ unsigned decode_ofp8_bits(unsigned code) {

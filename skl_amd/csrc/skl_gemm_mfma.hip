@@ -88,12 +88,17 @@ struct FusedSteps {
   T bias_j, running;
   size_t col;
   float q_scale_j;  // EXTRA: the current column's scale
+  const skl_fp8::Ofp8Format f8;  // modes 2 and 3: the constants of an fp8 copy (uniform; unused for an int8 copy)
   __device__ explicit FusedSteps(const MfmaArgs &p)
       : bias(reinterpret_cast<const T *>(p.bias)), max(reinterpret_cast<T *>(p.max)), rq(p.rq), bias_j(0), running(skl_lowest<T>()), col(0),
-        q_scale_j(0.0f) {}
-  // What a descriptor must look like for modes 2 and 3.
+        q_scale_j(0.0f), f8(p.rq.q_fmt) {}
+  // What a descriptor must look like for modes 2 and 3: a row-major copy on 4-byte boundaries, no activation beyond
+  // ReLU (the others cost too much code in each of a lane's 128 elements), and the copy's format the one these
+  // modes are built with for C's type - int8 behind an int32 C, OCP fp8 behind a floating-point C (an int8 product
+  // feeding an int8 layer, an fp8 product an fp8 layer; other pairings run on the bounds-checked kernels).
+  static constexpr bool kCopyIsFp8 = !std::is_same<T, int>::value;
   __host__ __device__ static bool dword_copy(const skl_requant &r) {
-    return r.q && r.q_fmt == 0 && r.csq == 1 && (r.rsq & 3) == 0 && ((uintptr_t)r.q & 3) == 0;
+    return r.q && r.act <= 1 && (r.q_fmt != 0) == kCopyIsFp8 && r.csq == 1 && (r.rsq & 3) == 0 && ((uintptr_t)r.q & 3) == 0;
   }
   __device__ __forceinline__ void column(size_t c) {
     col = c;
@@ -105,7 +110,8 @@ struct FusedSteps {
   }
   __device__ __forceinline__ T apply(T v) {
     if (bias) v = skl_add_bias(v, bias_j);
-    if constexpr (EXTRA != 0) v = skl_activate(v, rq.act);
+    if constexpr (EXTRA == 1) v = skl_activate(v, rq.act);
+    if constexpr (EXTRA >= 2) v = skl_activate(v, rq.act != 0);  // none or ReLU
     if (max && v > running) running = v;
     return v;
   }
@@ -132,7 +138,12 @@ struct FusedSteps {
     if constexpr (EXTRA >= 2) {
       unsigned packed = 0;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) packed |= ((unsigned)skl_requantise_int((float)v[i], q_scale_j, rq.q_zero) & 0xFFu) << (8 * i);
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (kCopyIsFp8)
+          packed |= skl_fp8::encode_ofp8(__float_as_uint(__fmul_rn((float)v[i], q_scale_j)), f8) << (8 * i);
+        else
+          packed |= ((unsigned)skl_requantise_int((float)v[i], q_scale_j, rq.q_zero) & 0xFFu) << (8 * i);
+      }
       const unsigned p0 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)packed, 0x00, 0xF, 0xF, true);  // quad_perm: lane 0 of the quad
       const unsigned p1 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)packed, 0x55, 0xF, 0xF, true);
       const unsigned p2 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)packed, 0xAA, 0xF, 0xF, true);
@@ -1219,8 +1230,8 @@ constexpr size_t kRingMinSlicesPerSplit = 64;  // below 8 KiB of K per row the p
 // The int8 streaming kernels for whole tiles also exist with the activation and requantisation steps, for a copy
 // that can be written as dwords (a quantised layer's int8 output at a quarter of C's bytes); every other call with
 // those steps goes to the bounds-checked kernels.
-template <int TA>
-constexpr bool kRingCarriesExtraSteps = TA == SKL_DT_I8;
+template <int TA, int TB>
+constexpr bool kRingCarriesExtraSteps = TA == TB && (TA == SKL_DT_I8 || TA == SKL_DT_F8E4M3 || TA == SKL_DT_F8E5M2);
 
 // An int32 C the streaming kernel writes 16 bytes per lane: blocks of 4 to 16 columns with contiguous rows, a
 // multiple of four rows per block, everything on 16-byte boundaries, no fused steps.
@@ -1231,7 +1242,7 @@ inline bool c_in_row_quads(const MfmaArgs &p) {
 
 template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0, bool CQUADS = false>
 int launch_ring(const MfmaArgs &args) {
-  if constexpr (EXTRA == 0 && kRingCarriesExtraSteps<TA> && !EDGE) {
+  if constexpr (EXTRA == 0 && kRingCarriesExtraSteps<TA, TB> && !EDGE) {
     if (args.rq.q) return args.rq.q_only ? launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 2>(args) : launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 3>(args);
   }
   if constexpr (TA == SKL_DT_I8 && TB == SKL_DT_I8 && A_KC && B_KC && !EDGE && EXTRA == 0 && !CQUADS) {  // what copies of blocked operands look like
@@ -1356,7 +1367,8 @@ int launch_tile(const MfmaArgs &p) {
   // can fill the 256 compute units, 256 x 128 tiles for the sizes below that; everything else runs
   // on the small, bounds-checked kernel.
   // activation / requantised copy: on the streaming kernel only int8 with a copy that goes out as dwords
-  const bool extra_steps = (p.rq.act || p.rq.q) && !(kRingCarriesExtraSteps<TA> && FusedSteps<int, 2>::dword_copy(p.rq));
+  using AccElem = decltype(typename Kind<TA>::Acc{}.x);
+  const bool extra_steps = (p.rq.act || p.rq.q) && !(kRingCarriesExtraSteps<TA, TB> && FusedSteps<AccElem, 2>::dword_copy(p.rq));
   if (!extra_steps && p.m % 256 == 0 && (p.k * ES) % 128 == 0) {
     const size_t tiles_m = p.m / 256;
     if (p.n % 256 == 0 && tiles_m * (p.n / 256) >= 200) {

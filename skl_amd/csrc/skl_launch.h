@@ -32,7 +32,10 @@ enum {
 
 /* alpha or beta in C's type. With a float in `f`, `skip_c_read` shares the 8 bytes: set on beta (by the host
  * layer, unless skl_hip_set_beta_zero_mode asked for the reference's evaluation) it lets a kernel leave C unread
- * when beta is zero. */
+ * when beta is zero - 1: except where alpha * acc is an exact zero, whose sign the old C decides; 2
+ * (SKL_C_UNTOUCHED): not even there, the old C counts as +0 (calls that do not write C either - q_only -, so that
+ * C need not exist). */
+#define SKL_C_UNTOUCHED 2u
 typedef union {
   int32_t i;
   float f;

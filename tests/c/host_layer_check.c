@@ -145,6 +145,17 @@ static void store_c(int dt, void *c, size_t i, double v) {
 static double scalar_of(int dt, skl_scalar s) { return dt == SKL_DT_I8 ? s.i : dt == SKL_DT_F64 ? s.d : s.f; }
 
 /* ------------------------------------------------------------------ plain loops over the two descriptors */
+/* A floating-point call that writes only the 8-bit copy, with beta == 0, neither writes nor reads C: the old C counts
+ * as +0 (include/skl-gfx950.h). `marked`: what the host layer put next to beta for the kernels (checked where the
+ * descriptor comes from the host layer). */
+static int c_is_unread(int dt, const skl_requant *rq, double beta, int from_host_layer, skl_scalar raw_beta, const char *who) {
+  const int unread = rq->q && rq->q_only && beta == 0 && dt != SKL_DT_I8 && dt != SKL_DT_F64 && dt != SKL_DT_F32 && dt != SKL_DT_F16H;
+  if (from_host_layer && unread != (dt != SKL_DT_I8 && dt != SKL_DT_F64 && raw_beta.fz.skip_c_read == 2)) {
+    fprintf(stderr, "FAIL: %s: beta is not marked as the call asks (C untouched: %d)\n", who, unread);
+    ++g_failures;
+  }
+  return unread;
+}
 /* The fused steps behind the alpha/beta step for element (i, j) of value v (include/skl-gfx950.h): bias, activation,
  * C unless q_only, the requantised copy, the maximum. Scales are powers of two and values small integers here, so
  * double arithmetic gives the float result exactly. */
@@ -179,9 +190,11 @@ static void gemm_over_desc(const skl_gemm_desc *d, int check, const char *who) {
       must_own(d->a, 0, (d->m1 - 1) * d->rsa1 + (d->k1 - 1) * d->csa1 + (d->m0 - 1) * d->rsa0 + (d->k0 - 1) * d->csa0, esa, who);
       must_own(d->b, 0, (d->k1 - 1) * d->rsb1 + (d->n1 - 1) * d->csb1 + (d->k0 - 1) * d->rsb0 + (d->n0 - 1) * d->csb0, esb, who);
     }
-    must_own(d->c, 0, (d->m1 - 1) * d->rsc1 + (d->n1 - 1) * d->csc1 + (d->m0 - 1) * d->rsc0 + (d->n0 - 1) * d->csc0, esc, who);
   }
   const double alpha = scalar_of(d->ta, d->alpha), beta = scalar_of(d->ta, d->beta);
+  const int c_unread = c_is_unread(d->ta, &d->rq, beta, check, d->beta, who);
+  if (check && !c_unread) /* a C that is neither written nor read need not exist */
+    must_own(d->c, 0, (d->m1 - 1) * d->rsc1 + (d->n1 - 1) * d->csc1 + (d->m0 - 1) * d->rsc0 + (d->n0 - 1) * d->csc0, esc, who);
   for (size_t I = 0; I < d->m1; ++I)
     for (size_t i = 0; i < d->m0; ++i)
       for (size_t J = 0; J < d->n1; ++J)
@@ -199,8 +212,8 @@ static void gemm_over_desc(const skl_gemm_desc *d, int check, const char *who) {
                        load_elem(d->tb, d->b, P * d->rsb1 + J * d->csb1 + p * d->rsb0 + j * d->csb0);
           }
           const size_t idx = I * d->rsc1 + J * d->csc1 + i * d->rsc0 + j * d->csc0;
-          fused_steps(d->ta, d->c, idx, I * d->m0 + i, J * d->n0 + j, beta * load_c(d->ta, d->c, idx) + alpha * acc, d->bias, d->max, &d->rq,
-                      who);
+          fused_steps(d->ta, d->c, idx, I * d->m0 + i, J * d->n0 + j, beta * (c_unread ? 0.0 : load_c(d->ta, d->c, idx)) + alpha * acc, d->bias,
+                      d->max, &d->rq, who);
         }
 }
 
@@ -209,6 +222,7 @@ static void gemm_over_canon(const skl_gemm_canon *g, int layout, const char *who
   const size_t esa = esize(g->ta), esb = esize(g->tb), esc = c_esize(g->ta);
   const size_t rmask = ((size_t)1 << g->c_row_shift) - 1, cmask = ((size_t)1 << g->c_col_shift) - 1;
   const double alpha = scalar_of(g->ta, g->alpha), beta = scalar_of(g->ta, g->beta);
+  const int c_unread = c_is_unread(g->ta, &g->rq, beta, 1, g->beta, who);
   size_t a_max = 0, b_max = 0, c_max = 0;
   ++g_launches;
   for (size_t i = 0; i < g->m; ++i)
@@ -231,21 +245,21 @@ static void gemm_over_canon(const skl_gemm_canon *g, int layout, const char *who
           const size_t i9 = g->m - 1, j9 = g->n - 1, p9 = g->k - 1;
           must_own(g->a, 0, layout == 1 ? i9 * g->a_s0 + p9 : (i9 / 64) * g->a_s1 + (i9 % 64) * g->a_s0 + p9 * g->a_sk, esa, who);
           must_own(g->b, 0, layout == 1 ? (p9 / 4) * g->b_sk + j9 * 4 + p9 % 4 : (j9 / 64) * g->b_s1 + (j9 % 64) * g->b_s0 + p9 * g->b_sk, esb, who);
-          must_own(g->c, 0, (i9 >> g->c_row_shift) * g->rsc1 + (i9 & rmask) * g->rsc0 + (j9 >> g->c_col_shift) * g->csc1 + (j9 & cmask) * g->csc0, esc, who);
+          if (!c_unread) must_own(g->c, 0, (i9 >> g->c_row_shift) * g->rsc1 + (i9 & rmask) * g->rsc0 + (j9 >> g->c_col_shift) * g->csc1 + (j9 & cmask) * g->csc0, esc, who);
           if (g_failures) return;
         }
         acc += load_elem(g->ta, g->a, ia) * load_elem(g->tb, g->b, ib);
       }
       const size_t idx = (i >> g->c_row_shift) * g->rsc1 + (i & rmask) * g->rsc0 + (j >> g->c_col_shift) * g->csc1 + (j & cmask) * g->csc0;
       if (idx > c_max) c_max = idx;
-      if (g->k == 0 && i == 0 && j == 0) must_own(g->c, 0, 0, esc, who);
-      fused_steps(g->ta, g->c, idx, i, j, beta * load_c(g->ta, g->c, idx) + alpha * acc, g->bias, g->max, &g->rq, who);
+      if (g->k == 0 && i == 0 && j == 0 && !c_unread) must_own(g->c, 0, 0, esc, who);
+      fused_steps(g->ta, g->c, idx, i, j, beta * (c_unread ? 0.0 : load_c(g->ta, g->c, idx)) + alpha * acc, g->bias, g->max, &g->rq, who);
     }
   if (g->k) {
     must_own(g->a, 0, a_max, esa, who);
     must_own(g->b, 0, b_max, esb, who);
   }
-  must_own(g->c, 0, c_max, esc, who);
+  if (!c_unread) must_own(g->c, 0, c_max, esc, who);
 }
 
 /* ------------------------------------------------------------------ the redirected GPU layer */

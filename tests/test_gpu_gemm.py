@@ -346,6 +346,7 @@ EXTRA_STEP_SHAPES = (
     (512, 768, 256, 1, "whole tiles, too few for the streaming kernel"),
     (2048, 2048, 128, 1, "streaming kernel, 256 x 128 tiles (int8 with a row-major copy; everything else: bounds-checked kernels)"),
     (2048, 9216, 128, 0, "streaming kernel, 256 x 256 tiles and a second launch of 256 x 128 on the last columns (int8)"),
+    (2048, 2048, 2560, 1, "streaming kernel, K beyond the exact fp8 kernels' range (int8 and fp8 kinds with a row-major copy)"),
     (1000, 1100, 520, 0, "ragged and large enough for padded copies: must stay on the bounds-checked kernels"),
     (16, 4096, 4096, 1, "a decode batch"),
     (40, 300, 8192, 1, "K shared between workgroups: the steps ride on the pass that adds the shares"),
@@ -397,7 +398,7 @@ def test_fused_activation_and_requantised_copy(gpu, ta, m, n, k, beta, what):
 
 
 @pytest.mark.parametrize("m,n,k,beta,what", EXTRA_STEP_SHAPES)
-@pytest.mark.parametrize("ta", ("i8", "bf16", "f8e5m2"))
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f8e4m3", "f8e5m2"))
 def test_fused_fp8_copy(gpu, ta, m, n, k, beta, what):
     """The 8-bit copy as OCP fp8 (q_format): each byte must be what the reference's fp32 -> fp8 conversion
     (skl_cvt_[sat_]f32_f8e4m3 / _f8e5m2, ref/cvt/cvt_ofp8.c:174-198, through the checker) makes of the value written to
@@ -425,7 +426,38 @@ def test_fused_fp8_copy(gpu, ta, m, n, k, beta, what):
             oq = np.arange(m)[:, None] * rsq + np.arange(n)[None, :] * csq
             codes = want_q[oq].view(np.uint8) & 0x7F
             beyond = {1: 0x7F, 2: 0x7E, 3: 0x7C, 4: 0x7B}[fmt]   # what a value past the largest becomes
-            assert np.count_nonzero(codes == beyond) > 0 and len(np.unique(codes)) > (40 if per_column else 3), tag
+            assert np.count_nonzero(codes == beyond) > 0 and len(np.unique(codes)) > (40 if per_column else 2), tag
+
+
+@pytest.mark.parametrize("ta,m,n,k,what", (
+    ("bf16", 300, 1100, 96, "bounds-checked tiles"),
+    ("f8e4m3", 2048, 2048, 2560, "streaming kernel"),
+    ("f8e5m2", 40, 300, 8192, "K shared between workgroups"),
+    ("bf16", 16, 4096, 4096, "a decode batch"),
+    ("f16", 1, 2048, 512, "M = 1"),
+))
+def test_q_only_with_beta_zero_leaves_c_untouched(gpu, ta, m, n, k, what):
+    """A floating-point call that writes only the 8-bit copy, with beta == 0, neither writes nor reads C
+    (include/skl-gfx950.h): rows of A that are all zero make exact zeros, whose sign an old C would decide - C holds
+    -1 everywhere and alpha is negative, so alpha * acc is -0 there and a kernel that looked at C would add the -0 that
+    0 * -1 is and write the fp8 code of -0 (0x80), as the call that also writes C does; an old C of +0 gives +0
+    (0x00). Everything else equals the call that also writes C, and C comes back bit for bit."""
+    rng = np.random.default_rng(m + n)
+    case = rowmajor_case(ta, m, n, k, alpha=-1.0, beta=0.0)
+    a, b, _ = case.make_inputs(int(rng.integers(1 << 30)))
+    zero_rows = sorted({0, m - 1, m // 2})
+    a.reshape(m, k)[zero_rows] = 0
+    c = np.full(m * n, -1.0, np.float32)
+    scale = np.array([0.125], np.float32)
+    for mode in MODES:
+        rq = dict(q=np.full(m * n, 0x55, np.int8), rsq=n, csq=1, scale=scale, format=2)
+        _, _, q_with_c = run_fused_gemm(gpu, "rc", case, a, b, c, None, None, mode, requant=rq)
+        got, _, q = run_fused_gemm(gpu, "rc", case, a, b, c, None, None, mode, requant=dict(rq, only=True))
+        assert np.array_equal(got.view(np.uint32), c.view(np.uint32)), (ta, what, mode)
+        q, q_with_c = q.reshape(m, n).view(np.uint8), q_with_c.reshape(m, n).view(np.uint8)
+        assert np.all(q_with_c[zero_rows] == 0x80) and np.all(q[zero_rows] == 0x00), (ta, what, mode)
+        rest = np.setdiff1d(np.arange(m), zero_rows)
+        assert np.array_equal(q[rest], q_with_c[rest]), (ta, what, mode)
 
 
 @pytest.mark.parametrize("act", (2, 3))

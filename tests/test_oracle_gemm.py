@@ -290,7 +290,10 @@ def fused_expectation(case, plain, bias, max_in, activation=0, requant=None):
     q = requant["q"].copy()
     scale = requant["scale"][None, :] if requant.get("per_column") else requant["scale"][0]
     oq = np.arange(m)[:, None] * requant["rsq"] + np.arange(n)[None, :] * requant["csq"]
-    q[oq] = requantised(want[oc], scale, requant.get("zero", 0), requant.get("format", 0))
+    values = want[oc]
+    if requant.get("only") and case.beta == 0 and not case.is_int:
+        values = np.where(values == 0, np.float32(0.0), values)   # C is not read then: an exact zero is +0 (include/skl-gfx950.h)
+    q[oq] = requantised(values, scale, requant.get("zero", 0), requant.get("format", 0))
     return want, top, q
 
 
