@@ -145,9 +145,7 @@ __device__ __forceinline__ int8_t skl_requantise(float v, float scale, int zero)
 // not) - a fused skl_cvt_[sat_]f32_f8e*.
 __device__ __forceinline__ int8_t skl_quantise(float v, float scale, int zero, int fmt) {
   if (fmt == 0) return skl_requantise(v, scale, zero);
-  const unsigned bits = __float_as_uint(__fmul_rn(v, scale));
-  const bool sat = fmt == 2 || fmt == 4;
-  return (int8_t)(fmt <= 2 ? skl_fp8::encode_ofp8<skl_fp8::E4M3>(bits, sat) : skl_fp8::encode_ofp8<skl_fp8::E5M2>(bits, sat));
+  return (int8_t)skl_fp8::encode_ofp8_hw(__fmul_rn(v, scale), skl_fp8::Ofp8Format(fmt));
 }
 // Element (row, col) of the requantised output, if there is one.
 template <typename T>

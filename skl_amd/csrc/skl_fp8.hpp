@@ -49,34 +49,32 @@ __device__ __forceinline__ unsigned encode_ofp8(unsigned bits, bool sat) {
   return sign | mag;
 }
 
-// The same conversion with the format as values instead of a type, and without a branch: for epilogues that convert
-// their accumulators in place, where one code path serves both formats (the constants are uniform across the wave)
-// and a branch per element would cost registers next to 128 live accumulators. `fmt`: 1 / 2 E4M3 without / with
-// saturation, 3 / 4 E5M2 likewise.
+// The same byte through the hardware's conversion, for epilogues that convert their accumulators in place (the
+// integer route above costs about 30 operations per element, which shows next to the matrix cores; in the
+// conversion kernels, which wait for memory, it does not). v_cvt_pk_fp8_f32 / v_cvt_pk_bf8_f32 round to nearest even
+// into the OCP codes, gradual underflow included, and never saturate: a value beyond the largest becomes the
+// format's NaN (E4M3) or infinity (E5M2) with its sign. That is the rule of ref/cvt/cvt_ofp8.c:97-172 except where
+// the rule leaves IEEE habits - every NaN is the sign-less 0x7F, E4M3's overflow without saturation drops the sign,
+// saturation ends at the largest finite code - and two selects restore those (compared with the integer route on the
+// hardware for every fp32 bit pattern and all four formats: no difference; the GEMM tests hold the copies to the
+// checker's conversion). The format comes as values, uniform across the wave, so one code path serves both.
+// `fmt`: 1 / 2 E4M3 without / with saturation, 3 / 4 E5M2 likewise.
 struct Ofp8Format {
-  int mant, bias, emin;
+  bool e5m2;
   unsigned max, overflow_sign, overflow_code;
   __host__ __device__ explicit Ofp8Format(int fmt) {
-    const bool e5 = fmt >= 3, sat = fmt == 2 || fmt == 4;
-    mant = e5 ? 2 : 3, bias = e5 ? 15 : 7, emin = e5 ? -14 : -6;
-    max = e5 ? 0x7Bu : 0x7Eu;
-    overflow_sign = (sat || e5) ? 0x80u : 0u;            // E4M3's overflow without saturation is the sign-less NaN
-    overflow_code = sat ? max : e5 ? 0x7Cu : 0x7Fu;
+    const bool sat = fmt == 2 || fmt == 4;
+    e5m2 = fmt >= 3;
+    max = e5m2 ? 0x7Bu : 0x7Eu;
+    overflow_sign = (sat || e5m2) ? 0x80u : 0u;            // E4M3's overflow without saturation is the sign-less NaN
+    overflow_code = sat ? max : e5m2 ? 0x7Cu : 0x7Fu;
   }
 };
-__host__ __device__ __forceinline__ unsigned encode_ofp8(unsigned bits, const Ofp8Format &f) {
-  const unsigned sign = (bits >> 24) & 0x80u, mag32 = bits & 0x7FFFFFFFu, field = mag32 >> 23;
-  const int e = field ? (int)field - 127 : -126;                             // fp32 subnormal: no hidden bit
-  const unsigned sig = field ? ((mag32 & 0x7FFFFFu) | 0x800000u) : mag32;
-  const int te = e > f.emin ? e : f.emin;
-  int shift = (te - f.mant) - (e - 23);
-  shift = shift > 31 ? 31 : shift;
-  unsigned q = sig >> shift;
-  const unsigned rem = sig & ((1u << shift) - 1u), half = 1u << (shift - 1);
-  q += (rem > half || (rem == half && (q & 1u))) ? 1u : 0u;
-  const unsigned mag = e < f.emin ? q : ((unsigned)(te + f.bias - 1) << f.mant) + q;   // inf / NaN: far beyond max
-  const unsigned finite = mag > f.max ? ((sign & f.overflow_sign) | f.overflow_code) : (sign | mag);
-  return mag32 > 0x7F800000u ? 0x7Fu : finite;
+__device__ __forceinline__ unsigned encode_ofp8_hw(float x, const Ofp8Format &f) {
+  const unsigned e4 = (unsigned)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false), e5 = (unsigned)__builtin_amdgcn_cvt_pk_bf8_f32(x, x, 0, false);
+  const unsigned hw = (f.e5m2 ? e5 : e4) & 0xFFu;
+  const unsigned out = (hw & 0x7Fu) > f.max ? ((hw & f.overflow_sign) | f.overflow_code) : hw;   // beyond the largest: overflow, infinity or NaN
+  return x != x ? 0x7Fu : out;
 }
 
 // OFP8 byte -> fp32 bit pattern. NaN codes give the sign-less quiet NaN.

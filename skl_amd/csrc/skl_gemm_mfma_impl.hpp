@@ -145,7 +145,7 @@ struct FusedSteps {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if constexpr (kCopyIsFp8)
-          packed |= skl_fp8::encode_ofp8(__float_as_uint(__fmul_rn((float)v[i], q_scale_j)), f8) << (8 * i);
+          packed |= skl_fp8::encode_ofp8_hw(__fmul_rn((float)v[i], q_scale_j), f8) << (8 * i);
         else
           packed |= ((unsigned)skl_requantise_int((float)v[i], q_scale_j, rq.q_zero) & 0xFFu) << (8 * i);
       }

@@ -460,6 +460,38 @@ def test_q_only_with_beta_zero_leaves_c_untouched(gpu, ta, m, n, k, what):
         assert np.array_equal(q[rest], q_with_c[rest]), (ta, what, mode)
 
 
+@pytest.mark.parametrize("ta,m,n,k,what", (
+    ("f8e4m3", 2048, 2048, 2560, "streaming kernel: four values per lane packed into a dword"),
+    ("bf16", 512, 1024, 64, "bounds-checked tiles: byte by byte"),
+))
+def test_fp8_copy_of_any_fp32_value(gpu, ta, m, n, k, what):
+    """The epilogues' fp32 -> fp8 conversion over fp32 values of every kind: with alpha = 0 and beta = 1 the value
+    written is C itself, so C can hold any bit pattern - every exponent with a spread of significands around the
+    rounding ties, both signs, zeros, subnormals, infinities, NaNs, the neighbourhood of each format's largest value,
+    and random patterns. Each byte of the copy must be the checker's conversion of what was written to C."""
+    from test_oracle_gemm import requantised
+    rng = np.random.default_rng(k)
+    case = rowmajor_case(ta, m, n, k, alpha=0.0, beta=1.0)
+    a, b, _ = case.make_inputs(3)
+    sig = np.array([0, 1, 0x7FFFFF, 0x400000, 0x400001, 0x3FFFFF, 0x100000, 0x080000, 0x0FFFFF, 0x200000, 0x600000, 0x700000,
+                    0x500000, 0x300000, 0x0FFFFE, 0x100001, 0x680000, 0x680001, 0x67FFFF], np.uint32)
+    special = (np.arange(256, dtype=np.uint32)[:, None, None] << 23 | np.array([0, 1], np.uint32)[None, :, None] << 31 | sig[None, None, :]).ravel()
+    near_max = np.concatenate([np.float32(x).view(np.uint32) + np.arange(-64, 65, dtype=np.int64).astype(np.uint32)
+                               for x in (448.0, 464.0, 480.0, 57344.0, 61440.0, 65536.0, 2.0 ** -6, 2.0 ** -9, 2.0 ** -10, 2.0 ** -14,
+                                         2.0 ** -16, 2.0 ** -17)])
+    near_max = np.concatenate([near_max, near_max | np.uint32(0x80000000)])
+    for fmt in (1, 2, 3, 4):
+        bits = rng.integers(0, 1 << 32, m * n, dtype=np.uint64).astype(np.uint32)
+        bits[:special.size] = special
+        bits[special.size:special.size + near_max.size] = near_max
+        c = bits.view(np.float32)
+        rq = dict(q=np.zeros(m * n, np.int8), rsq=n, csq=1, scale=np.array([1.0], np.float32), format=fmt)
+        got, _, q = run_fused_gemm(gpu, "rc", case, a, b, c, None, None, "device", requant=rq)
+        assert np.array_equal(q, requantised(got, np.float32(1.0), 0, fmt)), (ta, what, fmt)
+        same = ~np.isnan(c)
+        assert np.array_equal(got[same], c[same] + np.float32(0.0)), (ta, what, fmt)   # the values did arrive in the epilogue
+
+
 @pytest.mark.parametrize("act", (2, 3))
 def test_silu_and_gelu_values(gpu, act):
     """The activation alone: with alpha = 0 and beta = 1 the value it is applied to is C itself, so any fp32 value
