@@ -1232,11 +1232,11 @@ struct SequenceGuard {
 
 constexpr size_t kRingMinSlicesPerSplit = 64;  // below 8 KiB of K per row the pass over the planes costs what the split saves
 
-// The int8 streaming kernels for whole tiles also exist with the activation and requantisation steps, for a copy
-// that can be written as dwords (a quantised layer's int8 output at a quarter of C's bytes); every other call with
-// those steps goes to the bounds-checked kernels.
+// The streaming kernels for whole tiles also exist with the activation (none or ReLU) and requantisation steps, for a
+// copy that can be written as dwords (a quantised layer's 8-bit output at a quarter of C's bytes: int8 behind an
+// int32 C, fp8 behind an fp32 C); every other call with those steps goes to the bounds-checked kernels.
 template <int TA, int TB>
-constexpr bool kRingCarriesExtraSteps = TA == TB && (TA == SKL_DT_I8 || TA == SKL_DT_F8E4M3 || TA == SKL_DT_F8E5M2);
+constexpr bool kRingCarriesExtraSteps = TA == TB;   // every kind but the mixed fp8 pairings
 
 // An int32 C the streaming kernel writes 16 bytes per lane: blocks of 4 to 16 columns with contiguous rows, a
 // multiple of four rows per block, everything on 16-byte boundaries, no fused steps.

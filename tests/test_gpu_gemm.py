@@ -432,6 +432,7 @@ def test_fused_fp8_copy(gpu, ta, m, n, k, beta, what):
 @pytest.mark.parametrize("ta,m,n,k,what", (
     ("bf16", 300, 1100, 96, "bounds-checked tiles"),
     ("f8e4m3", 2048, 2048, 2560, "streaming kernel"),
+    ("f16", 2048, 2048, 128, "streaming kernel, 16-bit operands"),
     ("f8e5m2", 40, 300, 8192, "K shared between workgroups"),
     ("bf16", 16, 4096, 4096, "a decode batch"),
     ("f16", 1, 2048, 512, "M = 1"),
@@ -462,6 +463,8 @@ def test_q_only_with_beta_zero_leaves_c_untouched(gpu, ta, m, n, k, what):
 
 @pytest.mark.parametrize("ta,m,n,k,what", (
     ("f8e4m3", 2048, 2048, 2560, "streaming kernel: four values per lane packed into a dword"),
+    ("bf16", 2048, 2048, 128, "streaming kernel, 16-bit operands"),
+    ("f16", 2048, 9216, 64, "streaming kernel, 256 x 256 tiles and a second launch"),
     ("bf16", 512, 1024, 64, "bounds-checked tiles: byte by byte"),
 ))
 def test_fp8_copy_of_any_fp32_value(gpu, ta, m, n, k, what):
