@@ -181,18 +181,19 @@ SKL_GFX950_DECLARE_RCPRC(skl_gemm_f16rcprc_f16rcprc_f16rcprc_gfx950, skl_f16_t, 
  * functions") and leaves to them - the reference has no routine for either, the rules above define them here.
  * bias points to n = n1*n0 values of C's type, max to one, q_scale to n floats or one; all of them and q must be
  * memory of the same kind as C (device or host) and must not overlap C or each other; *max must not be NaN on
- * entry; q_zero lies in [-128, 127]. With q_only the call still reads C when beta is not zero (or skl_hip_set_beta_zero_mode asked for the reference's evaluation of beta * C). Members left zero
- * (e.g. by a designated initialiser that names only bias and max) switch their step off. ep == NULL: the plain GEMM. */
+ * entry; q_zero lies in [-128, 127]. With q_only the call still reads C when beta is not zero (or when
+ * skl_hip_set_beta_zero_mode asked for the reference's evaluation of beta * C). Members left zero (e.g. by a
+ * designated initialiser that names only bias and max) switch their step off. ep == NULL: the plain GEMM. */
 #define SKL_GFX950_ACT_NONE 0
 #define SKL_GFX950_ACT_RELU 1
 #define SKL_GFX950_ACT_SILU 2 /* floating-point C only */
 #define SKL_GFX950_ACT_GELU 3 /* floating-point C only */
-/* Every step off: `skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE; ep.bias = ...;` is valid C and C++. */
 #define SKL_GFX950_Q_INT8 0       /* what a byte of q holds: int8 by the rule above (default) */
 #define SKL_GFX950_Q_F8E4M3 1     /* OCP E4M3, overflow to the format's NaN like skl_cvt_f32_f8e4m3 */
 #define SKL_GFX950_Q_F8E4M3_SAT 2 /* ... saturating like skl_cvt_sat_f32_f8e4m3 */
-#define SKL_GFX950_Q_F8E5M2 3
-#define SKL_GFX950_Q_F8E5M2_SAT 4
+#define SKL_GFX950_Q_F8E5M2 3     /* OCP E5M2, overflow to infinity like skl_cvt_f32_f8e5m2 */
+#define SKL_GFX950_Q_F8E5M2_SAT 4 /* ... saturating like skl_cvt_sat_f32_f8e5m2 */
+/* Every step off: `skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE; ep.bias = ...;` is valid C and C++. */
 #define SKL_GFX950_EPILOGUE_NONE {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 typedef struct skl_gfx950_epilogue {
   const void *bias;
