@@ -345,6 +345,7 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   const int c_is_read = !(d->ta == SKL_DT_I8 && d->beta.i == 0) && !c_untouched(d);
   skl_gemm_canon h;
   char *scratch;
+  size_t flat;
   int r, c_in_place;
   if (esa > 2 || esb > 2 || M * N * K < ((size_t)1 << 18)) return DECLINED;
   memset(&h, 0, sizeof h);
@@ -364,10 +365,13 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
    * when C would otherwise travel three times (unpack, update, pack), not when an integer C with beta == 0 is only
    * packed - unless the streaming kernel takes the problem and writes such blocks 16 bytes per lane (8192^3: no
    * pack pass of 81 us). */
-  c_in_place = canonicalize_c(d, &h, 1);
-  if (c_in_place && !c_is_read) {
-    h.a = h.b = (const void *)(uintptr_t)256;
-    c_in_place = skl_hip_gemm_mfma_streams_c_quads(&h);
+  c_in_place = canonicalize_c(d, &h, 0); /* flat or in blocks of 64: the kernels' usual C */
+  if (!c_in_place && canonicalize_c(d, &h, 1)) {
+    c_in_place = 1;
+    if (!c_is_read) {
+      h.a = h.b = (const void *)(uintptr_t)256;
+      c_in_place = skl_hip_gemm_mfma_streams_c_quads(&h);
+    }
   }
   if (!c_in_place) {
     h.c = (void *)(uintptr_t)256;
@@ -381,11 +385,20 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
   if (r == TAKEN) {
     h.a = scratch, h.b = scratch + bytes_a;
     if (!c_in_place) h.c = scratch + bytes_a + bytes_b;
-    r = outcome(skl_hip_launch_realign((int)esa, M, K, d->a, d->m0, d->rsa0, d->rsa1, d->k0, d->csa0, d->csa1, scratch, kpa));
+    /* an operand whose K is flat in memory although the call describes it in blocks (the rows of the dot-product
+     * GEMM's A: groups of four k side by side) is copied as what it is */
+    if (flat_k(d->k0, d->k1, d->csa0, d->csa1, &flat))
+      r = outcome(skl_hip_launch_realign((int)esa, M, K, d->a, d->m0, d->rsa0, d->rsa1, 1, 0, flat, scratch, kpa));
+    else
+      r = outcome(skl_hip_launch_realign((int)esa, M, K, d->a, d->m0, d->rsa0, d->rsa1, d->k0, d->csa0, d->csa1, scratch, kpa));
   }
-  if (r == TAKEN)
-    r = outcome(skl_hip_launch_realign((int)esb, N, K, d->b, d->n0, d->csb0, d->csb1, d->k0, d->rsb0, d->rsb1,
-                                       scratch + bytes_a, kpb));
+  if (r == TAKEN) {
+    if (flat_k(d->k0, d->k1, d->rsb0, d->rsb1, &flat))
+      r = outcome(skl_hip_launch_realign((int)esb, N, K, d->b, d->n0, d->csb0, d->csb1, 1, 0, flat, scratch + bytes_a, kpb));
+    else
+      r = outcome(skl_hip_launch_realign((int)esb, N, K, d->b, d->n0, d->csb0, d->csb1, d->k0, d->rsb0, d->rsb1,
+                                         scratch + bytes_a, kpb));
+  }
   if (r == TAKEN && !c_in_place && c_is_read)
     r = outcome(skl_hip_launch_unpack(4, d->m0, d->n0, d->c, d->rsc0, d->csc0, d->rsc1, d->csc1, M, N, h.c, N, 1));
   if (r == TAKEN) r = gemm_fast_path(&h, fused, 1); /* the caller's C is untouched until this has launched */
@@ -396,13 +409,12 @@ static int gemm_through_copies(const skl_gemm_desc *d, int fused) {
 }
 
 /* K-packed B with more rows of A than one call of the decode-batch kernel takes (128): chunks of 128 rows, one pass
- * over B each. Up to 1024 rows that is cheaper than copying B into a layout the tile kernels read (the byte-wise
- * copy of 4096 x 11008 out of its groups of four k alone costs about 100 us). Every chunk is checked before the
- * first is launched. */
+ * over B each. Up to 256 rows that is cheaper than copying B into a layout the tile kernels read (a transpose of
+ * 32-bit groups, about one pass over B each way). Every chunk is checked before the first is launched. */
 static int k4_in_row_chunks(const skl_gemm_desc *d) {
   skl_gemm_canon g;
   int launch;
-  if (d->ta != SKL_DT_I8 || d->k0 != 4 || d->m0 != 1 || d->m1 <= 128 || d->m1 > 1024) return DECLINED;
+  if (d->ta != SKL_DT_I8 || d->k0 != 4 || d->m0 != 1 || d->m1 <= 128 || d->m1 > 256) return DECLINED;
   for (launch = 0; launch < 2; ++launch) {
     size_t i;
     /* A chunk that fails after others have run would leave C half updated: the one thing a chunk may lack, the

@@ -524,6 +524,13 @@ int skl_hip_launch_realign(int esize, size_t x, size_t k, const void *src, size_
       }
     }
   }
+  if (esize == 1 && x0 == 1 && s1 == 4 && k0 == 4 && sk0 == 1 && sk1 % 16 == 0 && k % 16 == 0 && kp == k && x % 4 == 0 &&
+      (((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
+    // K in groups of four bytes per x, the groups of neighbouring x side by side (the K-packed B of the dot-product
+    // GEMM, src/gemm/packed-gemm.md:178-219): as 32-bit elements that is a (k / 4) x x matrix with unit column
+    // stride, and the copy is its transpose - the vectorised transposing pack kernel with one block of k / 4 rows.
+    return skl_hip_launch_pack(4, k / 4, x, src, sk1 / 4, 1, k / 4, 1, dst, 1, 0, 0, kp / 4, 0);
+  }
   if (k0 > 1 && sk0 == 1 && (k0 * es) % 8 == 0 && pitch % 16 == 0 && ((uintptr_t)dst & 15) == 0 && k % k0 == 0 &&
       (((uintptr_t)src | (x0 > 1 ? s0 * es : 0) | (s1 * es) | (sk1 * es)) & 7) == 0) {
     // K in blocks whose k are contiguous: 8-byte pieces

@@ -129,6 +129,24 @@ def test_k_packed_int8_decode_batches(gpu, m):
                 assert np.array_equal(run_gemm(gpu, "dot4", case, a, b, c, mode), want), (m, n, k1, alpha, beta, mode)
 
 
+@pytest.mark.parametrize("m", (300, 600, 1100))
+def test_k_packed_int8_many_rows(gpu, m):
+    """The dot4 layout with more rows of A than the decode-batch kernels take in two passes over B: the K-packed B is
+    copied into rows contiguous in K - as 32-bit groups that is a transpose - and the tile kernels run on the copy
+    (A, K-contiguous already, is copied alongside; C is updated where it lies). Padded strides of A, B and C, alpha /
+    beta with wrap-around, both pointer modes; whole-buffer compare."""
+    rng = np.random.default_rng(900 + m)
+    for (n, k1, pad_a, pad_b, pad_c) in ((4100, 132, 16, 32, 5), (2052, 516, 48, 16, 0), (1024, 256, 0, 0, 0)):
+        for alpha, beta in ((1, 0), (0x01010101, -77)):
+            case = support.dot4_case(m, n, k1, alpha=alpha, beta=beta, rsa1=4 * k1 + pad_a, rsb1=4 * n + pad_b,
+                                     rsc1=n + pad_c)
+            a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+            c[:] = rng.integers(-2 ** 31, 2 ** 31, size=c.size)
+            want = run_oracle_gemm(case, a, b, c)
+            for mode in ("device", "host"):
+                assert np.array_equal(run_gemm(gpu, "dot4", case, a, b, c, mode), want), (m, n, k1, alpha, beta, mode)
+
+
 def _exact_int8_gemv(x, w, k, n):
     """x (k) times row-major w (k x n) in exact integer arithmetic, through fp64 BLAS in slices of K."""
     acc = np.zeros(n, np.float64)
