@@ -147,6 +147,30 @@ def _wl_small_batch(m):
     return build
 
 
+def _wl_decode_fused(m):
+    """A quantised layer at decode time: int8 in, bias, ReLU, int8 out (per-column scales), C not written."""
+    def build(lib, rng):
+        import skl_amd
+        k, n, nbuf = 4096, 11008, 8
+        w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+        x = DeviceBuffer.from_array(rand_i8(rng, m * k))
+        y = DeviceBuffer(16)  # not written
+        q = DeviceBuffer(m * n)
+        bias = DeviceBuffer.from_array(rng.integers(-1000, 1000, n).astype(np.int32))
+        scales = DeviceBuffer.from_array((rng.uniform(0.5, 2.0, n) / (74.0 * 74.0 * 64.0 * 0.4)).astype(np.float32))
+        ep = skl_amd.Epilogue(bias, None, activation=skl_amd.Epilogue.ACT_RELU, q=q, rsq=n, csq=1, q_scale=scales,
+                              q_scale_per_column=True, q_zero=-128, q_only=True)
+
+        def step(i):
+            lib.skl_gemm_fused_i8rc_i8rc_i32rc_gfx950(m, n, k, 1, x, k, 1, w[i % nbuf], n, 1, 0, y, n, 1, ep)
+
+        return dict(fn=step, bytes=k * n + m * k + m * n + 8 * n, ops=2 * m * k * n, bound="hbm", dtype="i8",
+                    keep=(w, x, y, q, bias, scales),
+                    name=f"int8 {m}x4096x11008 with bias, ReLU and requantised int8 output only (decode, batch of {m})",
+                    kernel="streaming kernel into a plane + gemm_split_reduce_kernel")
+    return build
+
+
 def wl_small_batch_bf16(lib, rng):
     """Decode with a batch of 8 against bf16 weights (90 MB): the stream over W with the matrix cores multiplying."""
     m, k, n, nbuf = 8, 4096, 11008, 4
@@ -562,6 +586,8 @@ WORKLOADS = {
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 10, 2, 64),
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 10, 2, 64),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 10, 2, 64),
+    "gemv_i8_fused_1x4096x11008": (_wl_decode_fused(1), 10, 2, 64),
+    "gemm_i8_fused_16x4096x11008": (_wl_decode_fused(16), 10, 2, 64),
     "gemm_i8_32x4096x11008": (_wl_small_batch(32), 10, 2, 64),
     "gemm_i8_64x4096x11008": (_wl_small_batch(64), 10, 2, 32),
     "gemm_i8_p4x1c_16x4096x11008": (_wl_small_batch_p4x1c(16), 10, 2, 64),

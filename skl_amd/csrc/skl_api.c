@@ -241,6 +241,34 @@ static int gemv_paths(const skl_gemm_canon *g, int launch) {
   return r;
 }
 
+/* A fused int8 call of a shape the streaming kernels take (a decode step: 1 to 16 rows): they have no fused steps,
+ * so the plain product goes to a row-major matrix in scratch memory and a second, small kernel computes
+ * beta*C + alpha*product and the steps from there - exact for integers, and a fraction of what the tile kernels
+ * take for such shapes (1 x 4096 x 11008 with bias, ReLU and int8 output: 13 against 28 us). */
+static int gemv_then_epilogue(const skl_gemm_canon *g) {
+  skl_gemm_canon h = *g;
+  void *product;
+  int r;
+  if (g->ta != SKL_DT_I8 || g->tb != SKL_DT_I8 || g->m > 16 || g->c_row_shift > 6 || g->c_col_shift > 6) return DECLINED;
+  h.c = (void *)(uintptr_t)256; /* stands for the scratch matrix while asking who would take it */
+  h.rsc0 = g->n, h.rsc1 = SKL_TE * g->n, h.csc0 = 1, h.csc1 = SKL_TE;
+  h.c_row_shift = h.c_col_shift = 6;
+  h.alpha.i = 1, h.beta.i = 0;
+  h.bias = NULL, h.max = NULL;
+  memset(&h.rq, 0, sizeof h.rq);
+  if (gemv_paths(&h, 0) != TAKEN) return DECLINED;
+  skl_hip_sequence_begin();
+  product = skl_hip_operand_scratch(g->m * g->n * 4);
+  r = product != NULL ? TAKEN : DECLINED;
+  if (r == TAKEN) {
+    h.c = product;
+    r = gemv_paths(&h, 1);
+  }
+  if (r == TAKEN) r = outcome(skl_hip_launch_gemm_epilogue(g, product)) == TAKEN ? TAKEN : FAILED; /* C is untouched until here */
+  skl_hip_sequence_end();
+  return r;
+}
+
 /* Streaming kernels, then the matrix-core tile kernels. */
 static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
   int r = DECLINED;
@@ -452,6 +480,7 @@ static int gemm_on_device(const skl_gemm_desc *d) {
     if (r == DECLINED) {
       if (canonicalize(d, &g)) {
         if (!fused) r = gemv_paths(&g, 1);
+        if (fused) r = gemv_then_epilogue(&g); /* uses the operand scratch itself: only here, on the caller's own operands */
         if (r == DECLINED) r = gemm_padded_to_tiles(&g);
         if (r == DECLINED) r = gemm_fast_path(&g, fused, 1);
         if (r == DECLINED) r = gemm_with_realigned_operands(&g, fused);

@@ -112,6 +112,37 @@ extern "C" int skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile
   }
 }
 
+// C = beta*C + alpha*P, then the fused steps (bias, activation, 8-bit copy, maximum), for a product P that another
+// kernel has left as a row-major M x N matrix of C's type in scratch memory: the pass that adds the shares of K,
+// given one share. What a streaming kernel without fused steps needs to serve a fused call (int32 C: the detour is
+// exact).
+extern "C" int skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void *product) {
+  if (g->ta != SKL_DT_I8 || g->tb != SKL_DT_I8 || g->m == 0 || g->n == 0 || !product || ((uintptr_t)g->c & 3) != 0 ||
+      ((uintptr_t)product & 3) != 0 || g->c_row_shift > 6 || g->c_col_shift > 6) {
+    skl_hip_record_error(-2, "gemm_epilogue: unsupported problem");
+    return -2;
+  }
+  MfmaArgs p;
+  p.a = p.b = nullptr;
+  p.c = (char *)g->c;
+  p.m = g->m, p.n = g->n, p.k = g->k;
+  p.a_s1 = p.a_s0 = p.a_sk = p.b_s1 = p.b_s0 = p.b_sk = 0;
+  p.rsc0 = g->rsc0, p.csc0 = g->csc0, p.rsc1 = g->rsc1, p.csc1 = g->csc1;
+  p.crs = g->c_row_shift, p.ccs = g->c_col_shift;
+  p.alpha = g->alpha, p.beta = g->beta;
+  p.bias = (const char *)g->bias, p.max = (char *)g->max;
+  p.rq = g->rq;
+  p.tiles_m = p.tiles_n = 0;
+  p.splits = 1, p.slices_per_split = 0, p.partial = (char *)product;
+  const size_t blocks = (p.m * p.n + 255) / 256;
+  if (blocks > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemm_epilogue: grid too large");
+    return -2;
+  }
+  gemm_split_reduce_kernel<int><<<(unsigned)blocks, 256, 0, skl_current_stream()>>>(p);
+  return skl_check_launch("gemm_epilogue");
+}
+
 extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
   if (!skl_hip_gemm_mfma_supported(g)) {
     skl_hip_record_error(-2, "gemm_mfma: unsupported problem");

@@ -118,6 +118,8 @@ int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g);
  * width (256 / 128) and the padded extents when that pays, else 0; the launch takes the canonical description of the
  * copies (K contiguous, rows *kp apart, k == *kp) with the true m, n and C. */
 int skl_hip_gemm_mfma_padded_plan(const skl_gemm_canon *g, size_t *mp, size_t *np, size_t *kp);
+/* C = beta*C + alpha*P and the fused steps of g, P a row-major m x n int32 matrix (int8 problems only). */
+int skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void *product);
 /* 1 when the streaming kernel would take this int8 problem where it lies and write its blocked C (4 to 16 columns
  * per block, contiguous rows) 16 bytes per lane - as cheaply as a row-major C. */
 int skl_hip_gemm_mfma_streams_c_quads(const skl_gemm_canon *g);

@@ -33,8 +33,8 @@ static int g_nranges;
 static long g_checked, g_launches;
 static int g_failures;
 /* how often each stand-in ran: the summary shows which routes of the dispatch the cases reached */
-enum { P_GENERIC, P_TILED, P_MFMA, P_PADDED, P_GEMV, P_GEMV_K4, P_ROWS, P_MFMA_ROWS, P_MFMA_ROWS_K4, P_KC, P_REALIGN, P_PACK, P_UNPACK, P_CVT, P_F4, P_SCARCE, P_COUNT };
-static const char *const kPathNames[P_COUNT] = {"any-stride", "register-tiled", "matrix-core", "padded tiles", "GEMV", "GEMV K-packed", "few rows",
+enum { P_GENERIC, P_TILED, P_MFMA, P_PADDED, P_EPILOGUE, P_GEMV, P_GEMV_K4, P_ROWS, P_MFMA_ROWS, P_MFMA_ROWS_K4, P_KC, P_REALIGN, P_PACK, P_UNPACK, P_CVT, P_F4, P_SCARCE, P_COUNT };
+static const char *const kPathNames[P_COUNT] = {"any-stride", "register-tiled", "matrix-core", "padded tiles", "epilogue pass", "GEMV", "GEMV K-packed", "few rows",
                                                 "decode batch", "decode batch K-packed", "dot-product GEMV", "operand copy", "pack", "unpack", "cvt", "4-bit weights",
                                                 "declined: no scratch"};
 static long g_path[P_COUNT];
@@ -301,6 +301,24 @@ int __wrap_skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
   EXPECT(skl_hip_gemm_mfma_supported(g), "matrix-core GEMM handed a problem it does not support");
   ++g_path[P_MFMA];
   gemm_over_canon(g, 0, "matrix-core GEMM");
+  return 0;
+}
+/* C = beta*C + alpha*product and the fused steps, the product a row-major m x n int32 matrix in scratch memory. */
+int __wrap_skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void *product) {
+  const size_t rmask = ((size_t)1 << g->c_row_shift) - 1, cmask = ((size_t)1 << g->c_col_shift) - 1;
+  const double alpha = scalar_of(g->ta, g->alpha), beta = scalar_of(g->ta, g->beta);
+  EXPECT(g->ta == SKL_DT_I8 && g->tb == SKL_DT_I8 && g->m && g->n, "epilogue pass: int8 problems only");
+  ++g_launches, ++g_path[P_EPILOGUE];
+  must_own(product, 0, g->m * g->n - 1, 4, "epilogue pass (product)");
+  must_own(g->c, 0, ((g->m - 1) >> g->c_row_shift) * g->rsc1 + ((g->m - 1) & rmask) * g->rsc0 + ((g->n - 1) >> g->c_col_shift) * g->csc1 +
+                        ((g->n - 1) & cmask) * g->csc0, 4, "epilogue pass (C)");
+  if (g_failures) return 0;
+  for (size_t i = 0; i < g->m; ++i)
+    for (size_t j = 0; j < g->n; ++j) {
+      const size_t idx = (i >> g->c_row_shift) * g->rsc1 + (i & rmask) * g->rsc0 + (j >> g->c_col_shift) * g->csc1 + (j & cmask) * g->csc0;
+      fused_steps(g->ta, g->c, idx, i, j, beta * load_c(g->ta, g->c, idx) + alpha * (double)((const int32_t *)product)[i * g->n + j], g->bias, g->max,
+                  &g->rq, "epilogue pass");
+    }
   return 0;
 }
 int __wrap_skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile_cols) {
@@ -924,7 +942,42 @@ static void run_rowmajor(int ta, size_t m, size_t n, size_t k, size_t pad_a, siz
   drop_buf(a), drop_buf(b), drop_buf(c), drop_buf(want);
 }
 
+/* A fused int8 call of a decode shape: bias, ReLU, the requantised copy (written next to C or alone) and the maximum. */
+static void run_rowmajor_fused(size_t m, size_t n, size_t k, int alpha, int beta, int q_only, const char *what) {
+  static const float kScales[4] = {0.25f, 0.5f, 1.0f, 2.0f};
+  skl_gemm_desc d, ref;
+  skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE;
+  memset(&d, 0, sizeof d);
+  d.ta = d.tb = SKL_DT_I8, d.m0 = d.n0 = d.k0 = 1, d.m1 = m, d.n1 = n, d.k1 = k;
+  d.rsa1 = k, d.csa1 = 1, d.rsb1 = n, d.csb1 = 1, d.rsc1 = n + 4, d.csc1 = 1;
+  const size_t nc = m * d.rsc1, nq = m * (n + 8);
+  buf_t a = new_buf(m * k, 1), b = new_buf(k * n, 1), c = new_buf(nc * 4, 1), want = new_buf(nc * 4, 0);
+  buf_t bias = new_buf(n * 4, 1), top = new_buf(4, 1), want_top = new_buf(4, 0), q = new_buf(nq, 1), want_q = new_buf(nq, 0), scales = new_buf(n * 4, 1);
+  for (size_t i = 0; i < m * k; ++i) store_small(SKL_DT_I8, a.ptr, i, small());
+  for (size_t i = 0; i < k * n; ++i) store_small(SKL_DT_I8, b.ptr, i, small());
+  for (size_t i = 0; i < nc; ++i) store_c(SKL_DT_I8, c.ptr, i, small());
+  for (size_t j = 0; j < n; ++j) store_c(SKL_DT_I8, bias.ptr, j, small()), ((float *)scales.ptr)[j] = kScales[rnd() % 4];
+  store_c(SKL_DT_I8, top.ptr, 0, -1000), store_c(SKL_DT_I8, want_top.ptr, 0, -1000);
+  memset(q.ptr, 0x5A, nq), memset(want_q.ptr, 0x5A, nq);
+  memcpy(want.ptr, c.ptr, c.bytes);
+  ep.bias = bias.ptr, ep.max = top.ptr, ep.activation = SKL_GFX950_ACT_RELU;
+  ep.q = (int8_t *)q.ptr, ep.rsq = n + 8, ep.csq = 1, ep.q_scale = (const float *)scales.ptr, ep.q_scale_per_column = 1, ep.q_zero = 3, ep.q_only = q_only;
+  d.a = a.ptr, d.b = b.ptr, d.c = c.ptr;
+  set_scalars(&d, alpha, beta);
+  ref = d;
+  ref.c = want.ptr, ref.bias = ep.bias, ref.max = want_top.ptr;
+  ref.rq.act = ep.activation, ref.rq.q_per_column = 1, ref.rq.q_only = q_only, ref.rq.q_zero = ep.q_zero;
+  ref.rq.q = (int8_t *)want_q.ptr, ref.rq.rsq = ep.rsq, ref.rq.csq = 1, ref.rq.q_scale = ep.q_scale;
+  gemm_over_desc(&ref, 0, "reference loops");
+  call_blocked(&d, &ep);
+  if (skl_hip_last_error() != 0) fail(skl_hip_last_error_string());
+  if (memcmp(want.ptr, c.ptr, c.bytes) != 0 || memcmp(want_q.ptr, q.ptr, nq) != 0 || memcmp(want_top.ptr, top.ptr, 4) != 0) fail(what);
+  drop_buf(a), drop_buf(b), drop_buf(c), drop_buf(want), drop_buf(bias), drop_buf(top), drop_buf(want_top), drop_buf(q), drop_buf(want_q), drop_buf(scales);
+}
+
 static int run_large_cases(void) {
+  run_rowmajor_fused(1, 4096, 1536, 1, 0, 1, "fused int8 GEMV (product into scratch, then the epilogue pass) differs");
+  run_rowmajor_fused(6, 2048, 2048, -1, 2, 0, "fused int8 decode batch (product into scratch, then the epilogue pass) differs");
   run_rowmajor(SKL_DT_I8, 1500, 2100, 120, 1, 5, 3, 2, -1, "large ragged int8 GEMM (tile-padded copies) differs");
   run_rowmajor(SKL_DT_BF16, 500, 600, 72, 8, 16, 1, 1, 1, "ragged mid-size bf16 GEMM differs");
   run_rowmajor(SKL_DT_I8, 3, 256, 100, 0, 0, 0, 1, 0, "int8 GEMM with three rows (few-rows kernel) differs");
