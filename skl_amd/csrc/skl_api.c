@@ -269,6 +269,35 @@ static int gemv_then_epilogue(const skl_gemm_canon *g) {
   return r;
 }
 
+/* The same for the K-packed B of the dot-product GEMM, which only the streaming kernels read in place (1 row, or 2
+ * to 128 rows in one pass over B). */
+static int k4_then_epilogue(const skl_gemm_desc *d) {
+  int rows;
+  for (rows = 0; rows < 2; ++rows) {
+    skl_gemm_canon g, e;
+    void *product;
+    int r;
+    if (!canonicalize_k4(d, &g, rows)) continue;
+    e = g; /* the second pass's view: the caller's C and scalars, and the fused operands */
+    e.bias = d->bias, e.max = d->max, e.rq = d->rq;
+    g.c = (void *)(uintptr_t)256; /* stands for the scratch matrix while asking */
+    g.rsc0 = g.n, g.rsc1 = SKL_TE * g.n, g.csc0 = 1, g.csc1 = SKL_TE;
+    g.alpha.i = 1, g.beta.i = 0;
+    if (!(rows ? skl_hip_gemv_mfma_rows_supported(&g, 1) : skl_hip_gemv_supported(&g, 1))) continue;
+    skl_hip_sequence_begin();
+    product = skl_hip_operand_scratch(g.m * g.n * 4);
+    r = product != NULL ? TAKEN : DECLINED;
+    if (r == TAKEN) {
+      g.c = product;
+      r = outcome(rows ? skl_hip_launch_gemv_mfma_rows(&g, 1) : skl_hip_launch_gemv(&g, 1));
+    }
+    if (r == TAKEN) r = outcome(skl_hip_launch_gemm_epilogue(&e, product)) == TAKEN ? TAKEN : FAILED;
+    skl_hip_sequence_end();
+    return r;
+  }
+  return DECLINED;
+}
+
 /* Streaming kernels, then the matrix-core tile kernels. */
 static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
   int r = DECLINED;
@@ -477,6 +506,7 @@ static int gemm_on_device(const skl_gemm_desc *d) {
     if (r == DECLINED && !fused && canonicalize_k4(d, &g, 1) && skl_hip_gemv_mfma_rows_supported(&g, 1))
       r = outcome(skl_hip_launch_gemv_mfma_rows(&g, 1));
     if (r == DECLINED && !fused) r = k4_in_row_chunks(d);
+    if (r == DECLINED && fused) r = k4_then_epilogue(d);
     if (r == DECLINED) {
       if (canonicalize(d, &g)) {
         if (!fused) r = gemv_paths(&g, 1);

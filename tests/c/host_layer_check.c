@@ -975,7 +975,42 @@ static void run_rowmajor_fused(size_t m, size_t n, size_t k, int alpha, int beta
   drop_buf(a), drop_buf(b), drop_buf(c), drop_buf(want), drop_buf(bias), drop_buf(top), drop_buf(want_top), drop_buf(q), drop_buf(want_q), drop_buf(scales);
 }
 
+/* The same on the K-packed B of the dot-product GEMM. */
+static void run_k4_fused(size_t m, size_t n, size_t k1, int alpha, int beta, int q_only, const char *what) {
+  static const float kScales[4] = {0.25f, 0.5f, 1.0f, 2.0f};
+  skl_gemm_desc d, ref;
+  skl_gfx950_epilogue_t ep = SKL_GFX950_EPILOGUE_NONE;
+  memset(&d, 0, sizeof d);
+  d.ta = d.tb = SKL_DT_I8, d.m0 = d.n0 = 1, d.k0 = 4, d.m1 = m, d.n1 = n, d.k1 = k1;
+  d.csa0 = 1, d.rsa1 = 4 * k1 + 16, d.csa1 = 4, d.rsb0 = 1, d.rsb1 = 4 * n, d.csb1 = 4, d.rsc1 = n + 2, d.csc1 = 1;
+  const size_t nc = m * d.rsc1, nq = m * (n + 8);
+  buf_t a = new_buf(m * d.rsa1, 1), b = new_buf(k1 * d.rsb1, 1), c = new_buf(nc * 4, 1), want = new_buf(nc * 4, 0);
+  buf_t bias = new_buf(n * 4, 1), top = new_buf(4, 1), want_top = new_buf(4, 0), q = new_buf(nq, 1), want_q = new_buf(nq, 0), scales = new_buf(n * 4, 1);
+  for (size_t i = 0; i < a.bytes; ++i) ((int8_t *)a.ptr)[i] = (int8_t)small();
+  for (size_t i = 0; i < b.bytes; ++i) ((int8_t *)b.ptr)[i] = (int8_t)small();
+  for (size_t i = 0; i < nc; ++i) ((int32_t *)c.ptr)[i] = small();
+  for (size_t j = 0; j < n; ++j) ((int32_t *)bias.ptr)[j] = small(), ((float *)scales.ptr)[j] = kScales[rnd() % 4];
+  *(int32_t *)top.ptr = *(int32_t *)want_top.ptr = -1000;
+  memset(q.ptr, 0x5A, nq), memset(want_q.ptr, 0x5A, nq);
+  memcpy(want.ptr, c.ptr, c.bytes);
+  ep.bias = bias.ptr, ep.max = top.ptr, ep.activation = SKL_GFX950_ACT_RELU;
+  ep.q = (int8_t *)q.ptr, ep.rsq = n + 8, ep.csq = 1, ep.q_scale = (const float *)scales.ptr, ep.q_scale_per_column = 1, ep.q_zero = -2, ep.q_only = q_only;
+  d.a = a.ptr, d.b = b.ptr, d.c = c.ptr;
+  set_scalars(&d, alpha, beta);
+  ref = d;
+  ref.c = want.ptr, ref.bias = ep.bias, ref.max = want_top.ptr;
+  ref.rq.act = ep.activation, ref.rq.q_per_column = 1, ref.rq.q_only = q_only, ref.rq.q_zero = ep.q_zero;
+  ref.rq.q = (int8_t *)want_q.ptr, ref.rq.rsq = ep.rsq, ref.rq.csq = 1, ref.rq.q_scale = ep.q_scale;
+  gemm_over_desc(&ref, 0, "reference loops");
+  call_blocked(&d, &ep);
+  if (skl_hip_last_error() != 0) fail(skl_hip_last_error_string());
+  if (memcmp(want.ptr, c.ptr, c.bytes) != 0 || memcmp(want_q.ptr, q.ptr, nq) != 0 || memcmp(want_top.ptr, top.ptr, 4) != 0) fail(what);
+  drop_buf(a), drop_buf(b), drop_buf(c), drop_buf(want), drop_buf(bias), drop_buf(top), drop_buf(want_top), drop_buf(q), drop_buf(want_q), drop_buf(scales);
+}
+
 static int run_large_cases(void) {
+  run_k4_fused(1, 1024, 264, 1, 0, 1, "fused int8 GEMV on K-packed B differs");
+  run_k4_fused(50, 1024, 264, 2, -1, 0, "fused int8 decode batch on K-packed B differs");
   run_rowmajor_fused(1, 4096, 1536, 1, 0, 1, "fused int8 GEMV (product into scratch, then the epilogue pass) differs");
   run_rowmajor_fused(6, 2048, 2048, -1, 2, 0, "fused int8 decode batch (product into scratch, then the epilogue pass) differs");
   run_rowmajor(SKL_DT_I8, 1500, 2100, 120, 1, 5, 3, 2, -1, "large ragged int8 GEMM (tile-padded copies) differs");

@@ -608,6 +608,32 @@ def test_fused_extra_steps_blocked_form_any_strides_and_refusals(gpu):
         dq.free()
 
 
+@pytest.mark.parametrize("m", (1, 16, 50))
+def test_fused_steps_on_k_packed_weights(gpu, m):
+    """A fused decode call on the K-packed B of the dot-product GEMM (src/gemm/packed-gemm.md:178-219), through the
+    blocked fused entry point with k0 = 4: the streaming kernels leave the plain product in scratch memory and a
+    second pass applies alpha / beta and the steps. C, the requantised copy and the maximum against the checker's
+    product plus the rules; padded strides, alpha / beta with wrap-around, both pointer modes, q_only."""
+    from test_oracle_gemm import fused_expectation
+    rng = np.random.default_rng(40 + m)
+    n, k1 = 4100, 132
+    for alpha, beta, only in ((1, 0, True), (0x01010101, -77, False)):
+        case = support.dot4_case(m, n, k1, alpha=alpha, beta=beta, rsa1=4 * k1 + 16, rsb1=4 * n + 32, rsc1=n + 5)
+        a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+        c[:] = rng.integers(-2 ** 31, 2 ** 31, size=c.size)
+        plain = run_oracle_gemm(case, a, b, c)
+        bias = rng.integers(-1 << 12, 1 << 12, n).astype(np.int32)
+        start = np.array([-(1 << 31)], np.int32)
+        spread = float(np.abs(plain.astype(np.float64)).max())
+        scales = (rng.uniform(0.5, 2.0, n) * 100.0 / spread).astype(np.float32)
+        for mode in MODES:
+            rq = dict(q=np.full(m * (n + 4), 0x55, np.int8), rsq=n + 4, csq=1, scale=scales, per_column=True, zero=3, only=only)
+            got, top, q = run_fused_gemm(gpu, "rcprc", case, a, b, c, bias, start, mode, activation=1, requant=rq)
+            want_c, want_top, want_q = fused_expectation(case, plain, bias, start, activation=1, requant=rq)
+            assert np.array_equal(q, want_q) and top[0] == want_top[0], (m, alpha, beta, mode)
+            assert np.array_equal(got, c if only else want_c), (m, alpha, beta, mode)
+
+
 def run_fused_gemm_expecting_refusal(gpu, case, a, b, c, activation=0, requant=None):
     before = c.copy()
     rq = requant or {}
