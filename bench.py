@@ -171,6 +171,27 @@ def _wl_decode_fused(m):
     return build
 
 
+def wl_gemv_f8_fused(lib, rng):
+    """An fp8 layer at decode time: E4M3 in, bias, saturating E4M3 out (per-column scales), C neither written nor read."""
+    import skl_amd
+    k, n, nbuf = 4096, 11008, 8
+    w = [_fp8_operand(lib, rng, k * n, "f8e4m3") for _ in range(nbuf)]
+    x = _fp8_operand(lib, rng, k, "f8e4m3")
+    y = DeviceBuffer(4 * n)
+    q = DeviceBuffer(n)
+    bias = DeviceBuffer.from_array(rng.uniform(-1, 1, n).astype(np.float32))
+    scales = DeviceBuffer.from_array(rng.uniform(0.5, 2.0, n).astype(np.float32) / 64.0)
+    ep = skl_amd.Epilogue(bias, None, q=q, rsq=n, csq=1, q_scale=scales, q_scale_per_column=True, q_only=True,
+                          q_format=skl_amd.Epilogue.Q_F8E4M3_SAT)
+
+    def step(i):
+        lib.skl_gemm_fused_f8e4m3rc_f8e4m3rc_f32rc_gfx950(1, n, k, 1.0, x, k, 1, w[i % nbuf], n, 1, 0.0, y, n, 1, ep)
+
+    return dict(fn=step, bytes=k * n + k + n + 8 * n, ops=2 * k * n, bound="hbm", dtype="f8", keep=(w, x, y, q, bias, scales),
+                name="fp8 E4M3 1x4096x11008 with bias and saturating E4M3 output only (decode)",
+                kernel="gemv_mfma_rows_kernel<fp8> + gemv_mfma_add_planes_kernel")
+
+
 def wl_small_batch_bf16(lib, rng):
     """Decode with a batch of 8 against bf16 weights (90 MB): the stream over W with the matrix cores multiplying."""
     m, k, n, nbuf = 8, 4096, 11008, 4
@@ -587,6 +608,7 @@ WORKLOADS = {
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 10, 2, 64),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 10, 2, 64),
     "gemv_i8_fused_1x4096x11008": (_wl_decode_fused(1), 10, 2, 64),
+    "gemv_f8e4m3_fused_1x4096x11008": (wl_gemv_f8_fused, 10, 2, 64),
     "gemm_i8_fused_16x4096x11008": (_wl_decode_fused(16), 10, 2, 64),
     "gemm_i8_32x4096x11008": (_wl_small_batch(32), 10, 2, 64),
     "gemm_i8_64x4096x11008": (_wl_small_batch(64), 10, 2, 32),

@@ -331,6 +331,9 @@ def test_fused_epilogue(gpu, ta, m, n, k, what):
                 if not use_bias:
                     support.assert_fp_gemm_close(case, a, b, c, got,
                                                  extra_rel=support.FP8_MFMA_REL if ta.startswith("f8") else 0.0)
+                else:  # the same kernel with and without the bias: one rounded addition apart
+                    unbiased, _ = run_fused_gemm(gpu, "rc", case, a, b, c, None, start, mode)
+                    assert np.array_equal(got, (unbiased + bias).astype(np.float32)), (what, mode)
                 if use_max:
                     assert top[0] == got.max(), (what, mode)
     # a maximum already above every element stays
