@@ -499,10 +499,13 @@ static int k4_in_row_chunks(const skl_gemm_desc *d) {
 /* 0, or nonzero when no kernel could be launched (the error is recorded). */
 static int gemm_on_device(const skl_gemm_desc *d) {
   skl_gemm_canon g;
-  const int fused = d->bias != NULL || d->max != NULL || d->rq.act != 0 || d->rq.q != NULL; /* the M = 1 kernels have no fused steps */
+  const int fused = d->bias != NULL || d->max != NULL || d->rq.act != 0 || d->rq.q != NULL;
   int r = DECLINED;
   if (d->k0 * d->k1 != 0 && d->ta <= SKL_DT_F8E5M2) {
-    if (!fused && canonicalize_k4(d, &g, 0) && skl_hip_gemv_supported(&g, 1)) r = outcome(skl_hip_launch_gemv(&g, 1));
+    if (canonicalize_k4(d, &g, 0) && skl_hip_gemv_supported(&g, 1)) { /* one row: the kernel applies fused steps itself */
+      g.bias = d->bias, g.max = d->max, g.rq = d->rq;
+      r = outcome(skl_hip_launch_gemv(&g, 1));
+    }
     if (r == DECLINED && !fused && canonicalize_k4(d, &g, 1) && skl_hip_gemv_mfma_rows_supported(&g, 1))
       r = outcome(skl_hip_launch_gemv_mfma_rows(&g, 1));
     if (r == DECLINED && !fused) r = k4_in_row_chunks(d);
@@ -510,7 +513,8 @@ static int gemm_on_device(const skl_gemm_desc *d) {
     if (r == DECLINED) {
       if (canonicalize(d, &g)) {
         if (!fused) r = gemv_paths(&g, 1);
-        if (fused) r = gemv_then_epilogue(&g); /* uses the operand scratch itself: only here, on the caller's own operands */
+        if (fused && g.m == 1 && skl_hip_gemv_supported(&g, 0)) r = outcome(skl_hip_launch_gemv(&g, 0)); /* applies the steps itself */
+        if (fused && r == DECLINED) r = gemv_then_epilogue(&g); /* uses the operand scratch itself: only here, on the caller's own operands */
         if (r == DECLINED) r = gemm_padded_to_tiles(&g);
         if (r == DECLINED) r = gemm_fast_path(&g, fused, 1);
         if (r == DECLINED) r = gemm_with_realigned_operands(&g, fused);

@@ -116,6 +116,9 @@ struct GemvArgs {
   unsigned *tickets; // floating point: one zero-initialised counter per strip ...
   float *planes;     // ... and `slabs` planes of n sums (the stream's workspace)
   unsigned tiles, slabs;
+  const char *bias;  // FUSED kernels: the steps behind alpha / beta (bias and maximum of y's type, or null) ...
+  char *max;
+  skl_requant rq;    // ... activation and 8-bit copy
 };
 
 // B is read once: a non-temporal 128-bit load.
@@ -203,7 +206,8 @@ __device__ __forceinline__ bool ordered_sum_over_slabs(float *planes, size_t pla
 // Lane pairs read 32 adjacent bytes of a row and the eight row groups of a wave sit inside each row of 16 lanes
 // (column lane = pair member + 2 * row of 16), so that the lanes that share columns are summed with DPP rotations
 // and only one partial sum per wave and column goes through LDS.
-template <int MODE, int LOADS>
+// FUSED: the thread that completes a column applies the fused steps (bias, activation, 8-bit copy, maximum) to it.
+template <int MODE, int LOADS, bool FUSED = false>
 __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
   using Md = Mode<MODE>;
   constexpr int kKPerLaneL = LOADS * Md::kKPerLoad, kKPerGroupL = kPartials * kKPerLaneL;
@@ -357,12 +361,33 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
   }
   // `total` is complete: the alpha/beta step with the old value that was asked for at the start (the initialising
   // mode reads it only now, and only where alpha * total is a zero).
+  Acc largest = skl_lowest<Acc>();  // FUSED: what this thread wrote, for the maximum
   auto finish = [&](Acc total) {
     Acc *y = yv + (tile_col0 + threadIdx.x) * p.y_s;
-    *y = y_is_read ? skl_combine(total, y_old, p.alpha, p.beta) : skl_initialise(total, y, p.alpha, p.beta);
+    Acc v = y_is_read ? skl_combine(total, y_old, p.alpha, p.beta) : skl_initialise(total, y, p.alpha, p.beta);
+    if constexpr (FUSED) {
+      const size_t j = tile_col0 + threadIdx.x;
+      if (p.bias) v = skl_add_bias(v, reinterpret_cast<const Acc *>(p.bias)[j]);
+      v = skl_activate(v, p.rq.act);
+      if (!p.rq.q_only) *y = v;
+      skl_emit_requantised(p.rq, v, 0, j);
+      if (v > largest) largest = v;
+    } else {
+      *y = v;
+    }
+  };
+  // FUSED: every thread of the workgroup comes here once it has finished what it finishes (most finish nothing);
+  // one atomic per wave that wrote something.
+  auto report_maximum = [&]() {
+    if constexpr (FUSED) {
+      if (!p.max) return;
+      const Acc best = skl_wave_max(largest);
+      if ((threadIdx.x & 63) == 0 && best > skl_lowest<Acc>()) skl_atomic_max(reinterpret_cast<Acc *>(p.max), best);
+    }
   };
   if (p.slabs == 1) {  // the strip is complete inside this workgroup
     if (owner) finish(sum);
+    report_maximum();
     return;
   }
   if constexpr (std::is_same<Acc, int>::value) {
@@ -385,6 +410,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
                                owner, sum, total) && owner)
       finish(total);
   }
+  report_maximum();
 }
 
 
@@ -1128,7 +1154,14 @@ int launch(const skl_gemm_canon *g, const Reduction &red) {
   if constexpr (!std::is_same<typename Md::Acc, int>::value) {
     if (p.slabs > 1 && !(p.planes = (float *)skl_workspace((size_t)p.slabs * p.n * sizeof(float)))) return -4;
   }
-  if (loads == 16)
+  p.bias = (const char *)g->bias, p.max = (char *)g->max;
+  p.rq = g->rq;
+  const bool fused = g->bias || g->max || g->rq.act || g->rq.q;
+  if (fused && loads == 16)
+    gemv_kernel<MODE, 16, true><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
+  else if (fused)
+    gemv_kernel<MODE, 8, true><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
+  else if (loads == 16)
     gemv_kernel<MODE, 16><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
   else
     gemv_kernel<MODE, 8><<<(unsigned)grid, kWaves * 64, 0, skl_current_stream()>>>(p);
