@@ -116,6 +116,27 @@ def wl_gemv_kc(lib, rng):
                 name="int8 GEMV 1x4096x11008, W with K contiguous ([n][k]), beta=0", kernel="gemv_kc_kernel<int8>")
 
 
+def wl_gemv_kc_fused(lib, rng):
+    """A quantised linear layer at decode time on its [out][in] weight: int8 in, bias, ReLU, int8 out, C not written."""
+    import skl_amd
+    k, n, nbuf = 4096, 11008, 8
+    w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+    x = DeviceBuffer.from_array(rand_i8(rng, k))
+    y = DeviceBuffer(16)  # not written
+    q = DeviceBuffer(n)
+    bias = DeviceBuffer.from_array(rng.integers(-1000, 1000, n).astype(np.int32))
+    scales = DeviceBuffer.from_array((rng.uniform(0.5, 2.0, n) / (74.0 * 74.0 * 64.0 * 0.4)).astype(np.float32))
+    ep = skl_amd.Epilogue(bias, None, activation=skl_amd.Epilogue.ACT_RELU, q=q, rsq=n, csq=1, q_scale=scales,
+                          q_scale_per_column=True, q_zero=-128, q_only=True)
+
+    def step(i):
+        lib.skl_gemm_fused_i8rc_i8rc_i32rc_gfx950(1, n, k, 1, x, k, 1, w[i % nbuf], 1, k, 0, y, n, 1, ep)
+
+    return dict(fn=step, bytes=k * n + k + n + 8 * n, ops=2 * k * n, bound="hbm", dtype="i8", keep=(w, x, y, q, bias, scales),
+                name="int8 1x4096x11008, W with K contiguous ([n][k]), with bias, ReLU and int8 output only (decode)",
+                kernel="gemv_kc_kernel<int8, FUSED>")
+
+
 def wl_gemv_kc_bf16(lib, rng):
     k, n, nbuf = 4096, 11008, 4
     w = [DeviceBuffer.from_array(bf16_bits(rng.normal(size=k * n) * 0.02)) for _ in range(nbuf)]
@@ -603,6 +624,7 @@ WORKLOADS = {
     "gemm_f8e4m3_mxf4_16x4096x11008": (_wl_ofp4(16, mx=True), 10, 2, 128),
     "gemv_i8_1x8192x28672": (wl_gemv_large, 10, 2, 32),
     "gemv_i8_kcontig": (wl_gemv_kc, 10, 2, 128),
+    "gemv_i8_kcontig_fused": (wl_gemv_kc_fused, 10, 2, 128),
     "gemv_bf16_kcontig": (wl_gemv_kc_bf16, 10, 2, 64),
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 10, 2, 64),
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 10, 2, 64),

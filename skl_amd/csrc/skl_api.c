@@ -513,7 +513,9 @@ static int gemm_on_device(const skl_gemm_desc *d) {
     if (r == DECLINED) {
       if (canonicalize(d, &g)) {
         if (!fused) r = gemv_paths(&g, 1);
-        if (fused && g.m == 1 && skl_hip_gemv_supported(&g, 0)) r = outcome(skl_hip_launch_gemv(&g, 0)); /* applies the steps itself */
+        /* these two apply the fused steps themselves: B with K contiguous (1 to 4 rows), B row-major (1 row) */
+        if (fused && skl_hip_gemv_kc_supported(&g)) r = outcome(skl_hip_launch_gemv_kc(&g));
+        if (fused && r == DECLINED && g.m == 1 && skl_hip_gemv_supported(&g, 0)) r = outcome(skl_hip_launch_gemv(&g, 0));
         if (fused && r == DECLINED) r = gemv_then_epilogue(&g); /* uses the operand scratch itself: only here, on the caller's own operands */
         if (r == DECLINED) r = gemm_padded_to_tiles(&g);
         if (r == DECLINED) r = gemm_fast_path(&g, fused, 1);

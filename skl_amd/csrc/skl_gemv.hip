@@ -990,6 +990,9 @@ struct GemvKcArgs {
   size_t y_row, y_s;
   size_t n, kbytes;
   skl_scalar alpha, beta;
+  const char *bias;  // FUSED kernels: the steps behind alpha / beta (bias and maximum of y's type, or null) ...
+  char *max;
+  skl_requant rq;    // ... activation and 8-bit copy
 };
 
 template <typename T>
@@ -1042,7 +1045,8 @@ __device__ __forceinline__ void dot16(const uint4 &w, const uint4 &x, typename M
   }
 }
 
-template <int MODE, int MR>
+// FUSED: the lane that writes an element applies the fused steps (bias, activation, 8-bit copy, maximum) to it.
+template <int MODE, int MR, bool FUSED = false>
 __global__ void __launch_bounds__(kKcWaves * 64) gemv_kc_kernel(GemvKcArgs p) {
   using Acc = typename Mode<MODE>::Acc;
   constexpr int kKcCols = kc_cols(MR);
@@ -1096,11 +1100,27 @@ __global__ void __launch_bounds__(kKcWaves * 64) gemv_kc_kernel(GemvKcArgs p) {
     for (int c = 0; c < kKcCols; ++c) acc[i][c] = wave_sum(acc[i][c]);
   if (lane == 0) {
     Acc *yv = reinterpret_cast<Acc *>(p.y);
+    Acc largest = skl_lowest<Acc>();
 #pragma unroll
     for (int i = 0; i < MR; ++i)
 #pragma unroll
-      for (int c = 0; c < kKcCols; ++c)
-        if (col0 + c < p.n) skl_update(acc[i][c], yv + (size_t)i * p.y_row + (col0 + c) * p.y_s, p.alpha, p.beta);
+      for (int c = 0; c < kKcCols; ++c) {
+        if (col0 + c >= p.n) continue;
+        Acc *y = yv + (size_t)i * p.y_row + (col0 + c) * p.y_s;
+        if constexpr (FUSED) {
+          Acc v = skl_beta_is_zero<Acc>(p.beta) ? skl_initialise(acc[i][c], y, p.alpha, p.beta) : skl_combine(acc[i][c], *y, p.alpha, p.beta);
+          if (p.bias) v = skl_add_bias(v, reinterpret_cast<const Acc *>(p.bias)[col0 + c]);
+          v = skl_activate(v, p.rq.act);
+          if (!p.rq.q_only) *y = v;
+          skl_emit_requantised(p.rq, v, (size_t)i, col0 + c);
+          if (v > largest) largest = v;
+        } else {
+          skl_update(acc[i][c], y, p.alpha, p.beta);
+        }
+      }
+    if constexpr (FUSED) {
+      if (p.max && largest > skl_lowest<Acc>()) skl_atomic_max(reinterpret_cast<Acc *>(p.max), largest);  // one per wave
+    }
   }
 }
 
@@ -1243,7 +1263,12 @@ int launch_kc(const skl_gemm_canon *g) {
     skl_hip_record_error(-2, "gemv: grid too large");
     return -2;
   }
-  gemv_kc_kernel<MODE, MR><<<(unsigned)grid, kKcWaves * 64, 0, skl_current_stream()>>>(p);
+  p.bias = (const char *)g->bias, p.max = (char *)g->max;
+  p.rq = g->rq;
+  if (g->bias || g->max || g->rq.act || g->rq.q)
+    gemv_kc_kernel<MODE, MR, true><<<(unsigned)grid, kKcWaves * 64, 0, skl_current_stream()>>>(p);
+  else
+    gemv_kc_kernel<MODE, MR><<<(unsigned)grid, kKcWaves * 64, 0, skl_current_stream()>>>(p);
   return skl_check_launch("gemv_kc");
 }
 

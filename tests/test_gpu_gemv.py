@@ -426,6 +426,40 @@ def test_k_contiguous_b_floating_point(gpu, ta, tb, m):
             assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
 
 
+@pytest.mark.parametrize("ta", ("i8", "bf16", "f8e4m3"))
+@pytest.mark.parametrize("m", (1, 3, 4))
+def test_k_contiguous_b_with_fused_steps(gpu, ta, m):
+    """A decode step on a linear layer's [out][in] weight with the fused steps of include/skl-gfx950.h: the kernel's
+    last stage applies bias, ReLU, the 8-bit copy (int8 behind int32, saturating E4M3 behind fp32) and the maximum.
+    int8 against the checker's product plus the rules; floating point against the plain call of the same kernel
+    (same sums, bit for bit) plus the rules. Row tails, padded strides, both pointer modes, q_only."""
+    from gpu_support import run_fused_gemm
+    from test_oracle_gemm import fused_expectation
+    rng = np.random.default_rng(70 + m)
+    for (n, k, pad) in ((11008, 4096, 0), (1037, 1040, 16), (70, 1008, 32)):
+        for beta, only in ((0, True), (1, False)):
+            case = _kc_case(ta, None, m, n, k, 2 if ta == "i8" else 0.5, beta, pad)
+            a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+            if case.is_int:
+                plain = run_oracle_gemm(case, a, b, c)
+                bias = rng.integers(-1 << 12, 1 << 12, n).astype(np.int32)
+                start = np.array([-(1 << 31)], np.int32)
+            else:
+                plain = run_gemm(gpu, "rc", case, a, b, c, "device")
+                bias = rng.uniform(-4, 4, n).astype(np.float32)
+                start = np.array([-np.inf], np.float32)
+            rows = np.arange(m)[:, None] * case.rsc1 + np.arange(n)[None, :]
+            spread = float(np.abs(plain[rows].astype(np.float64)).max())
+            scales = (rng.uniform(0.5, 2.0, n) * 100.0 / max(spread, 1e-3)).astype(np.float32)
+            rq = dict(q=np.full(m * (n + 3), 0x55, np.int8), rsq=n + 3, csq=1, scale=scales, per_column=True, zero=-5, only=only,
+                      format=0 if case.is_int else 2)
+            for mode in ("device", "host"):
+                got, top, q = run_fused_gemm(gpu, "rc", case, a, b, c, bias, start, mode, activation=1, requant=rq)
+                want_c, want_top, want_q = fused_expectation(case, plain, bias, start, activation=1, requant=rq)
+                assert np.array_equal(q, want_q) and top[0] == want_top[0], (ta, m, n, k, beta, mode)
+                assert np.array_equal(got.view(np.uint8), (c if only else want_c).view(np.uint8)), (ta, m, n, k, beta, mode)
+
+
 def _few_columns_case(ta, tb, m, n, k, alpha, beta, a_rows_contiguous, b_cols_contiguous, pad=0):
     """A tall problem with 1..8 columns: A row-major (lda = k + pad) or column-major (lda = m + pad); B column by
     column (a vector with unit stride when n == 1) or row-major; C row-major with a padded row."""
