@@ -1384,9 +1384,9 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int lay
   // rows against 11.2 / 12.9 / 14.6 us for 2 / 3 / 4 rows on the kernel that shares the byte transposes; fp8 13.7 us
   // against 17.9 us for 2 rows; bf16 20.5 us against 27.1 us. (One row: int8 12.8 against 10.3 us, fp8 13.5 against
   // 11.5 us, bf16 20.4 against 21.6 us - left to the M = 1 kernel, which uses no matrix cores.)
-  // A fused floating-point call with one row has no other streaming kernel (the M = 1 kernel has no fused steps):
-  // here it costs 13.5 / 20.4 us plus the pass over the planes for fp8 / bf16 weights of 4096 x 11008, on the tile
-  // kernels twice that.
+  // A fused floating-point call with one row that the M = 1 kernel does not take (its own conditions on B and y)
+  // still streams here rather than on the tile kernels: 13.5 / 20.4 us plus the pass over the planes for fp8 / bf16
+  // weights of 4096 x 11008, on the tile kernels twice that.
   const bool fused_single_row = mode != kI8RowMajor && g->m == 1 && (g->bias || g->max || g->rq.act || g->rq.q);
   const size_t min_rows = mode == kI8RowMajor ? kMfmaMinRowsInt8 : fused_single_row ? 1 : 2;
   if (g->m < min_rows || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;

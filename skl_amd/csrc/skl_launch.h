@@ -127,7 +127,8 @@ int skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile_cols);
 
 /* M == 1 streaming kernels: y[j*csc] = beta*y + alpha * sum_p x[p*x_sk] * B(p,j).
  * `layout`: 0 = B row-major (b_s0 == 1 within 64-blocks), 1 = K4-interleaved
- * int8 (`p4x1c`: B(p,j) at (p/4)*b_sk + j*4 + p%4). */
+ * int8 (`p4x1c`: B(p,j) at (p/4)*b_sk + j*4 + p%4). The launcher applies g's fused steps (bias, max, rq), if any,
+ * in the kernel's last stage. */
 int skl_hip_gemv_supported(const skl_gemm_canon *g, int layout);
 int skl_hip_launch_gemv(const skl_gemm_canon *g, int layout);
 /* 2 <= M <= 8 rows against a row-major int8 B: the same stream over B with the transposes shared by the rows. */
@@ -138,7 +139,8 @@ int skl_hip_launch_gemv_rows(const skl_gemm_canon *g);
  * kernels: 1 = K4-interleaved int8 B, 2 <= M <= 16. */
 int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int layout);
 int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g, int layout);
-/* 1 <= M <= 4 against a B with K contiguous (b_sk == 1): one dot product over contiguous memory per output. */
+/* 1 <= M <= 4 against a B with K contiguous (b_sk == 1): one dot product over contiguous memory per output; the
+ * launcher applies g's fused steps, if any, where the outputs are written. */
 int skl_hip_gemv_kc_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
 
