@@ -1,9 +1,10 @@
 #!/usr/bin/env python3
 """Benchmark of the GEMM / GEMV / pack / cvt hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--full] [--no-cpu] [--out FILE]
 
-Prints ONE JSON line. The headline (`value`) is the int8 GEMV decode shape
+Prints ONE compact JSON line (a few KB) and writes the full record of everything it measured to
+gpurun_out/bench_full.json (`--out`); `--full` also runs the workloads that are not benchmark configurations. The headline (`value`) is the int8 GEMV decode shape
 (1x4096 times 4096x11008, benchmark configuration 2) in GB/s of algorithmic bytes with
 all operands resident in HBM. A "step" is `config.calls_per_step` GEMV calls back to back,
 each on the next of eight weight matrices (their total size exceeds the 256 MiB last-level
@@ -12,8 +13,8 @@ around the step, not the kernel. `value` comes from the wall clock around the K 
 `roofline.achieved` from HIP events on the library's stream around the same calls.
 `roofline.configs` is the table of the other benchmark configurations (TOPS / TFLOP/s or GB/s and
 fraction of the roofline, each timed the same way), `roofline.measured_peak` what a plain read of
-the same buffers reaches on this device (and, per table row, what the matrix cores reach on register
-operands), `extra` the full records. `cpu_baseline` is the reference's scalar routine (or, where that
+the same buffers reaches on this device, `roofline.measured_peaks` all ceilings measured in the run (plain read;
+matrix cores alone on register operands). `cpu_baseline` is the reference's scalar routine (or, where that
 library was not built, the CPU checker) timed on this host for the same shape.
 """
 import argparse
@@ -83,7 +84,7 @@ def wl_gemv(lib, rng):
     def step(i):
         lib.skl_gemm_i8_i8_i32_gfx950(1, n, k, 1, x, k, w[i % nbuf], n, 0, y, n)
 
-    return dict(fn=step, bytes=k * n + k + 4 * n, ops=2 * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
+    return dict(fn=step, bytes=k * n + k + 4 * n, ops=2 * k * n, bound="hbm", dtype="i8", keep=(w, x, y), nbuf=nbuf,
                 name="int8 GEMV 1x4096x11008 (row-major W, beta=0)", kernel="gemv_kernel<int8 row-major>")
 
 
@@ -676,6 +677,7 @@ CONFIG_TABLE = {
     "C3 bf16 2048x4096x4096 beta=1": "gemm_bf16_2048x4096x4096",
     "C4 fp8 E4M3xE4M3 8192^3": "gemm_f8e4m3_8192",
     "C4 fp8 E4M3xE5M2 8192^3": "gemm_f8e4m3_f8e5m2_8192",
+    "C4 fp8 E4M3xE4M3 8192^3, K-contiguous A and B": "gemm_f8e4m3_8192_kcontig",
     "C5 f16 pack+GEMM+unpack 4096x4096x14336": "pipeline_f16_4096x4096x14336",
     "C5 pack A": "pack_e16_4096sq",
     "C5 pack B": "pack_e16_4096x14336_row_panels",
@@ -690,8 +692,9 @@ MEASURED_PEAK_OF = {"hbm": "peak_hbm_read", "i8": "peak_mfma_i8_random", "f8": "
 # HBM bytes per call from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, summed over the call's
 # kernels), FETCH_SIZE scaled by 1.998 (what it under-reads on a 64 MiB copy), WRITE_SIZE by 1.000; the runs are
 # summarised in profiles/gemv_cvt_gemm_hbm_traffic.pmc.txt.
+TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/gemv_cvt_gemm_hbm_traffic.pmc.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "gemv_i8": int((22061.0 * 1.998 + 817) * 1024),
+    "gemv_i8": int((22068.0 * 1.998 + 817) * 1024),
     "cvt_f32_f8e4m3_8192sq": int((131136.4 * 1.998 + 65536) * 1024),
     "gemm_i8_8192": int((401544.6 * 1.998 + 278814.8) * 1024),
     "copy_u32_4096sq": int((32800.9 * 1.998 + 65536) * 1024),
@@ -724,6 +727,9 @@ def measure(lib, key, steps=None, warmup=None, seed=0x5EED0000):
                    roofline=dict(bound="mfma", achieved=tops, peak=peak, unit=unit, frac=tops / peak, traffic=None,
                                  kernel=wl["kernel"], ops=wl["ops"]))
     out["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get(key)
+    if key in MEASURED_TRAFFIC_BYTES:
+        out["roofline"]["traffic_source"] = TRAFFIC_SOURCE
+    out["buffers_rotated"] = wl.get("nbuf", 1)
     out["peak_kind"] = "hbm" if wl["bound"] == "hbm" else wl["dtype"]
     for buf in _flatten(wl["keep"]):
         buf.free()
@@ -788,58 +794,41 @@ def cpu_baseline(budget_s=12.0):
     return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None)
-    ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
-    ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this library runs on one GPU; --gpus must be 1 (no multi-GPU path exists)")
+def config_rows(records, probes):
+    """`roofline.configs`: one short row per benchmark configuration - workload key, microseconds per call (HIP
+    events), achieved rate, fraction of the published peak and of the ceiling measured on this device."""
+    rows = {}
+    for label, key in CONFIG_TABLE.items():
+        r = records.get(key)
+        if r is None:
+            continue
+        if "error" in r:
+            rows[label] = {"key": key, "error": str(r["error"])[:80]}
+            continue
+        roof = r["roofline"]
+        probe = probes.get(MEASURED_PEAK_OF.get(r["peak_kind"]))
+        rows[label] = {"key": key, "us": round(r["event_ms_per_call"] * 1e3, 2), "achieved": round(roof["achieved"], 1),
+                       "unit": roof["unit"], "frac": round(roof["frac"], 4),
+                       "frac_of_measured": round(roof["achieved"] / probe["roofline"]["achieved"], 4) if probe else None}
+    return rows
 
-    lib = skl_amd.load()
-    if lib.skl_hip_init(0) != 0:
-        sys.exit("bench.py: no GPU: " + lib.skl_hip_last_error_string().decode())
-    lib.skl_hip_set_pointer_mode(1)  # device pointers only: no per-call pointer queries
 
-    head = measure(lib, args.workload, args.steps, args.warmup)
-    results = {args.workload: head}
-
-    def measured(key):
-        """The record of workload `key`, measured once; None (and an entry in `failed`) if it cannot be."""
-        if key not in results and key not in failed:
-            try:
-                results[key] = measure(lib, key)
-            except Exception as e:  # a failing extra must not hide the headline
-                failed[key] = str(e)
-        return results.get(key)
-
-    def with_measured_peak(rec):
-        """roofline of `rec` plus the ceiling measured on this device for its kind and the fraction of that."""
-        roof = dict(rec["roofline"])
-        probe = measured(MEASURED_PEAK_OF[rec["peak_kind"]]) if rec["peak_kind"] in MEASURED_PEAK_OF else None
-        if probe and not rec["workload"].startswith("peak_"):
-            roof["measured_peak"] = {"value": probe["roofline"]["achieved"], "unit": probe["roofline"]["unit"],
-                                     "workload": probe["workload"], "what": probe["name"]}
-            roof["frac_of_measured"] = roof["achieved"] / probe["roofline"]["achieved"]
-        return roof
-
-    failed = {}
-    roofline = with_measured_peak(head)
-    if not args.no_extra:
-        table = {}
-        for label, key in CONFIG_TABLE.items():
-            r = measured(key)
-            if r is None:
-                table[label] = {"error": failed[key]}
-                continue
-            roof = with_measured_peak(r)
-            table[label] = {"workload": key, "ms": r["event_ms_per_call"], "achieved": roof["achieved"], "unit": roof["unit"],
-                            "bound": roof["bound"], "frac": roof["frac"], "frac_of_measured": roof.get("frac_of_measured")}
-        roofline["configs"] = table
+def compact_result(head, records, cpu, device):
+    """The record of the final stdout line: the headline, its roofline with the measured ceilings and the table of
+    benchmark configurations, the CPU baseline and the device. Everything else goes to the results file. `records`
+    maps workload keys to measure() records (or {"error": ...})."""
+    probes = {k: r for k, r in records.items() if k.startswith("peak_") and "error" not in r}
+    roof = dict(head["roofline"])
+    probe = probes.get(MEASURED_PEAK_OF.get(head["peak_kind"]))
+    if probe and not head["workload"].startswith("peak_"):
+        roof["measured_peak"] = {"value": round(probe["roofline"]["achieved"], 1), "unit": probe["roofline"]["unit"],
+                                 "workload": probe["workload"]}
+        roof["frac_of_measured"] = round(roof["achieved"] / probe["roofline"]["achieved"], 4)
+    roof["measured_peaks"] = {k: {"value": round(r["roofline"]["achieved"], 1), "unit": r["roofline"]["unit"]}
+                              for k, r in probes.items()}
+    rows = config_rows(records, probes)
+    if rows:
+        roof["configs"] = rows
     result = {
         "metric": METRIC,
         "value": head["value"],
@@ -854,30 +843,71 @@ def main():
         "dtype": head["dtype"],
         "data": "synthetic",
         "config": {"workload": head["name"], "key": head["workload"], "resident": "HBM",
-                   "calls_per_step": head["calls_per_step"], "event_us_per_call": head["event_ms_per_call"] * 1e3,
-                   "weight_buffers_rotated": 8 if args.workload == "gemv_i8" else 1},
-        "roofline": roofline,
+                   "calls_per_step": head["calls_per_step"], "event_us_per_call": round(head["event_ms_per_call"] * 1e3, 3),
+                   "weight_buffers_rotated": head.get("buffers_rotated", 1)},
+        "roofline": roof,
     }
+    if cpu is not None:
+        result["cpu_baseline"] = cpu
+    result["device"] = device
+    return result
+
+
+def device_description(lib):
+    import ctypes
+    name, cus, mhz = ctypes.create_string_buffer(128), ctypes.c_int(0), ctypes.c_int(0)
+    lib.skl_hip_device_info(name, 128, ctypes.byref(cus), ctypes.byref(mhz))
+    return f"{name.value.decode().strip()}, {cus.value} CUs, {mhz.value} MHz"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extra", action="store_true", help="only the chosen workload: no table of configurations")
+    ap.add_argument("--full", action="store_true", help="also run every other workload (records go to the results file)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--out", default=os.path.join(ROOT, "gpurun_out", "bench_full.json"),
+                    help="file that receives the full records of everything measured")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this library runs on one GPU; --gpus must be 1 (no multi-GPU path exists)")
+
+    lib = skl_amd.load()
+    if lib.skl_hip_init(0) != 0:
+        sys.exit("bench.py: no GPU: " + lib.skl_hip_last_error_string().decode())
+    lib.skl_hip_set_pointer_mode(1)  # device pointers only: no per-call pointer queries
+
+    records = {args.workload: measure(lib, args.workload, args.steps, args.warmup)}
+    head = records[args.workload]
+
+    def measured(key):
+        if key not in records:
+            try:
+                records[key] = measure(lib, key)
+            except Exception as e:  # a failing extra must not hide the headline
+                records[key] = {"workload": key, "error": str(e)}
+
+    if head["peak_kind"] in MEASURED_PEAK_OF:
+        measured(MEASURED_PEAK_OF[head["peak_kind"]])
     if not args.no_extra:
-        extra = []
+        for key in list(CONFIG_TABLE.values()) + sorted(set(MEASURED_PEAK_OF.values())):
+            measured(key)
+    if args.full:
         for key in WORKLOADS:
-            if key == args.workload:
-                continue
-            r = measured(key)
-            if r is None:
-                extra.append({"workload": key, "error": failed[key]})
-                continue
-            extra.append({"workload": r["workload"], "name": r["name"], "value": r["value"], "unit": r["unit"],
-                          "ms_per_step": r["ms_per_step"], "steps": r["steps"], "calls_per_step": r["calls_per_step"],
-                          "event_us_per_call": r["event_ms_per_call"] * 1e3, "dtype": r["dtype"],
-                          "roofline": with_measured_peak(r)})
-        result["extra"] = extra
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline()
-    name = (lambda b: (lib.skl_hip_device_info(b, 128, None, None), b.value.decode())[1])(
-        __import__("ctypes").create_string_buffer(128))
-    result["device"] = name
-    print(json.dumps(result))
+            measured(key)
+    cpu = None if args.no_cpu else cpu_baseline()
+    result = compact_result(head, records, cpu, device_description(lib))
+    try:
+        os.makedirs(os.path.dirname(args.out), exist_ok=True)
+        with open(args.out, "w") as f:
+            json.dump({"line": result, "records": records}, f, indent=1)
+        result["full_results"] = os.path.relpath(args.out, ROOT)
+    except OSError:
+        pass
+    print(json.dumps(result, separators=(",", ":")), flush=True)
 
 
 if __name__ == "__main__":

@@ -350,7 +350,8 @@ int skl_hip_device_info(char *name, size_t name_len, int *compute_units, int *cl
   rc = skl_check_hip(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties");
   if (rc != 0) return rc;
   if (name && name_len) {
-    snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+    // Some driver stacks report no marketing name; the architecture string is always there.
+    snprintf(name, name_len, "%s (%s)", prop.name[0] ? prop.name : "unnamed AMD GPU", prop.gcnArchName);
   }
   if (compute_units) *compute_units = prop.multiProcessorCount;
   if (clock_mhz) *clock_mhz = prop.clockRate / 1000;
