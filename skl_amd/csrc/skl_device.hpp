@@ -81,6 +81,24 @@ __device__ __forceinline__ double skl_initialise(double acc, const double *c, sk
   return __dadd_rn(__longlong_as_double((long long)sign), x);
 }
 
+// The same in two steps, for kernels in which a lane writes many elements: a load that sits between two stores -
+// taken or not - makes the second store wait for the first to complete (one memory round trip per element). Such a
+// kernel first asks, for a batch of elements, whether any of them needs its old C at all, requests those values
+// together if so (a rare, wave-uniform branch), and then writes the batch. The old value matters only where
+// alpha*acc is the negative zero: (+0) + (+-0) is +0 whatever the sign of beta*c.
+__device__ __forceinline__ bool skl_initialise_needs_c(int, skl_scalar, skl_scalar) { return false; }
+__device__ __forceinline__ bool skl_initialise_needs_c(float acc, skl_scalar alpha, skl_scalar beta) {
+  return __float_as_uint(__fmul_rn(alpha.f, acc)) == 0x80000000u && beta.fz.skip_c_read != SKL_C_UNTOUCHED;
+}
+__device__ __forceinline__ int skl_initialise_with(int acc, int, skl_scalar alpha, skl_scalar) {
+  return (int)((unsigned)alpha.i * (unsigned)acc);
+}
+// `old`: the old C where skl_initialise_needs_c() said so, anything finite (+0) elsewhere.
+__device__ __forceinline__ float skl_initialise_with(float acc, float old, skl_scalar alpha, skl_scalar beta) {
+  const float x = __fmul_rn(alpha.f, acc);
+  return x == 0.0f ? __fadd_rn(__uint_as_float((__float_as_uint(old) ^ __float_as_uint(beta.f)) & 0x80000000u), x) : x;
+}
+
 template <typename T>
 __device__ __forceinline__ void skl_update(T acc, T *c, skl_scalar alpha, skl_scalar beta) {
   *c = skl_beta_is_zero<T>(beta) ? skl_initialise(acc, c, alpha, beta) : skl_combine(acc, *c, alpha, beta);

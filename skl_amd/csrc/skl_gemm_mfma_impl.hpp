@@ -105,14 +105,28 @@ struct FusedSteps {
   __host__ __device__ static bool dword_copy(const skl_requant &r) {
     return r.q && r.act <= 1 && (r.q_fmt != 0) == kCopyIsFp8 && r.csq == 1 && (r.rsq & 3) == 0 && ((uintptr_t)r.q & 3) == 0;
   }
-  __device__ __forceinline__ void column(size_t c) {
-    col = c;
-    if (bias) bias_j = bias[c];
-    if constexpr (EXTRA >= 2) q_scale_j = rq.q_scale[rq.q_per_column ? c : 0];
+  // What the steps need to know about column c, fetched ahead of the stores (a load issued behind a store has to
+  // wait for that store's acknowledgement before its value can be used) ...
+  struct Column {
+    T bias;
+    float q_scale;
+  };
+  __device__ __forceinline__ Column fetch(size_t c) const {
+    Column k{T(0), 0.0f};
+    if (bias) k.bias = bias[c];
+    if constexpr (EXTRA >= 2) k.q_scale = rq.q_scale[rq.q_per_column ? c : 0];
     if constexpr (EXTRA == 1) {
-      if (rq.q) q_scale_j = rq.q_scale[rq.q_per_column ? c : 0];
+      if (rq.q) k.q_scale = rq.q_scale[rq.q_per_column ? c : 0];
     }
+    return k;
   }
+  // ... and made current.
+  __device__ __forceinline__ void column(size_t c, const Column &k) {
+    col = c;
+    bias_j = k.bias;
+    q_scale_j = k.q_scale;
+  }
+  __device__ __forceinline__ void column(size_t c) { column(c, fetch(c)); }
   __device__ __forceinline__ T apply(T v) {
     if (bias) v = skl_add_bias(v, bias_j);
     if constexpr (EXTRA == 1) v = skl_activate(v, rq.act);
@@ -427,6 +441,135 @@ __device__ __forceinline__ auto read_frag(const char *tile, int row0, int kb) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// The epilogue of both kernels: one wave writes its MI x NI blocks of 32 x 32, lane l of a block holding column
+// l % 32 and rows 8 * (r / 4) + 4 * (l / 32) + r % 4 in register r, as C = beta*C + alpha*acc followed by the fused
+// steps. C is written once and not read again: non-temporal stores keep it out of the operands' caches.
+//
+// What decides the time is how the wave's loads and stores follow each other. On this target one counter covers
+// both, in issue order, so the value of a load cannot be used before every store issued in front of it has been
+// acknowledged - and under the write burst of a whole chip ending its tiles together that takes microseconds.
+// Hence: (1) when C is not read (beta == 0, and no element is the one case below) the 16 * MI * NI stores of a
+// lane go out with no load between them - the columns' bias values and scales are fetched first; (2) when C is
+// read, the old values of block b + kAhead are requested before block b is stored, so a wait only ever covers
+// loads that were issued in front of the stores still in flight.
+// beta == 0 in floating point reads C only where alpha*acc is the negative zero (skl_initialise_needs_c); whether
+// any element of the wave's tile is one is decided once, for the whole wave, before the first store.
+// CHECK: rows / columns beyond p.m / p.n are left alone.
+// ---------------------------------------------------------------------------
+template <int MI, int NI, bool CHECK, int EXTRA, typename Acc>
+__device__ __forceinline__ void write_wave_tile(const MfmaArgs &p, const Acc (&acc)[MI][NI], size_t row0, size_t col0) {
+  using AccElem = decltype(Acc{}.x);
+  using Steps = FusedSteps<AccElem, EXTRA>;
+  constexpr int kBlocks = MI * NI;            // block b: j = b / MI, i = b % MI (a column strip at a time)
+  constexpr int kAhead = kBlocks < 2 ? 1 : 2;
+  // The lane index from the execution mask rather than from threadIdx: nothing the epilogue needs is then computed
+  // in front of the main loop and held in a vector register across it (the loop uses every one of them).
+  const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  AccElem *c = reinterpret_cast<AccElem *>(p.c);
+  const size_t rmask = (size_t(1) << p.crs) - 1, cmask = (size_t(1) << p.ccs) - 1;
+  const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
+  bool read_c = !init;
+  if constexpr (!std::is_same<AccElem, int>::value) {
+    if (init) {
+      // alpha through a copy the compiler cannot identify with p.alpha: the products of this test are then not
+      // kept (all 16 * MI * NI of them, spilled) for the stores below, which multiply again.
+      skl_scalar alpha = p.alpha;
+      asm volatile("" : "+s"(alpha.i));
+      bool need = false;
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) need |= skl_initialise_needs_c(acc[i][j][r], alpha, p.beta);
+      read_c = __builtin_amdgcn_ballot_w64(need) != 0;
+    }
+  }
+  auto col_of = [&](int j) { return col0 + (size_t)j * 32 + (lane & 31); };
+  // first of the four consecutive rows of register group g (all in one block of C: blocks have a multiple of 4 rows)
+  auto first_row = [&](int i, int g) { return row0 + (size_t)i * 32 + g * 8 + (lane >> 5) * 4; };
+  auto inside = [&](int j, int i, int r) { return !CHECK || (col_of(j) < p.n && first_row(i, r >> 2) + (r & 3) < p.m); };
+  // The four row groups of block (i, j): where the first row of each starts.
+  struct Where {
+    AccElem *out[4];
+  };
+  auto where = [&](int j, int i) {
+    // A zero the compiler cannot see through, new at every use: the addresses of a block are then computed where
+    // the block is written and not, all 16 * MI * NI of them, ahead of the first block (which spills half of them).
+    unsigned opaque = 0;
+    asm volatile("" : "+s"(opaque));
+    const size_t col = col_of(j) + opaque, col_off = (col >> p.ccs) * p.csc1 + (col & cmask) * p.csc0;
+    Where w;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const size_t row = first_row(i, g);
+      w.out[g] = c + (row >> p.crs) * p.rsc1 + (row & rmask) * p.rsc0 + col_off;
+    }
+    return w;
+  };
+  Steps fused(p);
+  typename Steps::Column columns[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) columns[j] = (!CHECK || col_of(j) < p.n) ? fused.fetch(col_of(j)) : typename Steps::Column{AccElem(0), 0.0f};
+
+  // Block B. MODE 0: C is not read; 1: with the old values `old` (C is updated, or beta == 0 and they decide the sign of zeros).
+  // (Block numbers are compile-time constants throughout, so that the buffers of old values stay in registers.)
+  auto write_block = [&](auto mode, auto bc, const AccElem (&old)[16]) {
+    constexpr int MODE = decltype(mode)::value, B = decltype(bc)::value;
+    constexpr int j = B / MI, i = B % MI;
+    fused.column(col_of(j), columns[j]);
+    const Where w = where(j, i);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      AccElem four[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int r = 4 * g + q;
+        four[q] = AccElem(0);
+        if (inside(j, i, r)) {
+          AccElem v;
+          if constexpr (MODE == 0) v = skl_initialise_with(acc[i][j][r], AccElem(0), p.alpha, p.beta);
+          if constexpr (MODE == 1) {  // one path for both ways of using the old value: a select per element
+            const AccElem vi = skl_initialise_with(acc[i][j][r], old[r], p.alpha, p.beta), vc = skl_combine(acc[i][j][r], old[r], p.alpha, p.beta);
+            v = init ? vi : vc;
+          }
+          four[q] = fused.put(v, w.out[g] + q * p.rsc0, first_row(i, g) + q);
+        }
+      }
+      fused.rows4(four, first_row(i, g));
+    }
+    __builtin_amdgcn_sched_barrier(0);  // a block at a time: the addresses of later blocks are not computed (and held) early
+  };
+  // The blocks in order, block B + kAhead requested before block B is written.
+  auto update_blocks = [&](auto mode) {
+    AccElem old[kAhead + 1][16];
+    auto request = [&](auto bc) {
+      constexpr int B = decltype(bc)::value;
+      if constexpr (B < kBlocks) {
+        constexpr int j = B / MI, i = B % MI;
+        const Where w = where(j, i);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) old[B % (kAhead + 1)][r] = inside(j, i, r) ? w.out[r >> 2][(r & 3) * p.rsc0] : AccElem(0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    [&]<int... Bs>(std::integer_sequence<int, Bs...>) { (request(std::integral_constant<int, Bs>{}), ...); }(std::make_integer_sequence<int, kAhead>{});
+    [&]<int... Bs>(std::integer_sequence<int, Bs...>) {
+      ((request(std::integral_constant<int, Bs + kAhead>{}), write_block(mode, std::integral_constant<int, Bs>{}, old[Bs % (kAhead + 1)])), ...);
+    }(std::make_integer_sequence<int, kBlocks>{});
+  };
+  if (!read_c) {
+    const AccElem none[16] = {};
+    [&]<int... Bs>(std::integer_sequence<int, Bs...>) {
+      (write_block(std::integral_constant<int, 0>{}, std::integral_constant<int, Bs>{}, none), ...);
+    }(std::make_integer_sequence<int, kBlocks>{});
+  } else {
+    update_blocks(std::integral_constant<int, 1>{});
+  }
+  fused.finish();
+}
+
 // Tile index of a workgroup. Consecutive workgroup ids go to different XCDs
 // (eight of them, each with its own L2), so ids are first regrouped per XCD into
 // contiguous ranges, then walked in column-major groups of kGroupM tile rows so
@@ -457,7 +600,6 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
   constexpr int FRB = KB / 2;                   // fragment bytes per lane
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
   constexpr int MI = WM / 32, NI = WN / 32;     // MFMA blocks per wave
-  constexpr int kEpilogueBatch = MI < 2 ? MI : 2;  // blocks whose old C values are requested together
   using TileA = Tile<ES, BM, A_KC, NT>;
   using TileB = Tile<ES, BN, B_KC, NT>;
   constexpr int kStage = TileA::kBytes + TileB::kBytes;
@@ -468,7 +610,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
   const unsigned tiles = p.tiles_m * p.tiles_n, split = blockIdx.x / tiles;
   tile_of_block(blockIdx.x % tiles, p.tiles_m, p.tiles_n, tm, tn);
   const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;  // the wave index as a scalar: nothing derived from it occupies a vector register across the main loop
   const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
 
   Loader<ES, BM, A_KC, NT> la;
@@ -569,56 +711,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
     }
     return;
   }
-  // Epilogue. When C is
-  // updated, the old values of kEpilogueBatch blocks are all requested before the first of them is used
-  // (a load behind a store that may alias it would wait for that store: one exposed memory latency per
-  // element). C is written once and not read again: non-temporal stores keep it out of the operands' caches.
-  AccElem *c = reinterpret_cast<AccElem *>(p.c);
-  const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
-  FusedSteps<AccElem, EXTRA ? 1 : 0> fused(p);
-#pragma unroll
-  for (int j = 0; j < NI; ++j) {
-    const size_t col = n0 + wn + j * 32 + (lane & 31);
-    if (GUARDED && col >= p.n) continue;
-    fused.column(col);
-    const size_t col_off = (col >> p.ccs) * p.csc1 + (col & ((size_t(1) << p.ccs) - 1)) * p.csc0;
-#pragma unroll
-    for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
-      AccElem *out[kEpilogueBatch][4];
-#pragma unroll
-      for (int i = 0; i < kEpilogueBatch; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block (blocks have a multiple of 4 rows)
-          out[i][g] = c + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 + col_off;
-        }
-      auto row_of = [&](int i, int r) { return m0 + wm + (i0 + i) * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); };
-      auto in_range = [&](int i, int r) { return !GUARDED || row_of(i, r) < p.m; };
-      if (init) {
-#pragma unroll
-        for (int i = 0; i < kEpilogueBatch; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            if (in_range(i, r)) {
-              AccElem *dst = out[i][r >> 2] + (r & 3) * p.rsc0;
-              fused.put(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst, row_of(i, r));
-            }
-      } else {
-        AccElem old[kEpilogueBatch][16];
-#pragma unroll
-        for (int i = 0; i < kEpilogueBatch; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) old[i][r] = in_range(i, r) ? out[i][r >> 2][(r & 3) * p.rsc0] : (AccElem)0;
-#pragma unroll
-        for (int i = 0; i < kEpilogueBatch; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            if (in_range(i, r))
-              fused.put(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][r >> 2] + (r & 3) * p.rsc0, row_of(i, r));
-      }
-    }
-  }
-  fused.finish();
+  write_wave_tile<MI, NI, GUARDED, EXTRA ? 1 : 0>(p, acc, m0 + wm, n0 + wn);
 }
 
 // ===========================================================================
@@ -884,7 +977,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   const unsigned tiles = p.tiles_m * p.tiles_n, split = blockIdx.x / tiles;
   tile_of_block(blockIdx.x % tiles, p.tiles_m, p.tiles_n, tm, tn);
   const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;  // the wave index as a scalar: nothing derived from it occupies a vector register across the main loop
   const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
 
   LA la;
@@ -1124,69 +1217,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
     }
     return;
   }
-  // Epilogue, as in the kernel above: old values requested kEpilogueBatch blocks at a time, non-temporal stores.
-  AccElem *c = reinterpret_cast<AccElem *>(p.c);
-  const bool init = skl_beta_is_zero<AccElem>(p.beta);  // C is initialised, not updated
-  FusedSteps<AccElem, EXTRA> fused(p);
-#pragma unroll
-  for (int j = 0; j < NI; ++j) {
-    const size_t col = n0 + wn + j * 32 + (lane & 31);
-    if (EDGE && col >= p.n) continue;
-    fused.column(col);
-    const size_t col_off = (col >> p.ccs) * p.csc1 + (col & ((size_t(1) << p.ccs) - 1)) * p.csc0;
-#pragma unroll
-    for (int i0 = 0; i0 < MI; i0 += kEpilogueBatch) {
-      AccElem *out[kEpilogueBatch][4];
-      size_t first_row[kEpilogueBatch][4];
-#pragma unroll
-      for (int i = 0; i < kEpilogueBatch; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const size_t row = m0 + wm + (i0 + i) * 32 + g * 8 + (lane >> 5) * 4;  // four consecutive rows, all in one block (blocks have a multiple of 4 rows)
-          first_row[i][g] = row;
-          out[i][g] = c + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 + col_off;
-        }
-      auto inside = [&](int i, int r) { return !EDGE || first_row[i][r >> 2] + (r & 3) < p.m; };
-      // Four consecutive rows at a time: what put() wrote goes on to the requantised copy (rows4) while it is
-      // still in registers.
-      if (init) {
-#pragma unroll
-        for (int i = 0; i < kEpilogueBatch; ++i)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            AccElem four[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const int r = 4 * g + q;
-              AccElem *dst = out[i][g] + q * p.rsc0;
-              four[q] = inside(i, r) ? fused.put(skl_initialise(acc[i0 + i][j][r], dst, p.alpha, p.beta), dst, first_row[i][g] + q) : AccElem(0);
-            }
-            fused.rows4(four, first_row[i][g]);
-          }
-      } else {
-        AccElem old[kEpilogueBatch][16];
-#pragma unroll
-        for (int i = 0; i < kEpilogueBatch; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) old[i][r] = inside(i, r) ? out[i][r >> 2][(r & 3) * p.rsc0] : AccElem(0);
-#pragma unroll
-        for (int i = 0; i < kEpilogueBatch; ++i)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            AccElem four[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const int r = 4 * g + q;
-              four[q] = inside(i, r) ? fused.put(skl_combine(acc[i0 + i][j][r], old[i][r], p.alpha, p.beta), out[i][g] + q * p.rsc0,
-                                                 first_row[i][g] + q)
-                                     : AccElem(0);
-            }
-            fused.rows4(four, first_row[i][g]);
-          }
-      }
-    }
-  }
-  fused.finish();
+  write_wave_tile<MI, NI, EDGE, EXTRA>(p, acc, m0 + wm, n0 + wn);
 }
 
 // C = beta*C + alpha * (sum of the splits' planes, in split order), then the fused steps: the second
