@@ -734,6 +734,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaAr
 // ===========================================================================
 constexpr int kRingSlice = 64;   // bytes of K per stage
 constexpr int kRingStages = 4;
+// Stages of the ring for tiles of BN columns. The kernel's load schedule is written for any even number of stages;
+// four it is for both tile widths: six stages for the 256 x 128 tile (144 KiB; its slices take half the time, so
+// the same number of slices ahead is half the time ahead) measured no faster - bf16 2048 x 4096 x 4096 without its
+// epilogue 75 us against 71-74 us - i.e. that kernel does not wait for its loads.
+constexpr int ring_stages(int /*bn*/) { return kRingStages; }
 
 template <int ES, bool KC, int ROWS, int NS = kRingStages>
 struct STile {
@@ -917,7 +922,8 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   using Frag = typename M::Frag;
   using Acc = typename KA::Acc;
   using AccElem = decltype(Acc{}.x);
-  constexpr int SB = kRingSlice, STAGES = kRingStages;
+  constexpr int SB = kRingSlice, STAGES = ring_stages(BN);
+  static_assert(STAGES % 2 == 0, "pair loads fill two neighbouring stages");
   constexpr int ES = KA::ES, KB = KA::KB, FRB = KB / 2;
   // Eight waves: 2 x 4 blocks of 128 x 64 on a 256 x 256 tile, 4 x 2 blocks of 64 x 64 on a 256 x 128 one.
   constexpr int BM = 256, WAVES = 8, WAVES_N = BN == 256 ? 4 : 2, WAVES_M = WAVES / WAVES_N;
@@ -936,7 +942,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   // partner, and measured slower.)
   constexpr int NSA = STAGES, NSB = STAGES;
   constexpr int kExtra = kSteps == 1 ? 1 : 0;
-  constexpr int kEachAhead = 3 + kExtra, kPairAhead = 2 + kExtra;
+  constexpr int kEachAhead = STAGES - 1 + kExtra, kPairAhead = STAGES - 2 + kExtra;
   constexpr int kPairU = kPairAhead & 1;             // parity of the slices that issue pair loads
   constexpr int kPairsPrologue = (kPairU + kPairAhead) / 2;
   using LA = SLoader<ES, A_KC, WAVES, BM, NSA>;
@@ -956,9 +962,22 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   //   kExtra = 0: s even -> both from s-2: slice s-1 (odd, kEach).  s odd -> pairs from s-1: its kEach.
   //   kExtra = 1: s even -> both from s-3: slices s-2 (kEach) and s-1 (pairs + kEach).
   //               s odd  -> pairs from s-2: its kEach, and slice s-1 (kEach).
+  // In general (slice s of parity U, every-slice loads kEachAhead = kPairAhead + 1 slices ahead): the data of slice
+  // s+1 was requested in slice s - kPairAhead (every-slice loads; pair loads too when s is even) or, for pair loads
+  // with s odd, first thing in slice s + 1 - kPairAhead. Younger than that: for even s the loads of the
+  // kPairAhead - 1 slices s - kPairAhead + 1 .. s - 1; for odd s the every-slice loads of slice s + 1 - kPairAhead
+  // and the loads of the kPairAhead - 2 slices after it; and what slice s has issued in front of its barrier.
   constexpr int kPreOfU[2] = {ceil_div(kPre * kLoadsOfU[0], kSlots), ceil_div(kPre * kLoadsOfU[1], kSlots)};
-  constexpr int kInFlightOfU[2] = {(kExtra ? 2 * kEach + kPairs : kEach) + kPreOfU[0],
-                                   (kExtra ? 2 * kEach : kEach) + kPreOfU[1]};
+  constexpr auto younger = [](int u, const int (&loads)[2], int each, int pair_ahead) {
+    int n = u == 0 ? 0 : each;
+    for (int d = 1; d <= pair_ahead - 1 - u; ++d) n += loads[(u + d) % 2];
+    return n;
+  };
+  constexpr int kInFlightOfU[2] = {younger(0, kLoadsOfU, kEach, kPairAhead) + kPreOfU[0],
+                                   younger(1, kLoadsOfU, kEach, kPairAhead) + kPreOfU[1]};
+  static_assert(STAGES != 4 || (kInFlightOfU[0] == (kExtra ? 2 * kEach + kPairs : kEach) + kPreOfU[0] &&
+                                kInFlightOfU[1] == (kExtra ? 2 * kEach : kEach) + kPreOfU[1]),
+                "the four-stage counts, as derived by hand above");
   static_assert(kInFlightOfU[0] < 64 && kInFlightOfU[1] < 64, "vmcnt is a 6-bit counter");
 
   using RA = FragReader<ES, A_KC, FRB, KB, BM, NSA, MI>;
@@ -1067,8 +1086,9 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
             const size_t s = s0 + U;
             const size_t fill_slice = s + kEachAhead < slices ? s + kEachAhead : slices - 1;  // every-slice operands
             const size_t fill_pair = (s + kPairAhead) / 2 < pairs ? (s + kPairAhead) / 2 : pairs - 1;  // pair operands (s of parity kPairU)
-            const int cur_a = (int)(s % NSA), nxt_a = (int)((s + 1) % NSA), cur_b = (int)(s % NSB), nxt_b = (int)((s + 1) % NSB);
-            const int fill_a = (int)((s + (A_KC ? kPairAhead : kEachAhead)) % NSA), fill_b = (int)((s + (B_KC ? kPairAhead : kEachAhead)) % NSB);
+            const unsigned s32 = (unsigned)s;  // stage numbers from the low 32 bits: K / 64 fits, and a 32-bit remainder is a few scalar instructions
+            const int cur_a = (int)(s32 % NSA), nxt_a = (int)((s32 + 1) % NSA), cur_b = (int)(s32 % NSB), nxt_b = (int)((s32 + 1) % NSB);
+            const int fill_a = (int)((s32 + (A_KC ? kPairAhead : kEachAhead)) % NSA), fill_b = (int)((s32 + (B_KC ? kPairAhead : kEachAhead)) % NSB);
             [&]<int... KSs>(std::integer_sequence<int, KSs...>) {
               (
                   [&](auto ksc) {
@@ -1284,7 +1304,7 @@ int launch_ring(const MfmaArgs &args) {
   if constexpr (TA == SKL_DT_I8 && TB == SKL_DT_I8 && A_KC && B_KC && !EDGE && EXTRA == 0 && !CQUADS) {  // what copies of blocked operands look like
     if (c_in_row_quads(args)) return launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 0, true>(args);
   }
-  constexpr int lds = kRingStages * (256 + BN) * kRingSlice;
+  constexpr int lds = ring_stages(BN) * (256 + BN) * kRingSlice;
   auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE, EXTRA, CQUADS>;
   static bool configured = false;
   if (!configured) {
