@@ -99,6 +99,16 @@ __device__ __forceinline__ float skl_initialise_with(float acc, float old, skl_s
   return x == 0.0f ? __fadd_rn(__uint_as_float((__float_as_uint(old) ^ __float_as_uint(beta.f)) & 0x80000000u), x) : x;
 }
 
+// skl_initialise_with() for an element that does not need its old C (skl_initialise_needs_c() false: the product is
+// not the negative zero, or C counts as +0): a product that is a zero takes the sign (+0) + (+-0) has, which adding
+// the zero of beta's sign yields; every other value is unchanged by that sum.
+__device__ __forceinline__ int skl_initialise_plain(int acc, skl_scalar alpha, skl_scalar) {
+  return (int)((unsigned)alpha.i * (unsigned)acc);
+}
+__device__ __forceinline__ float skl_initialise_plain(float acc, skl_scalar alpha, skl_scalar beta) {
+  return __fadd_rn(__uint_as_float(__float_as_uint(beta.f) & 0x80000000u), __fmul_rn(alpha.f, acc));
+}
+
 template <typename T>
 __device__ __forceinline__ void skl_update(T acc, T *c, skl_scalar alpha, skl_scalar beta) {
   *c = skl_beta_is_zero<T>(beta) ? skl_initialise(acc, c, alpha, beta) : skl_combine(acc, *c, alpha, beta);

@@ -513,7 +513,8 @@ __device__ __forceinline__ void write_wave_tile(const MfmaArgs &p, const Acc (&a
 #pragma unroll
   for (int j = 0; j < NI; ++j) columns[j] = (!CHECK || col_of(j) < p.n) ? fused.fetch(col_of(j)) : typename Steps::Column{AccElem(0), 0.0f};
 
-  // Block B. MODE 0: C is not read; 1: with the old values `old` (C is updated, or beta == 0 and they decide the sign of zeros).
+  // Block B. MODE 0: C is not read; 1: with the old values `old` (C is updated, or beta == 0 and they decide the sign of
+  // zeros); 2: C is not read and there is no fused step (no bias, no maximum, no copy).
   // (Block numbers are compile-time constants throughout, so that the buffers of old values stay in registers.)
   auto write_block = [&](auto mode, auto bc, const AccElem (&old)[16]) {
     constexpr int MODE = decltype(mode)::value, B = decltype(bc)::value;
@@ -529,12 +530,17 @@ __device__ __forceinline__ void write_wave_tile(const MfmaArgs &p, const Acc (&a
         four[q] = AccElem(0);
         if (inside(j, i, r)) {
           AccElem v;
-          if constexpr (MODE == 0) v = skl_initialise_with(acc[i][j][r], AccElem(0), p.alpha, p.beta);
+          if constexpr (MODE == 0 || MODE == 2) v = skl_initialise_plain(acc[i][j][r], p.alpha, p.beta);
           if constexpr (MODE == 1) {  // one path for both ways of using the old value: a select per element
             const AccElem vi = skl_initialise_with(acc[i][j][r], old[r], p.alpha, p.beta), vc = skl_combine(acc[i][j][r], old[r], p.alpha, p.beta);
             v = init ? vi : vc;
           }
-          four[q] = fused.put(v, w.out[g] + q * p.rsc0, first_row(i, g) + q);
+          if constexpr (MODE == 2) {  // no fused step at all: the value as it is
+            __builtin_nontemporal_store(v, w.out[g] + q * p.rsc0);
+            four[q] = v;
+          } else {
+            four[q] = fused.put(v, w.out[g] + q * p.rsc0, first_row(i, g) + q);
+          }
         }
       }
       fused.rows4(four, first_row(i, g));
@@ -561,9 +567,15 @@ __device__ __forceinline__ void write_wave_tile(const MfmaArgs &p, const Acc (&a
   };
   if (!read_c) {
     const AccElem none[16] = {};
-    [&]<int... Bs>(std::integer_sequence<int, Bs...>) {
-      (write_block(std::integral_constant<int, 0>{}, std::integral_constant<int, Bs>{}, none), ...);
-    }(std::make_integer_sequence<int, kBlocks>{});
+    if (EXTRA == 0 && !p.bias && !p.max) {  // the plain product: two or three instructions and a store per element
+      [&]<int... Bs>(std::integer_sequence<int, Bs...>) {
+        (write_block(std::integral_constant<int, 2>{}, std::integral_constant<int, Bs>{}, none), ...);
+      }(std::make_integer_sequence<int, kBlocks>{});
+    } else {
+      [&]<int... Bs>(std::integer_sequence<int, Bs...>) {
+        (write_block(std::integral_constant<int, 0>{}, std::integral_constant<int, Bs>{}, none), ...);
+      }(std::make_integer_sequence<int, kBlocks>{});
+    }
   } else {
     update_blocks(std::integral_constant<int, 1>{});
   }
