@@ -37,7 +37,10 @@ extern "C" {
 #define SKL_HIP_ERR_NO_DEVICE (-3)
 #define SKL_HIP_ERR_WORKSPACE (-4)
 /* Advisory: the calling thread's stream has no scratch slot on this device (32 other streams hold one). The call
- * that recorded it has still completed, on kernels that need no scratch memory. See skl_hip_release_stream(). */
+ * that recorded it has still completed, on kernels that need no scratch memory (the 4-bit-weight GEMMs, which
+ * need a converted copy of their operands for more than 16 rows, through a buffer of their own that is released
+ * once the stream has drained: such a call returns after its work is done). See skl_hip_release_stream().
+ * SKL_HIP_ERR_WORKSPACE, by contrast, means that C was not written. */
 #define SKL_HIP_ERR_STREAM_SLOTS (-5)
 
 /* Pointer-classification modes for skl_hip_set_pointer_mode(). */

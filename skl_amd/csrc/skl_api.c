@@ -501,6 +501,7 @@ static int k4_in_row_chunks(const skl_gemm_desc *d) {
 static int gemm_on_device(const skl_gemm_desc *d) {
   skl_gemm_canon g;
   const int fused = d->bias != NULL || d->max != NULL || d->rq.act != 0 || d->rq.q != NULL;
+  const int pending = skl_hip_pending_error(); /* what an earlier call left unread is not this call's to withdraw */
   int r = DECLINED;
   if (d->k0 * d->k1 != 0 && d->ta <= SKL_DT_F8E5M2) {
     if (canonicalize_k4(d, &g, 0) && skl_hip_gemv_supported(&g, 1)) { /* one row: the kernel applies fused steps itself */
@@ -531,7 +532,7 @@ static int gemm_on_device(const skl_gemm_desc *d) {
     r = outcome(skl_hip_launch_gemm_tiled(&g));
   if (r == DECLINED) r = outcome(skl_hip_launch_gemm_generic(d)); /* needs no scratch memory */
   /* a kernel further down the list ran in place of one that could not get its scratch memory: the call succeeded */
-  if (r == TAKEN) skl_hip_withdraw_error(SKL_HIP_ERR_WORKSPACE);
+  if (r == TAKEN && pending != SKL_HIP_ERR_WORKSPACE) skl_hip_withdraw_error(SKL_HIP_ERR_WORKSPACE);
   return r == TAKEN ? 0 : -1;
 }
 
@@ -758,24 +759,42 @@ static int f4_gemm_on_device(size_t m, size_t n, size_t k, float alpha, const ui
     const size_t values = k ? (n - 1) * ldb + k : 0; /* 4-bit values from B's first to its last, gaps included */
     skl_gemm_desc d = {SKL_DT_F8E4M3, SKL_DT_F8E4M3, 1, 1, 1, m, n, k, a, 0, 0, rsa, csa, NULL, 0, 0, 1, ldb,
                        c, 0, 0, rsc, csc, {.f = alpha}, beta, NULL, NULL, {0}};
+    /* The converted operands live in the stream's scratch block; a stream without one (the 33rd on its device) or a
+     * refused allocation gets a buffer of its own for this call, released once the stream has drained - slower,
+     * but the call completes. Only when that fails too is C left unwritten, and then the error says so (a hard
+     * error in place of the advisory one the scratch request left). */
+    const size_t span_a = (values && scales) ? (m - 1) * rsa + (k - 1) * csa + 1 : 0, bytes_a = (2 * span_a + 255) / 256 * 256;
+    const size_t bytes = !values ? 0 : scales ? bytes_a + 2 * values : values;
+    const int pending = skl_hip_pending_error();
+    char *block = NULL, *own = NULL;
     skl_hip_sequence_begin(); /* the converted operands travel from one launch to the next through the stream's scratch */
-    if (values && !scales) { /* B as E4M3: exact */
-      uint8_t *b8 = (uint8_t *)skl_hip_converted_scratch(values);
-      rc = b8 ? skl_hip_launch_cvt_f4_f8e4m3(b8, b, values) : SKL_HIP_ERR_WORKSPACE;
-      d.b = b8;
+    if (bytes) {
+      block = (char *)skl_hip_converted_scratch(bytes);
+      if (!block) block = own = (char *)skl_hip_malloc(bytes);
+    }
+    if (bytes && !block) {
+      skl_hip_withdraw_error(SKL_HIP_ERR_STREAM_SLOTS);
+      skl_hip_record_error(SKL_HIP_ERR_WORKSPACE, "4-bit-weight GEMM: no memory for the converted operands, C not written");
+      rc = SKL_HIP_ERR_WORKSPACE;
+    } else if (values && !scales) { /* B as E4M3: exact */
+      rc = skl_hip_launch_cvt_f4_f8e4m3((uint8_t *)block, b, values);
+      d.b = block;
     } else if (values) { /* scaled values leave E4M3's range: both operands as bf16 (exact), then the bf16 GEMM */
-      const size_t span_a = (m - 1) * rsa + (k - 1) * csa + 1, bytes_a = (2 * span_a + 255) / 256 * 256;
-      char *block = (char *)skl_hip_converted_scratch(bytes_a + 2 * values);
-      rc = block ? skl_hip_launch_cvt_f8_bf16(SKL_DT_F8E4M3, (uint16_t *)block, a, span_a) : SKL_HIP_ERR_WORKSPACE;
+      rc = skl_hip_launch_cvt_f8_bf16(SKL_DT_F8E4M3, (uint16_t *)block, a, span_a);
       if (rc == 0) rc = skl_hip_launch_cvt_mxf4_bf16((uint16_t *)(block + bytes_a), b, scales, lds, n, k, ldb);
       d.ta = d.tb = SKL_DT_BF16;
       d.a = block;
-      d.b = block ? block + bytes_a : NULL;
+      d.b = block + bytes_a;
     } else {
       rc = 0;
     }
     if (rc == 0) rc = gemm_on_device(&d);
     skl_hip_sequence_end();
+    if (own) {
+      skl_hip_synchronize(); /* the kernels that read the buffer have finished */
+      skl_hip_free(own);
+      if (rc == 0 && pending != SKL_HIP_ERR_WORKSPACE) skl_hip_withdraw_error(SKL_HIP_ERR_WORKSPACE); /* the scratch block's refusal was made good */
+    }
     return rc;
   }
 }

@@ -32,6 +32,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <cstdlib>
 #include <utility>
 
@@ -1318,13 +1320,13 @@ int launch_ring(const MfmaArgs &args) {
   }
   constexpr int lds = ring_stages(BN) * (256 + BN) * kRingSlice;
   auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE, EXTRA, CQUADS>;
-  static bool configured = false;
-  if (!configured) {
+  static std::atomic<bool> configured{false};  // per instantiation; racing threads set the same value
+  if (!configured.load(std::memory_order_acquire)) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                            "gemm_mfma_ring: LDS size");
     if (rc != 0) return rc;
-    configured = true;
+    configured.store(true, std::memory_order_release);
   }
   MfmaArgs p = args;
   p.tiles_m = (unsigned)((p.m + (EDGE ? 255 : 0)) / 256);
@@ -1379,13 +1381,13 @@ int launch_one(const MfmaArgs &args) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int lds = 2 * (Tile<ES, BM, A_KC, NT>::kBytes + Tile<ES, BN, B_KC, NT>::kBytes);
   auto kernel = gemm_mfma_kernel<TA, TB, A_KC, B_KC, BM, BN, WAVES_M, WAVES_N, GUARDED, EXACT, EXTRA>;
-  static bool configured = false;  // per instantiation; racing threads would set the same value
-  if (!configured) {
+  static std::atomic<bool> configured{false};  // per instantiation; racing threads set the same value
+  if (!configured.load(std::memory_order_acquire)) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds),
                            "gemm_mfma: LDS size");
     if (rc != 0) return rc;
-    configured = true;
+    configured.store(true, std::memory_order_release);
   }
   MfmaArgs p = args;
   p.tiles_m = skl_div_up(p.m, BM);

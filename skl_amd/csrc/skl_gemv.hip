@@ -46,6 +46,8 @@
 // k, which v_dot4_i32_i8 consumes without any byte shuffling).
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <type_traits>
 
 #include <mutex>
@@ -1439,13 +1441,13 @@ int launch_mfma_rows(const GemvMfmaArgs &args) {
   using Sh = MfmaShape<(MODE == kBF16 || MODE == kF16) ? 2 : 1, MODE == kI8K4>;
   constexpr size_t kMfmaLds = Sh::kLds;
   auto kernel = gemv_mfma_rows_kernel<MODE>;
-  static bool configured = false;  // per instantiation; racing threads would set the same value
-  if (!configured) {
+  static std::atomic<bool> configured{false};  // per instantiation; racing threads set the same value
+  if (!configured.load(std::memory_order_acquire)) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLds),
                            "gemv_mfma_rows: LDS size");
     if (rc != 0) return rc;
-    configured = true;
+    configured.store(true, std::memory_order_release);
   }
   GemvMfmaArgs p = args;
   p.tiles = skl_div_up(p.n, Sh::kTileCols);

@@ -197,6 +197,8 @@ int skl_hip_launch_cvt_f4_f8e4m3(uint8_t *dst, const uint8_t *src, size_t n);
 void skl_hip_record_error(int code, const char *what);
 /* Forgets the calling thread's recorded error if it is `code` (a failure that a later step of the same call made good). */
 void skl_hip_withdraw_error(int code);
+/* The calling thread's recorded error, left in place (skl_hip_last_error() reads and clears it). */
+int skl_hip_pending_error(void);
 
 #ifdef __cplusplus
 }

@@ -32,6 +32,8 @@ struct StreamState {
   Scratch converted;       // an operand converted to another element type ahead of a GEMM that may itself copy operands
   void *zeroed = nullptr;  // block that is zero between launches (sums and counters shared by workgroups)
   size_t zeroed_bytes = 0;
+  std::vector<void *> retired;  // blocks this stream outgrew: kept while work that was handed their address may still
+                                // run, freed when the stream is released (or at shutdown)
 };
 
 // Streams with scratch of their own per device. A further stream gets none (its calls run on the kernels that need
@@ -40,7 +42,6 @@ constexpr size_t kMaxStreamStates = 32;
 
 struct DeviceState {
   std::vector<StreamState> streams;
-  std::vector<void *> retired;
 };
 
 constexpr size_t kWorkspaceBytes = size_t(64) << 20;
@@ -60,6 +61,8 @@ thread_local char t_error_text[256] = "no error";
 extern "C" void skl_hip_withdraw_error(int code) {
   if (t_error == code) t_error = SKL_HIP_OK;
 }
+
+extern "C" int skl_hip_pending_error(void) { return t_error; }
 
 extern "C" void skl_hip_record_error(int code, const char *what) {
   if (code == SKL_HIP_OK || t_error != SKL_HIP_OK) return;  // keep the first error until it is read
@@ -87,7 +90,7 @@ std::recursive_mutex g_sequence;
 
 // Under g_mutex. At least `floor` bytes, and at least twice the block replaced, so that retired blocks add up to
 // less than the live one.
-void *grow(DeviceState &st, Scratch &sc, size_t bytes, size_t floor, const char *what, bool record) {
+void *grow(StreamState &st, Scratch &sc, size_t bytes, size_t floor, const char *what, bool record) {
   if (sc.ptr && sc.bytes >= bytes) return sc.ptr;
   size_t want = bytes < floor ? floor : bytes;
   if (want < 2 * sc.bytes) want = 2 * sc.bytes;
@@ -131,7 +134,7 @@ void *skl_workspace(size_t bytes) {
   if (!st) return nullptr;
   std::lock_guard<std::mutex> lock(g_mutex);
   StreamState *ss = current_stream_state(*st);
-  return ss ? grow(*st, ss->workspace, bytes, kWorkspaceBytes, "skl_workspace", true) : nullptr;
+  return ss ? grow(*ss, ss->workspace, bytes, kWorkspaceBytes, "skl_workspace", true) : nullptr;
 }
 
 void *skl_zeroed_scratch(size_t bytes) {
@@ -189,7 +192,7 @@ void *skl_hip_operand_scratch(size_t bytes) {
   std::lock_guard<std::mutex> lock(g_mutex);
   // not recorded as an error: the caller falls back to a kernel that needs no copy
   StreamState *ss = current_stream_state(*st);
-  return ss ? grow(*st, ss->operands, bytes, kOperandBytes, "skl_hip_operand_scratch", false) : nullptr;
+  return ss ? grow(*ss, ss->operands, bytes, kOperandBytes, "skl_hip_operand_scratch", false) : nullptr;
 }
 
 int skl_hip_release_stream(void *stream) {
@@ -207,6 +210,7 @@ int skl_hip_release_stream(void *stream) {
     if (s.operands.ptr) (void)hipFree(s.operands.ptr);
     if (s.converted.ptr) (void)hipFree(s.converted.ptr);
     if (s.zeroed) (void)hipFree(s.zeroed);
+    for (void *p : s.retired) (void)hipFree(p);
     st->streams.erase(st->streams.begin() + (long)i);
     break;
   }
@@ -218,7 +222,7 @@ void *skl_hip_converted_scratch(size_t bytes) {
   if (!st) return nullptr;
   std::lock_guard<std::mutex> lock(g_mutex);
   StreamState *ss = current_stream_state(*st);
-  return ss ? grow(*st, ss->converted, bytes, kOperandBytes, "skl_hip_converted_scratch", true) : nullptr;
+  return ss ? grow(*ss, ss->converted, bytes, kOperandBytes, "skl_hip_converted_scratch", true) : nullptr;
 }
 
 void skl_hip_sequence_begin(void) { g_sequence.lock(); }
@@ -233,7 +237,7 @@ void skl_hip_shutdown(void) {
   }
   for (int d = 0; d < kMaxDevices; ++d) {
     DeviceState &st = g_devices[d];
-    if (st.streams.empty() && st.retired.empty()) continue;
+    if (st.streams.empty()) continue;
     if (hipSetDevice(d) == hipSuccess) {
       (void)hipDeviceSynchronize();
       for (StreamState &s : st.streams) {
@@ -241,8 +245,8 @@ void skl_hip_shutdown(void) {
         if (s.operands.ptr) (void)hipFree(s.operands.ptr);
         if (s.converted.ptr) (void)hipFree(s.converted.ptr);
         if (s.zeroed) (void)hipFree(s.zeroed);
+        for (void *p : s.retired) (void)hipFree(p);
       }
-      for (void *p : st.retired) (void)hipFree(p);
     }
     st = DeviceState{};
   }

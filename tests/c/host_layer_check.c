@@ -533,6 +533,11 @@ void *__wrap_skl_hip_malloc(size_t bytes) {
   range_add(p, bytes ? bytes : 1, 1);
   return p;
 }
+static long g_synchronized;
+int __wrap_skl_hip_synchronize(void) {
+  ++g_synchronized;
+  return 0;
+}
 void __wrap_skl_hip_free(void *p) {
   if (!p) return;
   range_remove(p);
@@ -1054,8 +1059,14 @@ int main(int argc, char **argv) {
       default: run_gemm_case(device_pointers); break;
     }
   }
-  g_scarce = 1;
+  g_scarce = 1; /* every scratch block refused: each call must still complete, on a kernel that needs none or a buffer of its own */
   for (int t = 0; t < cases / 4 && !g_failures; ++t) run_gemm_case((int)(rnd() % 2));
+  {
+    const long launches = g_launches, synchronized = g_synchronized;
+    for (int t = 0; t < cases / 8 && !g_failures; ++t) run_f4_case((int)(rnd() % 2));
+    if (!g_failures && cases >= 64 && (g_launches == launches || g_synchronized == synchronized))
+      fail("4-bit-weight GEMMs without a scratch block: no call went through a buffer of its own");
+  }
   g_scarce = 0;
   if (!g_failures && argc <= 2) run_large_cases();  /* with a seed: random cases only */
   if (g_nranges != (g_operand_scratch ? 1 : 0) + (g_converted_scratch ? 1 : 0)) fail("a buffer of the host layer was not released");

@@ -145,3 +145,65 @@ def test_ofp4_edges(gpu):
     gpu.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(4, 32, 64, 1.0, d, 64, 1, b4, 64, 0.0, c.copy(), 32, 1)
     assert gpu.skl_hip_last_error() == -1
     d.free()
+
+
+def test_converted_copy_without_a_scratch_slot(gpu):
+    """A stream beyond the 32 that hold scratch blocks on a device: a 4-bit-weight GEMM that needs a converted copy of
+    its operands (more than 16 rows) still writes the right C - through a buffer of its own - and leaves only the
+    advisory SKL_HIP_ERR_STREAM_SLOTS behind, with and without block scales."""
+    import ctypes as ct
+
+    hip = ct.CDLL("libamdhip64.so.7")
+    hip.hipStreamCreate.restype = hip.hipStreamDestroy.restype = ct.c_int
+    m, n, k = 40, 96, 512
+    case, a, b4, b8, c = f4.make_problem(4711, m, n, k, k, 1.25, 0.5, rsc=n + 1)
+    rng = np.random.default_rng(5)
+    scales = rng.integers(120, 135, size=n * (k // 32), dtype=np.uint8)
+    streams = []
+    gpu.skl_hip_last_error()
+    try:
+        # claim slots with an int8 GEMV (its workgroups meet in the stream's scratch) until one is refused
+        x, w, y = DeviceBuffer.from_array(np.ones(4096, np.int8)), DeviceBuffer.from_array(np.ones(4096 * 2048, np.int8)), DeviceBuffer(4 * 2048)
+        gpu.skl_hip_set_pointer_mode(1)
+        for _ in range(34):
+            stream = ct.c_void_p()
+            assert hip.hipStreamCreate(ct.byref(stream)) == 0
+            streams.append(stream)
+            gpu.skl_hip_set_stream(stream.value)
+            gpu.skl_gemm_i8_i8_i32_gfx950(1, 2048, 4096, 1, x, 4096, w, 2048, 0, y, 2048)
+            assert gpu.skl_hip_synchronize() == 0
+            if gpu.skl_hip_last_error() == -5:
+                break
+        else:
+            pytest.fail("no stream was refused a slot")
+        gpu.skl_hip_set_pointer_mode(0)
+        for sc in (None, scales):   # the stream set above is the one without a slot
+            bufs = [DeviceBuffer.from_array(v) if v is not None else None for v in (a, b4, c, sc)]
+            if sc is None:
+                gpu.skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(m, n, k, case.alpha, bufs[0], case.rsa1, case.csa1, bufs[1], k, case.beta, bufs[2],
+                                                           case.rsc1, case.csc1)
+            else:
+                gpu.skl_gemm_f8e4m3rc_mxf4e2m1c_f32rc_gfx950(m, n, k, case.alpha, bufs[0], case.rsa1, case.csa1, bufs[1], k, bufs[3], k // 32,
+                                                             case.beta, bufs[2], case.rsc1, case.csc1)
+            assert gpu.skl_hip_synchronize() == 0
+            assert gpu.skl_hip_last_error() in (0, -5)
+            got = bufs[2].download(c.dtype, c.size)
+            if sc is None:
+                support.assert_fp_gemm_close(case, a, b8, c, got)
+            else:
+                gpu.skl_hip_set_stream(None)
+                want = run(gpu, case, a, b4, c, "device", m, n, k, k, scales=sc, lds=k // 32)   # the same call on a stream with scratch
+                gpu.skl_hip_set_stream(streams[-1].value)
+                assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+            for d in bufs:
+                if d is not None:
+                    d.free()
+        for d in (x, w, y):
+            d.free()
+    finally:
+        gpu.skl_hip_set_stream(None)
+        gpu.skl_hip_set_pointer_mode(0)
+        for stream in streams:
+            gpu.skl_hip_release_stream(stream.value)
+            hip.hipStreamDestroy(stream)
+        gpu.skl_hip_last_error()
