@@ -223,11 +223,11 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
   constexpr size_t kRowStep = WHOLE ? kPartials : 1;  // rows from one load of a lane to its next
   using Acc = typename Md::Acc;
   constexpr int kCols = Md::kCols;
-  __shared__ Acc red[kWaves][Md::kTileCols + 4];
+  __shared__ __attribute__((aligned(16))) Acc red[kWaves][Md::kTileCols + 4];
   __shared__ unsigned ticket_s;
 
   const unsigned tile = WHOLE ? blockIdx.x : blockIdx.x % p.tiles, slab = WHOLE ? blockIdx.y : blockIdx.x / p.tiles;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int cl = (lane & 1) + 2 * (lane >> 4), rl = (lane >> 1) & 7;
   const int part = wave * kRowLanes + rl;
   const size_t k0 = (size_t)slab * kKPerGroupL + (WHOLE ? (size_t)part : (size_t)part * kKPerLaneL);  // the lane's first row
@@ -366,9 +366,10 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
   // sums to LDS, where the eight waves meet.
 #pragma unroll
   for (int j = 0; j < kCols; ++j) acc[j] = sum_over_row_groups(acc[j]);
-  if (rl == 0) {
+  if (rl == 0) {  // 16-byte stores: a row of `red` is a multiple of 16 bytes, a lane's columns start on one
+    typedef Acc acc4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int j = 0; j < kCols; ++j) red[wave][cl * kCols + j] = acc[j];
+    for (int j = 0; j < kCols; j += 4) *reinterpret_cast<acc4 *>(&red[wave][cl * kCols + j]) = acc4{acc[j], acc[j + 1], acc[j + 2], acc[j + 3]};
   }
   __syncthreads();
   Acc sum = 0;
