@@ -2,6 +2,7 @@
 """Benchmark of the GEMM / GEMV / pack / cvt hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--full] [--no-cpu] [--out FILE]
+    python bench.py --vendor-only      (the vendor BLAS through torch on three of the products, for comparison)
 
 Prints ONE compact JSON line (a few KB) and writes the full record of everything it measured to
 gpurun_out/bench_full.json (`--out`); `--full` also runs the workloads that are not benchmark configurations. The headline (`value`) is the int8 GEMV decode shape
@@ -704,13 +705,14 @@ MEASURED_PEAK_OF = {"hbm": "peak_hbm_read", "i8": "peak_mfma_i8_random", "f8": "
 # summarised in profiles/gemv_cvt_gemm_hbm_traffic.pmc.txt.
 TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/gemv_cvt_gemm_hbm_traffic.pmc.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "gemv_i8": int((22068.0 * 1.998 + 817) * 1024),
-    "cvt_f32_f8e4m3_8192sq": int((131136.4 * 1.998 + 65536) * 1024),
-    "gemm_i8_8192": int((401544.6 * 1.998 + 278814.8) * 1024),
+    "gemv_i8": int((22061.5 * 1.998 + 817.0) * 1024),
+    "cvt_f32_f8e4m3_8192sq": int((131136.4 * 1.998 + 65536.0) * 1024),
+    "gemm_i8_8192": int((393334.9 * 1.998 + 262434.0) * 1024),
+    "gemm_f8e4m3_8192_kcontig": int((393395.0 * 1.998 + 262727.1) * 1024),
     "copy_u32_4096sq": int((32800.9 * 1.998 + 65536) * 1024),
-    "gemm_i8_16x4096x11008": int(((22336.1 + 9.0) * 1.998 + 5504 + 688) * 1024),
-    "gemv_f8e4m3_f4_1x4096x11008": int((11058.5 * 1.998 + 43) * 1024),
-    "gemm_i8_p4x1c_112x4096x11008": int(((23879.6 + 9.0) * 1.998 + 19264 + 4816) * 1024),
+    "gemm_i8_16x4096x11008": int((22353.1 * 1.998 + 6192.0) * 1024),
+    "gemv_f8e4m3_f4_1x4096x11008": int((11058.5 * 1.998 + 43.0) * 1024),
+    "gemm_i8_p4x1c_112x4096x11008": int((23896.7 * 1.998 + 24080.0) * 1024),
 }
 
 
@@ -804,6 +806,56 @@ def cpu_baseline(budget_s=12.0):
     return out
 
 
+def vendor_blas():
+    """What the vendor's BLAS reaches on this device for three of the table's products, through torch (measurement
+    only: nothing of the library calls it). The same data distributions and the same sustained-clock warm-up as
+    the library's rows; microseconds per call from torch's events on torch's stream."""
+    import torch
+    dev = "cuda"
+    out = {}
+
+    def timed(fn, flops, key, calls=20):
+        try:
+            t0 = time.perf_counter()
+            while (time.perf_counter() - t0) * 1e3 < MFMA_WARM_MS:
+                for _ in range(4):
+                    fn()
+                torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(calls):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / calls * 1e3
+            out[key] = {"us": round(us, 2), "achieved": round(flops / us * 1e-6, 1)}
+        except Exception as e:  # a product this torch build does not offer
+            out[key] = {"error": str(e)[:80]}
+
+    n = 8192
+    try:
+        a8 = torch.randint(-128, 128, (n, n), device=dev, dtype=torch.int8)
+        b8 = torch.randint(-128, 128, (n, n), device=dev, dtype=torch.int8)
+        timed(lambda: torch._int_mm(a8, b8), 2.0 * n ** 3, "int8 8192^3 (row-major A and B)")
+        del a8, b8
+    except Exception as e:
+        out["int8 8192^3 (row-major A and B)"] = {"error": str(e)[:80]}
+    try:
+        af = torch.randn(n, n, device=dev).to(torch.float8_e4m3fn)
+        bf = torch.randn(n, n, device=dev).to(torch.float8_e4m3fn).t()   # K-contiguous B
+        one = torch.tensor(1.0, device=dev)
+        timed(lambda: torch._scaled_mm(af, bf, scale_a=one, scale_b=one, out_dtype=torch.float32), 2.0 * n ** 3,
+              "fp8 E4M3 8192^3 (K-contiguous A and B, fp32 out)")
+        del af, bf
+    except Exception as e:
+        out["fp8 E4M3 8192^3 (K-contiguous A and B, fp32 out)"] = {"error": str(e)[:80]}
+    a = torch.randn(2048, 4096, device=dev, dtype=torch.bfloat16)
+    b = (torch.randn(4096, 4096, device=dev) * 0.02).to(torch.bfloat16)
+    c = torch.randn(2048, 4096, device=dev, dtype=torch.float32)
+    timed(lambda: torch.addmm(c.to(torch.bfloat16), a, b), 2.0 * 2048 * 4096 * 4096, "bf16 2048x4096x4096 (bf16 out, beta=1)", calls=80)
+    return out
+
+
 def config_rows(records, probes):
     """`roofline.configs`: one short row per benchmark configuration - workload key, microseconds per call (HIP
     events), achieved rate, fraction of the published peak and of the ceiling measured on this device."""
@@ -879,12 +931,18 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the chosen workload: no table of configurations")
     ap.add_argument("--full", action="store_true", help="also run every other workload (records go to the results file)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--vendor-only", action="store_true",
+                    help="time the vendor BLAS (through torch) on three of the table's products and print that alone: a process "
+                         "of its own, since torch brings its own HIP runtime")
     ap.add_argument("--out", default=os.path.join(ROOT, "gpurun_out", "bench_full.json"),
                     help="file that receives the full records of everything measured")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this library runs on one GPU; --gpus must be 1 (no multi-GPU path exists)")
 
+    if args.vendor_only:
+        print(json.dumps({"vendor_blas": vendor_blas()}, separators=(",", ":")), flush=True)
+        return
     lib = skl_amd.load()
     if lib.skl_hip_init(0) != 0:
         sys.exit("bench.py: no GPU: " + lib.skl_hip_last_error_string().decode())
