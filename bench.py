@@ -423,6 +423,47 @@ def wl_gemm_i8_4000(lib, rng):
     return d
 
 
+def _wl_reference_bench(kind, m, n, k, beta):
+    """The shapes the reference's own benchmark rows use (column-major A through the `c` entry points):
+    test/gemm/xsfmm/skl_gemm_i8c_i8_i32_xsfmm32a8i.c:55-56 (128 x 128 x 8192, beta 0 and 1) and
+    test/gemm/xsfmm/skl_gemm_bf16c_bf16_f32_xsfmm32a16f.c:55-56 (128 x 128 x 4096). Launch-bound at GPU scale:
+    a single 128 x 128 tile of C - timed as what a caller of those rows would see."""
+    def build(lib, rng):
+        if kind == "i8":
+            a, b = DeviceBuffer.from_array(rand_i8(rng, m * k)), DeviceBuffer.from_array(rand_i8(rng, k * n))
+            c = DeviceBuffer.from_array(np.zeros(m * n, np.int32))
+
+            def step(i):
+                lib.skl_gemm_i8c_i8_i32_gfx950(m, n, k, 1, a, m, b, n, beta, c, n)
+            es = 1
+        else:
+            a = DeviceBuffer.from_array(bf16_bits(rng.normal(size=m * k)))
+            b = DeviceBuffer.from_array(bf16_bits(rng.normal(size=k * n) * 0.02))
+            c = DeviceBuffer.from_array(np.zeros(m * n, np.float32))
+
+            def step(i):
+                lib.skl_gemm_bf16c_bf16_f32_gfx950(m, n, k, 1.0, a, m, b, n, float(beta), c, n)
+            es = 2
+        return dict(fn=step, bytes=es * (m * k + k * n) + 4 * m * n * (2 if beta else 1), ops=2 * m * n * k, bound="mfma",
+                    dtype=kind, keep=(a, b, c), name=f"{kind} GEMM {m}x{n}x{k}, column-major A, beta={beta} (the reference's own benchmark row)",
+                    kernel="gemm_mfma_kernel (K shared between workgroups) + gemm_split_reduce_kernel")
+    return build
+
+
+def wl_reference_bench_dot4(lib, rng):
+    """test/gemm/xsfvqdotq/skl_gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.c:56: 126 x 128 with k1 = 64 groups of four k."""
+    m, n, k1 = 126, 128, 64
+    a = DeviceBuffer.from_array(rand_i8(rng, m * 4 * k1))
+    b = DeviceBuffer.from_array(rand_i8(rng, k1 * 4 * n))
+    c = DeviceBuffer.from_array(np.zeros(m * n, np.int32))
+
+    def step(i):
+        lib.skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(m, n, k1, 1, a, 4 * k1, 4, b, 4 * n, 0, c, n)
+
+    return dict(fn=step, bytes=m * 4 * k1 + 4 * k1 * n + 4 * m * n, ops=2 * m * n * 4 * k1, bound="mfma", dtype="i8", keep=(a, b, c),
+                name="int8 dot4 GEMM 126x128, k1=64 (K-packed B; the reference's own benchmark row)", kernel="gemv_k4_rowgroups_kernel")
+
+
 def wl_gemm_i8_512(lib, rng):
     return _dense(lib, rng, "int8 GEMM 512^3 (row-major, alpha=1, beta=0)", "skl_gemm_i8_i8_i32_gfx950", 512, 512, 512,
                   1, lambda n: rand_i8(rng, n), lambda n: rand_i8(rng, n), 1, 0, np.int32, "i8")
@@ -673,6 +714,10 @@ WORKLOADS = {
     "gemm_f64_4096": (wl_gemm_f64, 5, 1, 1),
     "pipeline_f16_4096x4096x14336": (wl_f16_pipeline, 10, 2, 1),
     "gemm_i8_512": (wl_gemm_i8_512, 10, 2, 64),
+    "ref_bench_i8c_128x128x8192_beta0": (_wl_reference_bench("i8", 128, 128, 8192, 0), 10, 2, 64),
+    "ref_bench_i8c_128x128x8192_beta1": (_wl_reference_bench("i8", 128, 128, 8192, 1), 10, 2, 64),
+    "ref_bench_bf16c_128x128x4096_beta0": (_wl_reference_bench("bf16", 128, 128, 4096, 0), 10, 2, 64),
+    "ref_bench_dot4_126x128x256": (wl_reference_bench_dot4, 10, 2, 64),
     "cvt_f32_f8e4m3_8192sq": (wl_cvt, 10, 2, 2),
     "pack_e16_4096sq": (wl_pack_a, 10, 2, 10),
     "pack_e16_4096x14336_row_panels": (wl_pack_b, 10, 2, 2),
