@@ -83,7 +83,10 @@ void skl_gemm_f8e4m3rc_f4e2m1c_f32rc_gfx950(size_t m, size_t n, size_t k, float 
                                             size_t rsa, size_t csa, const uint8_t *b, size_t ldb, float beta,
                                             float *c, size_t rsc, size_t csc);
 /* The same with OCP microscaling (MXFP4): every 32 consecutive k of a column share a scale 2^(s - 127), s = the
- * E8M0 byte scales[j * lds + p / 32] (1 <= s <= 254; s == 127 everywhere or scales == NULL is the call above). The
+ * E8M0 byte scales[j * lds + p / 32] (1 <= s <= 254; s == 127 everywhere or scales == NULL is the call above; the
+ * two codes outside that range - 0, E8M0's 2^-127, and 255, its NaN - are not part of this entry point's domain: the
+ * device cannot refuse them, and what a block that carries one contributes is unspecified - zero or 2^-127 times its
+ * values, infinity or NaN, depending on which kernel the shape selects). The
  * reference has no notion of block scales: the result is that of decoding both operands to fp32 - A by
  * ref/cvt/cvt_ofp8.c:18-52, B's E2M1 values times their scales, all exact - and calling
  * ref/gemm/gemm_f32rc_f32rc_f32rc.h:44 (sums in fp32), inside the error bound of the reference's fp8 GEMM test.
