@@ -246,7 +246,8 @@ void skl_gemm_i8_i8_i32_gfx950(size_t m, size_t n, size_t k, int32_t alpha, cons
  * each GPU instead of a block the library allocates. Anything else records SKL_HIP_ERR_BAD_ARGUMENT and does
  * nothing. The call itself allocates, frees and queries nothing (skl_hip_init on the device beforehand also
  * keeps the one address lookup out of it). All such calls on one GPU share that array: calls that overlap on the
- * device - different streams, or the branches of one graph - race. */
+ * device - different streams, or the branches of one graph - race, and leave sums behind that every later call
+ * would add to; skl_hip_noalloc_reset() (skl-hip.h) puts the array back to zero. */
 void skl_gemm_i8_i8_i32_noalloc_gfx950(size_t m, size_t n, size_t k, int32_t alpha, const int8_t *a, size_t rsa,
                                        const int8_t *b, size_t rsb, int32_t beta, int32_t *c, size_t rsc);
 /* src/gemm/gemm_bf16_bf16_f32_zvfbfwma.h:49, src/gemm/gemm_bf16_bf16_f32_zvfbfwma_x390.h:49 */

@@ -66,6 +66,11 @@ int skl_hip_memcpy_h2d(void *dst, const void *src, size_t bytes);
 int skl_hip_memcpy_d2h(void *dst, const void *src, size_t bytes);
 int skl_hip_memcpy_d2d(void *dst, const void *src, size_t bytes);
 int skl_hip_memset(void *dst, int byte, size_t bytes);
+/* Zeroes, on the current stream, the static array in which the calls of skl_gemm_i8_i8_i32_noalloc_gfx950 on the
+ * current device share their sums. Every such call leaves the array zero again, so this is only needed after calls
+ * that overlapped on the device (they race, see that entry point) or did not finish: slots left non-zero would be
+ * added to every later result. Allocates nothing; not to be recorded into a graph. Returns 0 or an error. */
+int skl_hip_noalloc_reset(void);
 
 /* The stream (a hipStream_t passed as void*) kernels of the calling thread are
  * enqueued on; NULL selects the default stream. */

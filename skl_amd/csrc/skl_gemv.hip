@@ -1609,6 +1609,15 @@ extern "C" int skl_hip_noalloc_setup(void) { return noalloc_slots_of_current_dev
 
 extern "C" size_t skl_hip_noalloc_max_sums(void) { return kNoAllocSlots; }
 
+// Puts the static sums back to zero on the current device, enqueued on the calling thread's stream: the way out
+// after no-alloc calls overlapped (or one was aborted) and left slots that are not zero - every later call would add
+// to them. Not for use under graph capture (a memset node); allocates nothing.
+extern "C" int skl_hip_noalloc_reset(void) {
+  unsigned long long *slots = noalloc_slots_of_current_device();
+  if (!slots) return -2;
+  return skl_check_hip(hipMemsetAsync(slots, 0, kNoAllocSlots * sizeof(unsigned long long), skl_current_stream()), "skl_hip_noalloc_reset");
+}
+
 extern "C" int skl_hip_launch_gemv_noalloc(const skl_gemm_canon *g) {
   if (g->ta != SKL_DT_I8 || g->tb != SKL_DT_I8 || g->m < 1 || g->m > (size_t)kMaxRows ||
       (g->m == 1 ? !skl_hip_gemv_supported(g, 0) : !skl_hip_gemv_rows_supported(g))) {

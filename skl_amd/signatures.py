@@ -189,6 +189,7 @@ RUNTIME = {
     "skl_hip_memcpy_d2h": (ctypes.c_int, "ppz"),
     "skl_hip_memcpy_d2d": (ctypes.c_int, "ppz"),
     "skl_hip_memset": (ctypes.c_int, "piz"),
+    "skl_hip_noalloc_reset": (ctypes.c_int, ""),
     "skl_hip_set_stream": (None, "p"),
     "skl_hip_get_stream": (ctypes.c_void_p, ""),
     "skl_hip_synchronize": (ctypes.c_int, ""),

@@ -62,3 +62,76 @@ def test_rejects_what_the_static_scratch_cannot_hold(gpu):
     assert np.array_equal(got, want)
     for d in (da, db, dc):
         d.free()
+
+
+def test_allocates_nothing_and_replays_from_a_graph(gpu):
+    """What the entry point exists for: on a stream that holds no scratch slot of the library, the call changes
+    nothing about the device's free memory, it can be recorded into a HIP graph, and every replay - with new
+    activations written in between and eager work of the process around it - gives the ordinary entry point's bits.
+    A spoiled array of sums is put right by skl_hip_noalloc_reset()."""
+    import ctypes as ct
+
+    lib = gpu
+    hip = ct.CDLL("libamdhip64.so.7")
+    for name in ("hipStreamCreate", "hipStreamBeginCapture", "hipStreamEndCapture", "hipGraphInstantiate", "hipGraphLaunch",
+                 "hipStreamSynchronize", "hipGraphExecDestroy", "hipGraphDestroy", "hipStreamDestroy", "hipMemGetInfo"):
+        getattr(hip, name).restype = ct.c_int
+
+    def free_bytes():
+        free, total = ct.c_size_t(), ct.c_size_t()
+        assert hip.hipMemGetInfo(ct.byref(free), ct.byref(total)) == 0
+        return free.value
+
+    m, n, k = 3, 4096, 2048
+    rng = np.random.default_rng(77)
+    b = rng.integers(-128, 128, size=k * n, dtype=np.int8)
+    c0 = rng.integers(-1000, 1000, size=m * n).astype(np.int32)
+    da, db, dc, dref = DeviceBuffer(m * k), DeviceBuffer.from_array(b), DeviceBuffer.from_array(c0), DeviceBuffer.from_array(c0)
+    stream, graph, executable = ct.c_void_p(), ct.c_void_p(), ct.c_void_p()
+    assert hip.hipStreamCreate(ct.byref(stream)) == 0
+    lib.skl_hip_set_pointer_mode(1)
+    try:
+        lib.skl_hip_set_stream(stream.value)
+        a = rng.integers(-128, 128, size=m * k, dtype=np.int8)
+        lib.skl_hip_memcpy_h2d(da, a, a.nbytes)
+        before = free_bytes()
+        lib.skl_gemm_i8_i8_i32_noalloc_gfx950(m, n, k, 2, da, k, db, n, 1, dc, n)     # eager, on the fresh stream
+        assert lib.skl_hip_synchronize() == 0 and lib.skl_hip_last_error() == 0
+        assert free_bytes() == before                                              # no scratch block, no workspace
+        assert hip.hipStreamBeginCapture(stream, 0) == 0
+        lib.skl_gemm_i8_i8_i32_noalloc_gfx950(m, n, k, 2, da, k, db, n, 1, dc, n)
+        assert hip.hipStreamEndCapture(stream, ct.byref(graph)) == 0
+        assert lib.skl_hip_last_error() == 0
+        assert hip.hipGraphInstantiate(ct.byref(executable), graph, None, None, 0) == 0
+        expected = None
+        for replay in range(3):
+            a = rng.integers(-128, 128, size=m * k, dtype=np.int8)
+            lib.skl_hip_memcpy_h2d(da, a, a.nbytes)
+            lib.skl_hip_memcpy_h2d(dc, c0, c0.nbytes)
+            assert hip.hipGraphLaunch(executable, stream) == 0
+            assert hip.hipStreamSynchronize(stream) == 0
+            lib.skl_hip_set_stream(None)                                           # the ordinary call, eagerly, on the default stream
+            lib.skl_hip_memcpy_h2d(dref, c0, c0.nbytes)
+            lib.skl_gemm_i8_i8_i32_gfx950(m, n, k, 2, da, k, db, n, 1, dref, n)
+            assert lib.skl_hip_synchronize() == 0
+            lib.skl_hip_set_stream(stream.value)
+            expected = dref.download(np.int32, c0.size)
+            assert np.array_equal(dc.download(np.int32, c0.size), expected), replay
+        # sums left behind (as overlapping calls would) spoil the next result; the reset puts them right
+        assert lib.skl_hip_noalloc_reset() == 0
+        lib.skl_hip_memcpy_h2d(dc, c0, c0.nbytes)
+        lib.skl_gemm_i8_i8_i32_noalloc_gfx950(m, n, k, 2, da, k, db, n, 1, dc, n)
+        assert lib.skl_hip_synchronize() == 0 and lib.skl_hip_last_error() == 0
+        assert np.array_equal(dc.download(np.int32, c0.size), expected)
+    finally:
+        lib.skl_hip_set_stream(None)
+        lib.skl_hip_set_pointer_mode(0)
+        if executable:
+            hip.hipGraphExecDestroy(executable)
+        if graph:
+            hip.hipGraphDestroy(graph)
+        lib.skl_hip_release_stream(stream.value)
+        hip.hipStreamDestroy(stream)
+        for d in (da, db, dc, dref):
+            d.free()
+        lib.skl_hip_last_error()
