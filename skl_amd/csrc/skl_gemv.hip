@@ -756,7 +756,9 @@ __global__ void __launch_bounds__(256) gemv_mfma_add_planes_kernel(GemvMfmaArgs 
   if (p.max && v > skl_lowest<float>()) skl_atomic_max(p.max, v);
 }
 
-template <int MODE>
+// WHOLE: n is a whole number of column tiles and k of workgroup ranges (checked by the launcher), so no load is
+// guarded - the guarded kernel's compares and selects on 32 addresses per lane cost 1.5 to 2 us of a 13 us call.
+template <int MODE, bool WHOLE = false>
 __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfmaArgs p) {
   constexpr bool kInt = MODE == kI8RowMajor || MODE == kI8K4, k16 = MODE == kBF16 || MODE == kF16;
   constexpr bool kPacked = MODE == kI8K4;
@@ -769,35 +771,37 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
   extern __shared__ __attribute__((aligned(16))) int mfma_red_raw[];
   Acc(*red)[16][Sh::kPitch] = reinterpret_cast<Acc(*)[16][Sh::kPitch]>(mfma_red_raw);
   const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int jl = lane & 15, g = lane >> 4;
   const size_t col = (size_t)tile * Sh::kTileCols + (size_t)jl * LC;  // the lane's columns: inside one block of 64
   const size_t kwave = ((size_t)slab * kMfmaWaves + wave) * (Sh::kBlockK * ITERS);
-  const bool col_ok = col < p.n;  // n is a multiple of the columns per lane
+  const bool col_ok = WHOLE || col < p.n;  // n is a multiple of the columns per lane
   const char *bp = kPacked ? p.b + col * 4 : p.b + (col >> 6) * p.b_s1 + (col & 63) * ES;
   constexpr int kLaneK = LR * Sh::kKPerLoad;  // k of a lane per block: 16 bytes of A
 
   uint4 rows[ITERS][LR];
   v4i xa[ITERS];
+  // A's pieces are requested ahead of B's: loads come back in the order of their requests, so with A behind B the
+  // first block's multiplications would wait for the last block's rows (0.75 us of a 15 us call).
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    // k is a multiple of a lane's k per block: a 16-byte piece of a row of A is inside or outside
+    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * kLaneK;
+    if ((size_t)jl < p.m && (WHOLE || k0 < p.k))
+      xa[it] = *reinterpret_cast<const v4i *>(p.a + (size_t)jl * p.a_row + k0 * ES);
+    else
+      xa[it] = v4i{0, 0, 0, 0};
+  }
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * kLaneK;
 #pragma unroll
     for (int r = 0; r < LR; ++r) {
-      if (col_ok && k0 + (size_t)r * Sh::kKPerLoad < p.k)
+      if (WHOLE || (col_ok && k0 + (size_t)r * Sh::kKPerLoad < p.k))
         rows[it][r] = stream_load(bp + (k0 / Sh::kKPerLoad + r) * p.b_sk);
       else
         rows[it][r] = make_uint4(0, 0, 0, 0);
     }
-  }
-#pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    // k is a multiple of a lane's k per block: a 16-byte piece of a row of A is inside or outside
-    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * kLaneK;
-    if ((size_t)jl < p.m && k0 < p.k)
-      xa[it] = *reinterpret_cast<const v4i *>(p.a + (size_t)jl * p.a_row + k0 * ES);
-    else
-      xa[it] = v4i{0, 0, 0, 0};
   }
   v4acc acc[LC];
 #pragma unroll
@@ -872,23 +876,40 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
   constexpr int kRowStep = kMfmaWaves * 64 / Sh::kTileCols;
   const int tc = threadIdx.x % Sh::kTileCols;
   const size_t j = (size_t)tile * Sh::kTileCols + tc;
-  if (j >= p.n) return;
-  if constexpr (kInt) {
-    for (size_t i = threadIdx.x / Sh::kTileCols; i < p.m; i += kRowStep) {
+  if (!WHOLE && j >= p.n) return;
+  // All rows' sums are read from LDS before the first goes out (a loop over the rows of A would pay an LDS round
+  // trip per row).
+  constexpr int kPasses = kMfmaMaxRows / kRowStep;
+  const int i0 = threadIdx.x / Sh::kTileCols;
+  Acc sums[kPasses];
+#pragma unroll
+  for (int q = 0; q < kPasses; ++q) {
+    const int i = i0 + q * kRowStep;
+    if constexpr (kInt) {
       unsigned sum = 0;
 #pragma unroll
       for (int w = 0; w < kMfmaWaves; ++w) sum += (unsigned)red[w][i][tc];
-      (void)__hip_atomic_fetch_add(p.c + i * p.c_row + j * p.c_s, (int)((unsigned)p.alpha.i * sum), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-    }
-  } else {
-    float *plane = p.planes + (size_t)slab * p.m * p.n;
-    for (size_t i = threadIdx.x / Sh::kTileCols; i < p.m; i += kRowStep) {
+      sums[q] = (int)((unsigned)p.alpha.i * sum);
+    } else {
       float sum = red[0][i][tc];
 #pragma unroll
       for (int w = 1; w < kMfmaWaves; ++w) sum = __fadd_rn(sum, red[w][i][tc]);
-      plane[i * p.n + j] = sum;
+      sums[q] = sum;
     }
+  }
+  if constexpr (kInt) {
+    int *cp = p.c + (size_t)i0 * p.c_row + j * p.c_s;
+#pragma unroll
+    for (int q = 0; q < kPasses; ++q)
+      if ((size_t)(i0 + q * kRowStep) < p.m)
+        (void)__hip_atomic_fetch_add(cp + (size_t)q * kRowStep * p.c_row, sums[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    // past the compute die's L2: the second kernel runs on every die, and lines left dirty here would have to be
+    // written back between the two kernels (16 x 4096 x 11008: 1 us of a 16 us call)
+    float *plane = p.planes + (size_t)slab * p.m * p.n + (size_t)i0 * p.n + j;
+#pragma unroll
+    for (int q = 0; q < kPasses; ++q)
+      if ((size_t)(i0 + q * kRowStep) < p.m) __builtin_nontemporal_store(sums[q], plane + (size_t)q * kRowStep * p.n);
   }
 }
 
@@ -983,6 +1004,127 @@ __global__ void __launch_bounds__(kMfmaWaves * 64, 2) gemv_k4_rowgroups_kernel(G
         (void)__hip_atomic_fetch_add(p.c + row * p.c_row + j * p.c_s, (int)((unsigned)p.alpha.i * sum), __ATOMIC_RELAXED,
                                      __HIP_MEMORY_SCOPE_AGENT);
       }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The K-packed B again, K <= 4096 and 2 to 128 rows of A: one workgroup of eight waves per 64 columns takes ALL of K
+// (512 k per wave: 32 loads per lane, the whole of B in flight from the start), so the sums of a column tile never
+// leave the workgroup - they meet in LDS, C is written once with the alpha / beta step applied in place, and neither
+// the kernel that scales C in front nor the atomic adds into C (one per element and quarter of K above: 19.7 MB next
+// to 45 MB of weights for 112 x 4096 x 11008) are needed. Loads are clamped into the operands instead of guarded -
+// a guard is a branch, and the compiler waits for every earlier load at a branch it cannot prove uniform; rows
+// beyond K meet zeros of A, columns beyond N are computed and not written.
+// Up to three row groups: the waves write their 16 x 64 sums side by side, one barrier per group (two blocks take
+// turns). From four groups on the waves add into one plane with LDS atomics and meet once at the end: barriers would
+// keep them in step, and out of step they hide each other's waits for the next group's pieces of A (an L2 round trip
+// each - every workgroup reads all of A, which is what bounds this kernel from about 64 rows on).
+// 4096 x 11008 weights: 16 rows 11.2 us (13.4 with the kernels above), 32 rows 13.0 (18.4), 112 rows 24.1 (30.4).
+// ---------------------------------------------------------------------------
+constexpr int kK4WholeWaves = 8, kK4WholeIters = 8, kK4WholePitch = 68;
+constexpr size_t kK4WholeMaxK = (size_t)kK4WholeWaves * kK4WholeIters * 64;
+constexpr size_t k4_whole_lds(int rg) {
+  return (rg >= 4 ? (size_t)rg * 16 : (size_t)2 * kK4WholeWaves * 16) * kK4WholePitch * sizeof(int);
+}
+
+template <int RG>
+__global__ void __launch_bounds__(kK4WholeWaves * 64) gemv_k4_wholek_kernel(GemvMfmaArgs p) {
+  constexpr bool kOnePlane = RG >= 4;
+  constexpr int ITERS = kK4WholeIters, W = kK4WholeWaves, PITCH = kK4WholePitch;
+  typedef int v4i __attribute__((ext_vector_type(4)));
+  extern __shared__ __attribute__((aligned(16))) int mfma_red_raw[];
+  const unsigned tile = blockIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int jl = lane & 15, g = lane >> 4;
+  const size_t col = (size_t)tile * 64 + (size_t)jl * 4;
+  const char *bp = p.b + (col < p.n ? col : p.n - 4) * 4;  // n is a multiple of four
+  const size_t kwave = (size_t)wave * (64 * ITERS);
+  // The lane's 16 k of row 16 rg + jl for each of the wave's blocks: loaded from inside A, zeroed beyond M and K.
+  auto fragment_of = [&](int rg, v4i(&xa)[ITERS]) {
+    const size_t row = (size_t)rg * 16 + jl;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const size_t k0 = kwave + (size_t)it * 64 + (size_t)g * 16;
+      const bool inside = row < p.m && k0 < p.k;  // k is a multiple of 16
+      const v4i v = *reinterpret_cast<const v4i *>(p.a + (row < p.m ? row : p.m - 1) * p.a_row + (k0 < p.k ? k0 : p.k - 16));
+      xa[it] = v4i{inside ? v.x : 0, inside ? v.y : 0, inside ? v.z : 0, inside ? v.w : 0};
+    }
+  };
+  v4i xa[2][ITERS];
+  fragment_of(0, xa[0]);  // ahead of B: loads come back in the order of their requests
+  uint4 rows[ITERS][4];
+  const size_t groups = p.k / 4;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const size_t k0 = kwave + (size_t)it * 64 + (size_t)g * 16;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const size_t group = k0 / 4 + r;
+      rows[it][r] = stream_load(bp + (group < groups ? group : groups - 1) * p.b_sk);
+    }
+  }
+  if constexpr (RG > 1) fragment_of(1, xa[1]);
+  __builtin_amdgcn_sched_barrier(0);  // every request is out before the first use (the scheduler would otherwise
+                                      // sink loads to their uses to save registers: 12 in flight instead of 32)
+  int(*plane)[PITCH] = reinterpret_cast<int(*)[PITCH]>(mfma_red_raw);
+  if constexpr (kOnePlane) {  // zeroed while the loads are under way
+    for (int idx = threadIdx.x; idx < RG * 16 * PITCH / 4; idx += W * 64) reinterpret_cast<v4i *>(mfma_red_raw)[idx] = v4i{0, 0, 0, 0};
+    __syncthreads();
+  }
+  const int tc = threadIdx.x & 63;
+  const size_t j = (size_t)tile * 64 + tc;
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) {
+    if ((size_t)rg * 16 >= p.m) break;  // the same for every thread of the workgroup
+    v4i acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = v4i{0, 0, 0, 0};
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const unsigned t[4][4] = {{rows[it][0].x, rows[it][0].y, rows[it][0].z, rows[it][0].w},
+                                {rows[it][1].x, rows[it][1].y, rows[it][1].z, rows[it][1].w},
+                                {rows[it][2].x, rows[it][2].y, rows[it][2].z, rows[it][2].w},
+                                {rows[it][3].x, rows[it][3].y, rows[it][3].z, rows[it][3].w}};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const v4i bw = {(int)t[0][c], (int)t[1][c], (int)t[2][c], (int)t[3][c]};
+        acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[rg & 1][it], bw, acc[c], 0, 0, 0);
+      }
+    }
+    if (rg + 2 < RG) fragment_of(rg + 2, xa[rg & 1]);
+    // acc[c][r] is row 16 rg + 4 g + r of C, column 4 jl + c of the tile.
+    if constexpr (kOnePlane) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          (void)__hip_atomic_fetch_add(&plane[rg * 16 + 4 * g + r][4 * jl + c], acc[c][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    } else {
+      // two blocks take turns: the next group's barrier stands between this group's readers and the writers of
+      // the group after it
+      int(*red)[16][PITCH] = reinterpret_cast<int(*)[16][PITCH]>(mfma_red_raw + (rg & 1) * W * 16 * PITCH);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) *reinterpret_cast<v4i *>(&red[wave][4 * g + r][4 * jl]) = v4i{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int il = (threadIdx.x >> 6) + W * q;
+        const size_t i = (size_t)rg * 16 + il;
+        unsigned sum = 0;
+#pragma unroll
+        for (int w = 0; w < W; ++w) sum += (unsigned)red[w][il][tc];
+        if (i < p.m && j < p.n) skl_update((int)sum, p.c + i * p.c_row + j * p.c_s, p.alpha, p.beta);
+      }
+    }
+  }
+  if constexpr (kOnePlane) {
+    __syncthreads();
+    if (j >= p.n) return;
+#pragma unroll
+    for (int q = 0; q < RG * 16 / W; ++q) {
+      const size_t i = (size_t)(threadIdx.x >> 6) + (size_t)q * W;
+      if (i < p.m) skl_update(plane[i][tc], p.c + i * p.c_row + j * p.c_s, p.alpha, p.beta);
     }
   }
 }
@@ -1441,13 +1583,16 @@ template <int MODE>
 int launch_mfma_rows(const GemvMfmaArgs &args) {
   using Sh = MfmaShape<(MODE == kBF16 || MODE == kF16) ? 2 : 1, MODE == kI8K4>;
   constexpr size_t kMfmaLds = Sh::kLds;
-  auto kernel = gemv_mfma_rows_kernel<MODE>;
-  static std::atomic<bool> configured{false};  // per instantiation; racing threads set the same value
+  const bool whole = args.n % Sh::kTileCols == 0 && args.k % Sh::kKPerGroup == 0;
+  auto kernel = whole ? gemv_mfma_rows_kernel<MODE, true> : gemv_mfma_rows_kernel<MODE, false>;
+  static std::atomic<bool> configured{false};  // per instantiation; racing threads set the same values
   if (!configured.load(std::memory_order_acquire)) {
-    int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLds),
-                           "gemv_mfma_rows: LDS size");
-    if (rc != 0) return rc;
+    for (auto k : {gemv_mfma_rows_kernel<MODE, true>, gemv_mfma_rows_kernel<MODE, false>}) {
+      int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLds),
+                             "gemv_mfma_rows: LDS size");
+      if (rc != 0) return rc;
+    }
     configured.store(true, std::memory_order_release);
   }
   GemvMfmaArgs p = args;
@@ -1457,6 +1602,33 @@ int launch_mfma_rows(const GemvMfmaArgs &args) {
   if (grid > 0x7FFFFFFFu || cells > 0x7FFFFFFFu) {
     skl_hip_record_error(-2, "gemv_mfma_rows: grid too large");
     return -2;
+  }
+  if constexpr (MODE == kI8K4) {
+    if (p.k <= kK4WholeMaxK) {  // all of K inside one workgroup: no sums between workgroups
+      const unsigned tiles = (unsigned)skl_div_up(p.n, (size_t)64);
+      hipStream_t st = skl_current_stream();
+      constexpr unsigned threads = kK4WholeWaves * 64;
+      static std::atomic<bool> whole_configured{false};
+      if (!whole_configured.load(std::memory_order_acquire)) {  // the kinds with two blocks of sums pass 64 KiB
+        for (const void *f : {reinterpret_cast<const void *>(gemv_k4_wholek_kernel<1>), reinterpret_cast<const void *>(gemv_k4_wholek_kernel<2>),
+                              reinterpret_cast<const void *>(gemv_k4_wholek_kernel<3>)}) {
+          int rc = skl_check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)k4_whole_lds(1)), "gemv_k4_wholek: LDS size");
+          if (rc != 0) return rc;
+        }
+        whole_configured.store(true, std::memory_order_release);
+      }
+      switch ((p.m + 15) / 16) {
+        case 1: gemv_k4_wholek_kernel<1><<<tiles, threads, k4_whole_lds(1), st>>>(p); break;
+        case 2: gemv_k4_wholek_kernel<2><<<tiles, threads, k4_whole_lds(2), st>>>(p); break;
+        case 3: gemv_k4_wholek_kernel<3><<<tiles, threads, k4_whole_lds(3), st>>>(p); break;
+        case 4: gemv_k4_wholek_kernel<4><<<tiles, threads, k4_whole_lds(4), st>>>(p); break;
+        case 5: gemv_k4_wholek_kernel<5><<<tiles, threads, k4_whole_lds(5), st>>>(p); break;
+        case 6: gemv_k4_wholek_kernel<6><<<tiles, threads, k4_whole_lds(6), st>>>(p); break;
+        case 7: gemv_k4_wholek_kernel<7><<<tiles, threads, k4_whole_lds(7), st>>>(p); break;
+        default: gemv_k4_wholek_kernel<8><<<tiles, threads, k4_whole_lds(8), st>>>(p); break;
+      }
+      return skl_check_launch("gemv_k4_wholek");
+    }
   }
   if constexpr (MODE == kI8RowMajor || MODE == kI8K4) {
     if (p.beta.i != 1) {  // beta == 1: C is the starting value as it is

@@ -112,13 +112,17 @@ def test_k_packed_int8_decode(gpu, n, k1):
 @pytest.mark.parametrize("m", (2, 3, 7, 16, 17, 33, 48, 100, 112, 128, 129, 200, 257))
 def test_k_packed_int8_decode_batches(gpu, m):
     """The dot4 layout with 2 or more rows of A (src/gemm/gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.c:645-660 has its own
-    kernels for these): the K-packed B is read in place by the decode-batch kernel - four loads give a lane 16 k of
-    four columns, no transposes; 17 to 128 rows take the variant that keeps B in registers for up to eight groups of
-    16 rows (ragged last group: 17, 33, 100), more rows go through it in chunks of 128 (a last chunk of one row
-    through the one-row kernel: 129, 257). The config-2 weights prepacked, N and K off the kernel's 1024 x 64
+    kernels for these): the K-packed B is read in place by the decode-batch kernels - four loads give a lane 16 k of
+    four columns, no transposes; B stays in registers for up to eight groups of 16 rows (ragged last group: 17, 33,
+    100), more rows go through in chunks of 128 (a last chunk of one row through the one-row kernel: 129, 257).
+    K <= 4096: one workgroup per 64 columns takes all of K and writes C once; beyond (one shape here) workgroups
+    share a column tile and meet in C. The config-2 weights prepacked, N and K off the kernel's 1024 x 64
     blocks, padded strides of A, B and C, alpha / beta with wrap-around, both pointer modes; whole-buffer compare."""
     rng = np.random.default_rng(600 + m)
-    for (n, k1, pad_a, pad_b, pad_c) in ((11008, 1024, 0, 0, 0), (4100, 132, 16, 32, 5), (2052, 516, 48, 16, 0)):
+    shapes = [(11008, 1024, 0, 0, 0), (4100, 132, 16, 32, 5), (2052, 516, 48, 16, 0)]
+    if m in (7, 100):
+        shapes.append((1028, 1284, 16, 0, 3))  # K = 5136 > 4096: the sums of a column tile meet in C, not in LDS
+    for (n, k1, pad_a, pad_b, pad_c) in shapes:
         for alpha, beta in ((1, 0), (0x01010101, -77), (-3, 1)):
             case = support.dot4_case(m, n, k1, alpha=alpha, beta=beta, rsa1=4 * k1 + pad_a, rsb1=4 * n + pad_b,
                                      rsc1=n + pad_c)
