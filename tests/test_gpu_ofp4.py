@@ -42,6 +42,8 @@ SHAPES = (
     # m, n, k, ldb, rsa, what
     (1, 11008, 4096, 4096, None, "decode, FP4 operand format of the matrix cores"),
     (16, 1000, 4352, 4384, 4368, "16 rows, n off the 16-column groups, K off the chunk of 1024"),
+    (16, 8200, 2592, 2624, 2608, "workgroups of 64 columns (n >= 8192, 3 rows or more): n off them, K off the chunk"),
+    (3, 8256, 2304, 2304, None, "workgroups of 64 columns, multiplied exactly"),
     (3, 500, 2304, 2304, None, "longest K multiplied exactly (operands widened to f16)"),
     (7, 48, 2336, 2336, None, "shortest K on the FP4 format"),
     (5, 48, 32, 32, None, "one piece of K"),
@@ -83,11 +85,12 @@ def test_mx_scaled_ofp4_weights(gpu, m, n, k, ldb, rsa, what):
             assert np.array_equal(got.view(np.uint32), again.view(np.uint32)), what
 
 
+@pytest.mark.parametrize("n", (48, 8208))
 @pytest.mark.parametrize("k", (2304, 2560))
-def test_scales_reach_their_blocks(gpu, k):
+def test_scales_reach_their_blocks(gpu, k, n):
     """A row of A that is 1.0 at one k reads B(k, :) times its block's scale back exactly: every block of 32 k gets the
-    scale stored for it, in both kernel variants."""
-    n, lds = 48, k // 32 + 1
+    scale stored for it, in both kernel variants and both workgroup widths (16 and, from n = 8192, 64 columns)."""
+    lds = k // 32 + 1
     rng = np.random.default_rng(k + 1)
     codes = rng.integers(1, 8, size=n * k, dtype=np.uint8)        # positive, non-zero values
     scales = rng.integers(117, 138, size=n * lds, dtype=np.uint8)
@@ -102,12 +105,12 @@ def test_scales_reach_their_blocks(gpu, k):
         assert np.array_equal(got.astype(np.float64), values[:, pos].T), (k, p0)
 
 
+@pytest.mark.parametrize("n", (64, 8256))
 @pytest.mark.parametrize("k", (2304, 2560))
-def test_every_position_and_code_is_read_back(gpu, k):
+def test_every_position_and_code_is_read_back(gpu, k, n):
     """A row of A that is 1.0 at one k and zero elsewhere reads B(k, :) back exactly: every position of a 256-k chunk
     (16 rows per call), every E2M1 code, both kernel variants (k = 2304: f16 instructions, 2560: FP4 format). This
-    is what fixes which nibble is which k and that A's and B's lanes hold the same k."""
-    n = 64
+    is what fixes which nibble is which k and that A's and B's lanes hold the same k. Both workgroup widths."""
     rng = np.random.default_rng(k)
     codes = rng.integers(0, 16, size=n * k, dtype=np.uint8)
     codes[:16 * k:k + 1] = np.arange(16)          # and every code at least once on a diagonal
