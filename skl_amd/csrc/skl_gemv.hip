@@ -245,20 +245,27 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
   const bool y_is_read = !skl_beta_is_zero<Acc>(p.beta);
   Acc y_old = 0;
 
-  if (WHOLE || (col < p.n && k0 < p.k)) {
-    // All of the lane's loads are requested before anything is consumed.
+  {
+    // All of the lane's loads are requested before anything is consumed. Without WHOLE they are clamped into B
+    // rather than guarded (a guard is a branch, and the compiler waits for the loads in flight at a branch it
+    // cannot prove uniform): a lane beyond N reads column 0 and writes nothing, a row beyond K is read as row 0 and
+    // meets a zero of x - or, in the floating-point kinds, where 0 * NaN would not be 0, is zeroed itself.
+    const size_t colc = (WHOLE || col < p.n) ? col : 0;
     const char *wp;
     if constexpr (MODE == kI8K4)
-      wp = p.b + (k0 / 4) * p.b_sk + col * 4;
+      wp = p.b + colc * 4;
     else
-      wp = p.b + (col >> 6) * p.b_s1 + (col & 63) * Md::kES + k0 * p.b_sk;
+      wp = p.b + (colc >> 6) * p.b_s1 + (colc & 63) * Md::kES;
     uint4 rows[LOADS];
 #pragma unroll
     for (int r = 0; r < LOADS; ++r) {
-      if (WHOLE || k0 + (size_t)r * Md::kKPerLoad < p.k)
-        rows[r] = stream_load(wp + (size_t)r * kRowStep * p.b_sk);
-      else
-        rows[r] = make_uint4(0, 0, 0, 0);
+      const size_t kr = k0 + (size_t)r * kRowStep * Md::kKPerLoad;
+      const bool inside = WHOLE || kr < p.k;
+      rows[r] = stream_load(wp + ((inside ? kr : 0) / Md::kKPerLoad) * p.b_sk);
+      if constexpr (!WHOLE && MODE != kI8RowMajor && MODE != kI8K4) {
+        rows[r].x = inside ? rows[r].x : 0u, rows[r].y = inside ? rows[r].y : 0u;
+        rows[r].z = inside ? rows[r].z : 0u, rows[r].w = inside ? rows[r].w : 0u;
+      }
     }
     if (owner && y_is_read) y_old = yv[(tile_col0 + threadIdx.x) * p.y_s];
     if constexpr (MODE == kI8RowMajor || MODE == kI8K4) {
@@ -325,7 +332,9 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
 #pragma unroll
       for (int r = 0; r < LOADS; ++r) {
         const size_t k = k0 + r * kRowStep;
-        const int xb = (WHOLE || k < p.k) ? (int)x[k * p.x_sk] : 0;
+        const bool inside = WHOLE || k < p.k;
+        const int xl = (int)x[(inside ? k : 0) * p.x_sk];
+        const int xb = inside ? xl : 0;  // code 0 is +0.0 in both formats
         const float xv = x_e5m2 ? __builtin_amdgcn_cvt_f32_bf8(xb, 0) : __builtin_amdgcn_cvt_f32_fp8(xb, 0);
         const unsigned w[4] = {rows[r].x, rows[r].y, rows[r].z, rows[r].w};
 #pragma unroll
@@ -350,7 +359,9 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
 #pragma unroll
       for (int r = 0; r < LOADS; ++r) {
         const size_t k = k0 + r * kRowStep;
-        const float xv = (WHOLE || k < p.k) ? widen16(x[k * p.x_sk], bf) : 0.0f;
+        const bool inside = WHOLE || k < p.k;
+        const float xl = widen16(x[(inside ? k : 0) * p.x_sk], bf);
+        const float xv = inside ? xl : 0.0f;
         const unsigned w[4] = {rows[r].x, rows[r].y, rows[r].z, rows[r].w};
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -359,8 +370,6 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kernel(GemvArgs p) {
         }
       }
     }
-  } else if (owner && y_is_read) {
-    y_old = yv[(tile_col0 + threadIdx.x) * p.y_s];
   }
   // The eight row groups of a wave are summed in registers (every lane takes part); the first hands the wave's
   // sums to LDS, where the eight waves meet.
@@ -483,15 +492,20 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
   const size_t col = (size_t)tile * Md::kTileCols + (size_t)cl * kCols;
   const bool live = col < p.n && k0 < p.k;
 
-  // B's bytes are loaded once and stay in registers for all passes.
+  // B's bytes are loaded once and stay in registers for all passes. The loads are clamped into B, not guarded (a
+  // guard is a branch, and the compiler waits for the loads in flight at a branch it cannot prove uniform): a lane
+  // beyond N reads column 0, a row beyond K row 0, and what they read is zeroed afterwards.
   uint4 rows[kLoadsPerLane];
+  {
+    const size_t colc = col < p.n ? col : 0;
+    const char *wp = p.b + (colc >> 6) * p.b_s1 + (colc & 63) * Md::kES;
 #pragma unroll
-  for (int r = 0; r < kLoadsPerLane; ++r) rows[r] = make_uint4(0, 0, 0, 0);
-  if (live) {
-    const char *wp = p.b + (col >> 6) * p.b_s1 + (col & 63) * Md::kES + k0 * p.b_sk;
-#pragma unroll
-    for (int r = 0; r < kLoadsPerLane; ++r)
-      if (k0 + (size_t)r < p.k) rows[r] = stream_load(wp + (size_t)r * p.b_sk);
+    for (int r = 0; r < kLoadsPerLane; ++r) {
+      const bool inside = col < p.n && k0 + (size_t)r < p.k;
+      rows[r] = stream_load(wp + (inside ? k0 + (size_t)r : 0) * p.b_sk);
+      rows[r].x = inside ? rows[r].x : 0u, rows[r].y = inside ? rows[r].y : 0u;
+      rows[r].z = inside ? rows[r].z : 0u, rows[r].w = inside ? rows[r].w : 0u;
+    }
   }
 #pragma unroll
   for (int i0 = 0; i0 < MR; i0 += kRowChunk) {
@@ -570,15 +584,15 @@ __global__ void __launch_bounds__(kWaves * 64, 2) gemv_rows_kernel(GemvRowsArgs 
           for (int i = 0; i < kRowChunk; ++i) {
             if (i0 + i >= MR) continue;
             const char *xr = p.x + (size_t)(i0 + i) * p.x_row;
-            float xv = 0.0f;
-            if (k < p.k) {
-              if constexpr (Md::kFp8) {
-                const int xb = (int)reinterpret_cast<const uint8_t *>(xr)[k];
-                xv = MODE == kF8E5M2 ? __builtin_amdgcn_cvt_f32_bf8(xb, 0) : __builtin_amdgcn_cvt_f32_fp8(xb, 0);
-              } else {
-                xv = widen16(reinterpret_cast<const unsigned short *>(xr)[k], MODE == kBF16);
-              }
+            float xv;  // loaded from inside the row, zeroed beyond K: no branch between the loads
+            const size_t kc = k < p.k ? k : 0;
+            if constexpr (Md::kFp8) {
+              const int xb = (int)reinterpret_cast<const uint8_t *>(xr)[kc];
+              xv = MODE == kF8E5M2 ? __builtin_amdgcn_cvt_f32_bf8(xb, 0) : __builtin_amdgcn_cvt_f32_fp8(xb, 0);
+            } else {
+              xv = widen16(reinterpret_cast<const unsigned short *>(xr)[kc], MODE == kBF16);
             }
+            xv = k < p.k ? xv : 0.0f;
 #pragma unroll
             for (int c = 0; c < kCols; ++c) acc[i][c] = __fmaf_rn(xv, wide[c], acc[i][c]);
           }
