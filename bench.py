@@ -275,7 +275,7 @@ def _wl_ofp4(m, mx=False):
         return dict(fn=step, bytes=k * n // 2 + (k * n // 32 if mx else 0) + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm",
                     dtype="f4e2m1", keep=(w, sc or [], x, y),
                     name=f"E4M3 x {'MXFP4' if mx else 'OFP4'} GEMM {m}x4096x11008 (4-bit weights, columns contiguous in K, beta=0)",
-                    kernel="gemv_f4_kernel")
+                    kernel="gemv_f4_kernel" if m <= 16 else "gemv_f4_rows_kernel, or a converted copy + the fp8 / bf16 GEMM")
     return build
 
 
@@ -673,6 +673,9 @@ WORKLOADS = {
     "gemv_f8e4m3": (wl_gemv_f8, 10, 2, 128),
     "gemv_f8e4m3_f4_1x4096x11008": (_wl_ofp4(1), 10, 2, 128),
     "gemm_f8e4m3_f4_16x4096x11008": (_wl_ofp4(16), 10, 2, 128),
+    "gemm_f8e4m3_f4_32x4096x11008": (_wl_ofp4(32), 10, 2, 64),
+    "gemm_f8e4m3_f4_64x4096x11008": (_wl_ofp4(64), 10, 2, 32),
+    "gemm_f8e4m3_f4_128x4096x11008": (_wl_ofp4(128), 10, 2, 32),
     "gemv_f8e4m3_mxf4_1x4096x11008": (_wl_ofp4(1, mx=True), 10, 2, 128),
     "gemm_f8e4m3_mxf4_16x4096x11008": (_wl_ofp4(16, mx=True), 10, 2, 128),
     "gemv_i8_1x8192x28672": (wl_gemv_large, 10, 2, 32),

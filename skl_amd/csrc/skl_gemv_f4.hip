@@ -188,14 +188,135 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_f4_kernel(F4Args p) {
   }
 }
 
+// 17 to 128 rows of A, K <= 4096: the same decomposition with B held in registers for all of K (one pass of the K
+// loop above: four chunks per wave) while up to eight groups of 16 rows take their turns - the 4-bit weights cross
+// HBM once and never exist as a converted copy (which cost 22.5 MB read, 45 MB written and a tile GEMM behind it:
+// 37 / 40 / 45 us for 32 / 64 / 128 x 4096 x 11008). Two groups of 16 columns per workgroup; a row group's pieces of A
+// are requested two groups ahead; its sums go through one of two LDS blocks, added in wave order (one barrier per
+// group: the next group's barrier stands between this group's readers and the writers of the group after it).
+constexpr int kRowsCG = 4, kMaxRowGroups = 8;
+constexpr size_t kRowsMaxK = (size_t)kWaves * kChunk * kInFlight;  // 4096
+
+template <bool EXACT, int RG>
+__global__ void __launch_bounds__(kWaves * 64) gemv_f4_rows_kernel(F4Args p) {
+  constexpr int CG = kRowsCG;
+  __shared__ float red[2][kWaves][kMaxRows][CG * kCols + 1];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int jl = lane & 15, g = lane >> 4;
+  const v4i zero = {0, 0, 0, 0};
+  // The pieces of A for row group rg: chunk u of this wave, as in the kernel above; loaded from inside A and zeroed
+  // beyond M and K.
+  auto fragment_of = [&](int rg, v4i(&a)[kInFlight][4]) {
+    const size_t row = (size_t)rg * 16 + jl;
+    const bool row_ok = row < p.m;
+    const char *ap = p.a + (row_ok ? row : p.m - 1) * p.a_row;
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const size_t kc = ((size_t)wave + (size_t)u * kWaves) * kChunk, kl = kc + (size_t)g * 64;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const size_t ka0 = EXACT ? kl + 32 * h : kc + 64 * (size_t)(g >> 1) + 32 * h + 16 * (size_t)(g & 1);
+        const size_t ka1 = EXACT ? ka0 + 16 : ka0 + 128;
+        const v4i a0 = *reinterpret_cast<const v4i *>(ap + (ka0 < p.k ? ka0 : p.k - 16));
+        const v4i a1 = *reinterpret_cast<const v4i *>(ap + (ka1 < p.k ? ka1 : p.k - 16));
+        a[u][2 * h] = ka0 < p.k && row_ok ? a0 : zero;
+        a[u][2 * h + 1] = ka1 < p.k && row_ok ? a1 : zero;
+      }
+    }
+  };
+  v4i a[2][kInFlight][4];
+  fragment_of(0, a[0]);  // ahead of B: loads come back in the order of their requests
+  v4i b[kInFlight][CG][2];
+  unsigned sc[kInFlight][CG][2];
+#pragma unroll
+  for (int cg = 0; cg < CG; ++cg) {
+    const size_t col = ((size_t)blockIdx.x * CG + cg) * kCols + jl;
+    const size_t colc = col < p.n ? col : p.n - 1;
+    const char *bp = p.b + colc * p.b_col;
+    const uint8_t *sp = p.s ? p.s + colc * p.s_col : nullptr;
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const size_t kl = ((size_t)wave + (size_t)u * kWaves) * kChunk + (size_t)g * 64;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const size_t kb = kl + 32 * h;
+        b[u][cg][h] = load16(bp + (kb < p.k ? kb : p.k - 32) / 2);
+      }
+      sc[u][cg][0] = sc[u][cg][1] = 127u;
+      if (p.s) {  // the same for every thread
+        const size_t last = p.k / 32 - 1, i0 = kl / 32, i1 = kl / 32 + 1;
+        sc[u][cg][0] = sp[i0 < last ? i0 : last];
+        sc[u][cg][1] = sp[i1 < last ? i1 : last];
+      }
+    }
+  }
+  if constexpr (RG > 1) fragment_of(1, a[1]);
+  __builtin_amdgcn_sched_barrier(0);  // every request is out before the first use
+  const int row = threadIdx.x >> 4, tc = threadIdx.x & 15;
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) {
+    if ((size_t)rg * 16 >= p.m) break;  // the same for every thread of the workgroup
+    v4f acc[CG];
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg) acc[cg] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const v4i(&ar)[4] = a[rg & 1][u];
+        if constexpr (EXACT) {
+          v8bf aw[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const v4i &ah = ar[2 * h + (q >> 1)];
+            aw[q] = widen_e4m3((unsigned)((q & 1) ? ah.z : ah.x), (unsigned)((q & 1) ? ah.w : ah.y));
+          }
+#pragma unroll
+          for (int cg = 0; cg < CG; ++cg) {
+            const float scale = __uint_as_float(sc[u][cg][h] << 23);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              acc[cg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aw[q], widen_f4((unsigned)b[u][cg][h][q], scale), acc[cg], 0, 0, 0);
+          }
+        } else {
+          const v8i av = {ar[2 * h].x, ar[2 * h].y, ar[2 * h].z, ar[2 * h].w, ar[2 * h + 1].x, ar[2 * h + 1].y, ar[2 * h + 1].z, ar[2 * h + 1].w};
+#pragma unroll
+          for (int cg = 0; cg < CG; ++cg) {
+            const v8i bv = {b[u][cg][h].x, b[u][cg][h].y, b[u][cg][h].z, b[u][cg][h].w, 0, 0, 0, 0};
+            acc[cg] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[cg], 0, 4, 0, 127, 0, (int)sc[u][cg][h]);
+          }
+        }
+      }
+    if (rg + 2 < RG) fragment_of(rg + 2, a[rg & 1]);
+    // acc[cg][r] is row 16 rg + 4 g + r of C, column 16 cg + jl of the workgroup's.
+    float(*block)[kMaxRows][CG * kCols + 1] = red[rg & 1];
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) block[wave][4 * g + r][cg * kCols + jl] = acc[cg][r];
+    __syncthreads();
+    const size_t i = (size_t)rg * 16 + row;
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg) {
+      float sum = block[0][row][cg * kCols + tc];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) sum = __fadd_rn(sum, block[w][row][cg * kCols + tc]);
+      const size_t j = ((size_t)blockIdx.x * CG + cg) * kCols + tc;
+      if (i < p.m && j < p.n) skl_update(sum, p.c + i * p.c_row + j * p.c_col, p.alpha, p.beta);
+    }
+  }
+}
+
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 }  // namespace
 
-// 1 to 16 rows of A, K a multiple of 32, rows of A and columns of B on 16-byte boundaries.
+// 1 to 16 rows of A (to 128 with K <= 4096), K a multiple of 32, rows of A and columns of B on 16-byte boundaries.
 extern "C" int skl_hip_gemv_f4_supported(size_t m, size_t n, size_t k, const void *a, size_t rsa, size_t csa, const void *b,
                                          size_t ldb) {
-  if (m < 1 || m > (size_t)kMaxRows || n == 0 || k == 0 || (k % 32) != 0) return 0;
+  if (m < 1 || m > (size_t)(kMaxRows * kMaxRowGroups) || n == 0 || k == 0 || (k % 32) != 0) return 0;
+  // beyond 16 rows: B stays in registers for all of K, and there must be enough of it to be worth a pass per 128 rows
+  if (m > (size_t)kMaxRows && (k > kRowsMaxK || n * k < (size_t(1) << 20))) return 0;
   if (csa != 1 || !aligned16(a) || (m > 1 && (rsa % 16) != 0)) return 0;
   if (!aligned16(b) || (n > 1 && (ldb % 32) != 0)) return 0;
   return 1;
@@ -207,6 +328,30 @@ extern "C" int skl_hip_launch_gemv_f4(size_t m, size_t n, size_t k, skl_scalar a
   if (!skl_hip_gemv_f4_supported(m, n, k, a, rsa, csa, b, ldb)) {
     skl_hip_record_error(-2, "gemv_f4: unsupported problem");
     return -2;
+  }
+  if (m > (size_t)kMaxRows) {
+    const size_t grid = (n + (size_t)kRowsCG * kCols - 1) / ((size_t)kRowsCG * kCols);
+    if (grid > 0x7FFFFFFFu) {
+      skl_hip_record_error(-2, "gemv_f4: grid too large");
+      return -2;
+    }
+    F4Args p = {(const char *)a, rsa, (const char *)b, ldb / 2, scales, lds, 0, c, rsc, csc, m, n, k, alpha, beta};
+    hipStream_t st = skl_current_stream();
+    const unsigned blocks = (unsigned)grid, threads = kWaves * 64;
+    const bool exact = k <= kExactMaxK;
+#define SKL_F4_ROWS(RG)                                                           \
+  case RG:                                                                        \
+    if (exact) gemv_f4_rows_kernel<true, RG><<<blocks, threads, 0, st>>>(p);      \
+    else gemv_f4_rows_kernel<false, RG><<<blocks, threads, 0, st>>>(p);           \
+    break;
+    switch ((m + 15) / 16) {
+      SKL_F4_ROWS(2) SKL_F4_ROWS(3) SKL_F4_ROWS(4) SKL_F4_ROWS(5) SKL_F4_ROWS(6) SKL_F4_ROWS(7)
+      default:
+        if (exact) gemv_f4_rows_kernel<true, 8><<<blocks, threads, 0, st>>>(p);
+        else gemv_f4_rows_kernel<false, 8><<<blocks, threads, 0, st>>>(p);
+    }
+#undef SKL_F4_ROWS
+    return skl_check_launch("gemv_f4_rows");
   }
   // Four groups of 16 columns per workgroup from three rows of A on, where that still leaves at least 128
   // workgroups: the pieces of A are what a wave loads most of then.
