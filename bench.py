@@ -174,7 +174,7 @@ def _wl_small_batch(m):
             lib.skl_gemm_i8_i8_i32_gfx950(m, n, k, 1, x, k, w[i % nbuf], n, 0, y, n)
 
         kernel = ("gemv_rows_kernel" if m <= 3 else "gemv_mfma_scale_c_kernel + gemv_mfma_rows_kernel" if m <= 16 else
-                  "gemm_mfma_kernel (K shared between workgroups) + gemm_split_reduce_kernel")
+                  "gemv_mfma_scale_c_kernel + gemv_rowgroups_kernel")
         return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
                     name=f"int8 GEMM {m}x4096x11008 (decode with a batch of {m}: still a stream over W)", kernel=kernel)
     return build
@@ -690,6 +690,7 @@ WORKLOADS = {
     "gemm_i8_fused_16x4096x11008": (_wl_decode_fused(16), 10, 2, 64),
     "gemm_i8_32x4096x11008": (_wl_small_batch(32), 10, 2, 64),
     "gemm_i8_64x4096x11008": (_wl_small_batch(64), 10, 2, 32),
+    "gemm_i8_128x4096x11008": (_wl_small_batch(128), 10, 2, 32),
     "gemm_i8_p4x1c_16x4096x11008": (_wl_small_batch_p4x1c(16), 10, 2, 64),
     "gemm_i8_p4x1c_32x4096x11008": (_wl_small_batch_p4x1c(32), 10, 2, 32),
     "gemm_i8_p4x1c_112x4096x11008": (_wl_small_batch_p4x1c(112), 10, 2, 32),

@@ -929,59 +929,84 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
 
 
 // ---------------------------------------------------------------------------
-// 17 to 128 rows of int8 A against the K-packed B: the kernel above with RG groups of 16 rows. B's bytes are loaded
-// once and stay in registers while the row groups take their turns (a pass over B per 16 rows, as chunked calls of
-// the kernel above cost, is what this saves: 112 x 4096 x 11008 took 110 us in seven passes). The A fragment of a
-// row group - 16 bytes per lane and block, from L2 - is requested two groups ahead; the sums of a group (16
-// registers) go through the same LDS block as above, one group at a time, and meet the other workgroups' in C.
+// 17 to 128 rows of int8 A: the kernel above with RG groups of 16 rows, for the K-packed B (any K beyond what the
+// whole-K kernel below takes) and for the row-major B. B's bytes are loaded once - and, row-major, transposed once -
+// and stay in registers while the row groups take their turns (a pass over B per 16 rows, as chunked calls of the
+// kernel above cost, is what this saves: K-packed 112 x 4096 x 11008 took 110 us in seven passes; the tile kernels
+// take 29 / 31 us for 32 / 64 rows against a row-major B). The A fragment of a row group - 16 bytes per lane and
+// block, from L2 - is requested two groups ahead; the sums of a group go through the same LDS block as above, one
+// group at a time, and meet the other workgroups' in C.
 // ---------------------------------------------------------------------------
 constexpr int kK4MaxRowGroups = 8;
+constexpr int kRowMajorMaxRows = 80;  // row-major B: rows of A up to which the row groups beat the tile kernels (32 rows 19.5 against
+                                      // 28.8 us, 64 rows 27.4 against 30.8, 128 rows 42.5 against 35.2 for 4096 x 11008 weights)
 
-template <int RG>
-__global__ void __launch_bounds__(kMfmaWaves * 64, 2) gemv_k4_rowgroups_kernel(GemvMfmaArgs p) {
-  using Sh = MfmaShape<1, true>;
+template <int MODE, int RG>
+__global__ void __launch_bounds__(kMfmaWaves * 64, 2) gemv_rowgroups_kernel(GemvMfmaArgs p) {
+  constexpr bool kPacked = MODE == kI8K4;
+  static_assert(kPacked || MODE == kI8RowMajor, "int8 only");
+  using Sh = MfmaShape<1, kPacked>;
   constexpr int LC = Sh::kLaneCols, LR = Sh::kLaneRows, ITERS = Sh::kIters;
-  static_assert(LC == 4 && LR == 4, "four columns x four k per 128-bit load");
+  constexpr int kLaneK = LR * Sh::kKPerLoad;  // 16
   typedef int v4i __attribute__((ext_vector_type(4)));
   extern __shared__ __attribute__((aligned(16))) int mfma_red_raw[];
   int(*red)[16][Sh::kPitch] = reinterpret_cast<int(*)[16][Sh::kPitch]>(mfma_red_raw);
   const unsigned tile = blockIdx.x % p.tiles, slab = blockIdx.x / p.tiles;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int jl = lane & 15, g = lane >> 4;
   const size_t col = (size_t)tile * Sh::kTileCols + (size_t)jl * LC;
   const size_t kwave = ((size_t)slab * kMfmaWaves + wave) * (Sh::kBlockK * ITERS);
-  const bool col_ok = col < p.n;  // n is a multiple of four
-  const char *bp = p.b + col * 4;
+  const size_t colc = col < p.n ? col : 0;  // n is a multiple of the columns per lane: a lane is inside or outside
+  const char *bp = kPacked ? p.b + colc * 4 : p.b + (colc >> 6) * p.b_s1 + (colc & 63);
 
-  uint4 rows[ITERS][LR];
-#pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * 16;
-#pragma unroll
-    for (int r = 0; r < LR; ++r) {
-      if (col_ok && k0 + (size_t)r * 4 < p.k)
-        rows[it][r] = stream_load(bp + (k0 / 4 + r) * p.b_sk);
-      else
-        rows[it][r] = make_uint4(0, 0, 0, 0);
-    }
-  }
-  // The lane's 16 k of row 16 rg + jl, for each of the wave's blocks; zeros beyond M and K.
+  // The lane's 16 k of row 16 rg + jl, for each of the wave's blocks: loaded from inside A, zeroed beyond M and K
+  // (k is a multiple of 16) - which is also what makes the rows of B beyond K, read as row 0, count for nothing.
   auto fragment_of = [&](int rg, v4i(&xa)[ITERS]) {
     const size_t row = (size_t)rg * 16 + jl;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * 16;
-      if (row < p.m && k0 < p.k)
-        xa[it] = *reinterpret_cast<const v4i *>(p.a + row * p.a_row + k0);
-      else
-        xa[it] = v4i{0, 0, 0, 0};
+      const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * kLaneK;
+      const bool inside = row < p.m && k0 < p.k;
+      const v4i v = *reinterpret_cast<const v4i *>(p.a + (row < p.m ? row : p.m - 1) * p.a_row + (k0 < p.k ? k0 : 0));
+      xa[it] = v4i{inside ? v.x : 0, inside ? v.y : 0, inside ? v.z : 0, inside ? v.w : 0};
     }
   };
   v4i xa[3][ITERS];
-  fragment_of(0, xa[0]);
+  fragment_of(0, xa[0]);  // ahead of B: loads come back in the order of their requests
+  uint4 rows[ITERS][LR];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const size_t k0 = kwave + (size_t)it * Sh::kBlockK + (size_t)g * kLaneK;
+#pragma unroll
+    for (int r = 0; r < LR; ++r) {
+      const size_t kr = k0 + (size_t)r * Sh::kKPerLoad;
+      rows[it][r] = stream_load(bp + ((kr < p.k ? kr : 0) / Sh::kKPerLoad) * p.b_sk);  // clamped, not guarded
+    }
+  }
   if constexpr (RG > 1) fragment_of(1, xa[1]);
-  constexpr int kRowStep = kMfmaWaves * 64 / Sh::kTileCols;  // 4
-  const int tc = threadIdx.x % Sh::kTileCols;
+  __builtin_amdgcn_sched_barrier(0);  // every request is out before the first use
+  // t[it][q][c]: dword q of the operand of column c in block it - the lane's 16 k of that column, ascending
+  unsigned t[ITERS][4][LC];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    if constexpr (kPacked) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) t[it][q][0] = rows[it][q].x, t[it][q][1] = rows[it][q].y, t[it][q][2] = rows[it][q].z, t[it][q][3] = rows[it][q].w;
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint4 r0 = rows[it][4 * q], r1 = rows[it][4 * q + 1], r2 = rows[it][4 * q + 2], r3 = rows[it][4 * q + 3];
+        const unsigned a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
+        const unsigned a2[4] = {r2.x, r2.y, r2.z, r2.w}, a3[4] = {r3.x, r3.y, r3.z, r3.w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          transpose4x4(a0[d], a1[d], a2[d], a3[d], t[it][q][4 * d], t[it][q][4 * d + 1], t[it][q][4 * d + 2], t[it][q][4 * d + 3]);
+      }
+    }
+  }
+  constexpr int kRowStep = kMfmaWaves * 64 / Sh::kTileCols;  // 4 (K-packed), 1 (row-major)
+  constexpr int kPasses = 16 / kRowStep;
+  const int tc = threadIdx.x % Sh::kTileCols, i0 = threadIdx.x / Sh::kTileCols;
   const size_t j = (size_t)tile * Sh::kTileCols + tc;
 #pragma unroll
   for (int rg = 0; rg < RG; ++rg) {
@@ -991,33 +1016,35 @@ __global__ void __launch_bounds__(kMfmaWaves * 64, 2) gemv_k4_rowgroups_kernel(G
 #pragma unroll
     for (int c = 0; c < LC; ++c) acc[c] = v4i{0, 0, 0, 0};
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const unsigned t[4][4] = {{rows[it][0].x, rows[it][0].y, rows[it][0].z, rows[it][0].w},
-                                {rows[it][1].x, rows[it][1].y, rows[it][1].z, rows[it][1].w},
-                                {rows[it][2].x, rows[it][2].y, rows[it][2].z, rows[it][2].w},
-                                {rows[it][3].x, rows[it][3].y, rows[it][3].z, rows[it][3].w}};
+    for (int it = 0; it < ITERS; ++it)
 #pragma unroll
       for (int c = 0; c < LC; ++c) {
-        const v4i bw = {(int)t[0][c], (int)t[1][c], (int)t[2][c], (int)t[3][c]};
+        const v4i bw = {(int)t[it][0][c], (int)t[it][1][c], (int)t[it][2][c], (int)t[it][3][c]};
         acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[rg % 3][it], bw, acc[c], 0, 0, 0);
       }
-    }
-    // acc[c][r] is row 16 rg + 4 g + r of C, column 4 jl + c of the tile.
+    // acc[c][r] is row 16 rg + 4 g + r of C, column LC jl + c of the tile.
     if (rg > 0) __syncthreads();  // the previous group's sums have been read
 #pragma unroll
     for (int r = 0; r < 4; ++r)
-      *reinterpret_cast<v4i *>(&red[wave][4 * g + r][LC * jl]) = v4i{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-    __syncthreads();
-    if (j < p.n) {
-      for (size_t i = threadIdx.x / Sh::kTileCols; i < 16; i += kRowStep) {
-        const size_t row = (size_t)rg * 16 + i;
-        if (row >= p.m) break;
-        unsigned sum = 0;
 #pragma unroll
-        for (int w = 0; w < kMfmaWaves; ++w) sum += (unsigned)red[w][i][tc];
-        (void)__hip_atomic_fetch_add(p.c + row * p.c_row + j * p.c_s, (int)((unsigned)p.alpha.i * sum), __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_AGENT);
-      }
+      for (int c4 = 0; c4 < LC / 4; ++c4)
+        *reinterpret_cast<v4i *>(&red[wave][4 * g + r][LC * jl + 4 * c4]) = v4i{acc[4 * c4][r], acc[4 * c4 + 1][r], acc[4 * c4 + 2][r], acc[4 * c4 + 3][r]};
+    __syncthreads();
+    // all of the thread's sums are read from LDS before the first goes out
+    int sums[kPasses];
+#pragma unroll
+    for (int q = 0; q < kPasses; ++q) {
+      unsigned sum = 0;
+#pragma unroll
+      for (int w = 0; w < kMfmaWaves; ++w) sum += (unsigned)red[w][i0 + q * kRowStep][tc];
+      sums[q] = (int)((unsigned)p.alpha.i * sum);
+    }
+    if (j < p.n) {
+      int *cp = p.c + ((size_t)rg * 16 + i0) * p.c_row + j * p.c_s;
+#pragma unroll
+      for (int q = 0; q < kPasses; ++q)
+        if ((size_t)rg * 16 + i0 + q * kRowStep < p.m)
+          (void)__hip_atomic_fetch_add(cp + (size_t)q * kRowStep * p.c_row, sums[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
@@ -1577,7 +1604,9 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int lay
   // weights of 4096 x 11008, on the tile kernels twice that.
   const bool fused_single_row = mode != kI8RowMajor && g->m == 1 && (g->bias || g->max || g->rq.act || g->rq.q);
   const size_t min_rows = mode == kI8RowMajor ? kMfmaMinRowsInt8 : fused_single_row ? 1 : 2;
-  if (g->m < min_rows || g->m > (size_t)kMfmaMaxRows || g->k == 0 || g->n == 0) return 0;
+  // int8 against a row-major B: beyond 16 rows in groups of 16 with B held in registers
+  const size_t max_rows = mode == kI8RowMajor && !(g->bias || g->max || g->rq.act || g->rq.q) ? (size_t)kRowMajorMaxRows : (size_t)kMfmaMaxRows;
+  if (g->m < min_rows || g->m > max_rows || g->k == 0 || g->n == 0) return 0;
   const size_t min_bytes = fused_single_row ? size_t(1) << 20 : mfma_rows_min_bytes(mode, g->m);
   if ((g->k % piece) != 0 || (g->n % piece) != 0 || g->k * g->n * es < min_bytes) return 0;
   if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % piece) != 0) return 0;
@@ -1650,22 +1679,30 @@ int launch_mfma_rows(const GemvMfmaArgs &args) {
       int rc = skl_check_launch("gemv_mfma_scale_c");
       if (rc != 0) return rc;
     }
-    if constexpr (MODE == kI8K4) {
-      if (p.m > (size_t)kMfmaMaxRows) {  // more than one group of 16 rows: one pass over B for all of them
-        constexpr unsigned threads = kMfmaWaves * 64;
-        static_assert(kMfmaLds <= 64 * 1024, "fits the default LDS limit of a launch");
-        hipStream_t st = skl_current_stream();
-        switch ((p.m + 15) / 16) {
-          case 2: gemv_k4_rowgroups_kernel<2><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
-          case 3: gemv_k4_rowgroups_kernel<3><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
-          case 4: gemv_k4_rowgroups_kernel<4><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
-          case 5: gemv_k4_rowgroups_kernel<5><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
-          case 6: gemv_k4_rowgroups_kernel<6><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
-          case 7: gemv_k4_rowgroups_kernel<7><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
-          default: gemv_k4_rowgroups_kernel<8><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+    if (p.m > (size_t)kMfmaMaxRows) {  // more than one group of 16 rows: one pass over B for all of them
+      constexpr unsigned threads = kMfmaWaves * 64;
+      hipStream_t st = skl_current_stream();
+      static std::atomic<bool> groups_configured{false};
+      if (!groups_configured.load(std::memory_order_acquire)) {
+        for (const void *f : {reinterpret_cast<const void *>(gemv_rowgroups_kernel<MODE, 2>), reinterpret_cast<const void *>(gemv_rowgroups_kernel<MODE, 3>),
+                              reinterpret_cast<const void *>(gemv_rowgroups_kernel<MODE, 4>), reinterpret_cast<const void *>(gemv_rowgroups_kernel<MODE, 5>),
+                              reinterpret_cast<const void *>(gemv_rowgroups_kernel<MODE, 6>), reinterpret_cast<const void *>(gemv_rowgroups_kernel<MODE, 7>),
+                              reinterpret_cast<const void *>(gemv_rowgroups_kernel<MODE, 8>)}) {
+          int rc = skl_check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLds), "gemv_rowgroups: LDS size");
+          if (rc != 0) return rc;
         }
-        return skl_check_launch("gemv_k4_rowgroups");
+        groups_configured.store(true, std::memory_order_release);
       }
+      switch ((p.m + 15) / 16) {
+        case 2: gemv_rowgroups_kernel<MODE, 2><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+        case 3: gemv_rowgroups_kernel<MODE, 3><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+        case 4: gemv_rowgroups_kernel<MODE, 4><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+        case 5: gemv_rowgroups_kernel<MODE, 5><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+        case 6: gemv_rowgroups_kernel<MODE, 6><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+        case 7: gemv_rowgroups_kernel<MODE, 7><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+        default: gemv_rowgroups_kernel<MODE, 8><<<(unsigned)grid, threads, kMfmaLds, st>>>(p); break;
+      }
+      return skl_check_launch("gemv_rowgroups");
     }
     kernel<<<(unsigned)grid, kMfmaWaves * 64, kMfmaLds, skl_current_stream()>>>(p);
     return skl_check_launch("gemv_mfma_rows");
