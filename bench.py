@@ -128,6 +128,30 @@ def wl_gemv_kc(lib, rng):
                 name="int8 GEMV 1x4096x11008, W with K contiguous ([n][k]), beta=0", kernel="gemv_kc_kernel<int8>")
 
 
+def _wl_batch_kc(m, kind="i8"):
+    """A decode batch against weights stored column by column (B with K contiguous, [out][in])."""
+    def build(lib, rng):
+        k, n, nbuf = 4096, 11008, 8
+        if kind == "i8":
+            w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
+            x = DeviceBuffer.from_array(rand_i8(rng, m * k))
+        else:
+            w = [DeviceBuffer.from_array(rng.integers(0, 0x78, size=k * n, dtype=np.uint8)) for _ in range(nbuf)]
+            x = DeviceBuffer.from_array(rng.integers(0, 0x78, size=m * k, dtype=np.uint8))
+        y = DeviceBuffer(4 * m * n)
+
+        def step(i):
+            if kind == "i8":
+                lib.skl_gemm_i8rc_i8rc_i32rc_gfx950(m, n, k, 1, x, k, 1, w[i % nbuf], 1, k, 0, y, n, 1)
+            else:
+                lib.skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950(m, n, k, 1.0, x, k, 1, w[i % nbuf], 1, k, 0.0, y, n, 1)
+
+        return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype=kind, keep=(w, x, y),
+                    name=f"{'int8' if kind == 'i8' else 'E4M3'} GEMM {m}x4096x11008, W with K contiguous ([n][k]), beta=0",
+                    kernel="gemv_kc_kernel (up to 4 rows), gemv_kc_rows_kernel (up to 128)")
+    return build
+
+
 def wl_gemv_kc_fused(lib, rng):
     """A quantised linear layer at decode time on its [out][in] weight: int8 in, bias, ReLU, int8 out, C not written."""
     import skl_amd
@@ -682,6 +706,10 @@ WORKLOADS = {
     "gemv_i8_kcontig": (wl_gemv_kc, 10, 2, 128),
     "gemv_i8_kcontig_fused": (wl_gemv_kc_fused, 10, 2, 128),
     "gemv_bf16_kcontig": (wl_gemv_kc_bf16, 10, 2, 64),
+    "gemm_i8_kcontig_4x4096x11008": (_wl_batch_kc(4), 10, 2, 64),
+    "gemm_i8_kcontig_16x4096x11008": (_wl_batch_kc(16), 10, 2, 64),
+    "gemm_i8_kcontig_64x4096x11008": (_wl_batch_kc(64), 10, 2, 32),
+    "gemm_f8e4m3_kcontig_16x4096x11008": (_wl_batch_kc(16, "f8"), 10, 2, 64),
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 10, 2, 64),
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 10, 2, 64),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 10, 2, 64),

@@ -192,6 +192,7 @@ static int outcome(int rc) { return rc == 0 ? TAKEN : rc == SKL_HIP_ERR_WORKSPAC
 static int gemv_on_device(const skl_gemm_canon *g) {
   int r = DECLINED;
   if (skl_hip_gemv_kc_supported(g) && (r = outcome(skl_hip_launch_gemv_kc(g))) != DECLINED) return r;
+  if (skl_hip_gemv_kc_rows_supported(g) && (r = outcome(skl_hip_launch_gemv_kc_rows(g))) != DECLINED) return r;
   if (g->m == 1 && skl_hip_gemv_supported(g, 0) && (r = outcome(skl_hip_launch_gemv(g, 0))) != DECLINED) return r;
   if (skl_hip_gemv_mfma_rows_supported(g, 0) && (r = outcome(skl_hip_launch_gemv_mfma_rows(g, 0))) != DECLINED) return r;
   if (skl_hip_gemv_rows_supported(g) && (r = outcome(skl_hip_launch_gemv_rows(g))) != DECLINED) return r;
@@ -199,7 +200,7 @@ static int gemv_on_device(const skl_gemm_canon *g) {
 }
 
 static int gemv_would_take(const skl_gemm_canon *g) {
-  return skl_hip_gemv_kc_supported(g) || (g->m == 1 && skl_hip_gemv_supported(g, 0)) ||
+  return skl_hip_gemv_kc_supported(g) || skl_hip_gemv_kc_rows_supported(g) || (g->m == 1 && skl_hip_gemv_supported(g, 0)) ||
          skl_hip_gemv_mfma_rows_supported(g, 0) || skl_hip_gemv_rows_supported(g);
 }
 

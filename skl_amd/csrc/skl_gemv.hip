@@ -1607,6 +1607,7 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int lay
   // int8 against a row-major B: beyond 16 rows in groups of 16 with B held in registers
   const size_t max_rows = mode == kI8RowMajor && !(g->bias || g->max || g->rq.act || g->rq.q) ? (size_t)kRowMajorMaxRows : (size_t)kMfmaMaxRows;
   if (g->m < min_rows || g->m > max_rows || g->k == 0 || g->n == 0) return 0;
+  if (g->m > 64 && (g->a_s1 != 64 * g->a_s0 || g->rsc1 != 64 * g->rsc0)) return 0;  // rows a fixed distance apart
   const size_t min_bytes = fused_single_row ? size_t(1) << 20 : mfma_rows_min_bytes(mode, g->m);
   if ((g->k % piece) != 0 || (g->n % piece) != 0 || g->k * g->n * es < min_bytes) return 0;
   if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % piece) != 0) return 0;

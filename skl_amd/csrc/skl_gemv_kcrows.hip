@@ -1,0 +1,232 @@
+// skl_gemv_kcrows.hip - decode batches against weights stored column by column: 5 to 128 rows of A (K contiguous)
+// times a B whose columns are contiguous in K - a linear layer's [out][in] weight -, int8 and the OCP fp8 kinds,
+// K <= 4096. The reference's generic kernels take any strides (ref/gemm/gemm_i8rc_i8rc_i32rc.c:9-24,
+// ref/gemm/gemm_f8rc_f8rc_f32rc.c); up to four rows skl_gemv.hip's gemv_kc_kernel streams such a B with dot
+// products, and without this file everything above went to the tile kernels (16 x 4096 x 11008: 27 us for 45 MB).
+//
+// With K contiguous in both operands a 16-byte load IS a matrix-core operand: 16 consecutive k of one column of B,
+// or of one row of A. A workgroup of eight waves owns 64 columns (four groups of 16) and ALL of K, 512 k per wave,
+// so the sums of a column tile never leave the workgroup: they meet in LDS in wave order - the same bits on every
+// run -, C is written once with the alpha / beta step applied in place, and no scratch memory is involved. All of
+// B is in flight from the start (32 loads per lane) and stays in registers while up to eight groups of 16 rows of A
+// take their turns; a group's pieces of A (from L2: every workgroup reads all of A) are requested two groups ahead.
+// Instruction t of a 256-k chunk takes k = chunk + 64 t + 16 g + (0..15) from the lanes of k group g: the four
+// groups read 64 consecutive bytes of a column per load. Which k meet in which instruction is free as long as
+// A's and B's lanes hold the same ones.
+// int8: v_mfma_i32_16x16x64_i8. fp8: every E4M3 / E5M2 value is an f16 value, so the bytes are widened in registers
+// and multiplied by v_mfma_f32_16x16x32_f16 - exact products, fp32 sums, inside the reference's bound for any K (the
+// fp8 instructions align the products of an instruction and drop low bits, which short K would show).
+// Loads are clamped into the operands instead of guarded (a guard is a branch, and the compiler waits for the loads in
+// flight at a branch it cannot prove uniform): k beyond K meets zeros of A, rows beyond M and columns beyond N are
+// computed and not written.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <type_traits>
+
+#include "skl_device.hpp"
+#include "skl_fp8.hpp"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 8, kColGroups = 4, kCols = 16 * kColGroups;  // 64 columns per workgroup
+constexpr int kChunk = 256, kChunks = 2;                           // k per wave: 512
+constexpr int kMaxRowGroups = 8, kMinRows = 5;
+constexpr size_t kMaxK = (size_t)kWaves * kChunks * kChunk;        // 4096
+constexpr int kPitch = kCols + 1;
+enum { kI8 = 0, kE4M3 = 1, kE5M2 = 2, kMixed = 3 };  // kMixed: E4M3 A with E5M2 B
+
+struct KcRowsArgs {
+  const char *a;  // row i at a + i * a_row (bytes), K contiguous
+  size_t a_row;
+  const char *b;  // column j at b + j * b_col (bytes), K contiguous
+  size_t b_col;
+  void *c;        // element (i, j) at i * c_row + j * c_col (elements)
+  size_t c_row, c_col;
+  size_t m, n, k;
+  skl_scalar alpha, beta;
+};
+
+__device__ __forceinline__ v4i load16(const char *p) { return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(p)); }
+
+template <int KIND, int RG>
+__global__ void __launch_bounds__(kWaves * 64) gemv_kc_rows_kernel(KcRowsArgs p) {
+  constexpr bool kInt = KIND == kI8;
+  using Acc = typename std::conditional<kInt, int, float>::type;
+  typedef Acc v4acc __attribute__((ext_vector_type(4)));
+  extern __shared__ __attribute__((aligned(16))) int kc_red_raw[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int jl = lane & 15, g = lane >> 4;
+  const size_t kwave = (size_t)wave * (kChunks * kChunk) + (size_t)g * 16;  // the lane's first k
+  const v4i zero = {0, 0, 0, 0};
+  // piece (u, t) of a lane: 16 k from kwave + 256 u + 64 t
+  auto fragment_of = [&](int rg, v4i(&xa)[kChunks][4]) {
+    const size_t row = (size_t)rg * 16 + jl;
+    const bool row_ok = row < p.m;
+    const char *ap = p.a + (row_ok ? row : p.m - 1) * p.a_row;
+#pragma unroll
+    for (int u = 0; u < kChunks; ++u)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const size_t k0 = kwave + (size_t)u * kChunk + (size_t)t * 64;  // k is a multiple of 16: inside or outside
+        const v4i v = *reinterpret_cast<const v4i *>(ap + (k0 < p.k ? k0 : 0));
+        xa[u][t] = k0 < p.k && row_ok ? v : zero;
+      }
+  };
+  v4i xa[2][kChunks][4];
+  fragment_of(0, xa[0]);  // ahead of B: loads come back in the order of their requests
+  v4i b[kColGroups][kChunks][4];
+#pragma unroll
+  for (int cg = 0; cg < kColGroups; ++cg) {
+    const size_t col = (size_t)blockIdx.x * kCols + (size_t)cg * 16 + jl;
+    const char *bp = p.b + (col < p.n ? col : p.n - 1) * p.b_col;
+#pragma unroll
+    for (int u = 0; u < kChunks; ++u)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const size_t k0 = kwave + (size_t)u * kChunk + (size_t)t * 64;
+        b[cg][u][t] = load16(bp + (k0 < p.k ? k0 : 0));
+      }
+  }
+  if constexpr (RG > 1) fragment_of(1, xa[1]);
+  __builtin_amdgcn_sched_barrier(0);  // every request is out before the first use
+  const int row = threadIdx.x >> 6, tc = threadIdx.x & 63;  // 512 threads: 8 rows x 64 columns at a time
+  const size_t j = (size_t)blockIdx.x * kCols + tc;
+  Acc *cbase = reinterpret_cast<Acc *>(p.c);
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) {
+    if ((size_t)rg * 16 >= p.m) break;  // the same for every thread of the workgroup
+    v4acc acc[kColGroups];
+#pragma unroll
+    for (int cg = 0; cg < kColGroups; ++cg) acc[cg] = v4acc{0, 0, 0, 0};
+#pragma unroll
+    for (int u = 0; u < kChunks; ++u)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const v4i av = xa[rg & 1][u][t];
+        if constexpr (kInt) {
+#pragma unroll
+          for (int cg = 0; cg < kColGroups; ++cg) acc[cg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, b[cg][u][t], acc[cg], 0, 0, 0);
+        } else {
+          constexpr bool a_e5m2 = KIND == kE5M2, b_e5m2 = KIND != kE4M3;
+          const auto a0 = skl_fp8::widen8_to_f16<a_e5m2>((unsigned)av.x, (unsigned)av.y);
+          const auto a1 = skl_fp8::widen8_to_f16<a_e5m2>((unsigned)av.z, (unsigned)av.w);
+#pragma unroll
+          for (int cg = 0; cg < kColGroups; ++cg) {
+            // an opaque copy: the widened form of B (twice the registers) must not be kept from one row group to
+            // the next
+            v4i bv = b[cg][u][t];
+            asm volatile("" : "+v"(bv));
+            acc[cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, skl_fp8::widen8_to_f16<b_e5m2>((unsigned)bv.x, (unsigned)bv.y), acc[cg], 0, 0, 0);
+            acc[cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, skl_fp8::widen8_to_f16<b_e5m2>((unsigned)bv.z, (unsigned)bv.w), acc[cg], 0, 0, 0);
+          }
+        }
+      }
+    if (rg + 2 < RG) fragment_of(rg + 2, xa[rg & 1]);
+    // acc[cg][r] is row 16 rg + 4 g + r of C, column 16 cg + jl of the workgroup's. Two blocks of sums take turns:
+    // the next group's barrier stands between this group's readers and the writers of the group after it.
+    Acc(*red)[16][kPitch] = reinterpret_cast<Acc(*)[16][kPitch]>(kc_red_raw + (rg & 1) * kWaves * 16 * kPitch);
+#pragma unroll
+    for (int cg = 0; cg < kColGroups; ++cg)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][4 * g + r][cg * 16 + jl] = acc[cg][r];
+    __syncthreads();
+    Acc sums[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int il = row + kWaves * q;
+      Acc sum = red[0][il][tc];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) {
+        if constexpr (kInt) sum = (int)((unsigned)sum + (unsigned)red[w][il][tc]);
+        else sum = __fadd_rn(sum, red[w][il][tc]);
+      }
+      sums[q] = sum;
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const size_t i = (size_t)rg * 16 + row + kWaves * q;
+      if (i < p.m && j < p.n) skl_update(sums[q], cbase + i * p.c_row + j * p.c_col, p.alpha, p.beta);
+    }
+  }
+}
+
+constexpr size_t kLds = (size_t)2 * kWaves * 16 * kPitch * 4;  // 66 560 bytes
+
+template <int KIND, int RG>
+int launch_groups(const KcRowsArgs &p, unsigned grid, hipStream_t st) {
+  static std::atomic<bool> configured{false};  // per instantiation; racing threads set the same value
+  if (!configured.load(std::memory_order_acquire)) {
+    int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_kc_rows_kernel<KIND, RG>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds), "gemv_kc_rows: LDS size");
+    if (rc != 0) return rc;
+    configured.store(true, std::memory_order_release);
+  }
+  gemv_kc_rows_kernel<KIND, RG><<<grid, kWaves * 64, kLds, st>>>(p);
+  return skl_check_launch("gemv_kc_rows");
+}
+
+template <int KIND>
+int launch_kind(const KcRowsArgs &p, unsigned grid) {
+  hipStream_t st = skl_current_stream();
+  switch ((p.m + 15) / 16) {
+    case 1: return launch_groups<KIND, 1>(p, grid, st);
+    case 2: return launch_groups<KIND, 2>(p, grid, st);
+    case 3: return launch_groups<KIND, 3>(p, grid, st);
+    case 4: return launch_groups<KIND, 4>(p, grid, st);
+    case 5: return launch_groups<KIND, 5>(p, grid, st);
+    case 6: return launch_groups<KIND, 6>(p, grid, st);
+    case 7: return launch_groups<KIND, 7>(p, grid, st);
+    default: return launch_groups<KIND, 8>(p, grid, st);
+  }
+}
+
+int kind_of(const skl_gemm_canon *g) {
+  if (g->ta == SKL_DT_I8 && g->tb == SKL_DT_I8) return kI8;
+  if (g->ta == SKL_DT_F8E4M3 && g->tb == SKL_DT_F8E4M3) return kE4M3;
+  if (g->ta == SKL_DT_F8E5M2 && g->tb == SKL_DT_F8E5M2) return kE5M2;
+  if (g->ta == SKL_DT_F8E4M3 && g->tb == SKL_DT_F8E5M2) return kMixed;
+  return -1;
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+}  // namespace
+
+// 5 to 128 rows of A and a B of at least 1 MiB, both with K contiguous (16-byte aligned rows and columns a fixed
+// distance apart, K a multiple of 16 up to 4096), C flat or in blocks of 64, no fused steps.
+extern "C" int skl_hip_gemv_kc_rows_supported(const skl_gemm_canon *g) {
+  if (kind_of(g) < 0) return 0;
+  if (g->bias || g->max || g->rq.act || g->rq.q) return 0;
+  if (g->c_row_shift != 6 || g->c_col_shift != 6) return 0;
+  if (g->m < (size_t)kMinRows || g->m > (size_t)(16 * kMaxRowGroups) || g->n == 0 || g->k == 0 || g->k > kMaxK) return 0;
+  if ((g->k % 16) != 0 || g->k * g->n < (size_t(1) << 20)) return 0;
+  if (g->a_sk != 1 || g->b_sk != 1) return 0;
+  if (!aligned16(g->a) || (g->a_s0 % 16) != 0 || (g->m > 64 && g->a_s1 != 64 * g->a_s0)) return 0;
+  if (!aligned16(g->b) || (g->b_s0 % 16) != 0 || (g->n > 64 && g->b_s1 != 64 * g->b_s0)) return 0;
+  if ((g->m > 64 && g->rsc1 != 64 * g->rsc0) || (g->n > 64 && g->csc1 != 64 * g->csc0)) return 0;
+  return 1;
+}
+
+extern "C" int skl_hip_launch_gemv_kc_rows(const skl_gemm_canon *g) {
+  if (!skl_hip_gemv_kc_rows_supported(g)) {
+    skl_hip_record_error(-2, "gemv_kc_rows: unsupported problem");
+    return -2;
+  }
+  const size_t grid = (g->n + kCols - 1) / kCols;
+  if (grid > 0x7FFFFFFFu) {
+    skl_hip_record_error(-2, "gemv_kc_rows: grid too large");
+    return -2;
+  }
+  const KcRowsArgs p = {(const char *)g->a, g->a_s0, (const char *)g->b, g->b_s0, g->c, g->rsc0, g->csc0,
+                        g->m, g->n, g->k, g->alpha, g->beta};
+  switch (kind_of(g)) {
+    case kI8: return launch_kind<kI8>(p, (unsigned)grid);
+    case kE4M3: return launch_kind<kE4M3>(p, (unsigned)grid);
+    case kE5M2: return launch_kind<kE5M2>(p, (unsigned)grid);
+    default: return launch_kind<kMixed>(p, (unsigned)grid);
+  }
+}

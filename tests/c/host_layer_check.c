@@ -362,6 +362,13 @@ int __wrap_skl_hip_launch_gemv_kc(const skl_gemm_canon *g) {
   gemm_over_canon(g, 0, "dot-product GEMV");
   return 0;
 }
+int __wrap_skl_hip_launch_gemv_kc_rows(const skl_gemm_canon *g) {
+  SCARCE("decode batch on K-contiguous weights (stand-in)");
+  EXPECT(skl_hip_gemv_kc_rows_supported(g), "decode batch on K-contiguous weights handed a problem it does not support");
+  ++g_path[P_KC];
+  gemm_over_canon(g, 0, "decode batch on K-contiguous weights");
+  return 0;
+}
 int __wrap_skl_hip_launch_gemv_noalloc(const skl_gemm_canon *g) {
   if (g->m < 1 || g->m > 8 || g->m * g->n > 65536 || (g->m == 1 ? !skl_hip_gemv_supported(g, 0) : !skl_hip_gemv_rows_supported(g))) {
     skl_hip_record_error(SKL_HIP_ERR_BAD_ARGUMENT, "noalloc (stand-in)");

@@ -419,6 +419,38 @@ def test_k_contiguous_b_int8_bit_exact(gpu, m):
                 assert np.array_equal(run_gemm(gpu, "rc", case, a, b, c, mode), want), (m, n, k, mode)
 
 
+@pytest.mark.parametrize("m", (5, 16, 17, 40, 100, 128))
+def test_k_contiguous_b_decode_batches_int8_bit_exact(gpu, m):
+    """5 to 128 rows of A against a B stored column by column, K <= 4096 (ref/gemm/gemm_i8rc_i8rc_i32rc.c:9-24 with
+    rsb = 1): one workgroup per 64 columns takes all of K on the matrix cores, row groups of 16 (ragged last groups:
+    5, 17, 40, 100), C written once. The config-2 width, N off the 64-column workgroups, K off the waves' 512 and the
+    chunks of 256, padded strides, alpha / beta with wrap-around on a C of extreme values, both pointer modes; a K
+    beyond 4096 (the tile kernels) for comparison."""
+    rng = np.random.default_rng(160 + m)
+    for (n, k, pad) in ((11008, 1024 if m > 16 else 4096, 0), (1037, 4080, 16), (300, 3504, 32), (4100, 272, 0), (260, 4112, 0)):
+        for alpha, beta in ((1, 0), (0x01010101, -77), (-3, 1)):
+            case = _kc_case("i8", None, m, n, k, alpha, beta, pad)
+            a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+            c[:] = rng.integers(-2 ** 31, 2 ** 31, size=c.size)
+            want = run_oracle_gemm(case, a, b, c)
+            for mode in ("device", "host"):
+                assert np.array_equal(run_gemm(gpu, "rc", case, a, b, c, mode), want), (m, n, k, alpha, beta, mode)
+
+
+@pytest.mark.parametrize("ta,tb", FP8_PAIRS)
+@pytest.mark.parametrize("m", (5, 16, 33, 128))
+def test_k_contiguous_b_decode_batches_fp8(gpu, ta, tb, m):
+    """The fp8 kinds of the same kernel (operands widened to f16 in registers: exact products, fp32 sums in a fixed
+    order): inside the reference's bound without any allowance, and the same bits on every run."""
+    for (n, k, pad) in ((11008, 1024 if m > 16 else 4096, 0), (1037, 2064, 16), (300, 3504, 32)):
+        case = _kc_case(ta, tb, m, n, k, 1.5, -0.5, pad)
+        a, b, c = case.make_inputs(m * 37 + n + k)
+        for mode in ("device", "host"):
+            got = run_gemm(gpu, "rc", case, a, b, c, mode)
+            support.assert_fp_gemm_close(case, a, b, c, got)
+            assert np.array_equal(got.view(np.uint8), run_gemm(gpu, "rc", case, a, b, c, mode).view(np.uint8))
+
+
 @pytest.mark.parametrize("ta,tb", (("bf16", "bf16"), ("f16", "f16")) + FP8_PAIRS)
 @pytest.mark.parametrize("m", (1, 4))
 def test_k_contiguous_b_floating_point(gpu, ta, tb, m):
