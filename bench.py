@@ -328,10 +328,10 @@ def _wl_small_batch_p4x1c(m):
         def step(i):
             lib.skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(m, n, k // 4, 1, x, k, 4, w[i % nbuf], 4 * n, 0, y, n)
 
-        kernel = "gemv_mfma_rows_kernel<int8 K-packed>" if m <= 16 else "gemv_k4_rowgroups_kernel"
+        kernel = "gemv_k4_wholek_kernel" if m <= 128 else "a copy of W with K contiguous + the tile kernels"
         return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype="i8", keep=(w, x, y),
                     name=f"int8 GEMM {m}x4096x11008 (W in the p4x1c K-packed layout, decode with a batch of {m})",
-                    kernel="gemv_mfma_scale_c_kernel + " + kernel)
+                    kernel=kernel)
     return build
 
 
@@ -782,14 +782,14 @@ MEASURED_PEAK_OF = {"hbm": "peak_hbm_read", "i8": "peak_mfma_i8_random", "f8": "
 # summarised in profiles/gemv_cvt_gemm_hbm_traffic.pmc.txt.
 TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/gemv_cvt_gemm_hbm_traffic.pmc.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "gemv_i8": int((22061.5 * 1.998 + 817.0) * 1024),
-    "cvt_f32_f8e4m3_8192sq": int((131136.4 * 1.998 + 65536.0) * 1024),
-    "gemm_i8_8192": int((393334.9 * 1.998 + 262434.0) * 1024),
-    "gemm_f8e4m3_8192_kcontig": int((393395.0 * 1.998 + 262727.1) * 1024),
+    "gemv_i8": int((22060.5 * 1.998 + 817.0) * 1024),
+    "cvt_f32_f8e4m3_8192sq": int((131136.5 * 1.998 + 65536.0) * 1024),
+    "gemm_i8_8192": int((393337.5 * 1.998 + 262375.7) * 1024),
+    "gemm_f8e4m3_8192_kcontig": int((393401.7 * 1.998 + 262659.2) * 1024),
     "copy_u32_4096sq": int((32800.9 * 1.998 + 65536) * 1024),
-    "gemm_i8_16x4096x11008": int((22353.1 * 1.998 + 6192.0) * 1024),
-    "gemv_f8e4m3_f4_1x4096x11008": int((11058.5 * 1.998 + 43.0) * 1024),
-    "gemm_i8_p4x1c_112x4096x11008": int((23896.7 * 1.998 + 24080.0) * 1024),
+    "gemm_i8_16x4096x11008": int((22349.1 * 1.998 + 6192.0) * 1024),
+    "gemv_f8e4m3_f4_1x4096x11008": int((11060.0 * 1.998 + 43.0) * 1024),
+    "gemm_i8_p4x1c_112x4096x11008": int((23911.2 * 1.998 + 4816.0) * 1024),
 }
 
 

@@ -304,8 +304,11 @@ static int k4_then_epilogue(const skl_gemm_desc *d) {
 static int gemm_fast_path(const skl_gemm_canon *g, int fused, int launch) {
   int r = DECLINED;
   if (!fused && (r = gemv_paths(g, launch)) != DECLINED) return r;
-  /* the decode-batch kernel of the floating-point kinds applies the fused steps itself, so that a call gives the
-   * same bits with and without them */
+  /* the kernels for a B with K contiguous and the decode-batch kernel of the floating-point kinds apply the fused
+   * steps themselves, so that a call gives the same bits with and without them */
+  if (fused && skl_hip_gemv_kc_supported(g) && (r = launch ? outcome(skl_hip_launch_gemv_kc(g)) : TAKEN) != DECLINED) return r;
+  if (fused && skl_hip_gemv_kc_rows_supported(g) && (r = launch ? outcome(skl_hip_launch_gemv_kc_rows(g)) : TAKEN) != DECLINED)
+    return r;
   if (fused && skl_hip_gemv_mfma_rows_supported(g, 0) &&
       (r = launch ? outcome(skl_hip_launch_gemv_mfma_rows(g, 0)) : TAKEN) != DECLINED)
     return r;
@@ -516,8 +519,9 @@ static int gemm_on_device(const skl_gemm_desc *d) {
     if (r == DECLINED) {
       if (canonicalize(d, &g)) {
         if (!fused) r = gemv_paths(&g, 1);
-        /* these two apply the fused steps themselves: B with K contiguous (1 to 4 rows), B row-major (1 row) */
+        /* these apply the fused steps themselves: B with K contiguous (1 to 4 rows, 5 to 128 rows), B row-major (1 row) */
         if (fused && skl_hip_gemv_kc_supported(&g)) r = outcome(skl_hip_launch_gemv_kc(&g));
+        if (fused && r == DECLINED && skl_hip_gemv_kc_rows_supported(&g)) r = outcome(skl_hip_launch_gemv_kc_rows(&g));
         if (fused && r == DECLINED && g.m == 1 && skl_hip_gemv_supported(&g, 0)) r = outcome(skl_hip_launch_gemv(&g, 0));
         if (fused && r == DECLINED) r = gemv_then_epilogue(&g); /* uses the operand scratch itself: only here, on the caller's own operands */
         if (r == DECLINED) r = gemm_padded_to_tiles(&g);

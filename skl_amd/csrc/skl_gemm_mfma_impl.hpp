@@ -464,7 +464,7 @@ __device__ __forceinline__ void write_wave_tile(const MfmaArgs &p, const Acc (&a
   using AccElem = decltype(Acc{}.x);
   using Steps = FusedSteps<AccElem, EXTRA>;
   constexpr int kBlocks = MI * NI;            // block b: j = b / MI, i = b % MI (a column strip at a time)
-  constexpr int kAhead = kBlocks < 2 ? 1 : 2;
+  constexpr int kAhead = (kBlocks < 2 || CHECK) ? 1 : 2;  // the bounds-checked kernels run four waves per SIMD: 128 registers
   // The lane index from the execution mask rather than from threadIdx: nothing the epilogue needs is then computed
   // in front of the main loop and held in a vector register across it (the loop uses every one of them).
   const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
@@ -603,7 +603,7 @@ __device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, un
 }
 
 template <int TA, int TB, bool A_KC, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool GUARDED, bool EXACT = false, bool EXTRA = false>
-__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gemm_mfma_kernel(MfmaArgs p) {
+__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, (BM == 128 ? 4 : 6)) gemm_mfma_kernel(MfmaArgs p) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   using KA = Kind<TA>;
   using M = typename std::conditional<EXACT, MmaF8Exact<TA, TB>, Mma<TA, TB>>::type;

@@ -7,7 +7,8 @@
 // With K contiguous in both operands a 16-byte load IS a matrix-core operand: 16 consecutive k of one column of B,
 // or of one row of A. A workgroup of eight waves owns 64 columns (four groups of 16) and ALL of K, 512 k per wave,
 // so the sums of a column tile never leave the workgroup: they meet in LDS in wave order - the same bits on every
-// run -, C is written once with the alpha / beta step applied in place, and no scratch memory is involved. All of
+// run -, C is written once with the alpha / beta step (and the fused steps of a fused call) applied in place, and no
+// scratch memory is involved. All of
 // B is in flight from the start (32 loads per lane) and stays in registers while up to eight groups of 16 rows of A
 // take their turns; a group's pieces of A (from L2: every workgroup reads all of A) are requested two groups ahead.
 // Instruction t of a 256-k chunk takes k = chunk + 64 t + 16 g + (0..15) from the lanes of k group g: the four
@@ -48,6 +49,9 @@ struct KcRowsArgs {
   size_t c_row, c_col;
   size_t m, n, k;
   skl_scalar alpha, beta;
+  const void *bias;  // fused steps behind alpha / beta (bias and maximum of C's type, or null) ...
+  void *max;
+  skl_requant rq;    // ... activation and 8-bit copy
 };
 
 __device__ __forceinline__ v4i load16(const char *p) { return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(p)); }
@@ -96,6 +100,8 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kc_rows_kernel(KcRowsArgs p)
   const int row = threadIdx.x >> 6, tc = threadIdx.x & 63;  // 512 threads: 8 rows x 64 columns at a time
   const size_t j = (size_t)blockIdx.x * kCols + tc;
   Acc *cbase = reinterpret_cast<Acc *>(p.c);
+  const bool fused = p.bias || p.max || p.rq.act || p.rq.q;  // the same for every thread
+  Acc largest = skl_lowest<Acc>();                           // what this thread wrote, for the maximum
 #pragma unroll
   for (int rg = 0; rg < RG; ++rg) {
     if ((size_t)rg * 16 >= p.m) break;  // the same for every thread of the workgroup
@@ -149,8 +155,23 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_kc_rows_kernel(KcRowsArgs p)
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       const size_t i = (size_t)rg * 16 + row + kWaves * q;
-      if (i < p.m && j < p.n) skl_update(sums[q], cbase + i * p.c_row + j * p.c_col, p.alpha, p.beta);
+      if (i >= p.m || j >= p.n) continue;
+      Acc *c = cbase + i * p.c_row + j * p.c_col;
+      if (!fused) {
+        skl_update(sums[q], c, p.alpha, p.beta);
+      } else {  // the steps of include/skl-gfx950.h's fused calls on the same sums: a fused call gives the plain call's bits plus the steps
+        Acc v = skl_beta_is_zero<Acc>(p.beta) ? skl_initialise(sums[q], c, p.alpha, p.beta) : skl_combine(sums[q], *c, p.alpha, p.beta);
+        if (p.bias) v = skl_add_bias(v, reinterpret_cast<const Acc *>(p.bias)[j]);
+        v = skl_activate(v, p.rq.act);
+        if (!p.rq.q_only) *c = v;
+        skl_emit_requantised(p.rq, v, i, j);
+        if (v > largest) largest = v;
+      }
     }
+  }
+  if (fused && p.max) {  // one atomic per wave that wrote something
+    const Acc best = skl_wave_max(largest);
+    if ((threadIdx.x & 63) == 0 && best > skl_lowest<Acc>()) skl_atomic_max(reinterpret_cast<Acc *>(p.max), best);
   }
 }
 
@@ -197,10 +218,9 @@ inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 }  // namespace
 
 // 5 to 128 rows of A and a B of at least 1 MiB, both with K contiguous (16-byte aligned rows and columns a fixed
-// distance apart, K a multiple of 16 up to 4096), C flat or in blocks of 64, no fused steps.
+// distance apart, K a multiple of 16 up to 4096), C flat or in blocks of 64; fused steps in the last stage.
 extern "C" int skl_hip_gemv_kc_rows_supported(const skl_gemm_canon *g) {
   if (kind_of(g) < 0) return 0;
-  if (g->bias || g->max || g->rq.act || g->rq.q) return 0;
   if (g->c_row_shift != 6 || g->c_col_shift != 6) return 0;
   if (g->m < (size_t)kMinRows || g->m > (size_t)(16 * kMaxRowGroups) || g->n == 0 || g->k == 0 || g->k > kMaxK) return 0;
   if ((g->k % 16) != 0 || g->k * g->n < (size_t(1) << 20)) return 0;
@@ -222,7 +242,7 @@ extern "C" int skl_hip_launch_gemv_kc_rows(const skl_gemm_canon *g) {
     return -2;
   }
   const KcRowsArgs p = {(const char *)g->a, g->a_s0, (const char *)g->b, g->b_s0, g->c, g->rsc0, g->csc0,
-                        g->m, g->n, g->k, g->alpha, g->beta};
+                        g->m, g->n, g->k, g->alpha, g->beta, g->bias, g->max, g->rq};
   switch (kind_of(g)) {
     case kI8: return launch_kind<kI8>(p, (unsigned)grid);
     case kE4M3: return launch_kind<kE4M3>(p, (unsigned)grid);

@@ -144,7 +144,7 @@ int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g, int layout);
 int skl_hip_gemv_kc_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
 /* 5 to 128 rows of A against a B with K contiguous, int8 and the fp8 kinds, K <= 4096: one workgroup per 64 columns
- * takes all of K on the matrix cores (skl_gemv_kcrows.hip). No fused steps, no scratch memory. */
+ * takes all of K on the matrix cores and applies the fused steps itself (skl_gemv_kcrows.hip). No scratch memory. */
 int skl_hip_gemv_kc_rows_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc_rows(const skl_gemm_canon *g);
 

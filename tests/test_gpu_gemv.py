@@ -466,10 +466,11 @@ def test_k_contiguous_b_floating_point(gpu, ta, tb, m):
 
 
 @pytest.mark.parametrize("ta", ("i8", "bf16", "f8e4m3"))
-@pytest.mark.parametrize("m", (1, 3, 4))
+@pytest.mark.parametrize("m", (1, 3, 4, 7, 40))
 def test_k_contiguous_b_with_fused_steps(gpu, ta, m):
     """A decode step on a linear layer's [out][in] weight with the fused steps of include/skl-gfx950.h: the kernel's
-    last stage applies bias, ReLU, the 8-bit copy (int8 behind int32, saturating E4M3 behind fp32) and the maximum.
+    last stage applies bias, ReLU, the 8-bit copy (int8 behind int32, saturating E4M3 behind fp32) and the maximum
+    (1 to 4 rows: the dot-product kernel; 7 and 40 rows: the matrix-core kernel for int8 and fp8, bf16 on the tile kernels).
     int8 against the checker's product plus the rules; floating point against the plain call of the same kernel
     (same sums, bit for bit) plus the rules. Row tails, padded strides, both pointer modes, q_only."""
     from gpu_support import run_fused_gemm
