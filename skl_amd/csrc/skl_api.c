@@ -519,7 +519,7 @@ static int gemm_on_device(const skl_gemm_desc *d) {
     if (r == DECLINED) {
       if (canonicalize(d, &g)) {
         if (!fused) r = gemv_paths(&g, 1);
-        /* these apply the fused steps themselves: B with K contiguous (1 to 4 rows, 5 to 128 rows), B row-major (1 row) */
+        /* these apply the fused steps themselves: B with K contiguous (1 to 4 rows, 5 to 96 rows), B row-major (1 row) */
         if (fused && skl_hip_gemv_kc_supported(&g)) r = outcome(skl_hip_launch_gemv_kc(&g));
         if (fused && r == DECLINED && skl_hip_gemv_kc_rows_supported(&g)) r = outcome(skl_hip_launch_gemv_kc_rows(&g));
         if (fused && r == DECLINED && g.m == 1 && skl_hip_gemv_supported(&g, 0)) r = outcome(skl_hip_launch_gemv(&g, 0));

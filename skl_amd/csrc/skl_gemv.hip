@@ -938,8 +938,8 @@ __global__ void __launch_bounds__(kMfmaWaves * 64) gemv_mfma_rows_kernel(GemvMfm
 // group at a time, and meet the other workgroups' in C.
 // ---------------------------------------------------------------------------
 constexpr int kK4MaxRowGroups = 8;
-constexpr int kRowMajorMaxRows = 80;  // row-major B: rows of A up to which the row groups beat the tile kernels (32 rows 19.5 against
-                                      // 28.8 us, 64 rows 27.4 against 30.8, 128 rows 42.5 against 35.2 for 4096 x 11008 weights)
+constexpr int kRowMajorMaxRows = 32;  // row-major B: rows of A up to which the row groups beat the tile kernels (4096 x 11008 weights: 32
+                                      // rows 19.5 against 20.3 us, 64 rows 27.4 against 24.1, 128 rows 42.5 against 28.8)
 
 template <int MODE, int RG>
 __global__ void __launch_bounds__(kMfmaWaves * 64, 2) gemv_rowgroups_kernel(GemvMfmaArgs p) {

@@ -1,4 +1,4 @@
-// skl_gemv_kcrows.hip - decode batches against weights stored column by column: 5 to 128 rows of A (K contiguous)
+// skl_gemv_kcrows.hip - decode batches against weights stored column by column: 5 to 96 rows of A (K contiguous)
 // times a B whose columns are contiguous in K - a linear layer's [out][in] weight -, int8 and the OCP fp8 kinds,
 // K <= 4096. The reference's generic kernels take any strides (ref/gemm/gemm_i8rc_i8rc_i32rc.c:9-24,
 // ref/gemm/gemm_f8rc_f8rc_f32rc.c); up to four rows skl_gemv.hip's gemv_kc_kernel streams such a B with dot
@@ -9,7 +9,7 @@
 // so the sums of a column tile never leave the workgroup: they meet in LDS in wave order - the same bits on every
 // run -, C is written once with the alpha / beta step (and the fused steps of a fused call) applied in place, and no
 // scratch memory is involved. All of
-// B is in flight from the start (32 loads per lane) and stays in registers while up to eight groups of 16 rows of A
+// B is in flight from the start (32 loads per lane) and stays in registers while up to six groups of 16 rows of A
 // take their turns; a group's pieces of A (from L2: every workgroup reads all of A) are requested two groups ahead.
 // Instruction t of a 256-k chunk takes k = chunk + 64 t + 16 g + (0..15) from the lanes of k group g: the four
 // groups read 64 consecutive bytes of a column per load. Which k meet in which instruction is free as long as
@@ -35,7 +35,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 8, kColGroups = 4, kCols = 16 * kColGroups;  // 64 columns per workgroup
 constexpr int kChunk = 256, kChunks = 2;                           // k per wave: 512
-constexpr int kMaxRowGroups = 8, kMinRows = 5;
+constexpr int kMaxRowGroups = 6, kMinRows = 5;  // 96 rows: beyond, the tile kernels are level (64 rows 21.5 against 23.5 us,
+                                                // a row group more costs 2.3 us, the tile kernels take 28-29 us for 128 rows)
 constexpr size_t kMaxK = (size_t)kWaves * kChunks * kChunk;        // 4096
 constexpr int kPitch = kCols + 1;
 enum { kI8 = 0, kE4M3 = 1, kE5M2 = 2, kMixed = 3 };  // kMixed: E4M3 A with E5M2 B
@@ -199,9 +200,7 @@ int launch_kind(const KcRowsArgs &p, unsigned grid) {
     case 3: return launch_groups<KIND, 3>(p, grid, st);
     case 4: return launch_groups<KIND, 4>(p, grid, st);
     case 5: return launch_groups<KIND, 5>(p, grid, st);
-    case 6: return launch_groups<KIND, 6>(p, grid, st);
-    case 7: return launch_groups<KIND, 7>(p, grid, st);
-    default: return launch_groups<KIND, 8>(p, grid, st);
+    default: return launch_groups<KIND, 6>(p, grid, st);
   }
 }
 
@@ -217,7 +216,7 @@ inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 }  // namespace
 
-// 5 to 128 rows of A and a B of at least 1 MiB, both with K contiguous (16-byte aligned rows and columns a fixed
+// 5 to 96 rows of A and a B of at least 1 MiB, both with K contiguous (16-byte aligned rows and columns a fixed
 // distance apart, K a multiple of 16 up to 4096), C flat or in blocks of 64; fused steps in the last stage.
 extern "C" int skl_hip_gemv_kc_rows_supported(const skl_gemm_canon *g) {
   if (kind_of(g) < 0) return 0;

@@ -200,11 +200,11 @@ def test_small_batch_rows_bit_exact(gpu, m):
                 assert np.array_equal(run_gemm(gpu, "rowmajor", case, a, b, c, mode), want), (m, n, k, mode)
 
 
-@pytest.mark.parametrize("m", (4, 5, 8, 9, 13, 16, 17, 33, 64, 70, 80, 81, 128))
+@pytest.mark.parametrize("m", (4, 5, 8, 9, 13, 16, 17, 25, 32, 33, 64, 128))
 def test_decode_batch_on_the_matrix_cores_bit_exact(gpu, m):
-    """4 to 80 rows of A against a row-major int8 B of at least 1 MiB (the stream over B whose multiply-adds run
-    on the matrix cores and whose workgroups add into C with atomics; beyond 16 rows in groups of 16 with B held in
-    registers, ragged last groups: 17, 33, 70), and row counts just beyond, which the tile kernels take: the config-2 weights, K and N off the kernel's 512 x 256 blocks, a K
+    """4 to 32 rows of A against a row-major int8 B of at least 1 MiB (the stream over B whose multiply-adds run
+    on the matrix cores and whose workgroups add into C with atomics; beyond 16 rows in two groups of 16 with B held
+    in registers, ragged second group: 17, 25), and row counts beyond, which the tile kernels take: the config-2 weights, K and N off the kernel's 512 x 256 blocks, a K
     of a single block, padded row strides of A, B and C (whole-buffer compare: the padding must survive), beta 0 / 1 /
     other with wrap-around, a C full of extreme values, both pointer modes."""
     rng = np.random.default_rng(400 + m)
@@ -419,11 +419,11 @@ def test_k_contiguous_b_int8_bit_exact(gpu, m):
                 assert np.array_equal(run_gemm(gpu, "rc", case, a, b, c, mode), want), (m, n, k, mode)
 
 
-@pytest.mark.parametrize("m", (5, 16, 17, 40, 100, 128))
+@pytest.mark.parametrize("m", (5, 16, 17, 40, 90, 96, 100, 128))
 def test_k_contiguous_b_decode_batches_int8_bit_exact(gpu, m):
-    """5 to 128 rows of A against a B stored column by column, K <= 4096 (ref/gemm/gemm_i8rc_i8rc_i32rc.c:9-24 with
+    """5 to 96 rows of A against a B stored column by column, K <= 4096 (ref/gemm/gemm_i8rc_i8rc_i32rc.c:9-24 with
     rsb = 1): one workgroup per 64 columns takes all of K on the matrix cores, row groups of 16 (ragged last groups:
-    5, 17, 40, 100), C written once. The config-2 width, N off the 64-column workgroups, K off the waves' 512 and the
+    5, 17, 40, 90), C written once; 100 and 128 rows: the tile kernels. The config-2 width, N off the 64-column workgroups, K off the waves' 512 and the
     chunks of 256, padded strides, alpha / beta with wrap-around on a C of extreme values, both pointer modes; a K
     beyond 4096 (the tile kernels) for comparison."""
     rng = np.random.default_rng(160 + m)
@@ -438,7 +438,7 @@ def test_k_contiguous_b_decode_batches_int8_bit_exact(gpu, m):
 
 
 @pytest.mark.parametrize("ta,tb", FP8_PAIRS)
-@pytest.mark.parametrize("m", (5, 16, 33, 128))
+@pytest.mark.parametrize("m", (5, 16, 33, 96))
 def test_k_contiguous_b_decode_batches_fp8(gpu, ta, tb, m):
     """The fp8 kinds of the same kernel (operands widened to f16 in registers: exact products, fp32 sums in a fixed
     order): inside the reference's bound without any allowance, and the same bits on every run."""
