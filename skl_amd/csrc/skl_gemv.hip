@@ -1,11 +1,14 @@
 // skl_gemv.hip - the M == 1 ("decode") path: y = beta*y + alpha * x*B, a pure
 // HBM stream over B. The one-row kernels use no matrix cores: they are bound by how
 // fast B's bytes arrive, so the design is about memory-level parallelism and coalescing.
-// Four kernels: gemv_kernel (M = 1, row-major or K-packed B; described below),
+// The kernels: gemv_kernel (M = 1, row-major or K-packed B; described below),
 // gemv_rows_kernel (a few rows of A against a row-major B), gemv_mfma_rows_kernel (up to
-// 16 rows of A against a row-major B: the same stream, B transposed in registers and
-// multiplied on the matrix cores) and gemv_kc_kernel (1 to 4 rows of A against a B with K
-// contiguous), each introduced where it is defined.
+// 16 rows of A against a row-major or K-packed B: the same stream, B transposed in registers
+// and multiplied on the matrix cores), gemv_rowgroups_kernel (the same with B held in
+// registers for several groups of 16 rows), gemv_k4_wholek_kernel (K-packed B with K <= 4096:
+// one workgroup per column tile takes all of K) and gemv_kc_kernel (1 to 4 rows of A against
+// a B with K contiguous), each introduced where it is defined. Decode batches on a B with K
+// contiguous: skl_gemv_kcrows.hip; 4-bit weights: skl_gemv_f4.hip.
 //
 // The reference has no separate GEMV API: M == 1 is a branch inside its GEMM
 // dispatchers (src/gemm/gemm_bf16_bf16_f32_zvfbfwma_x390.c:1220-1224,
