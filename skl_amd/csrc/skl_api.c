@@ -259,6 +259,23 @@ static int gemv_then_epilogue(const skl_gemm_canon *g) {
   h.bias = NULL, h.max = NULL;
   memset(&h.rq, 0, sizeof h.rq);
   if (gemv_paths(&h, 0) != TAKEN) return DECLINED;
+  /* The decode-batch kernel whose workgroups add into C: given the stream's block of sums - zero between calls - and
+   * beta == 1 it needs no kernel in front that clears the product, and the epilogue pass puts the zeros back. (The
+   * few-rows kernel keeps its own slots in that block: not for it.) */
+  if (g->m > 3 && !skl_hip_gemv_kc_supported(&h) && !skl_hip_gemv_kc_rows_supported(&h) && skl_hip_gemv_mfma_rows_supported(&h, 0)) {
+    skl_hip_sequence_begin();
+    product = skl_hip_zeroed_sums(g->m * g->n * 4);
+    if (product != NULL) {
+      h.c = product;
+      h.beta.i = 1;
+      r = outcome(skl_hip_launch_gemv_mfma_rows(&h, 0));
+      if (r == TAKEN) r = outcome(skl_hip_launch_gemm_epilogue_zeroing(g, product)) == TAKEN ? TAKEN : FAILED;
+      skl_hip_sequence_end();
+      return r;
+    }
+    skl_hip_sequence_end();
+    h.beta.i = 0;
+  }
   skl_hip_sequence_begin();
   product = skl_hip_operand_scratch(g->m * g->n * 4);
   r = product != NULL ? TAKEN : DECLINED;

@@ -116,7 +116,33 @@ extern "C" int skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile
 // kernel has left as a row-major M x N matrix of C's type in scratch memory: the pass that adds the shares of K,
 // given one share. What a streaming kernel without fused steps needs to serve a fused call (int32 C: the detour is
 // exact).
-extern "C" int skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void *product) {
+namespace {
+// The epilogue pass on a product that lives in the stream's block of sums: the same steps, and the element read is
+// put back to zero (the block is zero between calls).
+__global__ void __launch_bounds__(256) gemm_epilogue_zeroing_kernel(MfmaArgs p) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.m * p.n) return;
+  const size_t row = idx / p.n, col = idx % p.n;
+  int *product = reinterpret_cast<int *>(p.partial) + idx;
+  const int sum = *product;
+  *product = 0;
+  int *c = reinterpret_cast<int *>(p.c) + (row >> p.crs) * p.rsc1 + (row & ((size_t(1) << p.crs) - 1)) * p.rsc0 +
+           (col >> p.ccs) * p.csc1 + (col & ((size_t(1) << p.ccs) - 1)) * p.csc0;
+  int v = skl_beta_is_zero<int>(p.beta) ? skl_initialise(sum, c, p.alpha, p.beta) : skl_combine(sum, *c, p.alpha, p.beta);
+  if (p.bias) v = skl_add_bias(v, reinterpret_cast<const int *>(p.bias)[col]);
+  v = skl_activate(v, p.rq.act);
+  if (!p.rq.q_only) *c = v;
+  skl_emit_requantised(p.rq, v, row, col);
+  if (p.max && v > skl_lowest<int>()) skl_atomic_max(reinterpret_cast<int *>(p.max), v);
+}
+int launch_epilogue(const skl_gemm_canon *g, const void *product, bool zeroing);
+}  // namespace
+
+extern "C" int skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void *product) { return launch_epilogue(g, product, false); }
+extern "C" int skl_hip_launch_gemm_epilogue_zeroing(const skl_gemm_canon *g, void *product) { return launch_epilogue(g, product, true); }
+
+namespace {
+int launch_epilogue(const skl_gemm_canon *g, const void *product, bool zeroing) {
   if (g->ta != SKL_DT_I8 || g->tb != SKL_DT_I8 || g->m == 0 || g->n == 0 || !product || ((uintptr_t)g->c & 3) != 0 ||
       ((uintptr_t)product & 3) != 0 || g->c_row_shift > 6 || g->c_col_shift > 6) {
     skl_hip_record_error(-2, "gemm_epilogue: unsupported problem");
@@ -139,9 +165,13 @@ extern "C" int skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void 
     skl_hip_record_error(-2, "gemm_epilogue: grid too large");
     return -2;
   }
-  gemm_split_reduce_kernel<int><<<(unsigned)blocks, 256, 0, skl_current_stream()>>>(p);
+  if (zeroing)
+    gemm_epilogue_zeroing_kernel<<<(unsigned)blocks, 256, 0, skl_current_stream()>>>(p);
+  else
+    gemm_split_reduce_kernel<int><<<(unsigned)blocks, 256, 0, skl_current_stream()>>>(p);
   return skl_check_launch("gemm_epilogue");
 }
+}  // namespace
 
 extern "C" int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
   if (!skl_hip_gemm_mfma_supported(g)) {

@@ -1827,6 +1827,15 @@ unsigned long long *noalloc_slots_of_current_device() {
 }
 }  // namespace
 
+// The block of sums as an int32 matrix that is zero between calls: what a decode batch may add its product into
+// without a kernel in front that zeroes it, provided whoever reads the product puts the zeros back. NULL when the
+// product is larger than the block (or there is no block).
+extern "C" void *skl_hip_zeroed_sums(size_t bytes) {
+  Reduction red;
+  if (bytes > kMaxCols * 8 || !reduction_scratch(&red)) return nullptr;
+  return red.acc;
+}
+
 extern "C" int skl_hip_gemv_reserve_scratch(void) {
   Reduction red;
   return reduction_scratch(&red) ? 0 : -4;  // SKL_HIP_ERR_WORKSPACE

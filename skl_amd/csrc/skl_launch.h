@@ -120,6 +120,12 @@ int skl_hip_launch_gemm_mfma(const skl_gemm_canon *g);
 int skl_hip_gemm_mfma_padded_plan(const skl_gemm_canon *g, size_t *mp, size_t *np, size_t *kp);
 /* C = beta*C + alpha*P and the fused steps of g, P a row-major m x n int32 matrix (int8 problems only). */
 int skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void *product);
+/* The same with the product in the current stream's block of sums (skl_hip_zeroed_sums): every element is put back
+ * to zero once it has been read. */
+int skl_hip_launch_gemm_epilogue_zeroing(const skl_gemm_canon *g, void *product);
+/* The first `bytes` of the current stream's block of sums (zero between calls), or NULL when it is smaller or missing:
+ * a matrix that a decode-batch kernel can add into with beta == 1, without a kernel in front that clears it. */
+void *skl_hip_zeroed_sums(size_t bytes);
 /* 1 when the streaming kernel would take this int8 problem where it lies and write its blocked C (4 to 16 columns
  * per block, contiguous rows) 16 bytes per lane - as cheaply as a row-major C. */
 int skl_hip_gemm_mfma_streams_c_quads(const skl_gemm_canon *g);

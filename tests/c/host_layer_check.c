@@ -304,7 +304,7 @@ int __wrap_skl_hip_launch_gemm_mfma(const skl_gemm_canon *g) {
   return 0;
 }
 /* C = beta*C + alpha*product and the fused steps, the product a row-major m x n int32 matrix in scratch memory. */
-int __wrap_skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void *product) {
+static int epilogue_pass(const skl_gemm_canon *g, const void *product) {
   const size_t rmask = ((size_t)1 << g->c_row_shift) - 1, cmask = ((size_t)1 << g->c_col_shift) - 1;
   const double alpha = scalar_of(g->ta, g->alpha), beta = scalar_of(g->ta, g->beta);
   EXPECT(g->ta == SKL_DT_I8 && g->tb == SKL_DT_I8 && g->m && g->n, "epilogue pass: int8 problems only");
@@ -320,6 +320,31 @@ int __wrap_skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void *pro
                   &g->rq, "epilogue pass");
     }
   return 0;
+}
+int __wrap_skl_hip_launch_gemm_epilogue(const skl_gemm_canon *g, const void *product) { return epilogue_pass(g, product); }
+/* The stream's block of sums, zero between calls: handed out for a product only while it is zero, and whoever reads
+ * the product has to leave it zero again. */
+static int32_t *g_zeroed_sums;
+static size_t g_zeroed_sums_bytes;
+void *__wrap_skl_hip_zeroed_sums(size_t bytes) {
+  if (g_scarce) return NULL;
+  if (bytes > g_zeroed_sums_bytes) {
+    if (g_zeroed_sums) {
+      range_remove(g_zeroed_sums);
+      free(g_zeroed_sums);
+    }
+    g_zeroed_sums = calloc(1, bytes);
+    g_zeroed_sums_bytes = bytes;
+    range_add(g_zeroed_sums, bytes, 1);
+  }
+  for (size_t i = 0; i < g_zeroed_sums_bytes / 4; ++i) EXPECT(g_zeroed_sums[i] == 0, "block of sums handed out while not zero");
+  return g_zeroed_sums;
+}
+int __wrap_skl_hip_launch_gemm_epilogue_zeroing(const skl_gemm_canon *g, void *product) {
+  EXPECT(product == (void *)g_zeroed_sums, "zeroing epilogue pass on a product outside the block of sums");
+  const int rc = epilogue_pass(g, product);
+  if (!g_failures) memset(product, 0, g->m * g->n * 4);
+  return rc;
 }
 int __wrap_skl_hip_launch_gemm_mfma_padded(const skl_gemm_canon *g, int tile_cols) {
   SCARCE("padded GEMM (stand-in)");
@@ -1076,7 +1101,7 @@ int main(int argc, char **argv) {
   }
   g_scarce = 0;
   if (!g_failures && argc <= 2) run_large_cases();  /* with a seed: random cases only */
-  if (g_nranges != (g_operand_scratch ? 1 : 0) + (g_converted_scratch ? 1 : 0)) fail("a buffer of the host layer was not released");
+  if (g_nranges != (g_operand_scratch ? 1 : 0) + (g_converted_scratch ? 1 : 0) + (g_zeroed_sums ? 1 : 0)) fail("a buffer of the host layer was not released");
   printf("%s: %d cases, %ld launches carried out, %ld address ranges checked\n", g_failures ? "host layer check FAILED" : "host layer ok",
          cases, g_launches, g_checked);
   for (int q = 0; q < P_COUNT; ++q) printf("  %-24s %ld\n", kPathNames[q], g_path[q]);
