@@ -128,10 +128,10 @@ def wl_gemv_kc(lib, rng):
                 name="int8 GEMV 1x4096x11008, W with K contiguous ([n][k]), beta=0", kernel="gemv_kc_kernel<int8>")
 
 
-def _wl_batch_kc(m, kind="i8"):
+def _wl_batch_kc(m, kind="i8", k=4096, n=11008):
     """A decode batch against weights stored column by column (B with K contiguous, [out][in])."""
     def build(lib, rng):
-        k, n, nbuf = 4096, 11008, 8
+        nbuf = 8
         if kind == "i8":
             w = [DeviceBuffer.from_array(rand_i8(rng, k * n)) for _ in range(nbuf)]
             x = DeviceBuffer.from_array(rand_i8(rng, m * k))
@@ -147,7 +147,7 @@ def _wl_batch_kc(m, kind="i8"):
                 lib.skl_gemm_f8e4m3rc_f8e4m3rc_f32rc_gfx950(m, n, k, 1.0, x, k, 1, w[i % nbuf], 1, k, 0.0, y, n, 1)
 
         return dict(fn=step, bytes=k * n + m * k + 4 * m * n, ops=2 * m * k * n, bound="hbm", dtype=kind, keep=(w, x, y),
-                    name=f"{'int8' if kind == 'i8' else 'E4M3'} GEMM {m}x4096x11008, W with K contiguous ([n][k]), beta=0",
+                    name=f"{'int8' if kind == 'i8' else 'E4M3'} GEMM {m}x{k}x{n}, W with K contiguous ([n][k]), beta=0",
                     kernel="gemv_kc_kernel (up to 4 rows), gemv_kc_rows_kernel (up to 128)")
     return build
 
@@ -710,6 +710,7 @@ WORKLOADS = {
     "gemm_i8_kcontig_16x4096x11008": (_wl_batch_kc(16), 10, 2, 64),
     "gemm_i8_kcontig_64x4096x11008": (_wl_batch_kc(64), 10, 2, 32),
     "gemm_f8e4m3_kcontig_16x4096x11008": (_wl_batch_kc(16, "f8"), 10, 2, 64),
+    "gemm_i8_kcontig_16x11008x4096": (_wl_batch_kc(16, "i8", 11008, 4096), 10, 2, 64),
     "gemm_i8_4x4096x11008": (_wl_small_batch(4), 10, 2, 64),
     "gemm_i8_8x4096x11008": (_wl_small_batch(8), 10, 2, 64),
     "gemm_i8_16x4096x11008": (_wl_small_batch(16), 10, 2, 64),

@@ -75,7 +75,7 @@ void skl_gemm_f8e4m3rc_f8e5m2rc_f32rc_gfx950(size_t m, size_t n, size_t k, float
  * ref/cvt/cvt_ofp4.c:59-68 reads. The reference has no GEMM over 4-bit operands: it converts them first. The
  * result is that of skl_cvt_f4e2m1_f8e4m3 (ref/cvt/cvt_ofp4.c:59-68; exact - every E2M1 value is an E4M3 value) on
  * `b` followed by ref/gemm/gemm_f8e4m3rc_f8e4m3rc_f32rc.h:48 with rsb = 1, csb = ldb, inside that routine's
- * error bound. With 1 <= m <= 16 (up to 128 when k <= 4096 and B holds at least 2^20 values), csa = 1, k a
+ * error bound. With 1 <= m <= 16 (up to 128 when B holds at least 2^20 values), csa = 1, k a
  * multiple of 32 and 16-byte aligned rows of A and columns of B (ldb a multiple of 32) the weights are multiplied
  * as they are - decoded by the matrix cores' FP4 operand format, or widened to bf16 in registers when k <= 2304
  * (exact products) - so they cross memory at half a byte per element; every other call converts B once into

@@ -188,8 +188,8 @@ __global__ void __launch_bounds__(kWaves * 64) gemv_f4_kernel(F4Args p) {
   }
 }
 
-// 17 to 128 rows of A, K <= 4096: the same decomposition with B held in registers for all of K (one pass of the K
-// loop above: four chunks per wave) while up to eight groups of 16 rows take their turns - the 4-bit weights cross
+// 17 to 128 rows of A: the same decomposition with B held in registers for 4096 k (one pass of the K loop above:
+// four chunks per wave; a longer K takes one launch per 4096 k, the later ones adding to C) while up to eight groups of 16 rows take their turns - the 4-bit weights cross
 // HBM once and never exist as a converted copy (which cost 22.5 MB read, 45 MB written and a tile GEMM behind it:
 // 37 / 40 / 45 us for 32 / 64 / 128 x 4096 x 11008). Two groups of 16 columns per workgroup; a row group's pieces of A
 // are requested two groups ahead; its sums go through one of two LDS blocks, added in wave order (one barrier per
@@ -311,12 +311,12 @@ inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 }  // namespace
 
-// 1 to 16 rows of A (to 128 with K <= 4096), K a multiple of 32, rows of A and columns of B on 16-byte boundaries.
+// 1 to 16 rows of A (to 128 when B holds at least 2^20 values), K a multiple of 32, rows of A and columns of B on 16-byte boundaries.
 extern "C" int skl_hip_gemv_f4_supported(size_t m, size_t n, size_t k, const void *a, size_t rsa, size_t csa, const void *b,
                                          size_t ldb) {
   if (m < 1 || m > (size_t)(kMaxRows * kMaxRowGroups) || n == 0 || k == 0 || (k % 32) != 0) return 0;
-  // beyond 16 rows: B stays in registers for all of K, and there must be enough of it to be worth a pass per 128 rows
-  if (m > (size_t)kMaxRows && (k > kRowsMaxK || n * k < (size_t(1) << 20))) return 0;
+  // beyond 16 rows: B stays in registers for 4096 k at a time, and there must be enough of it to be worth a pass per 128 rows
+  if (m > (size_t)kMaxRows && n * k < (size_t(1) << 20)) return 0;
   if (csa != 1 || !aligned16(a) || (m > 1 && (rsa % 16) != 0)) return 0;
   if (!aligned16(b) || (n > 1 && (ldb % 32) != 0)) return 0;
   return 1;
@@ -335,23 +335,33 @@ extern "C" int skl_hip_launch_gemv_f4(size_t m, size_t n, size_t k, skl_scalar a
       skl_hip_record_error(-2, "gemv_f4: grid too large");
       return -2;
     }
-    F4Args p = {(const char *)a, rsa, (const char *)b, ldb / 2, scales, lds, 0, c, rsc, csc, m, n, k, alpha, beta};
     hipStream_t st = skl_current_stream();
     const unsigned blocks = (unsigned)grid, threads = kWaves * 64;
-    const bool exact = k <= kExactMaxK;
+    // A K beyond what the registers hold goes in passes of 4096 k: the first applies the caller's beta, the others
+    // add to C (beta = 1) - launches on one stream, in order; the same bits on every run.
+    for (size_t k0 = 0; k0 < k; k0 += kRowsMaxK) {
+      const size_t kk = k - k0 < kRowsMaxK ? k - k0 : kRowsMaxK;
+      skl_scalar pass_beta = beta;
+      if (k0 != 0) pass_beta.fz.value = 1.0f, pass_beta.fz.skip_c_read = 0;
+      F4Args p = {(const char *)a + k0, rsa, (const char *)b + k0 / 2, ldb / 2, scales ? scales + k0 / 32 : nullptr, lds, 0,
+                  c, rsc, csc, m, n, kk, alpha, pass_beta};
+      const bool exact = kk <= kExactMaxK;
 #define SKL_F4_ROWS(RG)                                                           \
   case RG:                                                                        \
     if (exact) gemv_f4_rows_kernel<true, RG><<<blocks, threads, 0, st>>>(p);      \
     else gemv_f4_rows_kernel<false, RG><<<blocks, threads, 0, st>>>(p);           \
     break;
-    switch ((m + 15) / 16) {
-      SKL_F4_ROWS(2) SKL_F4_ROWS(3) SKL_F4_ROWS(4) SKL_F4_ROWS(5) SKL_F4_ROWS(6) SKL_F4_ROWS(7)
-      default:
-        if (exact) gemv_f4_rows_kernel<true, 8><<<blocks, threads, 0, st>>>(p);
-        else gemv_f4_rows_kernel<false, 8><<<blocks, threads, 0, st>>>(p);
-    }
+      switch ((m + 15) / 16) {
+        SKL_F4_ROWS(2) SKL_F4_ROWS(3) SKL_F4_ROWS(4) SKL_F4_ROWS(5) SKL_F4_ROWS(6) SKL_F4_ROWS(7)
+        default:
+          if (exact) gemv_f4_rows_kernel<true, 8><<<blocks, threads, 0, st>>>(p);
+          else gemv_f4_rows_kernel<false, 8><<<blocks, threads, 0, st>>>(p);
+      }
 #undef SKL_F4_ROWS
-    return skl_check_launch("gemv_f4_rows");
+      const int rc = skl_check_launch("gemv_f4_rows");
+      if (rc != 0) return rc;
+    }
+    return 0;
   }
   // Four groups of 16 columns per workgroup from three rows of A on, where that still leaves at least 128
   // workgroups: the pieces of A are what a wave loads most of then.

@@ -149,8 +149,8 @@ int skl_hip_launch_gemv_mfma_rows(const skl_gemm_canon *g, int layout);
  * launcher applies g's fused steps, if any, where the outputs are written. */
 int skl_hip_gemv_kc_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc(const skl_gemm_canon *g);
-/* 5 to 96 rows of A against a B with K contiguous, int8 and the fp8 kinds, K <= 4096: one workgroup per 64 columns
- * takes all of K on the matrix cores and applies the fused steps itself (skl_gemv_kcrows.hip). No scratch memory. */
+/* 5 to 96 rows of A against a B with K contiguous, int8 and the fp8 kinds: one workgroup per 64 columns takes 4096 k
+ * (a longer K: a launch per 4096 k) on the matrix cores and applies the fused steps itself (skl_gemv_kcrows.hip). No scratch memory. */
 int skl_hip_gemv_kc_rows_supported(const skl_gemm_canon *g);
 int skl_hip_launch_gemv_kc_rows(const skl_gemm_canon *g);
 

@@ -422,12 +422,14 @@ def test_k_contiguous_b_int8_bit_exact(gpu, m):
 @pytest.mark.parametrize("m", (5, 16, 17, 40, 90, 96, 100, 128))
 def test_k_contiguous_b_decode_batches_int8_bit_exact(gpu, m):
     """5 to 96 rows of A against a B stored column by column, K <= 4096 (ref/gemm/gemm_i8rc_i8rc_i32rc.c:9-24 with
-    rsb = 1): one workgroup per 64 columns takes all of K on the matrix cores, row groups of 16 (ragged last groups:
-    5, 17, 40, 90), C written once; 100 and 128 rows: the tile kernels. The config-2 width, N off the 64-column workgroups, K off the waves' 512 and the
-    chunks of 256, padded strides, alpha / beta with wrap-around on a C of extreme values, both pointer modes; a K
-    beyond 4096 (the tile kernels) for comparison."""
+    rsb = 1): one workgroup per 64 columns takes 4096 k on the matrix cores, row groups of 16 (ragged last groups:
+    5, 17, 40, 90), C written once per 4096 k; 100 and 128 rows: the tile kernels. The config-2 width, N off the
+    64-column workgroups, K off the waves' 512 and the chunks of 256, padded strides, alpha / beta with wrap-around on
+    a C of extreme values, both pointer modes; a K beyond 4096 against a narrow B (the tile kernels) and against a
+    wide one (two launches, the second of 16 k)."""
     rng = np.random.default_rng(160 + m)
-    for (n, k, pad) in ((11008, 1024 if m > 16 else 4096, 0), (1037, 4080, 16), (300, 3504, 32), (4100, 272, 0), (260, 4112, 0)):
+    for (n, k, pad) in ((11008, 1024 if m > 16 else 4096, 0), (1037, 4080, 16), (300, 3504, 32), (4100, 272, 0), (260, 4112, 0),
+                        (8200, 4112, 0)):
         for alpha, beta in ((1, 0), (0x01010101, -77), (-3, 1)):
             case = _kc_case("i8", None, m, n, k, alpha, beta, pad)
             a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
@@ -442,7 +444,7 @@ def test_k_contiguous_b_decode_batches_int8_bit_exact(gpu, m):
 def test_k_contiguous_b_decode_batches_fp8(gpu, ta, tb, m):
     """The fp8 kinds of the same kernel (operands widened to f16 in registers: exact products, fp32 sums in a fixed
     order): inside the reference's bound without any allowance, and the same bits on every run."""
-    for (n, k, pad) in ((11008, 1024 if m > 16 else 4096, 0), (1037, 2064, 16), (300, 3504, 32)):
+    for (n, k, pad) in ((11008, 1024 if m > 16 else 4096, 0), (1037, 2064, 16), (300, 3504, 32), (8200, 4128, 0)):
         case = _kc_case(ta, tb, m, n, k, 1.5, -0.5, pad)
         a, b, c = case.make_inputs(m * 37 + n + k)
         for mode in ("device", "host"):
@@ -476,7 +478,7 @@ def test_k_contiguous_b_with_fused_steps(gpu, ta, m):
     from gpu_support import run_fused_gemm
     from test_oracle_gemm import fused_expectation
     rng = np.random.default_rng(70 + m)
-    for (n, k, pad) in ((11008, 4096, 0), (1037, 1040, 16), (70, 1008, 32)):
+    for (n, k, pad) in ((11008, 4096, 0), (1037, 1040, 16), (70, 1008, 32), (8200, 4128, 16)):
         for beta, only in ((0, True), (1, False)):
             case = _kc_case(ta, None, m, n, k, 2 if ta == "i8" else 0.5, beta, pad)
             a, b, c = case.make_inputs(int(rng.integers(1 << 30)))

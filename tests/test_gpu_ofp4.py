@@ -52,7 +52,8 @@ SHAPES = (
     (17, 4100, 512, 544, 528, "17 rows (two row groups, the second of one row), multiplied exactly, n off the 32-column workgroups"),
     (100, 1040, 4096, 4096, None, "100 rows in seven row groups, the longest K held in registers"),
     (128, 520, 2336, 2368, 2352, "eight full row groups on the FP4 format"),
-    (40, 300, 4128, 4128, None, "K beyond what the registers hold: through the converted copy"),
+    (40, 300, 4128, 4128, None, "K beyond what the registers hold: two passes, the second of one piece of K"),
+    (100, 520, 11008, 11040, 11024, "K of a down projection: three passes"),
     (300, 260, 1000, 1000, None, "a GEMM: through the converted copy"),
     (4, 64, 100, 101, None, "K off 32 and an odd column distance (columns start inside a byte): converted copy"),
     (2, 40, 64, 64, 67, "rows of A off 16 bytes: converted copy"),
