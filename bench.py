@@ -785,8 +785,8 @@ TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in pro
 MEASURED_TRAFFIC_BYTES = {
     "gemv_i8": int((22060.5 * 1.998 + 817.0) * 1024),
     "cvt_f32_f8e4m3_8192sq": int((131136.5 * 1.998 + 65536.0) * 1024),
-    "gemm_i8_8192": int((393338.8 * 1.998 + 262444.7) * 1024),
-    "gemm_f8e4m3_8192_kcontig": int((393354.7 * 1.998 + 262648.2) * 1024),
+    "gemm_i8_8192": int((393337.6 * 1.998 + 262504.5) * 1024),
+    "gemm_f8e4m3_8192_kcontig": int((393353.0 * 1.998 + 262726.9) * 1024),
     "copy_u32_4096sq": int((32800.9 * 1.998 + 65536) * 1024),
     "gemm_i8_16x4096x11008": int((22349.1 * 1.998 + 6192.0) * 1024),
     "gemv_f8e4m3_f4_1x4096x11008": int((11060.0 * 1.998 + 43.0) * 1024),
