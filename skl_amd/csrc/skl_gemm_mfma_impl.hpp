@@ -929,7 +929,20 @@ constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
 // the epilogue touches nothing beyond them.
 // CQUADS: an int32 C in small blocks with contiguous rows (the 4 x 4 blocks of src/gemm/packed-gemm.md:270-298, up to
 // 16 columns), no fused steps - see the epilogue.
-template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0, bool CQUADS = false>
+// SCAN (floating-point row-major C, beta == 0 evaluated like the reference's loops, whole tiles, K of at least 64
+// slices on the wide tile and 32 on the narrow one): whether 0 * c is a zero for every old c of the tile - i.e. no NaN,
+// no infinity - is found out while the tile is multiplied. Every even slice each wave requests 1 KiB of the tile's
+// old C (a row of the wide tile, two rows of the narrow one; wave w takes every eighth) into one of four slots of LDS
+// behind the operand stages; three and four slices later it reads them back, 8 bytes per lane and slice (its own
+// loads, its own counter: no barrier), and tests the exponents. After the loop the waves put their findings together.
+// A tile without such a value is then written as an initialised one (the sign of exact zeros is still taken from the
+// old c, see write_wave_tile); a tile with one takes the path that reads all of C. Either way the bits are those of
+// 0 * c + alpha * acc.
+// (Measured on fp8 8192^3, old C in memory: a first version - every wave its own block, lane addresses for any
+// layout of C, 64-bit block arithmetic per load - cost 62-70 us of 415 whether it loaded 4 bytes per lane every slice
+// or 16 every other one, 25-43 us of that with the rows already in cache: the instructions between two MFMAs, not the
+// loads. Hence contiguous rows, whose address is a scalar product and a shift of the lane index.)
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0, bool CQUADS = false, bool SCAN = false>
 __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   using KA = Kind<TA>;
   using M = Mma<TA, TB>;
@@ -968,29 +981,28 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   constexpr int kEachA = A_KC ? 0 : LA::kBlocks, kEachB = B_KC ? 0 : LB::kBlocks;
   constexpr int kEach = kEachA + kEachB, kPairs = kPairA + kPairB;
   constexpr int kLoadsOfU[2] = {(kPairU == 0 ? kPairs : 0) + kEach, (kPairU == 1 ? kPairs : 0) + kEach};
-  // At the barrier of slice s the data of slice s+1 must have landed; vmcnt may leave in flight what
-  // was requested after it. Every-slice loads: requested by slice s+1-kEachAhead. Pair loads: by the
-  // latest slice of parity kPairU not after s+1-kPairAhead, and first in that slice. Counted as younger
-  // (conservatively): the every-slice loads of that pair-issuing slice, all loads of the slices after
-  // the older of the two requesting slices, and what slice s itself has issued in front of its barrier.
-  //   kExtra = 0: s even -> both from s-2: slice s-1 (odd, kEach).  s odd -> pairs from s-1: its kEach.
-  //   kExtra = 1: s even -> both from s-3: slices s-2 (kEach) and s-1 (pairs + kEach).
-  //               s odd  -> pairs from s-2: its kEach, and slice s-1 (kEach).
-  // In general (slice s of parity U, every-slice loads kEachAhead = kPairAhead + 1 slices ahead): the data of slice
-  // s+1 was requested in slice s - kPairAhead (every-slice loads; pair loads too when s is even) or, for pair loads
-  // with s odd, first thing in slice s + 1 - kPairAhead. Younger than that: for even s the loads of the
-  // kPairAhead - 1 slices s - kPairAhead + 1 .. s - 1; for odd s the every-slice loads of slice s + 1 - kPairAhead
-  // and the loads of the kPairAhead - 2 slices after it; and what slice s has issued in front of its barrier.
+  // SCAN: one more load in every even slice, the first thing that slice requests (behind its first MFMA, in front
+  // of its pair loads): older than every load of its slice, so it has landed whenever the slice's own loads are
+  // waited for. It counts as younger wherever a whole slice counted below is an even one, and in front of the
+  // barrier of its own slice when that barrier is not in the slice's first k-step.
+  constexpr int kScanSlots = 4, kScanSlot = WAVES * 1024;
+  static_assert(!SCAN || (std::is_same<AccElem, float>::value && !EDGE && EXTRA == 0 && !CQUADS), "a plain floating-point product on whole tiles");
+  static_assert(kPairAhead <= 3, "the rows requested in slice 2q are read back in slices 2q + 3 and 2q + 4");
   constexpr int kPreOfU[2] = {ceil_div(kPre * kLoadsOfU[0], kSlots), ceil_div(kPre * kLoadsOfU[1], kSlots)};
-  constexpr auto younger = [](int u, const int (&loads)[2], int each, int pair_ahead) {
+  constexpr auto younger = [](int u, const int (&loads)[2], int each, int pair_ahead, bool scan, int pre_slots) {
     int n = u == 0 ? 0 : each;
-    for (int d = 1; d <= pair_ahead - 1 - u; ++d) n += loads[(u + d) % 2];
+    // the whole slices counted: t - pair_ahead + u + d for d = 1 .. pair_ahead - 1 - u, t (of parity u) being this slice
+    for (int d = 1; d <= pair_ahead - 1 - u; ++d) {
+      n += loads[(u + d) % 2];
+      if (scan && (pair_ahead + d) % 2 == 0) n += 1;
+    }
+    if (scan && u == 0 && pre_slots > 0) n += 1;  // this slice's own, requested in its first k-step
     return n;
   };
-  constexpr int kInFlightOfU[2] = {younger(0, kLoadsOfU, kEach, kPairAhead) + kPreOfU[0],
-                                   younger(1, kLoadsOfU, kEach, kPairAhead) + kPreOfU[1]};
-  static_assert(STAGES != 4 || (kInFlightOfU[0] == (kExtra ? 2 * kEach + kPairs : kEach) + kPreOfU[0] &&
-                                kInFlightOfU[1] == (kExtra ? 2 * kEach : kEach) + kPreOfU[1]),
+  constexpr int kInFlightOfU[2] = {younger(0, kLoadsOfU, kEach, kPairAhead, SCAN, kPre) + kPreOfU[0],
+                                   younger(1, kLoadsOfU, kEach, kPairAhead, SCAN, kPre) + kPreOfU[1]};
+  static_assert(STAGES != 4 || SCAN || (kInFlightOfU[0] == (kExtra ? 2 * kEach + kPairs : kEach) + kPreOfU[0] &&
+                                        kInFlightOfU[1] == (kExtra ? 2 * kEach : kEach) + kPreOfU[1]),
                 "the four-stage counts, as derived by hand above");
   static_assert(kInFlightOfU[0] < 64 && kInFlightOfU[1] < 64, "vmcnt is a 6-bit counter");
 
@@ -1033,6 +1045,54 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   // K is a whole number of slice pairs. Units beyond the end are requested as the last unit
   // again: in range, and the stage they land in is never read, which keeps the load counts static.
   const size_t slices = p.k * ES / SB, pairs = slices / 2;
+
+  // SCAN: the tile's old C, 1 KiB per wave and two slices (the host has checked that K has the slices for it and
+  // that C is row-major with 16-byte aligned rows).
+  unsigned long long scan_bad = 0;   // lanes that have seen a NaN or an infinity
+  v2i scan_pend = {0, 0};            // the 8 bytes read back during the k-step before
+  char *const scan_region = smem + TileA::kRegion + TileB::kRegion + wave * 1024;
+  const unsigned scan_addr = addr_b + TileB::kRegion + wave * 1024;
+  // (row of this wave's first load, and the bytes from one load's rows to the next: scalars, 64 x rsc0 fits 32 bits)
+  constexpr unsigned kScanRowsPerLoad = BN == 256 ? 1 : 2, kScanLoadsPerWave = BM / (WAVES * kScanRowsPerLoad);
+  // C in panels of 64 x 64 contiguous values (rsc0 == 64): 1 KiB is four rows of a panel; the tile's panels row by
+  // row, 16 such pieces each, piece 8 q + w is wave w's load q.
+  const bool scan_panels = p.rsc0 == 64 && p.rsc1 != 64 * 64;
+  const char *const scan_rows = scan_panels ? reinterpret_cast<const char *>(p.c) + ((m0 >> 6) * p.rsc1 + (n0 >> 6) * p.csc1) * 4
+                                            : reinterpret_cast<const char *>(p.c) + ((m0 + (size_t)wave * kScanRowsPerLoad) * p.rsc0 + n0) * 4;
+  const unsigned scan_step = (unsigned)p.rsc0 * (WAVES * kScanRowsPerLoad * 4u);
+  [[maybe_unused]] auto scan_issue = [&](size_t s) {  // s even: load s / 2 of this wave (the last one again beyond the tile)
+    const unsigned q = (unsigned)(s >> 1) < kScanLoadsPerWave ? (unsigned)(s >> 1) : kScanLoadsPerWave - 1;  // uniform
+    const char *rows = scan_rows + (size_t)q * scan_step;
+    if (scan_panels) {
+      const unsigned piece = q * WAVES + wave, panel = piece >> 4, pi = panel / (BN / 64), pj = panel % (BN / 64);
+      rows = scan_rows + ((size_t)pi * p.rsc1 + (size_t)pj * p.csc1) * 4 + (piece & 15u) * 1024u;
+    }
+    // The lane's own part of the address is computed anew for every load, from a lane index the compiler cannot
+    // follow: held across the loop it would be a register that the loop does not have.
+    unsigned l = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(l));
+    unsigned mine;
+    if constexpr (BN == 256)
+      mine = l * 16u;                                                                // 64 lanes x 16 bytes: one row of 256 columns
+    else
+      mine = (l & 31u) * 16u + ((unsigned)((int)(l << 26) >> 31) & (scan_panels ? 512u : (unsigned)p.rsc0 * 4u));  // lanes 32-63: the row below (panels: the next 512 bytes)
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(rows + mine),
+                                     (__attribute__((address_space(3))) void *)(scan_region + (unsigned)((s >> 1) % kScanSlots) * kScanSlot), 16, 0, 0);
+  };
+  [[maybe_unused]] auto scan_read = [&](unsigned slot, unsigned half) {  // 512 of this wave's 1024 bytes in `slot`; the value counts from the next lgkmcnt(0) on
+    unsigned l = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(l));
+    const unsigned addr = scan_addr + slot * kScanSlot + half * 512 + l * 8;
+    asm volatile("ds_read_b64 %0, %1" : "=v"(scan_pend) : "v"(addr) : "memory");
+  };
+  [[maybe_unused]] auto scan_check = [&]() {  // behind an lgkmcnt(0): NaN or infinity, either sign, in either dword
+    asm volatile("" : "+v"(scan_pend));
+    unsigned long long x, y;
+    asm volatile("v_cmp_class_f32_e64 %0, %1, %2" : "=s"(x) : "v"(scan_pend.x), "s"(0x207));
+    asm volatile("v_cmp_class_f32_e64 %0, %1, %2" : "=s"(y) : "v"(scan_pend.y), "s"(0x207));
+    scan_bad |= x | y;
+  };
+
   if constexpr (A_KC) {
 #pragma unroll
     for (int i = 0; i < kPairsPrologue; ++i) la.issue(region_a, 2 * i, (size_t)i < pairs ? (size_t)i : pairs - 1);
@@ -1046,6 +1106,13 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   } else {
 #pragma unroll
     for (int i = 0; i < kEachAhead; ++i) lb.issue(region_b, i, (size_t)i < slices ? (size_t)i : slices - 1);
+  }
+  if constexpr (SCAN) {  // the slots start as zeros: the first slices read slots that no load has filled yet
+#pragma unroll
+    for (int slot = 0; slot < kScanSlots; ++slot)
+#pragma unroll
+      for (int quarter = 0; quarter < 4; ++quarter)
+        *reinterpret_cast<float *>(scan_region + slot * kScanSlot + quarter * 256 + (threadIdx.x & 63) * 4) = 0.0f;
   }
   wait_loads_upto<0>();
   __syncthreads();
@@ -1133,6 +1200,14 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
                             constexpr int Q = decltype(qc)::value, kSlot = KS * kMfmas + Q;
                             constexpr int i = Q / NI, j = Q % NI;
                             acc[i][j] = M::run(fa[i], fb[j], acc[i][j]);
+                            // SCAN: the MFMA first, what follows in its shadow - the waves have just left a barrier together, and
+                            // instructions in front of a slice's first MFMA are a gap in every SIMD's matrix core at once.
+                            if constexpr (SCAN && kSlot <= 1) __builtin_amdgcn_sched_barrier(0);
+                            if constexpr (SCAN && U == 0 && kSlot == 0) scan_issue(s);
+                            if constexpr (SCAN && kSlot == 1) scan_check();  // what the last slot of the k-step before has read, behind this k-step's lgkmcnt(0)
+                            // Behind the barrier of slice 2q + 3 the rows requested in slice 2q have landed: half of them is
+                            // read back in that slice, half in the next (the first slices find zeros).
+                            if constexpr (SCAN && kSlot == kSlots - 1) scan_read(((s32 >> 1) + kScanSlots - (U == 1 ? 1 : 2)) % kScanSlots, U == 1 ? 0 : 1);
                             // this slot's share of the next k-step's reads
                             [&]<int... Rs>(std::integer_sequence<int, Rs...>) {
                               (
@@ -1176,6 +1251,19 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
     }(std::make_integer_sequence<int, 2>{});
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  if constexpr (SCAN) {
+    // The last rows requested have not been read back or in part only, and the last 8 bytes read have not been
+    // tested: all slots once more (a row tested twice changes nothing).
+    scan_check();
+#pragma unroll
+    for (int slot = 0; slot < kScanSlots; ++slot)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        scan_read(slot, half);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        scan_check();
+      }
+  }
 
   if (p.splits > 1) {  // a share of K: the raw sums go to this split's M x N plane
     AccElem *plane = reinterpret_cast<AccElem *>(p.partial) + (size_t)split * p.m * p.n;
@@ -1251,7 +1339,21 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
     }
     return;
   }
-  write_wave_tile<MI, NI, EDGE, EXTRA>(p, acc, m0 + wm, n0 + wn);
+  if constexpr (SCAN) {
+    // What the eight waves have found, put together: each wave's word where its first slot began (its own reads of
+    // the slots are over), a barrier, and everybody reads all eight.
+    unsigned *const found = reinterpret_cast<unsigned *>(smem + TileA::kRegion + TileB::kRegion);
+    found[wave * 256] = scan_bad != 0;
+    __syncthreads();
+    unsigned any = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) any |= found[w * 256];
+    MfmaArgs q = p;
+    if (any == 0) q.beta.fz.skip_c_read = 1;  // 0 * c is a zero everywhere in this tile
+    write_wave_tile<MI, NI, EDGE, EXTRA>(q, acc, m0 + wm, n0 + wn);
+  } else {
+    write_wave_tile<MI, NI, EDGE, EXTRA>(p, acc, m0 + wm, n0 + wn);
+  }
 }
 
 // C = beta*C + alpha * (sum of the splits' planes, in split order), then the fused steps: the second
@@ -1310,7 +1412,7 @@ inline bool c_in_row_quads(const MfmaArgs &p) {
          (((uintptr_t)p.c | (p.rsc0 * 4) | (p.rsc1 * 4) | (p.csc1 * 4)) & 15) == 0;
 }
 
-template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0, bool CQUADS = false>
+template <int TA, int TB, bool A_KC, bool B_KC, int BN, bool EDGE = false, int EXTRA = 0, bool CQUADS = false, bool SCAN = false>
 int launch_ring(const MfmaArgs &args) {
   if constexpr (EXTRA == 0 && kRingCarriesExtraSteps<TA, TB> && !EDGE) {
     if (args.rq.q) return args.rq.q_only ? launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 2>(args) : launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 3>(args);
@@ -1318,8 +1420,26 @@ int launch_ring(const MfmaArgs &args) {
   if constexpr (TA == SKL_DT_I8 && TB == SKL_DT_I8 && A_KC && B_KC && !EDGE && EXTRA == 0 && !CQUADS) {  // what copies of blocked operands look like
     if (c_in_row_quads(args)) return launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, 0, true>(args);
   }
-  constexpr int lds = ring_stages(BN) * (256 + BN) * kRingSlice;
-  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE, EXTRA, CQUADS>;
+  constexpr int ES = Kind<TA>::ES;
+  using AccElem = decltype(typename Kind<TA>::Acc{}.x);
+  if constexpr (std::is_same<AccElem, float>::value && !EDGE && EXTRA == 0 && !CQUADS && !SCAN) {
+    // beta == 0 evaluated as the reference's loops do (0 * c: a NaN or an infinity in C stays a NaN): the old C is
+    // looked through while the tile is multiplied, 8 KiB of it per two slices - needs 64 slices on the wide tile, 32
+    // on the narrow one, a tile to itself (no shared K) and a row-major C.
+    const size_t scan_slices = args.k * ES / kRingSlice, scan_tiles = (args.m / 256) * (args.n / BN);
+    const bool shared_k = scan_tiles <= 128 && scan_slices % 4 == 0 && scan_slices / 2 >= kRingMinSlicesPerSplit;
+    // C row-major: rows and columns at one stride each across the blocks, rows of 16-byte aligned starts ...
+    const bool row_major = args.csc0 == 1 && args.csc1 == (size_t(1) << args.ccs) && args.rsc1 == (args.rsc0 << args.crs) &&
+                           (((uintptr_t)args.c | (args.rsc0 * 4)) & 15) == 0 && args.rsc0 < (size_t(1) << 26) &&
+                           !(args.rsc0 == 64 && args.rsc1 != 64 * 64);
+    // ... or in panels of 64 x 64 contiguous values on 16-byte boundaries
+    const bool panels = args.csc0 == 1 && args.rsc0 == 64 && args.crs == 6 && args.ccs == 6 && args.rsc1 != 64 * 64 &&
+                        (((uintptr_t)args.c | (args.rsc1 * 4) | (args.csc1 * 4)) & 15) == 0;
+    if (args.beta.f == 0.0f && args.beta.fz.skip_c_read == 0 && !shared_k && (row_major || panels) && scan_slices >= (BN == 256 ? 64 : 32))
+      return launch_ring<TA, TB, A_KC, B_KC, BN, EDGE, EXTRA, CQUADS, true>(args);
+  }
+  constexpr int lds = ring_stages(BN) * (256 + BN) * kRingSlice + (SCAN ? 4 * 8 * 1024 : 0);
+  auto kernel = gemm_mfma_ring_kernel<TA, TB, A_KC, B_KC, BN, EDGE, EXTRA, CQUADS, SCAN>;
   static std::atomic<bool> configured{false};  // per instantiation; racing threads set the same value
   if (!configured.load(std::memory_order_acquire)) {
     int rc = skl_check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -1334,7 +1454,6 @@ int launch_ring(const MfmaArgs &args) {
   const size_t tiles = (size_t)p.tiles_m * p.tiles_n;
   // Tiles for at most half of the 256 compute units: K is shared between two workgroups per tile (each at least
   // kRingMinSlicesPerSplit slices long) and a second pass adds the two planes and applies alpha / beta.
-  constexpr int ES = Kind<TA>::ES;
   const size_t slices = p.k * ES / kRingSlice;
   p.splits = (tiles <= 128 && slices % 4 == 0 && slices / 2 >= kRingMinSlicesPerSplit) ? 2 : 1;
   SequenceGuard sequence(p.splits > 1);
@@ -1351,7 +1470,6 @@ int launch_ring(const MfmaArgs &args) {
   kernel<<<(unsigned)grid, 512, lds, skl_current_stream()>>>(p);
   int rc = skl_check_launch("gemm_mfma_ring");
   if (rc != 0 || p.splits == 1) return rc;
-  using AccElem = decltype(typename Kind<TA>::Acc{}.x);
   const size_t blocks = (p.m * p.n + 255) / 256;
   if (blocks > 0x7FFFFFFFu) {
     skl_hip_record_error(-2, "gemm_mfma: grid too large");

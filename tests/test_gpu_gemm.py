@@ -253,6 +253,65 @@ def test_beta_zero_initialises_c(gpu, ta, m, n, k, what):
         assert np.array_equal(got.view(np.uint8), reference_mode.view(np.uint8)), (ta, mode)
 
 
+SCANNED_C_SHAPES = (
+    # ta, layout of C, m, n, k, what serves it
+    ("f8e4m3", "row", 4096, 4096, 4096, "256 x 256 tiles, exactly the slices of K it takes to look through a wave's block (64)"),
+    ("f8e4m3", "row", 4096, 4096, 4096 + 128, "256 x 256 tiles, two slices more"),
+    ("f8e4m3", "row", 4096, 4096, 8192, "256 x 256 tiles, twice the slices: the last rows are requested again"),
+    ("bf16", "row", 1024, 3072, 1024, "256 x 128 tiles, exactly the slices it takes (32)"),
+    ("bf16", "row", 1024, 3072, 2048 + 64, "256 x 128 tiles"),
+    ("f16", "column", 4096, 4096, 4096, "column-major C"),
+    ("bf16", "panel", 4096, 4096, 4096, "C in 64 x 64 panels, 256 x 256 tiles"),
+    ("bf16", "panel", 1024, 3072, 1024 + 64, "C in 64 x 64 panels, 256 x 128 tiles"),
+)
+
+
+@pytest.mark.parametrize("ta,layout,m,n,k,what", SCANNED_C_SHAPES)
+def test_beta_zero_as_the_reference_scans_c_under_the_product(gpu, ta, layout, m, n, k, what):
+    """The streaming kernel with a long K looks through the old C while it multiplies (four rows of every wave's block
+    per two slices of K) instead of reading all of it in the epilogue. Single NaNs and infinities planted in a few blocks - first
+    and last row of a block, first and last column, neighbouring blocks, the matrix's corners - become NaN exactly
+    there (ref/gemm/gemm_bf16rc_bf16rc_f32rc.c:21: 0 * c), every other element has the bits of the same call on a
+    clean C and of the initialising mode's call, and rows of exact zeros (a zeroed row of A) take their sign from the
+    old C in blocks with and without a planted value."""
+    rng = np.random.default_rng(79)
+    if layout == "panel":
+        case = support.panel_case(ta, m // support.TE, n // support.TE, k, -1.5, 0.0)
+        kind = "rcprc"
+    else:
+        case = rowmajor_case(ta, m, n, k, -1.5, 0.0)
+        if layout == "column":
+            case.rsc1, case.csc1 = 1, m
+        kind = "rc"
+    a, b, c = case.make_inputs(int(rng.integers(1 << 30)))
+    if layout != "panel":  # row 5 and the last row of A: exact zeros in those rows of C
+        for i in (5, m - 1):
+            a[i * k:(i + 1) * k] = 0
+    c[::3] = -c[::3]
+    oc = support.blocked_offsets(case.m1, case.n1, case.m0, case.n0, case.rsc0, case.csc0, case.rsc1, case.csc1)
+    spots = [(0, 0), (127, 63), (128, 64), (255, 255), (256 + 63, 191), (256 + 64, 192), (m - 1, n - 1), (m - 1, 0),
+             (0, n - 1), (m // 2 + 31, n // 2 + 33), (m - 129, n - 65), (700, 1500)]
+    spoiled = c.copy()
+    for idx, (i, j) in enumerate(spots):
+        spoiled[oc[i, j]] = (np.nan, np.inf, -np.inf)[idx % 3]
+    nan_want = np.zeros(c.size, dtype=bool)
+    nan_want[[oc[i, j] for i, j in spots]] = True
+    initialised = run_gemm(gpu, kind, case, a, b, c, "device")
+    assert np.all(np.isfinite(initialised))
+    gpu.skl_hip_set_beta_zero_mode(1)
+    try:
+        clean = run_gemm(gpu, kind, case, a, b, c, "device")
+        again = run_gemm(gpu, kind, case, a, b, spoiled, "device")
+    finally:
+        gpu.skl_hip_set_beta_zero_mode(0)
+    assert np.array_equal(clean.view(np.uint8), initialised.view(np.uint8)), (ta, layout)
+    assert np.array_equal(np.isnan(again), nan_want), (ta, layout, int(np.isnan(again).sum()))
+    assert np.array_equal(again[~nan_want].view(np.uint8), clean[~nan_want].view(np.uint8)), (ta, layout)
+    if layout != "panel":  # the zero rows hold zeros of both signs, following the old C
+        zeros = clean[oc[5, :]]
+        assert np.all(zeros == 0) and np.signbit(zeros).any() and not np.signbit(zeros).all()
+
+
 @pytest.mark.parametrize("ta,tb", (("f8e4m3", "f8e4m3"), ("f8e5m2", "f8e5m2"), ("f8e4m3", "f8e5m2")))
 @pytest.mark.parametrize("a_rowmajor", (True, False))
 def test_fp8_short_k_is_multiplied_exactly(gpu, ta, tb, a_rowmajor):
