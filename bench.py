@@ -590,6 +590,25 @@ def wl_f16_pipeline(lib, rng):
                 name="f16 pack->GEMM->unpack 4096x4096x14336 (TE=64 panels)", kernel="gemm_mfma_ring_kernel")
 
 
+def _beta_zero_as_reference(builder):
+    """The same workload with beta == 0 evaluated as the reference's loops do (0 * c + alpha * acc: a NaN or an
+    infinity in the old C stays a NaN, ref/gemm/gemm_bf16rc_bf16rc_f32rc.c:21) instead of the default, which
+    initialises C. The switch is per thread and set around every call."""
+    def build(lib, rng):
+        wl = builder(lib, rng)
+        inner = wl["fn"]
+
+        def step(i):
+            lib.skl_hip_set_beta_zero_mode(1)
+            inner(i)
+            lib.skl_hip_set_beta_zero_mode(0)
+
+        wl["fn"] = step
+        wl["name"] += ", beta == 0 as the reference evaluates it"
+        return wl
+    return build
+
+
 def wl_cvt(lib, rng):
     n = 8192 * 8192
     src = DeviceBuffer.from_array(rng.normal(size=n).astype(np.float32))
@@ -741,6 +760,9 @@ WORKLOADS = {
     "gemm_f8e4m3_f8e5m2_8192": (lambda lib, rng: wl_gemm_f8_8192(lib, rng, "f8e5m2"), 20, 2, 1),
     "gemm_f8e4m3_8192_rowmajor_a": (wl_gemm_f8_layout(True, False), 20, 2, 1),
     "gemm_f8e4m3_8192_kcontig": (wl_gemm_f8_layout(True, True), 20, 2, 1),
+    "gemm_f8e4m3_8192_kcontig_beta0_as_reference": (_beta_zero_as_reference(wl_gemm_f8_layout(True, True)), 20, 2, 1),
+    "gemm_f8e4m3_8192_beta0_as_reference": (_beta_zero_as_reference(wl_gemm_f8_8192), 20, 2, 1),
+    "pipeline_f16_4096x4096x14336_beta0_as_reference": (_beta_zero_as_reference(wl_f16_pipeline), 10, 2, 1),
     "gemm_i8_4000": (wl_gemm_i8_4000, 10, 2, 2),
     "gemm_bf16_2048x4096x4096": (wl_gemm_bf16, 20, 2, 4),
     "gemm_f32_4096": (wl_gemm_f32, 5, 1, 1),

@@ -89,8 +89,9 @@ int skl_hip_get_pointer_mode(void);
  *   for every finite C; an Inf or NaN in C - or whatever uninitialised memory holds - is overwritten.
  * SKL_HIP_BETA_ZERO_AS_REFERENCE: beta*C + alpha*A*B is evaluated as the reference's routines evaluate it
  *   (ref/gemm/gemm_bf16rc_bf16rc_f32rc.c:21): the old C is read and multiplied by zero, so an Inf or NaN in it
- *   makes the result NaN, exactly where the reference's result is NaN. Costs the read of C (8192^3 fp8: 256 MiB,
- *   about a quarter on top of the call).
+ *   makes the result NaN, exactly where the reference's result is NaN. Costs the read of C (8192^3 fp8: 256 MiB;
+ *   looked through under the product on the large tile kernels, about 8 % on top of the call; up to a fifth where
+ *   it is read in the epilogue).
  * Integer GEMMs give the same result either way and never read C when beta == 0; f64 GEMMs always read it. */
 #define SKL_HIP_BETA_ZERO_INITIALISES 0
 #define SKL_HIP_BETA_ZERO_AS_REFERENCE 1
