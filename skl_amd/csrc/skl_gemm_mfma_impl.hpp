@@ -1200,9 +1200,12 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
                             constexpr int Q = decltype(qc)::value, kSlot = KS * kMfmas + Q;
                             constexpr int i = Q / NI, j = Q % NI;
                             acc[i][j] = M::run(fa[i], fb[j], acc[i][j]);
-                            // SCAN: the MFMA first, what follows in its shadow - the waves have just left a barrier together, and
-                            // instructions in front of a slice's first MFMA are a gap in every SIMD's matrix core at once.
-                            if constexpr (SCAN && kSlot <= 1) __builtin_amdgcn_sched_barrier(0);
+                            // The MFMA first, what belongs to its slot in its shadow. Left to itself the compiler moves a slot's address
+                            // arithmetic, reads and loads in front of the MFMA - and behind a barrier, which the waves leave together,
+                            // instructions in front of the first MFMA are a gap in every SIMD's matrix core at once (measured, same job,
+                            // alternating libraries: int8 8192^3 -1.5 %, fp8 with column-major A -3 %, bf16 config 3 -2.3 %; for the
+                            // extra instructions of SCAN the difference between +43 and +14 us).
+                            __builtin_amdgcn_sched_barrier(0);
                             if constexpr (SCAN && U == 0 && kSlot == 0) scan_issue(s);
                             if constexpr (SCAN && kSlot == 1) scan_check();  // what the last slot of the k-step before has read, behind this k-step's lgkmcnt(0)
                             // Behind the barrier of slice 2q + 3 the rows requested in slice 2q have landed: half of them is
