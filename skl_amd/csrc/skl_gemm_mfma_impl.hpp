@@ -790,7 +790,9 @@ struct SLoader {
   unsigned lds[kBlocks];   // LDS byte offsets (inside the operand's region, stage 0) of the blocks
 
   __device__ void init(const char *base, size_t mn0, size_t s1, size_t s0, size_t sk) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // The wave index as a scalar: the LDS address of a block (which goes into M0) is then scalar arithmetic, not a
+    // vector add and a v_readfirstlane per load, and lds[] lives in scalar registers.
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     tile_base = base + (mn0 >> 6) * s1 * ES;
 #pragma unroll
     for (int i = 0; i < kBlocks; ++i) {
@@ -808,7 +810,10 @@ struct SLoader {
         lds[i] = b * 1024;
       }
     }
-    k_step = KC ? (size_t)(2 * kRingSlice) : (size_t)(kRingSlice / ES) * sk * ES;
+    // (spelled out as a scalar: as a member next to per-lane offsets it otherwise ends up in a vector register, and
+    // every load of an MN-contiguous operand pays a 64-bit vector multiply-add for its address)
+    const size_t step = KC ? (size_t)(2 * kRingSlice) : (size_t)(kRingSlice / ES) * sk * ES;
+    k_step = ((size_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(step >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)step);
   }
 
   // Requests block `i` of `unit`; it lands in stage `stage` (the even one of the pair for KC) of `region`.
@@ -1010,7 +1015,7 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
   using RB = FragReader<ES, B_KC, FRB, KB, BN, NSB, NI>;
   constexpr int PA = RA::kPieces, PB = RB::kPieces;
   constexpr int kReads = MI * PA + NI * PB;      // LDS instructions per k-step
-  constexpr int kReadSlots = kMfmas / 2;         // ... issued behind the first half of its MFMAs, the rest is time to land
+  constexpr int kReadSlots = kMfmas / 2;         // ... issued behind the first half of its MFMAs, the rest is time to land (all of them behind the first of four MFMAs on the narrow tile: 73.5-74.0 against 72.7-73.0 us)
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char *region_a = smem, *region_b = smem + TileA::kRegion;
@@ -1044,7 +1049,9 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 
   // K is a whole number of slice pairs. Units beyond the end are requested as the last unit
   // again: in range, and the stage they land in is never read, which keeps the load counts static.
-  const size_t slices = p.k * ES / SB, pairs = slices / 2;
+  // (32-bit counters - the host refuses a K of 2^31 slices or more: a 64-bit "less than" of two scalars is a vector
+  // compare and two vector registers)
+  const unsigned slices = (unsigned)(p.k * ES / SB), pairs = slices / 2;
 
   // SCAN: the tile's old C, 1 KiB per wave and two slices (the host has checked that K has the slices for it and
   // that C is row-major with 16-byte aligned rows).
@@ -1095,17 +1102,17 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 
   if constexpr (A_KC) {
 #pragma unroll
-    for (int i = 0; i < kPairsPrologue; ++i) la.issue(region_a, 2 * i, (size_t)i < pairs ? (size_t)i : pairs - 1);
+    for (int i = 0; i < kPairsPrologue; ++i) la.issue(region_a, 2 * i, (unsigned)i < pairs ? (unsigned)i : pairs - 1);
   } else {
 #pragma unroll
-    for (int i = 0; i < kEachAhead; ++i) la.issue(region_a, i, (size_t)i < slices ? (size_t)i : slices - 1);
+    for (int i = 0; i < kEachAhead; ++i) la.issue(region_a, i, (unsigned)i < slices ? (unsigned)i : slices - 1);
   }
   if constexpr (B_KC) {
 #pragma unroll
-    for (int i = 0; i < kPairsPrologue; ++i) lb.issue(region_b, 2 * i, (size_t)i < pairs ? (size_t)i : pairs - 1);
+    for (int i = 0; i < kPairsPrologue; ++i) lb.issue(region_b, 2 * i, (unsigned)i < pairs ? (unsigned)i : pairs - 1);
   } else {
 #pragma unroll
-    for (int i = 0; i < kEachAhead; ++i) lb.issue(region_b, i, (size_t)i < slices ? (size_t)i : slices - 1);
+    for (int i = 0; i < kEachAhead; ++i) lb.issue(region_b, i, (unsigned)i < slices ? (unsigned)i : slices - 1);
   }
   if constexpr (SCAN) {  // the slots start as zeros: the first slices read slots that no load has filled yet
 #pragma unroll
@@ -1158,16 +1165,16 @@ __global__ void __launch_bounds__(512) gemm_mfma_ring_kernel(MfmaArgs p) {
 
   // Two slices per trip: the parity of the slice decides which loads it issues, and (for the
   // operand kinds with one k-step per slice) which fragment buffer a k-step uses.
-  for (size_t s0 = 0; s0 < slices; s0 += 2) {
+  for (unsigned s0 = 0; s0 < slices; s0 += 2) {
     [&]<int... Us>(std::integer_sequence<int, Us...>) {
       (
           [&](auto uc) {
             constexpr int U = decltype(uc)::value;
             constexpr int kLoads = kLoadsOfU[U];
-            const size_t s = s0 + U;
-            const size_t fill_slice = s + kEachAhead < slices ? s + kEachAhead : slices - 1;  // every-slice operands
-            const size_t fill_pair = (s + kPairAhead) / 2 < pairs ? (s + kPairAhead) / 2 : pairs - 1;  // pair operands (s of parity kPairU)
-            const unsigned s32 = (unsigned)s;  // stage numbers from the low 32 bits: K / 64 fits, and a 32-bit remainder is a few scalar instructions
+            const unsigned s = s0 + U;
+            const unsigned fill_slice = s + kEachAhead < slices ? s + kEachAhead : slices - 1;  // every-slice operands
+            const unsigned fill_pair = (s + kPairAhead) / 2 < pairs ? (s + kPairAhead) / 2 : pairs - 1;  // pair operands (s of parity kPairU)
+            const unsigned s32 = s;
             const int cur_a = (int)(s32 % NSA), nxt_a = (int)((s32 + 1) % NSA), cur_b = (int)(s32 % NSB), nxt_b = (int)((s32 + 1) % NSB);
             const int fill_a = (int)((s32 + (A_KC ? kPairAhead : kEachAhead)) % NSA), fill_b = (int)((s32 + (B_KC ? kPairAhead : kEachAhead)) % NSB);
             [&]<int... KSs>(std::integer_sequence<int, KSs...>) {
@@ -1458,6 +1465,10 @@ int launch_ring(const MfmaArgs &args) {
   // Tiles for at most half of the 256 compute units: K is shared between two workgroups per tile (each at least
   // kRingMinSlicesPerSplit slices long) and a second pass adds the two planes and applies alpha / beta.
   const size_t slices = p.k * ES / kRingSlice;
+  if (slices >= (size_t(1) << 31)) {
+    skl_hip_record_error(-2, "gemm_mfma: K too long");
+    return -2;
+  }
   p.splits = (tiles <= 128 && slices % 4 == 0 && slices / 2 >= kRingMinSlicesPerSplit) ? 2 : 1;
   SequenceGuard sequence(p.splits > 1);
   if (p.splits > 1) {
