@@ -819,7 +819,12 @@ struct SLoader {
   // Requests block `i` of `unit`; it lands in stage `stage` (the even one of the pair for KC) of `region`.
   __device__ __forceinline__ void issue_one(char *region, int stage, size_t unit, int i) const {
     const char *g = tile_base + unit * k_step;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(g + off[i]),
+    // The lane's offset through a copy the compiler cannot follow: it otherwise widens every offset to 64 bits ahead
+    // of the loop (two registers each) and adds the scalar base with a 64-bit vector add per load; this way the load
+    // takes the scalar base and the 32-bit offset as they are.
+    unsigned o = off[i];
+    asm volatile("" : "+v"(o));
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(g + o),
                                      (__attribute__((address_space(3))) void *)(region + stage * T::kStageStep + lds[i]),
                                      16, 0, 0);
   }
