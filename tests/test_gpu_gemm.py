@@ -259,6 +259,7 @@ SCANNED_C_SHAPES = (
     ("f8e4m3", "row", 4096, 4096, 4096 + 128, "256 x 256 tiles, two slices more"),
     ("f8e4m3", "row", 4096, 4096, 8192, "256 x 256 tiles, twice the slices: the last rows are requested again"),
     ("bf16", "row", 1024, 3072, 1024, "256 x 128 tiles, exactly the slices it takes (32)"),
+    ("f8e4m3", "row", 1024, 16640, 4096, "260 tiles: 256-column tiles and, for the last 256 columns, 128-column ones (two launches)"),
     ("bf16", "row", 1024, 3072, 2048 + 64, "256 x 128 tiles"),
     ("f16", "column", 4096, 4096, 4096, "column-major C"),
     ("bf16", "panel", 4096, 4096, 4096, "C in 64 x 64 panels, 256 x 256 tiles"),
