@@ -485,7 +485,7 @@ def wl_reference_bench_dot4(lib, rng):
         lib.skl_gemm_i8rcp1x4_i8p4x1c_i32_gfx950(m, n, k1, 1, a, 4 * k1, 4, b, 4 * n, 0, c, n)
 
     return dict(fn=step, bytes=m * 4 * k1 + 4 * k1 * n + 4 * m * n, ops=2 * m * n * 4 * k1, bound="mfma", dtype="i8", keep=(a, b, c),
-                name="int8 dot4 GEMM 126x128, k1=64 (K-packed B; the reference's own benchmark row)", kernel="gemv_k4_rowgroups_kernel")
+                name="int8 dot4 GEMM 126x128, k1=64 (K-packed B; the reference's own benchmark row)", kernel="gemv_k4_wholek_kernel<1> on a grid of column tiles x groups of 16 rows")
 
 
 def wl_gemm_i8_512(lib, rng):

@@ -512,7 +512,9 @@ static int k4_in_row_chunks(const skl_gemm_desc *d) {
         if (!canonicalize_k4(&part, &g, 1) || !skl_hip_gemv_mfma_rows_supported(&g, 1)) return DECLINED;
         if (launch) rc = skl_hip_launch_gemv_mfma_rows(&g, 1);
       }
-      if (rc != 0) return FAILED; /* a launch error of the device: recorded, C is not to be relied on */
+      /* A first chunk that could not get scratch memory has launched nothing: the call goes on to the next kernel.
+       * Any other error, or a later chunk's: recorded, C is not to be relied on. */
+      if (rc != 0) return i == 0 ? outcome(rc) : FAILED;
     }
   }
   return TAKEN;

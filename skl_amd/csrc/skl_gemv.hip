@@ -1079,6 +1079,11 @@ __global__ void __launch_bounds__(kK4WholeWaves * 64) gemv_k4_wholek_kernel(Gemv
   typedef int v4i __attribute__((ext_vector_type(4)));
   extern __shared__ __attribute__((aligned(16))) int mfma_red_raw[];
   const unsigned tile = blockIdx.x;
+  // A second grid dimension deals the groups of RG * 16 rows out to workgroups of their own (problems with so few
+  // column tiles that the chip is empty otherwise: B is small then, and read once per workgroup).
+  const size_t row0 = (size_t)blockIdx.y * (RG * 16), m = p.m - row0;
+  const char *const a = p.a + row0 * p.a_row;
+  int *const c = p.c + row0 * p.c_row;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int jl = lane & 15, g = lane >> 4;
   const size_t col = (size_t)tile * 64 + (size_t)jl * 4;
@@ -1090,8 +1095,8 @@ __global__ void __launch_bounds__(kK4WholeWaves * 64) gemv_k4_wholek_kernel(Gemv
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const size_t k0 = kwave + (size_t)it * 64 + (size_t)g * 16;
-      const bool inside = row < p.m && k0 < p.k;  // k is a multiple of 16
-      const v4i v = *reinterpret_cast<const v4i *>(p.a + (row < p.m ? row : p.m - 1) * p.a_row + (k0 < p.k ? k0 : p.k - 16));
+      const bool inside = row < m && k0 < p.k;  // k is a multiple of 16
+      const v4i v = *reinterpret_cast<const v4i *>(a + (row < m ? row : m - 1) * p.a_row + (k0 < p.k ? k0 : p.k - 16));
       xa[it] = v4i{inside ? v.x : 0, inside ? v.y : 0, inside ? v.z : 0, inside ? v.w : 0};
     }
   };
@@ -1120,7 +1125,7 @@ __global__ void __launch_bounds__(kK4WholeWaves * 64) gemv_k4_wholek_kernel(Gemv
   const size_t j = (size_t)tile * 64 + tc;
 #pragma unroll
   for (int rg = 0; rg < RG; ++rg) {
-    if ((size_t)rg * 16 >= p.m) break;  // the same for every thread of the workgroup
+    if ((size_t)rg * 16 >= m) break;  // the same for every thread of the workgroup
     v4i acc[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) acc[c] = v4i{0, 0, 0, 0};
@@ -1158,7 +1163,7 @@ __global__ void __launch_bounds__(kK4WholeWaves * 64) gemv_k4_wholek_kernel(Gemv
         unsigned sum = 0;
 #pragma unroll
         for (int w = 0; w < W; ++w) sum += (unsigned)red[w][il][tc];
-        if (i < p.m && j < p.n) skl_update((int)sum, p.c + i * p.c_row + j * p.c_s, p.alpha, p.beta);
+        if (i < m && j < p.n) skl_update((int)sum, c + i * p.c_row + j * p.c_s, p.alpha, p.beta);
       }
     }
   }
@@ -1168,7 +1173,7 @@ __global__ void __launch_bounds__(kK4WholeWaves * 64) gemv_k4_wholek_kernel(Gemv
 #pragma unroll
     for (int q = 0; q < RG * 16 / W; ++q) {
       const size_t i = (size_t)(threadIdx.x >> 6) + (size_t)q * W;
-      if (i < p.m) skl_update(plane[i][tc], p.c + i * p.c_row + j * p.c_s, p.alpha, p.beta);
+      if (i < m) skl_update(plane[i][tc], c + i * p.c_row + j * p.c_s, p.alpha, p.beta);
     }
   }
 }
@@ -1591,7 +1596,11 @@ extern "C" int skl_hip_gemv_mfma_rows_supported(const skl_gemm_canon *g, int lay
     // B(4P + p, j) at P * b_sk + 4 j + p; 2 to 128 rows (no other kernel reads this layout with more than one row)
     if (g->c_row_shift != 6 || g->c_col_shift != 6 || g->bias || g->max || g->rq.act || g->rq.q) return 0;
     if (g->m < 2 || g->m > (size_t)(16 * kK4MaxRowGroups) || g->k == 0 || g->n == 0) return 0;
-    if ((g->k % 16) != 0 || (g->n % 4) != 0 || g->k * g->n < (size_t(1) << 20)) return 0;
+    if ((g->k % 16) != 0 || (g->n % 4) != 0) return 0;
+    // A small B (under 1 MiB) only where the whole-K kernel runs a workgroup per column tile and group of 16 rows:
+    // elsewhere the tile kernels are faster on it.
+    const bool side_by_side = g->k <= kK4WholeMaxK && skl_div_up(g->n, (size_t)64) * ((g->m + 15) / 16) <= 256;
+    if (g->k * g->n < (size_t(1) << 20) && !side_by_side) return 0;
     if (g->a_sk != 1 || !aligned16(g->a) || (g->a_s0 % 16) != 0) return 0;
     if (!aligned16(g->b) || (g->b_sk % 16) != 0) return 0;
     return g->csc1 == 64 * g->csc0;
@@ -1664,7 +1673,14 @@ int launch_mfma_rows(const GemvMfmaArgs &args) {
         }
         whole_configured.store(true, std::memory_order_release);
       }
-      switch ((p.m + 15) / 16) {
+      const unsigned row_groups = (unsigned)((p.m + 15) / 16);
+      if (row_groups > 1 && (size_t)tiles * row_groups <= 256) {
+        // So few column tiles that all row groups side by side still leave compute units free: a workgroup per
+        // column tile and group of 16 rows (B is small then; each workgroup reads its 64 columns of it).
+        gemv_k4_wholek_kernel<1><<<dim3(tiles, row_groups), threads, k4_whole_lds(1), st>>>(p);
+        return skl_check_launch("gemv_k4_wholek");
+      }
+      switch (row_groups) {
         case 1: gemv_k4_wholek_kernel<1><<<tiles, threads, k4_whole_lds(1), st>>>(p); break;
         case 2: gemv_k4_wholek_kernel<2><<<tiles, threads, k4_whole_lds(2), st>>>(p); break;
         case 3: gemv_k4_wholek_kernel<3><<<tiles, threads, k4_whole_lds(3), st>>>(p); break;

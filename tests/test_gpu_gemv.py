@@ -116,10 +116,13 @@ def test_k_packed_int8_decode_batches(gpu, m):
     four columns, no transposes; B stays in registers for up to eight groups of 16 rows (ragged last group: 17, 33,
     100), more rows go through in chunks of 128 (a last chunk of one row through the one-row kernel: 129, 257).
     K <= 4096: one workgroup per 64 columns takes all of K and writes C once; beyond (one shape here) workgroups
-    share a column tile and meet in C. The config-2 weights prepacked, N and K off the kernel's 1024 x 64
+    share a column tile and meet in C. Problems with few column tiles (the reference's own benchmark shape, 126 x 128
+    with k1 = 64, test/gemm/xsfvqdotq/skl_gemm_i8rcp1x4_i8p4x1c_i32_xsfvqdotq.c:56) run a workgroup per tile and group of
+    16 rows. The config-2 weights prepacked, N and K off the kernel's 1024 x 64
     blocks, padded strides of A, B and C, alpha / beta with wrap-around, both pointer modes; whole-buffer compare."""
     rng = np.random.default_rng(600 + m)
-    shapes = [(11008, 1024, 0, 0, 0), (4100, 132, 16, 32, 5), (2052, 516, 48, 16, 0)]
+    shapes = [(11008, 1024, 0, 0, 0), (4100, 132, 16, 32, 5), (2052, 516, 48, 16, 0),
+              (128, 64, 0, 0, 0), (132, 68, 16, 16, 3)]  # few column tiles: a workgroup per tile and group of 16 rows
     if m in (7, 100):
         shapes.append((1028, 1284, 16, 0, 3))  # K = 5136 > 4096: the sums of a column tile meet in C, not in LDS
     for (n, k1, pad_a, pad_b, pad_c) in shapes:
