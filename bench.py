@@ -807,12 +807,12 @@ TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in pro
 MEASURED_TRAFFIC_BYTES = {
     "gemv_i8": int((22060.5 * 1.998 + 817.0) * 1024),
     "cvt_f32_f8e4m3_8192sq": int((131136.6 * 1.998 + 65536.0) * 1024),
-    "gemm_i8_8192": int((393325.2 * 1.998 + 262463.2) * 1024),
-    "gemm_f8e4m3_8192_kcontig": int((393343.5 * 1.998 + 262758.9) * 1024),
+    "gemm_i8_8192": int((393337.8 * 1.998 + 262443.1) * 1024),
+    "gemm_f8e4m3_8192_kcontig": int((393391.2 * 1.998 + 262875.0) * 1024),
     "copy_u32_4096sq": int((32800.9 * 1.998 + 65536) * 1024),
     "gemm_i8_16x4096x11008": int((22349.1 * 1.998 + 6192.0) * 1024),
     "gemv_f8e4m3_f4_1x4096x11008": int((11060.0 * 1.998 + 43.0) * 1024),
-    "gemm_i8_p4x1c_112x4096x11008": int((23911.2 * 1.998 + 4816.0) * 1024),
+    "gemm_i8_p4x1c_112x4096x11008": int((23911.7 * 1.998 + 4816.0) * 1024),
 }
 
 
