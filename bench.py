@@ -4,8 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--full] [--no-cpu] [--out FILE]
     python bench.py --vendor-only      (the vendor BLAS through torch on three of the products, for comparison)
 
-Prints ONE compact JSON line (a few KB) and writes the full record of everything it measured to
-gpurun_out/bench_full.json (`--out`); `--full` also runs the workloads that are not benchmark configurations. The headline (`value`) is the int8 GEMV decode shape
+Prints ONE compact JSON line (a few KB) and writes the full record of everything it measured to the file that
+`--out` names; `--full` also runs the workloads that are not benchmark configurations. The headline (`value`) is the int8 GEMV decode shape
 (1x4096 times 4096x11008, benchmark configuration 2) in GB/s of algorithmic bytes with
 all operands resident in HBM. A "step" is `config.calls_per_step` GEMV calls back to back,
 each on the next of eight weight matrices (their total size exceeds the 256 MiB last-level
