@@ -92,7 +92,9 @@ int skl_hip_get_pointer_mode(void);
  *   makes the result NaN, exactly where the reference's result is NaN. Costs the read of C (8192^3 fp8: 256 MiB;
  *   looked through under the product on the large tile kernels, about 8 % on top of the call; up to a fifth where
  *   it is read in the epilogue).
- * Integer GEMMs give the same result either way and never read C when beta == 0; f64 GEMMs always read it. */
+ * Integer GEMMs give the same result either way and never read C when beta == 0; f64 GEMMs always read it.
+ * A thread that has not called the setter takes the process's default: SKL_HIP_BETA_ZERO_INITIALISES, or, with
+ * SKL_HIP_BETA_ZERO=reference in the environment when the library is first asked, SKL_HIP_BETA_ZERO_AS_REFERENCE. */
 #define SKL_HIP_BETA_ZERO_INITIALISES 0
 #define SKL_HIP_BETA_ZERO_AS_REFERENCE 1
 void skl_hip_set_beta_zero_mode(int mode);

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -52,7 +53,7 @@ DeviceState g_devices[kMaxDevices];
 
 thread_local hipStream_t t_stream = nullptr;
 thread_local int t_pointer_mode = SKL_HIP_POINTERS_AUTO;
-thread_local int t_beta_zero_mode = SKL_HIP_BETA_ZERO_INITIALISES;
+thread_local int t_beta_zero_mode = -1;  // not set by this thread: the process's default (the environment) counts
 thread_local int t_error = SKL_HIP_OK;
 thread_local char t_error_text[256] = "no error";
 
@@ -301,7 +302,15 @@ int skl_hip_get_pointer_mode(void) { return t_pointer_mode; }
 void skl_hip_set_beta_zero_mode(int mode) {
   t_beta_zero_mode = (mode == SKL_HIP_BETA_ZERO_AS_REFERENCE) ? SKL_HIP_BETA_ZERO_AS_REFERENCE : SKL_HIP_BETA_ZERO_INITIALISES;
 }
-int skl_hip_get_beta_zero_mode(void) { return t_beta_zero_mode; }
+int skl_hip_get_beta_zero_mode(void) {
+  // A thread that has not chosen takes the process's default: SKL_HIP_BETA_ZERO=reference in the environment makes
+  // the reference's evaluation the default for callers that cannot be changed to call the setter.
+  static const int process_default = [] {
+    const char *e = std::getenv("SKL_HIP_BETA_ZERO");
+    return (e && std::strcmp(e, "reference") == 0) ? SKL_HIP_BETA_ZERO_AS_REFERENCE : SKL_HIP_BETA_ZERO_INITIALISES;
+  }();
+  return t_beta_zero_mode < 0 ? process_default : t_beta_zero_mode;
+}
 
 int skl_hip_pointer_is_device(const void *ptr) {
   if (t_pointer_mode == SKL_HIP_POINTERS_DEVICE) return 1;

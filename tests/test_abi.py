@@ -42,6 +42,24 @@ def test_tile_edge_and_error_channel_without_gpu():
     assert lib.skl_hip_get_pointer_mode() == 0
 
 
+def test_beta_zero_default_follows_the_environment():
+    """A thread that has not called skl_hip_set_beta_zero_mode takes the process's default: the initialising evaluation,
+    or the reference's (ref/gemm/gemm_bf16rc_bf16rc_f32rc.c:21 evaluates 0 * c) with SKL_HIP_BETA_ZERO=reference in the
+    environment; the setter overrides either for its thread. No GPU needed: each case in a process of its own."""
+    import subprocess
+    import sys
+    code = ("import skl_amd; lib = skl_amd.load(); first = lib.skl_hip_get_beta_zero_mode(); "
+            "lib.skl_hip_set_beta_zero_mode(1 - first); print(first, lib.skl_hip_get_beta_zero_mode())")
+    for env_value, want in ((None, "0 1"), ("reference", "1 0"), ("something else", "0 1")):
+        env = dict(os.environ)
+        env.pop("SKL_HIP_BETA_ZERO", None)
+        if env_value is not None:
+            env["SKL_HIP_BETA_ZERO"] = env_value
+        out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        assert out.stdout.strip().splitlines()[-1] == want, (env_value, out.stdout)
+
+
 def test_missing_library_fails_loudly(tmp_path):
     from skl_amd import binding
     try:
